@@ -1,0 +1,410 @@
+#!/usr/bin/env python3
+"""Benchmark of the packed-kernel hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload ce|rmsnorm|add_rmsnorm|kl|topk|route]
+                    [--no-extras] [--no-cpu]
+
+A step is one pass of the hot path (forward + backward) over one batch of synthetic,
+seeded input that is already resident in HBM, launched straight through the C ABI of
+libfmhip.so with pre-allocated outputs (no allocator, no autograd in the timed region).
+The headline workload is the fused cross entropy of the reference's loss path at
+logits bf16 [8192, 32000]; `value` is algorithmic bytes per step / time per step.
+
+Prints ONE JSON line. Besides the headline it carries
+  roofline      the dominant kernel of the headline workload against the 8 TB/s HBM peak,
+                timed with HIP events around that kernel's launches;
+  cpu_baseline  the CPU oracle (the reference's torch expression) on a bounded row sample,
+                on the host's cores -- a reported baseline, never a target;
+  workloads     the same measurement for the other shapes of the hot path.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E, published
+METRIC = "HBM GB/s & % roofline: RMSNorm, CE/KL fwd+bwd; MoE top-k rows/s"
+
+# HBM bytes per launch of the dominant kernels, from `rocprofv3 --pmc FETCH_SIZE` and
+# `--pmc WRITE_SIZE` runs of this file (summaries under profiles/), each scaled by what the
+# same counter reads for a copy of known size; None until measured.
+MEASURED_TRAFFIC_BYTES = {
+    "ce": None,
+}
+
+
+def parse():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawTextHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="ce",
+                    choices=["ce", "rmsnorm", "add_rmsnorm", "kl", "topk", "route"])
+    ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
+                    help="only run a plain device copy of this many MiB (counter calibration)")
+    return ap.parse_args()
+
+
+# ---------------------------------------------------------------------------- workloads
+class Workload:
+    """Pre-allocated tensors plus closures that enqueue the launches of one step."""
+
+    name = ""
+    desc = ""
+    unit = "GB/s"
+    dominant = ""          # kernel the roofline object is about
+
+    def step(self):        # forward + backward of the hot path
+        raise NotImplementedError
+
+    def dominant_launch(self):
+        raise NotImplementedError
+
+
+def _check(rc, what):
+    if rc != 0:
+        from forgeminds_amd.kernels import _hip
+        raise RuntimeError(f"{what}: status {rc}: {_hip.lib().fm_last_error().decode()}")
+
+
+def make_workload(name, torch, L, dev):
+    from forgeminds_amd.kernels import _hip
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator(device=dev)
+    BF, F32c = _hip.BF16, _hip.F32
+    w = Workload()
+    w.name = name
+
+    if name == "rmsnorm":
+        n, d = 8192, 1024
+        g.manual_seed(1001)
+        sets = 8     # rotate through > 256 MB so the Infinity Cache cannot serve a step
+        xs = [torch.randn(n, d, device=dev, generator=g).bfloat16() for _ in range(sets)]
+        dys = [torch.randn(n, d, device=dev, generator=g).bfloat16() for _ in range(sets)]
+        ys = [torch.empty_like(xs[0]) for _ in range(sets)]
+        dxs = [torch.empty_like(xs[0]) for _ in range(sets)]
+        wt = (1 + 0.02 * torch.randn(d, device=dev, generator=g))
+        rstd = torch.empty(n, device=dev)
+        dw = torch.empty_like(wt)
+        nb = L.fm_rmsnorm_bwd_workspace(n, d, BF)
+        ws = torch.empty(nb, device=dev, dtype=torch.uint8)
+        state = {"i": 0}
+
+        def fwd(i):
+            _check(L.fm_rmsnorm_fwd(xs[i].data_ptr(), wt.data_ptr(), ys[i].data_ptr(), rstd.data_ptr(),
+                                    n, d, BF, F32c, 1e-6, st), "fm_rmsnorm_fwd")
+
+        def bwd(i):
+            _check(L.fm_rmsnorm_bwd(xs[i].data_ptr(), wt.data_ptr(), rstd.data_ptr(), dys[i].data_ptr(),
+                                    dxs[i].data_ptr(), dw.data_ptr(), ws.data_ptr(), nb, n, d, BF, F32c,
+                                    st), "fm_rmsnorm_bwd")
+
+        def step():
+            i = state["i"] = (state["i"] + 1) % sets
+            fwd(i)
+            bwd(i)
+
+        def warm_step():
+            fwd(0)
+            bwd(0)
+
+        w.step, w.warm_step = step, warm_step
+        w.dominant_launch = lambda: bwd(state["i"])
+        w.dominant = "norm_bwd_kernel<bf16,f32,64,2> + colsum"
+        w.dominant_bytes = n * d * 6
+        w.bytes = n * d * 10
+        w.desc = f"RMSNorm fwd+bwd x bf16 [{n},{d}], w fp32, eps 1e-6 (rotating {sets} buffer sets)"
+        w.rows = n
+        return w
+
+    if name == "add_rmsnorm":
+        n, d = 16384, 8192
+        g.manual_seed(1004)
+        x = torch.randn(n, d, device=dev, generator=g).bfloat16()
+        dl = torch.randn(n, d, device=dev, generator=g).bfloat16()
+        gy = torch.randn(n, d, device=dev, generator=g).bfloat16()
+        gxn = torch.randn(n, d, device=dev, generator=g).bfloat16()
+        wt = (1 + 0.02 * torch.randn(d, device=dev, generator=g))
+        xn, y, dx = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+        rstd = torch.empty(n, device=dev)
+        dw = torch.empty_like(wt)
+        nb = L.fm_rmsnorm_bwd_workspace(n, d, BF)
+        ws = torch.empty(nb, device=dev, dtype=torch.uint8)
+
+        def fwd():
+            _check(L.fm_add_rmsnorm_fwd(x.data_ptr(), dl.data_ptr(), wt.data_ptr(), xn.data_ptr(),
+                                        y.data_ptr(), rstd.data_ptr(), n, d, BF, F32c, 1e-5, st),
+                   "fm_add_rmsnorm_fwd")
+
+        def bwd():
+            _check(L.fm_add_rmsnorm_bwd(xn.data_ptr(), wt.data_ptr(), rstd.data_ptr(), gy.data_ptr(),
+                                        gxn.data_ptr(), dx.data_ptr(), None, dw.data_ptr(), ws.data_ptr(),
+                                        nb, n, d, BF, F32c, st), "fm_add_rmsnorm_bwd")
+
+        def step():
+            fwd()
+            bwd()
+
+        w.step = step
+        w.dominant_launch = bwd
+        w.dominant = "norm_bwd_kernel<bf16,f32,512,2> + colsum"
+        w.dominant_bytes = n * d * 8
+        w.bytes = n * d * 16
+        w.desc = f"add-RMSNorm fwd+bwd x,delta bf16 [{n},{d}], w fp32, eps 1e-5, with residual grad"
+        w.rows = n
+        return w
+
+    if name == "ce":
+        n, v = 8192, 32000
+        g.manual_seed(1002)
+        lg = (2 * torch.randn(n, v, device=dev, generator=g)).bfloat16()
+        y = torch.randint(0, v, (n,), device=dev, generator=g)
+        y[torch.rand(n, device=dev, generator=g) < 0.05] = -100
+        lse, rl = torch.empty(n, device=dev), torch.empty(n, device=dev)
+        sc = torch.empty(2, device=dev)
+        dlg = torch.empty_like(lg)
+
+        def fwd():
+            _check(L.fm_ce_fwd(lg.data_ptr(), y.data_ptr(), lse.data_ptr(), rl.data_ptr(), sc.data_ptr(),
+                               sc.data_ptr() + 4, n, v, BF, -100, 2, st), "fm_ce_fwd")
+
+        def bwd():
+            _check(L.fm_ce_bwd(lg.data_ptr(), y.data_ptr(), lse.data_ptr(), sc.data_ptr() + 4, None,
+                               dlg.data_ptr(), n, v, BF, -100, st), "fm_ce_bwd")
+
+        def step():
+            fwd()
+            bwd()
+
+        w.step = step
+        w.dominant_launch = bwd
+        w.dominant = "ce_bwd_kernel<bf16,512,4>"
+        w.dominant_bytes = n * v * 4
+        w.bytes = n * v * 6
+        w.desc = (f"fused CE fwd+bwd logits bf16 [{n},{v}], 5% ignore_index, mean; "
+                  "dataflow fwd(read) + bwd(read, write) = 6 B/logit")
+        w.rows = n
+        w.tensors = (lg, y)
+        return w
+
+    if name in ("kl", "topk"):
+        n, v = 4096, 128256
+        g.manual_seed(1005)
+        s = (3 * torch.randn(n, v, device=dev, generator=g)).bfloat16()
+        t = (s.float() + 0.5 * torch.randn(n, v, device=dev, generator=g)).bfloat16()
+        if name == "topk":
+            del s
+            idx = torch.empty(n, 64, device=dev, dtype=torch.int32)
+
+            def step():
+                _check(L.fm_topk(t.data_ptr(), None, idx.data_ptr(), n, v, 64, BF, 32, st), "fm_topk")
+
+            w.step = step
+            w.dominant_launch = step
+            w.dominant = "topk_kernel<bf16,1024,16>"
+            w.dominant_bytes = w.bytes = n * v * 2
+            w.desc = f"top-64 of teacher logits bf16 [{n},{v}], int32 indices (separate launch)"
+            w.rows = n
+            return w
+        b3 = torch.empty(3, n, device=dev)
+        ls = torch.empty((), device=dev)
+        gs = torch.empty_like(s)
+
+        def fwd():
+            _check(L.fm_kl_fwd(s.data_ptr(), t.data_ptr(), b3[0].data_ptr(), b3[1].data_ptr(),
+                               b3[2].data_ptr(), ls.data_ptr(), n, v, BF, 0.5, 2, st), "fm_kl_fwd")
+
+        def bwd():
+            _check(L.fm_kl_bwd(s.data_ptr(), t.data_ptr(), b3[0].data_ptr(), b3[1].data_ptr(), None, 0,
+                               gs.data_ptr(), n, v, BF, BF, 0.5, 1.0 / n, st), "fm_kl_bwd")
+
+        def step():
+            fwd()
+            bwd()
+
+        w.step = step
+        w.dominant_launch = bwd
+        w.dominant = "kl_bwd_kernel<bf16,bf16,1024,2>"
+        w.dominant_bytes = n * v * 6
+        w.bytes = n * v * 10
+        w.desc = f"KL(teacher||student) fwd+bwd bf16 [{n},{v}], T=2, mean"
+        w.rows = n
+        return w
+
+    if name == "route":
+        n, e, k = 16384, 64, 2
+        g.manual_seed(1003)
+        lg = torch.round(torch.randn(n, e, device=dev, generator=g) * 4096) / 4096
+        idx = torch.empty(n, k, device=dev, dtype=torch.int32)
+        wt = torch.empty(n, k, device=dev)
+        cnt = torch.empty(e, device=dev, dtype=torch.int32)
+        sl = torch.empty(n * k, device=dev, dtype=torch.int32)
+        od = torch.empty(n * k, device=dev, dtype=torch.int32)
+        nb = L.fm_route_workspace(n, e, k)
+        ws = torch.empty(max(nb, 16), device=dev, dtype=torch.uint8)
+
+        def step():
+            _check(L.fm_route(lg.data_ptr(), idx.data_ptr(), wt.data_ptr(), cnt.data_ptr(), sl.data_ptr(),
+                              od.data_ptr(), ws.data_ptr(), nb, n, e, k, F32c, st), "fm_route")
+
+        w.step = step
+        w.dominant_launch = step
+        w.dominant = "route_kernel + permute_kernel"
+        w.dominant_bytes = w.bytes = n * (e * 4 + k * 4 * 4)
+        w.desc = f"router softmax + top-{k} + counts + stable permutation, logits fp32 [{n},{e}]"
+        w.unit = "rows/s"
+        w.rows = n
+        return w
+
+    raise ValueError(name)
+
+
+def time_steps(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps     # ms per step
+
+
+def time_kernel_events(torch, fn, steps):
+    """Average duration of the launches `fn` enqueues, HIP events on the launch stream."""
+    pairs = []
+    for _ in range(steps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        pairs.append((a, b))
+    torch.cuda.synchronize()
+    times = sorted(a.elapsed_time(b) for a, b in pairs)
+    return sum(times) / len(times), times[0], times[len(times) // 2]
+
+
+def measure(torch, w, steps, warmup):
+    ms = time_steps(torch, w.step, steps, warmup)
+    avg, best, med = time_kernel_events(torch, w.dominant_launch, steps)
+    out = {
+        "desc": w.desc,
+        "ms_per_step": round(ms, 5),
+        "algorithmic_bytes": w.bytes,
+        "gbps": round(w.bytes / ms / 1e6, 1),
+        "frac_of_hbm_peak": round(w.bytes / ms / 1e6 / HBM_PEAK_GBPS, 4),
+        "rows_per_s": round(w.rows / ms * 1e3, 1),
+        "dominant_kernel": w.dominant,
+        "dominant_ms_avg": round(avg, 5), "dominant_ms_min": round(best, 5),
+        "dominant_gbps": round(w.dominant_bytes / avg / 1e6, 1),
+    }
+    if hasattr(w, "warm_step"):      # same buffers every step: served by the Infinity Cache
+        wm = time_steps(torch, w.warm_step, steps, warmup)
+        out["warm_cache_ms_per_step"] = round(wm, 5)
+        out["warm_cache_gbps"] = round(w.bytes / wm / 1e6, 1)
+    return out
+
+
+# ---------------------------------------------------------------------------- CPU baseline
+def cpu_baseline(torch):
+    """The CPU oracle's CE forward + backward on a bounded sample of the headline workload."""
+    from oracle import oracle as O
+    rows, v = 1024, 32000
+    g = torch.Generator(device="cpu").manual_seed(1002)
+    lg = (2 * torch.randn(rows, v, generator=g)).bfloat16()
+    y = torch.randint(0, v, (rows,), generator=g)
+    y[torch.rand(rows, generator=g) < 0.05] = -100
+    cores = torch.get_num_threads()
+    O.cross_entropy(lg, y)                       # warm-up
+    best = float("inf")
+    t_all = time.perf_counter()
+    for _ in range(3):
+        t0 = time.perf_counter()
+        O.cross_entropy(lg, y)
+        best = min(best, time.perf_counter() - t0)
+        if time.perf_counter() - t_all > 25:
+            break
+    return {
+        "value": round(rows * v * 6 / best / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+        "sample": f"oracle.cross_entropy fwd+bwd on {rows} of 8192 rows x {v} bf16 logits, "
+                  f"min of 3, {best * 1e3:.1f} ms, same 6 B/logit accounting",
+    }
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print(f"bench.py: this path is measured on ONE MI355X (no sharding, no collectives); "
+              f"--gpus {a.gpus} is not a supported configuration", file=sys.stderr)
+        return 2
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    from forgeminds_amd.kernels import _hip
+    L = _hip.lib()          # raises if libfmhip.so is not built: never a silent fallback
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    if a.copy_probe:
+        n = a.copy_probe << 20
+        src = torch.empty(n, device=dev, dtype=torch.uint8).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(max(a.steps, 1)):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_probe_bytes_read": n, "copy_probe_bytes_written": n, "launches": max(a.steps, 1)}))
+        return 0
+
+    head = make_workload(a.workload, torch, L, dev)
+    res = measure(torch, head, a.steps, a.warmup)
+    avg_ms = res["dominant_ms_avg"]
+    achieved = head.dominant_bytes / avg_ms / 1e6
+    line = {
+        "metric": METRIC,
+        "value": res["rows_per_s"] if head.unit == "rows/s" else res["gbps"],
+        "unit": head.unit,
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": res["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if a.workload != "route" else "f32", "data": "synthetic",
+        "config": {"workload": head.desc, "name": a.workload,
+                   "timing": "K steps between two device synchronisations, inputs resident in HBM"},
+        "roofline": {
+            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload),
+            "kernel": head.dominant, "algorithmic_bytes_per_launch": head.dominant_bytes,
+            "avg_launch_ms": avg_ms,
+        },
+        "frac_of_hbm_peak": res["frac_of_hbm_peak"],
+    }
+    del head
+    torch.cuda.empty_cache()
+    if not a.no_extras:
+        extras = {a.workload: res}
+        for name in ["rmsnorm", "add_rmsnorm", "ce", "kl", "topk", "route"]:
+            if name == a.workload:
+                continue
+            wl = make_workload(name, torch, L, dev)
+            extras[name] = measure(torch, wl, a.steps, a.warmup)
+            del wl
+            torch.cuda.empty_cache()
+        line["workloads"] = extras
+    line["cpu_baseline"] = None if a.no_cpu else cpu_baseline(torch)
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

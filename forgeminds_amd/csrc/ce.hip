@@ -1,0 +1,264 @@
+// Vocabulary-wide cross entropy, forward and backward, for gfx950.
+//
+// Reference semantics: forgemind/loss.py:54-70 (sum of per-row CE over the valid rows,
+// divided by max(1, n_valid); ignored rows contribute nothing and get a zero gradient).
+//
+// Forward: one workgroup per row, one read of the row. Each thread runs an online
+// (max, sum-exp) over its share of the row in the base-2 domain, the workgroup merges
+// the pairs, and lse[row] is saved. Backward: the softmax is recomputed from lse instead of
+// being stored, so the whole fwd+bwd moves 2 + 2 + 2 bytes per bf16 logit.
+#include "fm_vocab.cuh"
+
+using namespace fm;
+
+namespace {
+
+template <typename T, int THREADS, int UNROLL>
+__global__ __launch_bounds__(THREADS) void ce_fwd_kernel(const T* __restrict__ logits,
+                                                          const int64_t* __restrict__ labels,
+                                                          float* __restrict__ lse,
+                                                          float* __restrict__ row_loss, int v,
+                                                          int64_t ignore_index, bool vec_ok) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int NW = THREADS / 64;
+  __shared__ float smem[2 * NW];
+  const int64_t row = blockIdx.x;
+  const T* rp = logits + row * (int64_t)v;
+  const RowSplit sp = split_row<EPV>(row, v, vec_ok);
+  const int tid = threadIdx.x;
+
+  MaxSum st{kNegBig, 0.f};
+  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+    u32x4 raw[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
+    }
+    float z[UNROLL][EPV];
+    float cm = st.m;
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) {
+        Elem<T>::unpack(raw[u], z[u]);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) { z[u][e] *= kLog2e; cm = fmaxf(cm, z[u][e]); }
+      } else {
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) z[u][e] = -INFINITY;
+      }
+    }
+    float acc = st.s * fast_exp2(st.m - cm);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) acc += fast_exp2(z[u][e] - cm);
+    }
+    st.m = cm;
+    st.s = acc;
+  }
+  const int ne = edge_count(sp, v);
+  for (int e = tid; e < ne; e += THREADS) {
+    const float z = Elem<T>::load1(rp + edge_col(sp, e)) * kLog2e;
+    const float cm = fmaxf(st.m, z);
+    st.s = st.s * fast_exp2(st.m - cm) + fast_exp2(z - cm);
+    st.m = cm;
+  }
+  const MaxSum tot = block_merge<NW>(st, smem);
+  if (tid == 0) {
+    const float l = (tot.m + fast_log2(tot.s)) * kLn2;
+    lse[row] = l;
+    const int64_t y = labels[row];
+    float loss = 0.f;
+    if (y != ignore_index) {
+      loss = (y >= 0 && y < v) ? l - Elem<T>::load1(rp + y) : __builtin_nanf("");
+    }
+    row_loss[row] = loss;
+  }
+}
+
+// loss = sum(row_loss) [/ max(1, n_valid)] in a fixed order: thread i adds rows i, i+1024, ...,
+// then lanes and waves are combined in index order.
+__global__ __launch_bounds__(1024) void ce_finalize_kernel(const float* __restrict__ row_loss,
+                                                           const int64_t* __restrict__ labels,
+                                                           int64_t n, int64_t ignore_index,
+                                                           int mean, float* __restrict__ loss,
+                                                           float* __restrict__ n_valid) {
+  __shared__ float sf[16];
+  __shared__ int si[16];
+  float a = 0.f;
+  int cnt = 0;
+  for (int64_t i = threadIdx.x; i < n; i += 1024) {
+    a += row_loss[i];
+    cnt += labels[i] != ignore_index ? 1 : 0;
+  }
+  a = wave_sum(a);
+  cnt = wave_sum_i(cnt);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) { sf[wave] = a; si[wave] = cnt; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float t = sf[0];
+    int c = si[0];
+    for (int i = 1; i < 16; ++i) { t += sf[i]; c += si[i]; }
+    const float nv = c > 0 ? (float)c : 1.f;
+    *n_valid = nv;
+    *loss = mean ? t / nv : t;
+  }
+}
+
+template <typename T, int THREADS, int UNROLL>
+__global__ __launch_bounds__(THREADS) void ce_bwd_kernel(const T* __restrict__ logits,
+                                                          const int64_t* __restrict__ labels,
+                                                          const float* __restrict__ lse,
+                                                          const float* __restrict__ n_valid,
+                                                          const float* __restrict__ grad_out,
+                                                          T* __restrict__ dlogits, int v,
+                                                          int64_t ignore_index, bool vec_ok) {
+  constexpr int EPV = Elem<T>::kVec;
+  const int64_t row = blockIdx.x;
+  const T* rp = logits + row * (int64_t)v;
+  T* gp = dlogits + row * (int64_t)v;
+  const RowSplit sp = split_row<EPV>(row, v, vec_ok);
+  const int tid = threadIdx.x;
+  const int64_t y64 = labels[row];
+  const int ne = edge_count(sp, v);
+
+  if (y64 == ignore_index) {  // ignored row: zeros, and the logits are never read
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    for (int c = tid; c < sp.nvec; c += THREADS) store16_stream(gp + sp.head + (int64_t)c * EPV, zero);
+    for (int e = tid; e < ne; e += THREADS) Elem<T>::store1(gp + edge_col(sp, e), 0.f);
+    return;
+  }
+  const int y = (y64 >= 0 && y64 < v) ? (int)y64 : -1;
+  const float scale = (grad_out != nullptr ? *grad_out : 1.f) / (n_valid != nullptr ? *n_valid : 1.f);
+  const float l2 = lse[row] * kLog2e;
+
+  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+    u32x4 raw[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) {
+        float z[EPV], o[EPV];
+        Elem<T>::unpack(raw[u], z);
+        const int col0 = sp.head + c * EPV;
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] = fast_exp2(z[e] * kLog2e - l2);
+        if (y >= col0 && y < col0 + EPV) {
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) o[e] -= (col0 + e == y) ? 1.f : 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] *= scale;
+        store16_stream(gp + col0, Elem<T>::pack(o));
+      }
+    }
+  }
+  for (int e = tid; e < ne; e += THREADS) {
+    const int col = edge_col(sp, e);
+    float p = fast_exp2(Elem<T>::load1(rp + col) * kLog2e - l2);
+    if (col == y) p -= 1.f;
+    Elem<T>::store1(gp + col, p * scale);
+  }
+}
+
+template <typename T>
+int launch_fwd(const void* logits, const int64_t* labels, float* lse, float* row_loss, int64_t n,
+               int v, int64_t ignore_index, bool vec_ok, hipStream_t st) {
+  const T* lp = static_cast<const T*>(logits);
+  const int threads = fm_host::vocab_threads(v, sizeof(T));
+  const dim3 grid((unsigned)n);
+  if (threads == 1024)
+    hipLaunchKernelGGL((ce_fwd_kernel<T, 1024, 4>), grid, dim3(1024), 0, st, lp, labels, lse,
+                       row_loss, v, ignore_index, vec_ok);
+  else if (threads == 512)
+    hipLaunchKernelGGL((ce_fwd_kernel<T, 512, 4>), grid, dim3(512), 0, st, lp, labels, lse, row_loss,
+                       v, ignore_index, vec_ok);
+  else
+    hipLaunchKernelGGL((ce_fwd_kernel<T, 256, 4>), grid, dim3(256), 0, st, lp, labels, lse, row_loss,
+                       v, ignore_index, vec_ok);
+  return FM_OK;
+}
+
+template <typename T>
+int launch_bwd(const void* logits, const int64_t* labels, const float* lse, const float* n_valid,
+               const float* grad_out, void* dlogits, int64_t n, int v, int64_t ignore_index,
+               bool vec_ok, hipStream_t st) {
+  const T* lp = static_cast<const T*>(logits);
+  T* gp = static_cast<T*>(dlogits);
+  const int threads = fm_host::vocab_threads(v, sizeof(T));
+  const dim3 grid((unsigned)n);
+  if (threads == 1024)
+    hipLaunchKernelGGL((ce_bwd_kernel<T, 1024, 4>), grid, dim3(1024), 0, st, lp, labels, lse,
+                       n_valid, grad_out, gp, v, ignore_index, vec_ok);
+  else if (threads == 512)
+    hipLaunchKernelGGL((ce_bwd_kernel<T, 512, 4>), grid, dim3(512), 0, st, lp, labels, lse, n_valid,
+                       grad_out, gp, v, ignore_index, vec_ok);
+  else
+    hipLaunchKernelGGL((ce_bwd_kernel<T, 256, 4>), grid, dim3(256), 0, st, lp, labels, lse, n_valid,
+                       grad_out, gp, v, ignore_index, vec_ok);
+  return FM_OK;
+}
+
+int check_shape(const char* what, int64_t n, int64_t v, int dtype) {
+  FM_CHECK_ARG(n >= 0 && v > 0, "%s: bad shape n=%lld v=%lld", what, (long long)n, (long long)v);
+  FM_CHECK_ARG(dtype == FM_F32 || dtype == FM_F16 || dtype == FM_BF16, "%s: bad dtype %d", what,
+               dtype);
+  if (n > 0x7fffffffLL || v > 0x7fffffffLL) {
+    fm_host::set_error("%s: n and v must be below 2^31", what);
+    return FM_ERR_UNSUPPORTED;
+  }
+  return FM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fm_ce_fwd(const void* logits, const int64_t* labels, float* lse, float* row_loss, float* loss,
+              float* n_valid, int64_t n, int64_t v, int dtype, int64_t ignore_index, int reduction,
+              fm_stream_t stream) {
+  int rc = check_shape("fm_ce_fwd", n, v, dtype);
+  if (rc != FM_OK) return rc;
+  FM_CHECK_ARG(reduction == FM_REDUCE_SUM || reduction == FM_REDUCE_MEAN,
+               "fm_ce_fwd: reduction must be sum or mean (got %d)", reduction);
+  FM_CHECK_ARG(loss && n_valid, "fm_ce_fwd: NULL scalar output");
+  FM_CHECK_ARG(n == 0 || (logits && labels && lse && row_loss), "fm_ce_fwd: NULL pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (n > 0) {
+    const bool vec_ok = fm_host::aligned16(logits);
+    if (dtype == FM_F32) launch_fwd<float>(logits, labels, lse, row_loss, n, (int)v, ignore_index, vec_ok, st);
+    else if (dtype == FM_BF16) launch_fwd<bf16_t>(logits, labels, lse, row_loss, n, (int)v, ignore_index, vec_ok, st);
+    else launch_fwd<f16_t>(logits, labels, lse, row_loss, n, (int)v, ignore_index, vec_ok, st);
+    FM_CHECK_LAUNCH("fm_ce_fwd");
+  }
+  hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, st, row_loss, labels, n,
+                     ignore_index, reduction == FM_REDUCE_MEAN ? 1 : 0, loss, n_valid);
+  FM_CHECK_LAUNCH("fm_ce_fwd(finalize)");
+  return FM_OK;
+}
+
+int fm_ce_bwd(const void* logits, const int64_t* labels, const float* lse, const float* n_valid,
+              const float* grad_out, void* dlogits, int64_t n, int64_t v, int dtype,
+              int64_t ignore_index, fm_stream_t stream) {
+  int rc = check_shape("fm_ce_bwd", n, v, dtype);
+  if (rc != FM_OK) return rc;
+  if (n == 0) return FM_OK;
+  FM_CHECK_ARG(logits && labels && lse && dlogits, "fm_ce_bwd: NULL pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool vec_ok = fm_host::aligned16(logits) && fm_host::aligned16(dlogits);
+  if (dtype == FM_F32) launch_bwd<float>(logits, labels, lse, n_valid, grad_out, dlogits, n, (int)v, ignore_index, vec_ok, st);
+  else if (dtype == FM_BF16) launch_bwd<bf16_t>(logits, labels, lse, n_valid, grad_out, dlogits, n, (int)v, ignore_index, vec_ok, st);
+  else launch_bwd<f16_t>(logits, labels, lse, n_valid, grad_out, dlogits, n, (int)v, ignore_index, vec_ok, st);
+  FM_CHECK_LAUNCH("fm_ce_bwd");
+  return FM_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,274 @@
+// MoE router: softmax + top-k + renormalised weights + per-expert counts + the stable
+// (by expert) dispatch permutation, for gfx950.
+//
+// Reference semantics: forgemind/moe.py:86-91 (softmax -> topk -> renormalise),
+// moe.py:52-60 (per-expert histogram), moe.py:232-236 (stable sort of the flat assignments).
+// Ties are resolved in the canonical order of forgemind/kernels/topk.py:13-16: equal
+// probabilities go to the lowest expert index.
+//
+// Two launches, integer-only bookkeeping:
+//   route_kernel    one wave per row, experts spread over the lanes (lane l owns experts
+//                   l, l+64, ...). Wave max / sum give the softmax; each of the k picks is a
+//                   wave max over order-preserving integer keys followed by a wave min over
+//                   the tied expert indices. Each workgroup owns a contiguous tile of rows
+//                   and leaves its expert histogram in `hist[tile][e]`.
+//   permute_kernel  every workgroup sums the histograms of the tiles before it (and of all
+//                   tiles, for the expert bases), then walks its own tile in ascending flat
+//                   position and gives each assignment the slot
+//                     base[e] + (#assignments to e in earlier tiles) + (rank inside the tile),
+//                   which is exactly the position a stable sort by expert would assign.
+#include "fm_common.cuh"
+
+using namespace fm;
+
+namespace {
+
+constexpr int kMaxE = 512;
+constexpr int kMaxK = 8;
+constexpr int kMaxTiles = 1024;
+
+__device__ __forceinline__ uint32_t key_of(float f) {
+  if (f != f) return 0xFFFFFFFFu;
+  f = f + 0.0f;
+  const uint32_t b = __builtin_bit_cast(uint32_t, f);
+  return b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);
+}
+
+template <typename T, int EPL>
+__global__ __launch_bounds__(256) void route_kernel(const T* __restrict__ logits,
+                                                     int32_t* __restrict__ idx,
+                                                     float* __restrict__ weights,
+                                                     int32_t* __restrict__ hist, int64_t n, int e,
+                                                     int k, int tile_rows) {
+  __shared__ int lh[kMaxE];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < e; i += 256) lh[i] = 0;
+  __syncthreads();
+  const int64_t row0 = (int64_t)blockIdx.x * tile_rows;
+  const int64_t row1 = row0 + tile_rows < n ? row0 + tile_rows : n;
+  for (int64_t row = row0 + wave; row < row1; row += 4) {
+    float z[EPL];
+    float m = -INFINITY;
+#pragma unroll
+    for (int q = 0; q < EPL; ++q) {
+      const int ex = lane + 64 * q;
+      z[q] = ex < e ? Elem<T>::load1(logits + row * (int64_t)e + ex) : -INFINITY;
+      m = fmaxf(m, z[q]);
+    }
+    m = wave_max(m);
+    float p[EPL];
+    float s = 0.f;
+#pragma unroll
+    for (int q = 0; q < EPL; ++q) {
+      p[q] = fast_exp2((z[q] - m) * kLog2e);
+      s += p[q];
+    }
+    s = wave_sum(s);
+    uint32_t key[EPL];
+#pragma unroll
+    for (int q = 0; q < EPL; ++q) {
+      p[q] = p[q] / s;
+      key[q] = (lane + 64 * q) < e ? key_of(p[q]) : 0u;   // 0 is below every real key
+    }
+    int sel_i[kMaxK];
+    float sel_p[kMaxK];
+    float wsum = 0.f;
+#pragma unroll
+    for (int j = 0; j < kMaxK; ++j) {
+      if (j < k) {
+        uint32_t bk = key[0];
+        int bq = 0;
+#pragma unroll
+        for (int q = 1; q < EPL; ++q) {
+          if (key[q] > bk) { bk = key[q]; bq = q; }
+        }
+        const uint32_t wk = wave_max_u(bk);
+        const int cand = (bk == wk) ? lane + 64 * bq : 0x7fffffff;
+        const int wi = wave_min_i(cand);
+        const int wq = wi >> 6, wl = wi & 63;
+        float pv = p[0];
+#pragma unroll
+        for (int q = 1; q < EPL; ++q) pv = (q == wq) ? p[q] : pv;
+        pv = __shfl(pv, wl, 64);
+#pragma unroll
+        for (int q = 0; q < EPL; ++q) {
+          if (lane == wl && q == wq) key[q] = 0u;
+        }
+        sel_i[j] = wi;
+        sel_p[j] = pv;
+        wsum += pv;
+      }
+    }
+    int my_i = 0;
+    float my_p = 0.f;
+#pragma unroll
+    for (int j = 0; j < kMaxK; ++j) {
+      if (j < k && lane == j) { my_i = sel_i[j]; my_p = sel_p[j]; }
+    }
+    if (lane < k) {
+      idx[row * (int64_t)k + lane] = my_i;
+      weights[row * (int64_t)k + lane] = my_p / wsum;
+      atomicAdd(&lh[my_i], 1);
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < e; i += 256) hist[(int64_t)blockIdx.x * e + i] = lh[i];
+}
+
+__global__ __launch_bounds__(256) void permute_kernel(const int32_t* __restrict__ idx,
+                                                       const int32_t* __restrict__ hist,
+                                                       int32_t* __restrict__ counts,
+                                                       int32_t* __restrict__ slot,
+                                                       int32_t* __restrict__ order, int64_t n, int e,
+                                                       int k, int tile_rows, int ntiles, int emit) {
+  __shared__ int part_b[4][kMaxE];
+  __shared__ int part_t[4][kMaxE];
+  __shared__ int total[kMaxE];
+  __shared__ int offs[kMaxE];      // next free slot of each expert for this tile
+  __shared__ int wcnt[4][kMaxE];   // per-wave assignment counts of the current chunk
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int me = blockIdx.x;
+
+  for (int c0 = 0; c0 < e; c0 += 64) {
+    const int col = c0 + lane;
+    int bef = 0, tot = 0;
+    if (col < e) {
+      for (int t = wave; t < ntiles; t += 4) {
+        const int h = hist[(int64_t)t * e + col];
+        tot += h;
+        bef += t < me ? h : 0;
+      }
+      part_b[wave][col] = bef;
+      part_t[wave][col] = tot;
+    }
+  }
+  for (int i = tid; i < 4 * kMaxE; i += 256) (&wcnt[0][0])[i] = 0;
+  __syncthreads();
+  for (int col = tid; col < e; col += 256) {
+    total[col] = (part_t[0][col] + part_t[1][col]) + (part_t[2][col] + part_t[3][col]);
+    part_b[0][col] = (part_b[0][col] + part_b[1][col]) + (part_b[2][col] + part_b[3][col]);
+  }
+  __syncthreads();
+  for (int col = tid; col < e; col += 256) {
+    int base = 0;
+    for (int c = 0; c < col; ++c) base += total[c];
+    offs[col] = base + part_b[0][col];
+    if (me == 0) counts[col] = total[col];
+  }
+  __syncthreads();
+  if (!emit) return;
+
+  const int64_t p0 = (int64_t)me * tile_rows * k;
+  int64_t p1 = p0 + (int64_t)tile_rows * k;
+  const int64_t pend = n * (int64_t)k;
+  if (p1 > pend) p1 = pend;
+  for (int64_t c0 = p0; c0 < p1; c0 += 256) {
+    const int64_t p = c0 + tid;
+    const bool act = p < p1;
+    const int ex = act ? idx[p] : -1;
+    // rank among equal experts inside the wave, in lane (= flat position) order
+    int rank = 0;
+    unsigned long long todo = __ballot(act);
+    while (todo != 0ull) {
+      const int leader = __builtin_ctzll(todo);
+      const int e0 = __builtin_amdgcn_readlane(ex, leader);
+      const unsigned long long same = __ballot(act && ex == e0);
+      if (act && ex == e0) {
+        rank = __builtin_popcountll(same & ((1ull << lane) - 1ull));
+        if (lane == leader) wcnt[wave][e0] = __builtin_popcountll(same);
+      }
+      todo &= ~same;
+    }
+    __syncthreads();
+    if (act) {
+      int prior = offs[ex];
+      for (int w = 0; w < wave; ++w) prior += wcnt[w][ex];
+      const int s = prior + rank;
+      if (slot != nullptr) slot[p] = s;
+      if (order != nullptr) order[s] = (int32_t)p;
+    }
+    __syncthreads();
+    for (int col = tid; col < e; col += 256) {
+      offs[col] += (wcnt[0][col] + wcnt[1][col]) + (wcnt[2][col] + wcnt[3][col]);
+      wcnt[0][col] = 0; wcnt[1][col] = 0; wcnt[2][col] = 0; wcnt[3][col] = 0;
+    }
+    __syncthreads();
+  }
+}
+
+struct Tiling {
+  int tile_rows;
+  int ntiles;
+};
+
+Tiling make_tiling(int64_t n) {
+  Tiling t;
+  int64_t rows = 64;
+  if ((n + rows - 1) / rows > kMaxTiles) rows = (n + kMaxTiles - 1) / kMaxTiles;
+  rows = (rows + 3) / 4 * 4;
+  t.tile_rows = (int)rows;
+  t.ntiles = (int)((n + rows - 1) / rows);
+  if (t.ntiles < 1) t.ntiles = 1;
+  return t;
+}
+
+template <typename T>
+int launch_route(const void* logits, int32_t* idx, float* weights, int32_t* hist, int64_t n, int e,
+                 int k, const Tiling& tl, hipStream_t st) {
+  const T* lp = static_cast<const T*>(logits);
+  const dim3 grid((unsigned)tl.ntiles), block(256);
+#define GO(EPL) \
+  hipLaunchKernelGGL((route_kernel<T, EPL>), grid, block, 0, st, lp, idx, weights, hist, n, e, k, tl.tile_rows)
+  if (e <= 64) GO(1);
+  else if (e <= 128) GO(2);
+  else if (e <= 256) GO(4);
+  else GO(8);
+#undef GO
+  return FM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t fm_route_workspace(int64_t n, int e, int k) {
+  (void)k;
+  if (n <= 0 || e <= 0) return 0;
+  const Tiling tl = make_tiling(n);
+  return (size_t)tl.ntiles * (size_t)e * sizeof(int32_t);
+}
+
+int fm_route(const void* logits, int32_t* idx, float* weights, int32_t* counts, int32_t* slot,
+             int32_t* order, void* workspace, size_t workspace_bytes, int64_t n, int e, int k,
+             int dtype, fm_stream_t stream) {
+  FM_CHECK_ARG(n >= 0 && e > 0 && k >= 1, "fm_route: bad shape n=%lld e=%d k=%d", (long long)n, e, k);
+  FM_CHECK_ARG(dtype == FM_F32 || dtype == FM_F16 || dtype == FM_BF16, "fm_route: bad dtype %d", dtype);
+  FM_CHECK_ARG(k <= e, "fm_route: selected index k out of range (got %d vs %d)", k, e);
+  if (e > kMaxE || k > kMaxK || n * (int64_t)k >= 0x7fffffffLL) {
+    fm_host::set_error("fm_route: e <= %d, k <= %d and n*k < 2^31 required (e=%d k=%d n=%lld)", kMaxE,
+                       kMaxK, e, k, (long long)n);
+    return FM_ERR_UNSUPPORTED;
+  }
+  FM_CHECK_ARG(counts != nullptr, "fm_route: NULL counts");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const Tiling tl = make_tiling(n);
+  const size_t need = (size_t)tl.ntiles * (size_t)e * sizeof(int32_t);
+  if (workspace == nullptr || workspace_bytes < need) {
+    fm_host::set_error("fm_route: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    return FM_ERR_WORKSPACE;
+  }
+  FM_CHECK_ARG(n == 0 || (logits && idx && weights), "fm_route: NULL pointer");
+  int32_t* hist = static_cast<int32_t*>(workspace);
+  // with n == 0 the single tile has no rows and leaves an all-zero histogram
+  if (dtype == FM_F32) launch_route<float>(logits, idx, weights, hist, n, e, k, tl, st);
+  else if (dtype == FM_BF16) launch_route<bf16_t>(logits, idx, weights, hist, n, e, k, tl, st);
+  else launch_route<f16_t>(logits, idx, weights, hist, n, e, k, tl, st);
+  FM_CHECK_LAUNCH("fm_route");
+  const int emit = (slot != nullptr || order != nullptr) && n > 0 ? 1 : 0;
+  hipLaunchKernelGGL(permute_kernel, dim3(emit ? (unsigned)tl.ntiles : 1u), dim3(256), 0, st, idx, hist,
+                     counts, slot, order, n, e, k, tl.tile_rows, tl.ntiles, emit);
+  FM_CHECK_LAUNCH("fm_route(permute)");
+  return FM_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,113 @@
+// Row softmax over the last dimension for gfx950.
+//
+// Reference semantics: forgemind/kernels/softmax.py:27-80 (y = exp(x - max) / sum, fp32
+// math, stored in x's dtype; NaN propagates, a row of -inf yields NaN like torch).
+// One workgroup per row: an online (max, sum-exp) pass, then a second pass over the row
+// (served by L2 for rows that fit) that writes exp2(z - m) / s.
+#include "fm_vocab.cuh"
+
+using namespace fm;
+
+namespace {
+
+template <typename T, int THREADS, int UNROLL>
+__global__ __launch_bounds__(THREADS) void softmax_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                           int v, bool vec_ok) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int NW = THREADS / 64;
+  __shared__ float smem[2 * NW];
+  const int64_t row = blockIdx.x;
+  const T* rp = x + row * (int64_t)v;
+  T* op = y + row * (int64_t)v;
+  const RowSplit sp = split_row<EPV>(row, v, vec_ok);
+  const int tid = threadIdx.x;
+  const int ne = edge_count(sp, v);
+
+  MaxSum st{kNegBig, 0.f};
+  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+    u32x4 raw[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) raw[u] = load16(rp + sp.head + (int64_t)c * EPV);
+    }
+    float z[UNROLL][EPV];
+    float cm = st.m;
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) {
+        Elem<T>::unpack(raw[u], z[u]);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) { z[u][e] *= kLog2e; cm = fmaxf(cm, z[u][e]); }
+      } else {
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) z[u][e] = -INFINITY;
+      }
+    }
+    float acc = st.s * fast_exp2(st.m - cm);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) acc += fast_exp2(z[u][e] - cm);
+    }
+    st.m = cm;
+    st.s = acc;
+  }
+  for (int e = tid; e < ne; e += THREADS) {
+    const float z = Elem<T>::load1(rp + edge_col(sp, e)) * kLog2e;
+    const float cm = fmaxf(st.m, z);
+    st.s = st.s * fast_exp2(st.m - cm) + fast_exp2(z - cm);
+    st.m = cm;
+  }
+  const MaxSum tot = block_merge<NW>(st, smem);
+  // a row whose maximum is -inf has sum 0: 0 * inf = NaN, which is what torch returns
+  const float inv = 1.f / tot.s;
+  for (int c = tid; c < sp.nvec; c += THREADS) {
+    float z[EPV], o[EPV];
+    Elem<T>::unpack(load16(rp + sp.head + (int64_t)c * EPV), z);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) o[e] = fast_exp2(z[e] * kLog2e - tot.m) * inv;
+    store16_stream(op + sp.head + (int64_t)c * EPV, Elem<T>::pack(o));
+  }
+  for (int e = tid; e < ne; e += THREADS) {
+    const int col = edge_col(sp, e);
+    Elem<T>::store1(op + col, fast_exp2(Elem<T>::load1(rp + col) * kLog2e - tot.m) * inv);
+  }
+}
+
+template <typename T>
+void launch(const void* x, void* y, int64_t n, int v, bool vec_ok, hipStream_t st) {
+  const T* xp = static_cast<const T*>(x);
+  T* yp = static_cast<T*>(y);
+  const int threads = fm_host::vocab_threads(v, sizeof(T));
+  const dim3 grid((unsigned)n);
+  if (threads == 1024)
+    hipLaunchKernelGGL((softmax_kernel<T, 1024, 4>), grid, dim3(1024), 0, st, xp, yp, v, vec_ok);
+  else if (threads == 512)
+    hipLaunchKernelGGL((softmax_kernel<T, 512, 4>), grid, dim3(512), 0, st, xp, yp, v, vec_ok);
+  else
+    hipLaunchKernelGGL((softmax_kernel<T, 256, 2>), grid, dim3(256), 0, st, xp, yp, v, vec_ok);
+}
+
+}  // namespace
+
+extern "C" int fm_softmax_fwd(const void* x, void* y, int64_t n, int64_t v, int dtype,
+                              fm_stream_t stream) {
+  FM_CHECK_ARG(n >= 0 && v > 0, "fm_softmax_fwd: bad shape n=%lld v=%lld", (long long)n, (long long)v);
+  FM_CHECK_ARG(dtype == FM_F32 || dtype == FM_F16 || dtype == FM_BF16, "fm_softmax_fwd: bad dtype %d",
+               dtype);
+  if (n > 0x7fffffffLL || v > 0x7fffffffLL) {
+    fm_host::set_error("fm_softmax_fwd: n and v must be below 2^31");
+    return FM_ERR_UNSUPPORTED;
+  }
+  if (n == 0) return FM_OK;
+  FM_CHECK_ARG(x && y, "fm_softmax_fwd: NULL pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool vec_ok = fm_host::aligned16(x) && fm_host::aligned16(y);
+  if (dtype == FM_F32) launch<float>(x, y, n, (int)v, vec_ok, st);
+  else if (dtype == FM_BF16) launch<bf16_t>(x, y, n, (int)v, vec_ok, st);
+  else launch<f16_t>(x, y, n, (int)v, vec_ok, st);
+  FM_CHECK_LAUNCH("fm_softmax_fwd");
+  return FM_OK;
+}

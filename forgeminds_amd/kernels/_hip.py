@@ -1,0 +1,295 @@
+"""ctypes binding of ``libfmhip.so`` (the C ABI declared in ``include/fm_hip.h``).
+
+Nothing here computes: each wrapper checks shapes the kernels assume, resolves the current
+device and stream of the tensor, passes raw device pointers and raises ``RuntimeError`` with
+the library's message on a non-zero status. Outputs are allocated by the callers in
+``norm.py`` / ``ce.py`` / ... with ``torch.empty``; the library itself never allocates.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import os
+import threading
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "_lib", "libfmhip.so")
+
+F32, F16, BF16 = 0, 1, 2
+REDUCE = {"none": 0, "sum": 1, "mean": 2}
+_DT = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
+
+_lib = None
+_lib_err: "str | None" = None
+_lock = threading.Lock()
+
+_vp, _i64, _int, _f32, _sz = C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_size_t
+
+# name -> (restype, argtypes); mirrors include/fm_hip.h one to one
+SIGNATURES = {
+    "fm_version": (_int, []),
+    "fm_last_error": (C.c_char_p, []),
+    "fm_set_param": (_int, [C.c_char_p, _int]),
+    "fm_rmsnorm_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _f32, _vp]),
+    "fm_rmsnorm_bwd_workspace": (_sz, [_i64, _i64, _int]),
+    "fm_rmsnorm_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64, _int, _int, _vp]),
+    "fm_add_rmsnorm_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _f32, _vp]),
+    "fm_add_rmsnorm_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64,
+                                  _int, _int, _vp]),
+    "fm_ce_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _i64, _int, _vp]),
+    "fm_ce_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _i64, _vp]),
+    "fm_kl_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _f32, _int, _vp]),
+    "fm_kl_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _i64, _i64, _int, _int, _f32, _f32, _vp]),
+    "fm_topk": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _int, _vp]),
+    "fm_softmax_fwd": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
+    "fm_route_workspace": (_sz, [_i64, _int, _int]),
+    "fm_route": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _int, _int, _int, _vp]),
+}
+
+
+def _load():
+    global _lib, _lib_err
+    with _lock:
+        if _lib is not None or _lib_err is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            _lib_err = (f"{LIB_PATH} is missing; build it with "
+                        "`python -m forgeminds_amd.build` (needs hipcc)")
+            return None
+        try:
+            lib = C.CDLL(LIB_PATH)
+            for name, (res, args) in SIGNATURES.items():
+                fn = getattr(lib, name)
+                fn.restype, fn.argtypes = res, args
+        except (OSError, AttributeError) as exc:
+            _lib_err = f"could not load {LIB_PATH}: {exc}"
+            return None
+        _lib = lib
+        return _lib
+
+
+def loaded() -> bool:
+    """True when ``libfmhip.so`` is built and loads in this process."""
+    # lock-free once resolved: this sits on the dispatch path, which dynamo also traces
+    if _lib is not None:
+        return True
+    if _lib_err is not None:
+        return False
+    return _load() is not None
+
+
+def load_error() -> "str | None":
+    _load()
+    return _lib_err
+
+
+def lib():
+    """The loaded library; raises if it is missing -- the GPU path never degrades silently."""
+    l = _lib if _lib is not None else _load()
+    if l is None:
+        raise RuntimeError(f"forgeminds_amd: HIP extension unavailable: {_lib_err}")
+    return l
+
+
+def reset_for_tests() -> None:
+    """Forget a failed load (used after the test-suite builds the library)."""
+    global _lib, _lib_err
+    with _lock:
+        _lib, _lib_err = None, None
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _DT[dt]
+    except KeyError:
+        raise RuntimeError(f"forgeminds_amd: dtype {dt} is not supported by the HIP kernels") from None
+
+
+def _ptr(t: "torch.Tensor | None"):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = lib().fm_last_error()
+        raise RuntimeError(f"{what} failed (status {rc}): {msg.decode() if msg else ''}")
+
+
+def _dense(*ts):
+    for t in ts:
+        if t is not None and not t.is_contiguous():
+            raise RuntimeError("forgeminds_amd: the HIP kernels take contiguous tensors")
+
+
+def set_param(name: str, value: int) -> None:
+    _check(lib().fm_set_param(name.encode(), int(value)), "fm_set_param")
+
+
+# ------------------------------------------------------------------ norm
+def rmsnorm_fwd(x2: torch.Tensor, w: torch.Tensor, eps: float):
+    """x2 [n, d] contiguous, w [d] -> (y [n, d], rstd [n] fp32)."""
+    _dense(x2, w)
+    n, d = x2.shape
+    y = torch.empty_like(x2)
+    rstd = torch.empty(n, device=x2.device, dtype=torch.float32)
+    with torch.cuda.device(x2.device):
+        _check(lib().fm_rmsnorm_fwd(_ptr(x2), _ptr(w), _ptr(y), _ptr(rstd), n, d,
+                                    dtype_code(x2.dtype), dtype_code(w.dtype), float(eps),
+                                    _stream(x2)), "fm_rmsnorm_fwd")
+    return y, rstd
+
+
+def _norm_ws(n: int, d: int, x: torch.Tensor, want_dw: bool):
+    if not want_dw:
+        return None, 0
+    nbytes = int(lib().fm_rmsnorm_bwd_workspace(n, d, dtype_code(x.dtype)))
+    return torch.empty(max(nbytes, 16), device=x.device, dtype=torch.uint8), nbytes
+
+
+def rmsnorm_bwd(x2, w, rstd, dy2, want_dw: bool = True):
+    """-> (dx [n, d], dw [d] in w.dtype or None)."""
+    _dense(x2, w, rstd, dy2)
+    n, d = x2.shape
+    dx = torch.empty_like(x2)
+    dw = torch.empty_like(w) if want_dw else None
+    with torch.cuda.device(x2.device):
+        ws, nbytes = _norm_ws(n, d, x2, want_dw)
+        _check(lib().fm_rmsnorm_bwd(_ptr(x2), _ptr(w), _ptr(rstd), _ptr(dy2), _ptr(dx), _ptr(dw),
+                                    _ptr(ws), nbytes, n, d, dtype_code(x2.dtype),
+                                    dtype_code(w.dtype), _stream(x2)), "fm_rmsnorm_bwd")
+    return dx, dw
+
+
+def add_rmsnorm_fwd(x2, delta2, w, eps: float):
+    """-> (xn [n, d], y [n, d], rstd [n] fp32)."""
+    _dense(x2, delta2, w)
+    n, d = x2.shape
+    xn = torch.empty_like(x2)
+    y = torch.empty_like(x2)
+    rstd = torch.empty(n, device=x2.device, dtype=torch.float32)
+    with torch.cuda.device(x2.device):
+        _check(lib().fm_add_rmsnorm_fwd(_ptr(x2), _ptr(delta2), _ptr(w), _ptr(xn), _ptr(y),
+                                        _ptr(rstd), n, d, dtype_code(x2.dtype),
+                                        dtype_code(w.dtype), float(eps), _stream(x2)),
+               "fm_add_rmsnorm_fwd")
+    return xn, y, rstd
+
+
+def add_rmsnorm_bwd(xn2, w, rstd, gy2, gxn2, want_dw: bool = True):
+    """-> (dx [n, d] (== ddelta), dw or None). gxn2 may be None (no gradient on the sum)."""
+    _dense(xn2, w, rstd, gy2, gxn2)
+    n, d = xn2.shape
+    dx = torch.empty_like(xn2)
+    dw = torch.empty_like(w) if want_dw else None
+    with torch.cuda.device(xn2.device):
+        ws, nbytes = _norm_ws(n, d, xn2, want_dw)
+        _check(lib().fm_add_rmsnorm_bwd(_ptr(xn2), _ptr(w), _ptr(rstd), _ptr(gy2), _ptr(gxn2),
+                                        _ptr(dx), None, _ptr(dw), _ptr(ws), nbytes, n, d,
+                                        dtype_code(xn2.dtype), dtype_code(w.dtype),
+                                        _stream(xn2)), "fm_add_rmsnorm_bwd")
+    return dx, dw
+
+
+# ------------------------------------------------------------------ cross entropy
+def ce_fwd(logits2, labels, ignore_index: int, reduction: str):
+    """logits2 [n, v], labels [n] int64 -> (loss fp32 scalar, lse [n], n_valid fp32 scalar)."""
+    _dense(logits2, labels)
+    n, v = logits2.shape
+    dev = logits2.device
+    lse = torch.empty(n, device=dev, dtype=torch.float32)
+    row_loss = torch.empty(n, device=dev, dtype=torch.float32)
+    scal = torch.empty(2, device=dev, dtype=torch.float32)
+    with torch.cuda.device(dev):
+        _check(lib().fm_ce_fwd(_ptr(logits2), _ptr(labels), _ptr(lse), _ptr(row_loss),
+                               scal.data_ptr(), scal.data_ptr() + 4, n, v,
+                               dtype_code(logits2.dtype), int(ignore_index), REDUCE[reduction],
+                               _stream(logits2)), "fm_ce_fwd")
+    return scal[0], lse, scal[1], row_loss
+
+
+def ce_bwd(logits2, labels, lse, n_valid, grad_out, ignore_index: int):
+    """-> dlogits [n, v]; n_valid / grad_out are fp32 device scalars or None."""
+    _dense(logits2, labels, lse)
+    n, v = logits2.shape
+    dl = torch.empty_like(logits2)
+    with torch.cuda.device(logits2.device):
+        _check(lib().fm_ce_bwd(_ptr(logits2), _ptr(labels), _ptr(lse), _ptr(n_valid),
+                               _ptr(grad_out), _ptr(dl), n, v, dtype_code(logits2.dtype),
+                               int(ignore_index), _stream(logits2)), "fm_ce_bwd")
+    return dl
+
+
+# ------------------------------------------------------------------ KL
+def kl_fwd(s2, t2, inv_temperature: float, reduction: str):
+    """-> (loss fp32 scalar or None, row_kl [n], lse_s [n], lse_t [n])."""
+    _dense(s2, t2)
+    n, v = s2.shape
+    dev = s2.device
+    buf = torch.empty(3, n, device=dev, dtype=torch.float32)
+    loss = torch.empty((), device=dev, dtype=torch.float32) if reduction != "none" else None
+    with torch.cuda.device(dev):
+        _check(lib().fm_kl_fwd(_ptr(s2), _ptr(t2), buf[0].data_ptr(), buf[1].data_ptr(),
+                               buf[2].data_ptr(), _ptr(loss), n, v, dtype_code(s2.dtype),
+                               float(inv_temperature), REDUCE[reduction], _stream(s2)), "fm_kl_fwd")
+    return loss, buf[2], buf[0], buf[1]
+
+
+def kl_bwd(s2, t2, lse_s, lse_t, grad_out, per_row: bool, grad_dtype, inv_temperature: float,
+           scale: float):
+    _dense(s2, t2, lse_s, lse_t, grad_out)
+    n, v = s2.shape
+    g = torch.empty((n, v), device=s2.device, dtype=grad_dtype)
+    with torch.cuda.device(s2.device):
+        _check(lib().fm_kl_bwd(_ptr(s2), _ptr(t2), _ptr(lse_s), _ptr(lse_t), _ptr(grad_out),
+                               1 if per_row else 0, _ptr(g), n, v, dtype_code(s2.dtype),
+                               dtype_code(grad_dtype), float(inv_temperature), float(scale),
+                               _stream(s2)), "fm_kl_bwd")
+    return g
+
+
+# ------------------------------------------------------------------ top-k / softmax / router
+def topk(x2, k: int, index_dtype=torch.int64, want_values: bool = True):
+    _dense(x2)
+    n, v = x2.shape
+    vals = torch.empty((n, k), device=x2.device, dtype=x2.dtype) if want_values else None
+    idx = torch.empty((n, k), device=x2.device, dtype=index_dtype)
+    bits = 64 if index_dtype == torch.int64 else 32
+    with torch.cuda.device(x2.device):
+        _check(lib().fm_topk(_ptr(x2), _ptr(vals), _ptr(idx), n, v, int(k), dtype_code(x2.dtype),
+                             bits, _stream(x2)), "fm_topk")
+    return vals, idx
+
+
+def softmax_fwd(x2):
+    _dense(x2)
+    n, v = x2.shape
+    y = torch.empty_like(x2)
+    with torch.cuda.device(x2.device):
+        _check(lib().fm_softmax_fwd(_ptr(x2), _ptr(y), n, v, dtype_code(x2.dtype), _stream(x2)),
+               "fm_softmax_fwd")
+    return y
+
+
+def route(logits2, k: int, want_permutation: bool = True):
+    """-> (idx int32 [n, k], weights fp32 [n, k], counts int32 [e], slot, order int32 [n*k])."""
+    _dense(logits2)
+    n, e = logits2.shape
+    dev = logits2.device
+    idx = torch.empty((n, k), device=dev, dtype=torch.int32)
+    wts = torch.empty((n, k), device=dev, dtype=torch.float32)
+    counts = torch.empty(e, device=dev, dtype=torch.int32)
+    slot = torch.empty(n * k, device=dev, dtype=torch.int32) if want_permutation else None
+    order = torch.empty(n * k, device=dev, dtype=torch.int32) if want_permutation else None
+    with torch.cuda.device(dev):
+        nbytes = int(lib().fm_route_workspace(n, e, k))
+        ws = torch.empty(max(nbytes, 16), device=dev, dtype=torch.uint8)
+        _check(lib().fm_route(_ptr(logits2), _ptr(idx), _ptr(wts), _ptr(counts), _ptr(slot),
+                              _ptr(order), _ptr(ws), nbytes, n, e, int(k),
+                              dtype_code(logits2.dtype), _stream(logits2)), "fm_route")
+    return idx, wts, counts, slot, order

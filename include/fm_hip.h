@@ -1,0 +1,170 @@
+/* C ABI of libfmhip.so: hand-written HIP kernels (gfx950 / MI355X) for ForgeMind's
+ * packed-kernel hot path.
+ *
+ * Conventions shared by every entry point
+ *   - plain pointers and sizes only; all tensor pointers are DEVICE pointers to
+ *     row-major, densely packed data (row stride == row width);
+ *   - the caller owns every buffer, including scratch ("workspace"); the library never
+ *     allocates, frees, retains a pointer or synchronises, so each call is a pure enqueue on
+ *     `stream` (a hipStream_t passed as void*; NULL = the default stream) and can be
+ *     captured into a HIP graph;
+ *   - the device that is current on the calling thread must own the buffers;
+ *   - inputs are never written;
+ *   - return value 0 (FM_OK) on success, otherwise an fm_status code; fm_last_error()
+ *     returns a thread-local message for the last failure on the calling thread;
+ *   - element types are selected with fm_dtype codes; math is fp32 with one rounding at
+ *     the store, and every reduction runs in a fixed order (no float atomics), so results
+ *     are bit-reproducible run to run.
+ *
+ * "Reference" below is xygamer179-boop/ForgeMinds; each entry point names the reference
+ * interface (file:line) it stands in for.
+ */
+#ifndef FM_HIP_H_
+#define FM_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* fm_stream_t; /* hipStream_t */
+
+enum fm_dtype { FM_F32 = 0, FM_F16 = 1, FM_BF16 = 2 };
+
+enum fm_status {
+  FM_OK = 0,
+  FM_ERR_INVALID = 1,     /* bad argument (null pointer, non-positive size, bad enum) */
+  FM_ERR_UNSUPPORTED = 2, /* shape or dtype outside what the kernels handle */
+  FM_ERR_LAUNCH = 3,      /* the HIP runtime rejected a launch */
+  FM_ERR_WORKSPACE = 4    /* workspace pointer missing or too small */
+};
+
+enum fm_reduction { FM_REDUCE_NONE = 0, FM_REDUCE_SUM = 1, FM_REDUCE_MEAN = 2 };
+
+/* ABI version (bumped on any signature change) and last error text. */
+int fm_version(void);
+const char* fm_last_error(void);
+
+/* Tuning hook used by the benchmark sweeps; unknown names return FM_ERR_INVALID.
+ * value <= 0 restores the built-in heuristic. Not part of the reference surface. */
+int fm_set_param(const char* name, int value);
+
+/* ------------------------------------------------------------------ RMSNorm
+ * Replaces _launch_rms_fwd / _rms_layernorm_forward (forgemind/kernels/norm.py:1095-1101,
+ * 133-175); semantics of _fallback.rms_norm (forgemind/kernels/_fallback.py:26-30):
+ *   r = rsqrt(mean(x^2) + eps);  y = ((x * r) * w) rounded once to x's dtype;  rstd[i] = r.
+ * x, y: [n, d] of x_dtype; w: [d] of w_dtype (x_dtype or FM_F32); rstd: [n] fp32. */
+int fm_rmsnorm_fwd(const void* x, const void* w, void* y, float* rstd, int64_t n, int64_t d,
+                   int x_dtype, int w_dtype, float eps, fm_stream_t stream);
+
+/* Bytes of scratch fm_rmsnorm_bwd / fm_add_rmsnorm_bwd need for the fp32 partial weight
+ * gradients (the reference's `[programs, n_cols]` buffer, norm.py:845-870, 1143-1146). */
+size_t fm_rmsnorm_bwd_workspace(int64_t n, int64_t d, int x_dtype);
+
+/* Replaces _launch_rms_bwd / _rms_layernorm_backward + _rms_sum_dw_partials
+ * (norm.py:1104-1115, 179-231, 234-316, 571-593):
+ *   xh = x * rstd; g = dy * w; dx = rstd * (g - xh * mean(g * xh));  dw = sum_rows dy * xh.
+ * dx: [n, d] of x_dtype; dw: [d] of w_dtype (fp32 accumulation, fixed summation order).
+ * dw may be NULL (frozen weight): then no workspace is needed. */
+int fm_rmsnorm_bwd(const void* x, const void* w, const float* rstd, const void* dy, void* dx,
+                   void* dw, void* workspace, size_t workspace_bytes, int64_t n, int64_t d,
+                   int x_dtype, int w_dtype, fm_stream_t stream);
+
+/* Replaces _launch_addrms_fwd / _addrms_fwd (norm.py:1118-1131, 1001-1047) with the
+ * rounding points of _fallback.add_rms_norm (_fallback.py:33-35):
+ *   xn = x + delta rounded to x's dtype; y = rms_norm(xn, w, eps) computed from the rounded xn. */
+int fm_add_rmsnorm_fwd(const void* x, const void* delta, const void* w, void* xn, void* y,
+                       float* rstd, int64_t n, int64_t d, int x_dtype, int w_dtype, float eps,
+                       fm_stream_t stream);
+
+/* Replaces _launch_addrms_bwd / _addrms_bwd (norm.py:1134-1148, 1050-1086):
+ *   dx = rstd * (gy*w - xh * mean(gy*w*xh)) + gxn;  ddelta == dx;  dw = sum_rows gy * xh.
+ * gxn (gradient of the residual output) may be NULL (treated as zero). ddelta may be NULL or
+ * equal to dx (the two gradients are the same values; a second buffer is only written when
+ * a distinct pointer is given). dw may be NULL. */
+int fm_add_rmsnorm_bwd(const void* xn, const void* w, const float* rstd, const void* gy,
+                       const void* gxn, void* dx, void* ddelta, void* dw, void* workspace,
+                       size_t workspace_bytes, int64_t n, int64_t d, int x_dtype, int w_dtype,
+                       fm_stream_t stream);
+
+/* ------------------------------------------------------------------ cross entropy
+ * Replaces the F.cross_entropy(reduction="sum") / n reduction of logits_cross_entropy and
+ * chunked_cross_entropy (forgemind/loss.py:54-70, 23-51):
+ *   row_loss[i] = logsumexp(logits[i,:]) - logits[i, labels[i]]   (0 where labels[i] == ignore_index)
+ *   n_valid = max(1, #{labels != ignore_index})
+ *   loss = sum(row_loss) / n_valid for FM_REDUCE_MEAN (loss.py:63-70),
+ *          sum(row_loss) for FM_REDUCE_SUM (one chunk of loss.py:36-38)
+ * logits: [n, v] of dtype; labels: [n] int64; lse, row_loss: [n] fp32 (lse is what the
+ * backward re-uses instead of a stored softmax); loss, n_valid: fp32 scalars on device.
+ * One read of logits. n == 0 yields loss 0 and n_valid 1. */
+int fm_ce_fwd(const void* logits, const int64_t* labels, float* lse, float* row_loss,
+              float* loss, float* n_valid, int64_t n, int64_t v, int dtype,
+              int64_t ignore_index, int reduction, fm_stream_t stream);
+
+/* Backward of the above (what autograd derives for loss.py:65-70):
+ *   dlogits[i,j] = (exp(logits[i,j] - lse[i]) - [j == labels[i]]) * grad_out / n_valid
+ * for rows with a valid label, 0 for ignored rows (those rows are not read).
+ * grad_out: device fp32 scalar, or NULL for 1. n_valid: the scalar fm_ce_fwd wrote, or NULL
+ * for 1 (the gradient of the FM_REDUCE_SUM loss). dlogits: [n, v] of dtype. */
+int fm_ce_bwd(const void* logits, const int64_t* labels, const float* lse, const float* n_valid,
+              const float* grad_out, void* dlogits, int64_t n, int64_t v, int dtype,
+              int64_t ignore_index, fm_stream_t stream);
+
+/* ------------------------------------------------------------------ distillation KL
+ * Replaces _kl_fwd_bwd_kernel's loss half (forgemind/kernels/kl.py:73-135, 143-179);
+ * semantics of _fallback.kl_div_logits (_fallback.py:52-69) on logits scaled by
+ * inv_temperature:  row_kl[i] = sum_j p_t (log p_t - log p_s),  p = softmax(logits * inv_temperature).
+ * One pass over both rows (online max / sum-exp); lse_s, lse_t ([n] fp32, of the scaled
+ * logits) are saved for the backward. loss (device fp32 scalar, may be NULL) receives
+ * sum(row_kl) for FM_REDUCE_SUM, sum/n for FM_REDUCE_MEAN and is left untouched for
+ * FM_REDUCE_NONE. */
+int fm_kl_fwd(const void* student, const void* teacher, float* lse_s, float* lse_t,
+              float* row_kl, float* loss, int64_t n, int64_t v, int dtype,
+              float inv_temperature, int reduction, fm_stream_t stream);
+
+/* Gradient wrt the (unscaled) student logits, recomputed from the saved lse values
+ * (the reference stores it from the forward, kl.py:112-134, and rescales it in
+ * _KLDivFn.backward, kl.py:181-191):
+ *   dstudent[i,j] = (p_s - p_t) * inv_temperature * scale * g_i
+ * g_i = grad_out[i] when grad_per_row != 0, grad_out[0] otherwise, 1 when grad_out is NULL;
+ * `scale` carries the 1/n of the mean reduction. dstudent: [n, v] of grad_dtype. */
+int fm_kl_bwd(const void* student, const void* teacher, const float* lse_s, const float* lse_t,
+              const float* grad_out, int grad_per_row, void* dstudent, int64_t n, int64_t v,
+              int dtype, int grad_dtype, float inv_temperature, float scale, fm_stream_t stream);
+
+/* ------------------------------------------------------------------ top-k
+ * Replaces _fused / _topk_threshold_kernel + _topk_select_kernel
+ * (forgemind/kernels/topk.py:234-251, 59-218). Exact top-k over the last dim in the canonical
+ * order of topk.py:13-16: value descending, index ascending inside ties, smallest indices
+ * win at the k-th value; NaN counts as the largest value and is passed through.
+ * x: [n, v] of dtype; values: [n, k] of dtype (may be NULL); indices: [n, k] int32 when
+ * index_bits == 32, int64 when index_bits == 64. 1 <= k <= min(v, 512). */
+int fm_topk(const void* x, void* values, void* indices, int64_t n, int64_t v, int k, int dtype,
+            int index_bits, fm_stream_t stream);
+
+/* ------------------------------------------------------------------ softmax (last dim)
+ * Replaces _softmax_kernel (forgemind/kernels/softmax.py:27-80): y = exp(x - max) / sum. */
+int fm_softmax_fwd(const void* x, void* y, int64_t n, int64_t v, int dtype, fm_stream_t stream);
+
+/* ------------------------------------------------------------------ MoE router + dispatch permutation
+ * Replaces the aten sequence of Router.forward and MoE.forward
+ * (forgemind/moe.py:86-91, 52-60, 232-236): probs = softmax(logits) in fp32; top-k of probs
+ * in the canonical order above (lowest expert index wins ties); weights renormalised to sum
+ * to 1; per-expert counts; and the stable sort of the flat assignments by expert:
+ *   flat[p] = idx[p / k][p % k];  slot[p] = position of p after the stable sort;
+ *   order[slot[p]] = p  (== torch.sort(flat, stable=True).indices).
+ * logits: [n, e] of dtype (fp32 math inside); idx: [n, k] int32; weights: [n, k] fp32;
+ * counts: [e] int32; slot, order: [n*k] int32 (either may be NULL: then only routing and
+ * counts are produced when both are NULL). 1 <= k <= 8, k <= e <= 512, n*k < 2^31. */
+size_t fm_route_workspace(int64_t n, int e, int k);
+int fm_route(const void* logits, int32_t* idx, float* weights, int32_t* counts, int32_t* slot,
+             int32_t* order, void* workspace, size_t workspace_bytes, int64_t n, int e, int k,
+             int dtype, fm_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* FM_HIP_H_ */

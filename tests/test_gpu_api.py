@@ -1,0 +1,318 @@
+"""The public ``fm.kernels`` surface on a GPU: the HIP path is the one that runs (``stats()``
+counts it as fast), autograd / custom-op / torch.compile plumbing gives the same numbers as the
+direct launches, and the module-level callers (nn.RMSNorm, loss, moe.Router) sit on top of it.
+"""
+
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+import forgeminds_amd as fm
+from forgeminds_amd import kernels
+from forgeminds_amd.kernels import _hip, _ops
+from forgeminds_amd.loss import chunked_cross_entropy, logits_cross_entropy
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu_and_library():
+    assert torch.cuda.is_available() and _hip.loaded(), _hip.load_error()
+    assert kernels.available()
+
+
+def close(a, b, rel=1e-2):
+    a, b = a.detach().float().cpu(), b.detach().float().cpu()
+    return ((a - b).abs().max() / b.abs().max().clamp_min(1e-30)).item() <= rel
+
+
+def test_gpu_calls_take_the_hip_path():
+    kernels.reset_stats()
+    x = torch.randn(64, 256, device=DEV, dtype=torch.bfloat16)
+    w = torch.ones(256, device=DEV)
+    kernels.rms_norm(x, w)
+    kernels.add_rms_norm(x, x, w)
+    kernels.cross_entropy(torch.randn(8, 100, device=DEV), torch.randint(0, 100, (8,), device=DEV))
+    kernels.kl_div_logits(torch.randn(8, 100, device=DEV), torch.randn(8, 100, device=DEV))
+    kernels.topk(torch.randn(8, 100, device=DEV), 5)
+    kernels.softmax(torch.randn(8, 100, device=DEV))
+    kernels.moe_route(torch.randn(8, 16, device=DEV), 2)
+    st = kernels.stats()
+    assert st["fast"] == 7 and st["fallback"] == 0, st
+    kernels.set_backend("fallback")
+    kernels.rms_norm(x, w)
+    assert kernels.stats()["reasons"] == {"backend=fallback": 1}
+    kernels.set_backend("triton")              # the reference's name for "force the kernels"
+    kernels.rms_norm(x, w)
+    assert kernels.stats()["fast"] == 8
+    kernels.set_backend("auto")
+    kernels.rms_norm(x.double(), w.double())   # float64 stays with torch, and says why
+    assert "dtype torch.float64" in kernels.stats()["reasons"]
+
+
+@pytest.mark.parametrize("dt,wdt", [(torch.bfloat16, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                    (torch.float32, torch.float32), (torch.float16, torch.float16)])
+def test_rms_norm_autograd_matches_oracle(dt, wdt):
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(3, 50, 512, generator=g).to(dt)
+    w = (1 + 0.1 * torch.randn(512, generator=g)).to(wdt)
+    dy = torch.randn(3, 50, 512, generator=g).to(dt)
+    xd = x.to(DEV).requires_grad_(True)
+    wd = w.to(DEV).requires_grad_(True)
+    y = kernels.rms_norm(xd, wd, 1e-6)
+    y.backward(dy.to(DEV))
+    oy, _ = O.rms_norm(x, w)
+    odx, odw = O.rms_norm_bwd(x, w, dy)
+    assert y.shape == x.shape and y.dtype == dt
+    assert close(y, oy) and close(xd.grad, odx) and close(wd.grad, odw)
+    assert wd.grad.dtype == wdt
+    # non-contiguous input (reference tests/test_edge_cases.py:106-111)
+    xt = torch.randn(512, 40, device=DEV).t()
+    assert not xt.is_contiguous()
+    assert close(kernels.rms_norm(xt, torch.ones(512, device=DEV)), F.rms_norm(xt, (512,), None, 1e-6), 1e-5)
+
+
+def test_add_rms_norm_autograd_and_partial_use():
+    g = torch.Generator().manual_seed(1)
+    x, dl = torch.randn(40, 768, generator=g).bfloat16(), torch.randn(40, 768, generator=g).bfloat16()
+    w = 1 + 0.1 * torch.randn(768, generator=g)
+    gy, gxn = torch.randn(40, 768, generator=g).bfloat16(), torch.randn(40, 768, generator=g).bfloat16()
+    xd, dd, wd = (t.to(DEV).requires_grad_(True) for t in (x, dl, w))
+    xn, y = kernels.add_rms_norm(xd, dd, wd, 1e-5)
+    torch.autograd.backward([xn, y], [gxn.to(DEV), gy.to(DEV)])
+    oxn, oy, _ = O.add_rms_norm(x, dl, w, 1e-5)
+    odx, odw = O.add_rms_norm_bwd(oxn, w, gy, gxn, 1e-5)
+    assert torch.equal(xn.cpu(), oxn) and close(y, oy)
+    assert close(xd.grad, odx) and torch.equal(xd.grad, dd.grad) and close(wd.grad, odw)
+    assert xd.grad.data_ptr() != dd.grad.data_ptr()          # leaves do not share storage
+    # only the normalised output used / only the residual used
+    xd2, dd2 = (t.to(DEV).requires_grad_(True) for t in (x, dl))
+    _, y2 = kernels.add_rms_norm(xd2, dd2, w.to(DEV), 1e-5)
+    y2.backward(gy.to(DEV))
+    assert close(xd2.grad, O.add_rms_norm_bwd(oxn, w, gy, None, 1e-5)[0])
+    xd3, dd3 = (t.to(DEV).requires_grad_(True) for t in (x, dl))
+    xn3, _ = kernels.add_rms_norm(xd3, dd3, w.to(DEV), 1e-5)
+    xn3.backward(gxn.to(DEV))
+    assert torch.equal(xd3.grad.cpu(), gxn)
+
+
+def test_op_path_equals_eager_path_bit_for_bit():
+    # reference tests/test_kernel_ops.py:94-109
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(6, 64, generator=g).to(DEV)
+    w = torch.randn(64, generator=g).to(DEV)
+
+    def run(mode, fn):
+        _ops.use_custom_ops(mode)
+        ins = [t.clone().requires_grad_(True) for t in (x, x * 0.5, w)]
+        out = fn(ins)
+        out.square().sum().backward()
+        return out.detach().clone(), [t.grad.clone() for t in ins if t.grad is not None]
+
+    for fn in (lambda t: kernels.rms_norm(t[0], t[2], 1e-6),
+               lambda t: sum(kernels.add_rms_norm(t[0], t[1], t[2], 1e-6))):
+        ye, ge = run(False, fn)
+        yo, go = run(True, fn)
+        assert torch.equal(ye, yo) and len(ge) == len(go)
+        assert all(torch.equal(a, b) for a, b in zip(ge, go))
+    _ops.use_custom_ops(True)
+    with torch.no_grad():
+        assert not kernels.rms_norm(x, w).requires_grad
+
+
+def test_compile_fullgraph_and_export_keep_the_kernel():
+    # reference tests/test_kernel_ops.py:120-153
+    x = torch.randn(6, 64, device=DEV)
+    w = torch.randn(64, device=DEV)
+
+    def fn(t, ww):
+        a, b = kernels.add_rms_norm(t, t * 2, ww, 1e-6)
+        return kernels.rms_norm(a + b, ww, 1e-6)
+
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    fn(xr, wr).square().sum().backward()
+    xc, wc = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    out = torch.compile(fn, backend="aot_eager", fullgraph=True)(xc, wc)
+    out.square().sum().backward()
+    assert torch.allclose(out, fn(x, w), atol=2e-6, rtol=1e-5)
+    assert torch.allclose(xc.grad, xr.grad, atol=1e-4, rtol=1e-4)
+    assert torch.allclose(wc.grad, wr.grad, atol=1e-4, rtol=1e-4)
+
+    class M(nn.Module):
+        def forward(self, t):
+            return kernels.rms_norm(t, w, 1e-6)
+
+    ep = torch.export.export(M(), (x,))
+    targets = [str(n.target) for n in ep.graph.nodes if n.op == "call_function"]
+    assert "forgemind.rms_norm.default" in targets, targets
+
+
+def test_cross_entropy_autograd_and_callers():
+    g = torch.Generator().manual_seed(3)
+    lg = (2 * torch.randn(300, 4000, generator=g)).bfloat16()
+    y = torch.randint(0, 4000, (300,), generator=g)
+    y[::7] = -100
+    ol, og = O.cross_entropy(lg, y)
+    lgd = lg.to(DEV).requires_grad_(True)
+    loss = kernels.cross_entropy(lgd, y.to(DEV))
+    (loss * 3.0).backward()
+    assert loss.dtype == torch.float32 and loss.item() == pytest.approx(ol.item(), rel=1e-4)
+    assert close(lgd.grad, og.float() * 3.0)
+    # logits_cross_entropy on [B, T, V] (reference tests/test_edge_cases.py:50-56)
+    l3 = logits_cross_entropy(lg.to(DEV).view(3, 100, 4000), y.to(DEV).view(3, 100))
+    assert l3.item() == pytest.approx(ol.item(), rel=1e-4)
+    # chunked CE over h @ W^T equals the unchunked one, and trains both operands
+    h = torch.randn(70, 64, generator=g).to(DEV).requires_grad_(True)
+    wt = torch.randn(500, 64, generator=g).to(DEV).requires_grad_(True)
+    yy = torch.randint(0, 500, (70,), generator=g).to(DEV)
+    yy[3] = -100
+    a = chunked_cross_entropy(h, wt, yy, chunk=32)
+    a.backward()
+    ref = F.cross_entropy(h.detach() @ wt.detach().t(), yy, ignore_index=-100)
+    assert a.item() == pytest.approx(ref.item(), rel=1e-4)
+    assert h.grad is not None and wt.grad is not None
+    # all ignored: 0.0 and a usable backward (reference tests/test_edge_cases.py:21-28)
+    h2 = torch.randn(6, 64, device=DEV, requires_grad=True)
+    z = chunked_cross_entropy(h2, wt, torch.full((6,), -100, device=DEV), chunk=4)
+    z.backward()
+    assert z.item() == 0.0 and h2.grad is not None and not h2.grad.any()
+
+
+def test_kl_autograd_reductions_and_temperature():
+    g = torch.Generator().manual_seed(4)
+    s = (3 * torch.randn(20, 3000, generator=g)).bfloat16()
+    t = (s.float() + 0.5 * torch.randn(20, 3000, generator=g)).bfloat16()
+    for red in ("mean", "sum", "none"):
+        sd = s.to(DEV).requires_grad_(True)
+        out = kernels.kl_div_logits(sd, t.to(DEV), red, temperature=2.0)
+        ol, og = O.kl_div(s, t, red, 2.0)
+        assert torch.allclose(out.cpu(), ol, rtol=1e-4, atol=1e-6)
+        (out.sum() * 2.0).backward()
+        assert close(sd.grad, og.float() * 2.0) and sd.grad.dtype == torch.bfloat16
+    sd = s.to(DEV).requires_grad_(True)
+    keep = sd.detach().clone()
+    kernels.kl_div_logits(sd, t.to(DEV), grad_dtype=torch.float32).backward()
+    assert torch.equal(sd.detach(), keep)                    # inputs are never written
+    # distillation loop (reference tests/test_kernels.py:143-166)
+    hs = torch.randn(16, 32, generator=g).to(DEV).requires_grad_(True)
+    ht = torch.randn(16, 32, generator=g).to(DEV)
+    w = torch.randn(200, 32, generator=g).to(DEV)
+    wt = torch.randn(200, 32, generator=g).to(DEV).requires_grad_(True)
+    loss = kernels.kl_distill_loss(hs, ht, w, lambda zz: zz @ wt.t(), chunk=5)
+    loss.backward()
+    ref, _ = O.kl_div((hs.detach() @ w.t()).cpu(), (ht @ wt.detach().t()).cpu(), "mean")
+    assert loss.item() == pytest.approx(ref.item(), rel=1e-4) and wt.grad is None
+
+
+def test_topk_softmax_surface_on_gpu():
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(2, 30, 5000, generator=g)
+    xd = x.to(DEV).requires_grad_(True)
+    v, idx = kernels.topk(xd, 12)
+    ov, oi = O.topk(x, 12)
+    assert idx.dtype == torch.int64 and torch.equal(idx.cpu(), oi) and torch.equal(v.detach().cpu(), ov)
+    (v * 2).sum().backward()
+    assert int((xd.grad != 0).sum()) == 2 * 30 * 12
+    with pytest.raises(RuntimeError, match="selected index k out of range"):
+        kernels.topk(xd, 5001)
+    tv, ti = torch.topk(xd.detach(), 2, dim=0)
+    v0, i0 = kernels.topk(xd.detach(), 2, dim=0)
+    assert torch.equal(v0, tv) and torch.equal(i0, ti)
+    kernels.reset_stats()
+    kernels.topk(torch.randn(2, 2048, device=DEV), 600)       # k > 512: torch path, counted
+    assert kernels.stats()["fallback"] == 1
+    xs = torch.randn(4, 256, device=DEV, requires_grad=True)
+    y = kernels.softmax(xs)
+    gr = torch.randn(4, 256, device=DEV)
+    y.backward(gr)
+    xr = xs.detach().clone().requires_grad_(True)
+    torch.softmax(xr, -1).backward(gr)
+    assert torch.allclose(y, torch.softmax(xr, -1), rtol=1e-5, atol=1e-6)
+    assert torch.allclose(xs.grad, xr.grad, rtol=1e-4, atol=1e-6)
+    fn = torch.compile(lambda t: kernels.topk(kernels.softmax(t), 8)[0].sum(), fullgraph=True, backend="eager")
+    fn(xs)                                                   # traces to aten, no graph break
+
+
+def test_router_module_and_route_backward():
+    g = torch.Generator().manual_seed(6)
+    router = fm.moe.Router(64, 16, 2).to(DEV)
+    x = torch.randn(300, 64, generator=g).to(DEV)
+    w, idx, aux, z = router(x)
+    logits = router.gate(x).float()
+    oi, ow, oc, oslot, oorder = O.router(logits.detach().cpu(), 2)
+    assert torch.equal(idx.cpu(), oi) and torch.allclose(w.cpu(), ow, rtol=1e-5)
+    plan = router.last_plan
+    assert torch.equal(plan.order.cpu(), oorder) and torch.equal(plan.counts.cpu(), oc)
+    assert torch.equal(plan.offsets.cpu().long(), oc.cumsum(0))
+    # gradient of the renormalised weights wrt the logits == autograd through the torch expression
+    lg = logits.detach().clone().requires_grad_(True)
+    r = kernels.moe_route(lg, 2)
+    gw = torch.randn(300, 2, generator=g).to(DEV)
+    r.weights.backward(gw)
+    lr = logits.detach().clone().requires_grad_(True)
+    p = lr.softmax(-1)
+    pk = p.gather(1, r.idx.long())
+    (pk / pk.sum(-1, keepdim=True)).backward(gw)
+    assert torch.allclose(lg.grad, lr.grad, rtol=1e-4, atol=1e-7)
+    (w.sum() + aux + z).backward()
+    assert router.gate.weight.grad is not None
+
+
+def test_modules_on_gpu():
+    m = fm.nn.RMSNorm(256, eps=1e-5).to(DEV)
+    ref = nn.RMSNorm(256, eps=1e-5).to(DEV)
+    x = torch.randn(4, 9, 256, device=DEV, dtype=torch.bfloat16)
+    kernels.reset_stats()
+    y = m(x)                                  # fp32 parameter, bf16 activations: still the kernel
+    assert kernels.stats()["fast"] == 1
+    assert close(y, ref(x.float()).bfloat16())
+    normed, res = m.forward_with_residual(x, x)
+    assert torch.equal(res, x + x) and close(normed, ref((x + x).float()))
+    net = nn.Sequential(nn.Linear(256, 256), nn.RMSNorm(256)).to(DEV)
+    exp = net(x.float())
+    kernels.enable(net)
+    assert net._fm_fused["norm"] == 1 and torch.allclose(net(x.float()), exp, atol=1e-5, rtol=1e-5)
+    kernels.revert(net)
+
+
+def test_launches_are_graph_capturable():
+    """No allocation, no sync, no memset node inside the library: a captured fwd+bwd replays
+    to the same bits as the eager launches, replay after replay."""
+    n, d = 512, 1024
+    x = torch.randn(n, d, device=DEV).bfloat16()
+    w = torch.randn(d, device=DEV)
+    dy = torch.randn(n, d, device=DEV).bfloat16()
+    y, rstd = torch.empty_like(x), torch.empty(n, device=DEV)
+    dx, dw = torch.empty_like(x), torch.empty_like(w)
+    L = _hip.lib()
+    nb = L.fm_rmsnorm_bwd_workspace(n, d, _hip.BF16)
+    ws = torch.empty(nb, device=DEV, dtype=torch.uint8)
+
+    def launch(stream):
+        assert L.fm_rmsnorm_fwd(x.data_ptr(), w.data_ptr(), y.data_ptr(), rstd.data_ptr(), n, d,
+                                _hip.BF16, _hip.F32, 1e-6, stream) == 0
+        assert L.fm_rmsnorm_bwd(x.data_ptr(), w.data_ptr(), rstd.data_ptr(), dy.data_ptr(),
+                                dx.data_ptr(), dw.data_ptr(), ws.data_ptr(), nb, n, d, _hip.BF16,
+                                _hip.F32, stream) == 0
+
+    launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    ref = [t.clone() for t in (y, dx, dw)]
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch(side.cuda_stream)                         # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            launch(side.cuda_stream)
+    for _ in range(3):
+        for t in (y, dx, dw):
+            t.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, b) for a, b in zip((y, dx, dw), ref))

@@ -1,0 +1,365 @@
+"""Parity of the HIP kernels with the CPU oracle, through the C ABI (the thin ctypes wrappers
+of forgeminds_amd.kernels._hip pass raw device pointers to libfmhip.so and nothing else).
+
+Bars: bit-exact for indices, counts and permutations; <= 1e-2 relative for bf16/fp16 tensors
+(relative to the largest magnitude of the reference tensor, plus an elementwise bf16-ulp
+check); <= 1e-4 relative for fp32 losses against fp32/fp64 math on the same input values.
+Inputs are seeded on the CPU generator and moved to the GPU, so both sides see the same bits.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from forgeminds_amd.kernels import _hip
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+BF16, F16, F32 = torch.bfloat16, torch.float16, torch.float32
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu_and_library():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    assert _hip.loaded(), f"libfmhip.so must be built before GPU tests: {_hip.load_error()}"
+
+
+def gen(seed):
+    return torch.Generator(device="cpu").manual_seed(seed)
+
+
+def rel_max(got, ref):
+    got, ref = got.detach().float().cpu(), ref.detach().float().cpu()
+    return ((got - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item()
+
+
+def assert_close_lowp(got, ref, dt, what, ulps=2.0, cancel=0.0):
+    """<= 1e-2 of the tensor's scale, and elementwise within a few ulps of the dtype.
+
+    `cancel` is the magnitude of the fp32 terms the result is a difference of (g - xh*c in the
+    norm backward, p_s - p_t in the KL gradient): each term carries ~2**-23 relative rounding
+    (and ~2**-22 from the hardware exp2), so where the exact answer cancels towards 0 the
+    honest absolute tolerance is a few 2**-23 of that magnitude, not of the tiny result."""
+    got, ref = got.detach().float().cpu(), ref.detach().float().cpu()
+    assert got.shape == ref.shape, what
+    cancel = float(cancel)
+    scale = ref.abs().max().clamp_min(max(1e-3 * cancel, 1e-30))
+    assert ((got - ref).abs().max() / scale).item() <= 1e-2, what
+    eps = {BF16: 2.0 ** -8, F16: 2.0 ** -11, F32: 2.0 ** -20}[dt]
+    quantum = {BF16: 0.0, F16: 2.0 ** -24, F32: 0.0}[dt]      # fp16 subnormal spacing
+    bound = ulps * eps * ref.abs() + 1e-6 * scale + 8 * 2.0 ** -23 * cancel + quantum
+    bad = ((got - ref).abs() > bound)
+    assert not bad.any(), f"{what}: {int(bad.sum())} elements beyond {ulps} ulp"
+
+
+# ------------------------------------------------------------------ RMSNorm
+NORM_CASES = [
+    # n, d, x dtype, w dtype, eps      (first one: BASELINE config 1 at 1/8 of the rows)
+    (1024, 1024, BF16, F32, 1e-6), (64, 8192, BF16, BF16, 1e-6), (33, 768, F16, F16, 1e-5),
+    (17, 100, F32, F32, 1e-6), (5, 7, BF16, F32, 1e-6), (300, 5120, BF16, F32, 1e-6),
+    (16, 64, BF16, BF16, 1e-6), (3, 1, F32, F32, 1e-6), (6, 8, F32, F32, 1e-6), (1, 3, F32, F32, 1e-6),
+    (9, 16384, BF16, F32, 1e-6), (4, 40000, F16, F32, 1e-6), (130, 3072, F32, F32, 1e-6),
+    (7, 12288, BF16, BF16, 1e-5), (2, 24576, BF16, F32, 1e-5),
+]
+
+
+@pytest.mark.parametrize("n,d,dt,wdt,eps", NORM_CASES)
+def test_rmsnorm_fwd_bwd(n, d, dt, wdt, eps):
+    g = gen(1001)
+    x = torch.randn(n, d, generator=g).to(dt)
+    w = (1 + 0.02 * torch.randn(d, generator=g)).to(wdt)
+    dy = torch.randn(n, d, generator=g).to(dt)
+    oy, orstd = O.rms_norm(x, w, eps)
+    odx, odw = O.rms_norm_bwd(x, w, dy, eps)
+    xd, wd, dyd = x.to(DEV), w.to(DEV), dy.to(DEV)
+    y, rstd = _hip.rmsnorm_fwd(xd, wd, eps)
+    dx, dw = _hip.rmsnorm_bwd(xd, wd, rstd, dyd)
+    torch.cuda.synchronize()
+    assert y.dtype == dt and dx.dtype == dt and dw.dtype == wdt
+    assert_close_lowp(y, oy, dt, "y")
+    natural = (dy.float().abs().max() * w.float().abs().max() * orstd.max()).item()
+    assert_close_lowp(dx, odx, dt, "dx", ulps=3.0, cancel=natural)
+    assert rel_max(rstd, orstd) < 1e-5
+    # dw: fp32 accumulation on both sides; compare against the fp64 sum too
+    _, odw64 = O.rms_norm_bwd(x, w.double(), dy, eps, acc=torch.float64)
+    assert rel_max(dw, odw64) <= (1e-2 if wdt != F32 else 1e-4)
+    assert rel_max(dw, odw) <= 1e-2
+    # frozen weight: no dw, same dx
+    dx2, none = _hip.rmsnorm_bwd(xd, wd, rstd, dyd, want_dw=False)
+    assert none is None and torch.equal(dx2, dx)
+
+
+def test_rmsnorm_is_deterministic_and_leaves_inputs_alone():
+    g = gen(7)
+    x = torch.randn(2048, 1024, generator=g).bfloat16().to(DEV)
+    w = torch.randn(1024, generator=g).to(DEV)
+    dy = torch.randn(2048, 1024, generator=g).bfloat16().to(DEV)
+    keep = x.clone()
+    y1, r1 = _hip.rmsnorm_fwd(x, w, 1e-6)
+    dx1, dw1 = _hip.rmsnorm_bwd(x, w, r1, dy)
+    y2, r2 = _hip.rmsnorm_fwd(x, w, 1e-6)
+    dx2, dw2 = _hip.rmsnorm_bwd(x, w, r2, dy)
+    assert torch.equal(y1, y2) and torch.equal(dx1, dx2) and torch.equal(dw1, dw2)   # bit for bit
+    assert torch.equal(x, keep)
+
+
+def test_rmsnorm_unaligned_views_take_the_any_width_path():
+    g = gen(8)
+    base = torch.randn(6 * 512 + 3, generator=g).bfloat16().to(DEV)
+    x = base[3:].view(6, 512)                        # data pointer is 6 bytes off a 16-byte line
+    w = torch.ones(512, device=DEV)
+    y, _ = _hip.rmsnorm_fwd(x, w, 1e-6)
+    oy, _ = O.rms_norm(x.cpu(), w.cpu(), 1e-6)
+    assert_close_lowp(y, oy, BF16, "y on an unaligned view")
+
+
+ADD_CASES = [(256, 8192, BF16, F32, 1e-5), (9, 24, F32, F32, 1e-6), (10, 33, BF16, BF16, 1e-6),
+             (6, 8, F32, F32, 1e-6), (5, 7, F32, F32, 1e-6), (40, 4096, F16, F16, 1e-5),
+             (12, 2048, BF16, F32, 1e-5)]
+
+
+@pytest.mark.parametrize("n,d,dt,wdt,eps", ADD_CASES)
+def test_add_rmsnorm_fwd_bwd(n, d, dt, wdt, eps):
+    g = gen(1004)
+    x = torch.randn(n, d, generator=g).to(dt)
+    dl = torch.randn(n, d, generator=g).to(dt)
+    w = (1 + 0.02 * torch.randn(d, generator=g)).to(wdt)
+    gy = torch.randn(n, d, generator=g).to(dt)
+    gxn = torch.randn(n, d, generator=g).to(dt)
+    oxn, oy, orstd = O.add_rms_norm(x, dl, w, eps)
+    odx, odw = O.add_rms_norm_bwd(oxn, w, gy, gxn, eps)
+    odx0, _ = O.add_rms_norm_bwd(oxn, w, gy, None, eps)
+    xn, y, rstd = _hip.add_rmsnorm_fwd(x.to(DEV), dl.to(DEV), w.to(DEV), eps)
+    dx, dw = _hip.add_rmsnorm_bwd(xn, w.to(DEV), rstd, gy.to(DEV), gxn.to(DEV))
+    dx0, dw0 = _hip.add_rmsnorm_bwd(xn, w.to(DEV), rstd, gy.to(DEV), None)
+    torch.cuda.synchronize()
+    assert torch.equal(xn.cpu(), oxn), "xn must be exactly x + delta in x's dtype"
+    assert_close_lowp(y, oy, dt, "y")
+    natural = (gy.float().abs().max() * w.float().abs().max() * orstd.max()).item()
+    assert_close_lowp(dx, odx, dt, "dx", ulps=3.0, cancel=natural)
+    assert_close_lowp(dx0, odx0, dt, "dx without a residual gradient", ulps=3.0, cancel=natural)
+    assert rel_max(dw, odw) <= 1e-2 and torch.equal(dw, dw0)
+    assert rel_max(rstd, orstd) < 1e-5
+
+
+# ------------------------------------------------------------------ cross entropy
+CE_CASES = [(512, 32000, BF16), (7, 50257, BF16), (5, 1000, F32), (4, 7, F16), (9, 16, F32),
+            (3, 128256, BF16), (6, 32001, F32), (33, 4096, F16), (2, 1, F32), (64, 50257, F32)]
+
+
+@pytest.mark.parametrize("n,v,dt", CE_CASES)
+def test_ce_fwd_bwd(n, v, dt):
+    g = gen(1002)
+    lg = (2 * torch.randn(n, v, generator=g)).to(dt)
+    y = torch.randint(0, v, (n,), generator=g)
+    y[torch.rand(n, generator=g) < 0.2] = -100
+    o32, ograd = O.cross_entropy(lg, y)
+    o64, _ = O.cross_entropy(lg, y, acc=torch.float64)
+    lgd, yd = lg.to(DEV), y.to(DEV)
+    loss, lse, nv, rows = _hip.ce_fwd(lgd, yd, -100, "mean")
+    go = torch.tensor(0.5, device=DEV)
+    dl = _hip.ce_bwd(lgd, yd, lse, nv, go, -100)
+    total, _, _, _ = _hip.ce_fwd(lgd, yd, -100, "sum")
+    torch.cuda.synchronize()
+    n_valid = max(1, int((y != -100).sum()))
+    assert nv.item() == n_valid
+    assert loss.item() == pytest.approx(o64.item(), rel=1e-4, abs=1e-7)
+    assert loss.item() == pytest.approx(o32.item(), rel=1e-4, abs=1e-7)
+    assert total.item() == pytest.approx(o64.item() * n_valid, rel=1e-4, abs=1e-6)
+    assert_close_lowp(dl, ograd.float() * 0.5, dt, "dlogits", ulps=3.0, cancel=0.5 / n_valid)
+    ign = (y == -100)
+    assert not dl.cpu()[ign].any(), "ignored rows get exact zeros"
+    if (~ign).any():                      # softmax - onehot sums to zero on every valid row
+        assert dl.float().cpu()[~ign].sum(-1).abs().max() < (2e-2 if dt != F32 else 1e-5) * 0.5 / n_valid * 8
+    lse_ref = torch.logsumexp(lg.double(), -1)
+    assert torch.allclose(lse.cpu().double(), lse_ref, rtol=1e-5, atol=1e-5)
+
+
+def test_ce_known_answers_on_gpu():
+    # all ignored -> 0.0 and a zero gradient; reference tests/test_edge_cases.py:21-28
+    lg = torch.randn(6, 16, device=DEV)
+    y = torch.full((6,), -100, device=DEV)
+    loss, lse, nv, _ = _hip.ce_fwd(lg, y, -100, "mean")
+    dl = _hip.ce_bwd(lg, y, lse, nv, None, -100)
+    assert loss.item() == 0.0 and nv.item() == 1.0 and not dl.any()
+    # uniform logits -> log(V)
+    loss, *_ = _hip.ce_fwd(torch.zeros(3, 10, device=DEV), torch.tensor([0, 5, 9], device=DEV), -100, "mean")
+    assert loss.item() == pytest.approx(math.log(10), rel=1e-6)
+    # a different ignore_index
+    y2 = torch.tensor([1, 2, 3, 2, 2, 0], device=DEV)
+    loss2, *_ = _hip.ce_fwd(lg, y2, 2, "mean")
+    ref, _ = O.cross_entropy(lg.cpu(), y2.cpu(), ignore_index=2)
+    assert loss2.item() == pytest.approx(ref.item(), rel=1e-5)
+
+
+# ------------------------------------------------------------------ KL
+KL_CASES = [(64, 128256, BF16, 2.0), (6, 5000, F32, 1.0), (3, 1, F32, 1.0), (5, 50257, BF16, 1.0),
+            (4, 7, F32, 1.0), (4, 64, F32, 1.0), (4, 1000, F32, 1.0), (9, 32000, F16, 1.5),
+            (2, 5000, F32, 4.0)]
+
+
+@pytest.mark.parametrize("n,v,dt,T", KL_CASES)
+def test_kl_fwd_bwd(n, v, dt, T):
+    g = gen(1005)
+    s = (3 * torch.randn(n, v, generator=g)).to(dt)
+    t = (s.float() + 0.5 * torch.randn(n, v, generator=g)).to(dt)
+    o64, _ = O.kl_div(s, t, "mean", T, acc=torch.float64)
+    orow, _ = O.kl_div(s, t, "none", T, acc=torch.float64)
+    _, ograd = O.kl_div(s, t, "mean", T)
+    sd, td = s.to(DEV), t.to(DEV)
+    loss, rows, ls, lt = _hip.kl_fwd(sd, td, 1.0 / T, "mean")
+    total, *_ = _hip.kl_fwd(sd, td, 1.0 / T, "sum")
+    gs = _hip.kl_bwd(sd, td, ls, lt, None, False, dt, 1.0 / T, 1.0 / n)
+    torch.cuda.synchronize()
+    assert loss.item() == pytest.approx(o64.item(), rel=1e-4, abs=2e-7)
+    assert total.item() == pytest.approx(o64.item() * n, rel=1e-4, abs=2e-6)
+    assert torch.allclose(rows.cpu().double(), orow, rtol=2e-4, atol=2e-6)
+    assert_close_lowp(gs, ograd, dt, "dstudent", ulps=3.0, cancel=1.0 / (T * n))
+    assert torch.allclose(ls.cpu().double(), torch.logsumexp(s.double() / T, -1), rtol=1e-5, atol=1e-5)
+    assert torch.allclose(lt.cpu().double(), torch.logsumexp(t.double() / T, -1), rtol=1e-5, atol=1e-5)
+    # per-row upstream gradients and an fp32 gradient buffer
+    up = torch.rand(n, generator=g)
+    gs32 = _hip.kl_bwd(sd, td, ls, lt, up.to(DEV), True, F32, 1.0 / T, 1.0)
+    _, g_none = O.kl_div(s.float(), t.float(), "none", T)
+    want = g_none * up[:, None]
+    tol = (1e-2 if dt != F32 else 1e-4) * want.abs().max().item() + 1e-6 / T
+    assert (gs32.cpu() - want).abs().max().item() <= tol
+
+
+def test_kl_known_answers_on_gpu():
+    s = torch.randn(5, 777, device=DEV)
+    loss, rows, ls, lt = _hip.kl_fwd(s, s.clone(), 1.0, "mean")
+    gs = _hip.kl_bwd(s, s.clone(), ls, lt, None, False, F32, 1.0, 0.2)
+    assert abs(loss.item()) < 1e-6 and gs.abs().max().item() < 1e-7   # identical -> 0
+    t = torch.randn(5, 777, device=DEV)
+    _, rows, _, _ = _hip.kl_fwd(s, t, 1.0, "none")
+    assert (rows > 0).all()                                           # Gibbs
+    keep = s.clone()
+    assert torch.equal(s, keep)
+
+
+# ------------------------------------------------------------------ top-k
+TOPK_CASES = [(32, 128256, 64, BF16), (8, 4096, 64, F32), (4, 64, 8, F32), (3, 5000, 512, BF16),
+              (4, 20000, 100, F16), (2, 300000, 17, BF16), (3, 9000, 5, F32), (2, 100, 99, F32),
+              (1, 512, 512, F32), (5, 1, 1, F32), (2, 600, 4, F32), (4, 5000, 512, F32),
+              (2, 1025, 3, BF16), (3, 70000, 512, F32), (6, 50257, 64, BF16), (2, 140000, 64, F32)]
+
+
+@pytest.mark.parametrize("n,v,k,dt", TOPK_CASES)
+def test_topk_is_bit_exact(n, v, k, dt):
+    g = gen(1006)
+    x = (3 * torch.randn(n, v, generator=g)).to(dt)
+    ov, oi = O.topk(x, k)
+    vals, idx = _hip.topk(x.to(DEV), k, torch.int32)
+    vals64, idx64 = _hip.topk(x.to(DEV), k, torch.int64)
+    torch.cuda.synchronize()
+    assert idx.dtype == torch.int32 and idx64.dtype == torch.int64
+    assert torch.equal(idx.cpu().long(), oi) and torch.equal(idx64.cpu(), oi)
+    assert torch.equal(vals.cpu(), ov) and torch.equal(vals64.cpu(), ov)
+
+
+def test_topk_ties_nans_zeros_and_degenerate_rows():
+    def run(t, k):
+        _, i = _hip.topk(t.to(DEV), k, torch.int64)
+        return i.cpu()
+    # reference tests/test_topk.py:68-85
+    assert run(torch.tensor([[1.0, 3.0, 3.0, 2.0, 3.0]]), 3).tolist() == [[1, 2, 4]]
+    assert run(torch.tensor([[float("nan"), 1.0, 2.0, float("nan"), 0.0]]), 3).tolist() == [[0, 3, 2]]
+    assert run(torch.tensor([[float("inf"), float("nan"), 0.0, -0.0, 0.0]]), 5).tolist() == [[1, 0, 2, 3, 4]]
+    # long runs of equal values force the exact path (every element is a candidate)
+    for dt in (BF16, F32):
+        for v, k in ((5000, 7), (131000, 64), (2049, 512)):
+            z = torch.zeros(3, v, dtype=dt)
+            assert torch.equal(run(z, k), torch.arange(k).expand(3, k))
+    g = gen(11)
+    x = torch.randint(0, 3, (4, 40000), generator=g).to(BF16)         # three distinct values
+    assert torch.equal(run(x, 300), O.topk(x, 300)[1])
+    x = torch.randint(0, 50, (4, 70000), generator=g).float()
+    x[:, ::7] = float("nan")
+    x[:, 5::11] = float("-inf")
+    assert torch.equal(run(x, 512), O.topk(x, 512)[1])
+    # negative NaN payloads and a row of -inf
+    x = torch.full((2, 3000), float("-inf"))
+    x[0, 17] = -torch.tensor(float("nan"))
+    assert torch.equal(run(x, 4), O.topk(x, 4)[1])
+
+
+def test_topk_unaligned_rows():
+    g = gen(12)
+    for dt, v in ((BF16, 50257), (F32, 32001), (F16, 4099)):
+        x = (3 * torch.randn(5, v, generator=g)).to(dt)
+        _, idx = _hip.topk(x.to(DEV), 33, torch.int32)
+        assert torch.equal(idx.cpu().long(), O.topk(x, 33)[1])
+    base = (3 * torch.randn(3 * 9000 + 1, generator=g)).bfloat16().to(DEV)
+    x = base[1:].view(3, 9000)                                        # base pointer off by 2 bytes
+    _, idx = _hip.topk(x, 20, torch.int32)
+    assert torch.equal(idx.cpu().long(), O.topk(x.cpu(), 20)[1])
+
+
+# ------------------------------------------------------------------ softmax
+@pytest.mark.parametrize("n,v,dt", [(4, 64, F32), (5, 1000, F32), (3, 4096, F32), (7, 1, F32),
+                                     (8, 50257, BF16), (6, 300, F16), (2, 128256, BF16)])
+def test_softmax(n, v, dt):
+    x = torch.randn(n, v, generator=gen(21)).to(dt)
+    y = _hip.softmax_fwd(x.to(DEV))
+    ref = O.softmax(x)
+    assert_close_lowp(y, ref, dt, "softmax", ulps=2.0)
+    assert torch.allclose(y.float().sum(-1).cpu(), torch.ones(n), atol=1e-2)
+
+
+def test_softmax_nan_and_neg_inf_rows():
+    y = _hip.softmax_fwd(torch.tensor([[float("nan"), 1.0, 2.0]], device=DEV))
+    assert math.isnan(y[0, 0].item())
+    y = _hip.softmax_fwd(torch.full((1, 3), float("-inf"), device=DEV))
+    assert all(math.isnan(v) for v in y[0].tolist())
+
+
+# ------------------------------------------------------------------ router
+def router_inputs(n, e, seed, dtype=F32):
+    """Logits on a 2**-12 grid (distinct values differ by far more than any exp rounding), 1% of
+    the rows with four copies of the row maximum and four copies of another value."""
+    g = gen(seed)
+    lg = torch.round(torch.randn(n, e, generator=g) * 4096) / 4096
+    rows = torch.randperm(n, generator=g)[: max(1, n // 100)]
+    for r in rows.tolist():
+        cols = torch.randperm(e, generator=g)[: min(8, e)]
+        lg[r, cols[: len(cols) // 2]] = lg[r].max().clone()
+        lg[r, cols[len(cols) // 2:]] = lg[r, cols[-1]].clone()
+    return lg.to(dtype)
+
+
+ROUTE_CASES = [(16384, 64, 2), (1000, 8, 2), (513, 128, 4), (100, 300, 8), (1, 64, 2), (70000, 16, 1),
+               (257, 512, 8), (4099, 64, 6), (3, 2, 2)]
+
+
+@pytest.mark.parametrize("n,e,k", ROUTE_CASES)
+def test_route_is_bit_exact(n, e, k):
+    lg = router_inputs(n, e, 1003)
+    oi, ow, oc, oslot, oorder = O.router(lg, k)
+    idx, w, counts, slot, order = _hip.route(lg.to(DEV), k)
+    torch.cuda.synchronize()
+    assert idx.dtype == torch.int32 and counts.dtype == torch.int32
+    assert torch.equal(idx.cpu().long(), oi), "expert indices"
+    assert torch.equal(counts.cpu().long(), oc), "per-expert counts"
+    assert torch.equal(slot.cpu().long(), oslot), "token -> slot permutation"
+    assert torch.equal(order.cpu().long(), oorder), "slot -> token permutation"
+    assert torch.allclose(w.cpu(), ow, rtol=1e-5, atol=0)
+    i2, w2, c2, none_a, none_b = _hip.route(lg.to(DEV), k, want_permutation=False)
+    assert none_a is None and none_b is None and torch.equal(i2, idx) and torch.equal(c2, counts)
+
+
+def test_route_half_precision_logits_and_all_equal_rows():
+    lg = router_inputs(300, 64, 5, BF16)
+    oi, ow, oc, oslot, oorder = O.router(lg, 2)
+    idx, w, counts, slot, order = _hip.route(lg.to(DEV), 2)
+    assert torch.equal(idx.cpu().long(), oi) and torch.equal(order.cpu().long(), oorder)
+    z = torch.zeros(130, 64, device=DEV)
+    idx, w, counts, slot, order = _hip.route(z, 2)
+    assert torch.equal(idx.cpu(), torch.tensor([[0, 1]], dtype=torch.int32).expand(130, 2))
+    assert counts.cpu().tolist() == [130, 130] + [0] * 62
+    assert torch.allclose(w.cpu(), torch.full((130, 2), 0.5))
+    assert order.cpu().tolist() == list(range(0, 260, 2)) + list(range(1, 260, 2))

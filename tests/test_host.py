@@ -1,0 +1,372 @@
+"""Host-side behaviour of the ``fm.kernels`` surface on CPU: gate, stats, dispatch, the torch
+path's numbers (checked against the oracle), module wrappers and the op registrations.
+
+These mirror the reference's CPU suite (tests/test_kernels.py, test_kernel_ops.py,
+test_nn_blocks.py, test_edge_cases.py, test_topk.py, test_softmax.py) at the level of
+behaviour: same names, same arguments, same errors.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+import forgeminds_amd as fm
+from forgeminds_amd import kernels
+from forgeminds_amd.kernels import _ops
+from forgeminds_amd.loss import chunked_cross_entropy, logits_cross_entropy
+from oracle import oracle as O
+
+
+# ------------------------------------------------------------------ surface
+def test_public_surface_has_the_reference_names():
+    # forgemind/kernels/__init__.py:42-48 plus the two additions of this build
+    for name in ["HAS_TRITON", "set_backend", "get_backend", "stats", "reset_stats", "rms_norm",
+                 "add_rms_norm", "qk_norm_rope", "swiglu", "swiglu_split", "kl_div_logits", "kl_div",
+                 "kl_distill_loss", "distill_kl", "newton_schulz", "topk", "softmax", "enable",
+                 "patch", "revert", "available", "use_custom_ops", "cross_entropy", "moe_route"]:
+        assert hasattr(kernels, name), name
+        assert name in kernels.__all__, name
+    assert kernels.available() is (torch.cuda.is_available() and kernels._common.extension_available())
+
+
+def test_backend_switch_and_stats():
+    with pytest.raises(ValueError, match="unknown kernel backend"):
+        kernels.set_backend("cuda")
+    for name in ("auto", "fallback", "triton", "hip"):
+        kernels.set_backend(name)
+        assert kernels.get_backend() == name
+    kernels.set_backend("auto")
+    kernels.reset_stats()
+    kernels.rms_norm(torch.randn(4, 8), torch.randn(8), 1e-6)
+    st = kernels.stats()
+    assert st["fast"] == 0 and st["fallback"] == 1 and st["reasons"] == {"not cuda": 1}
+    kernels.set_backend("fallback")
+    kernels.reset_stats()
+    kernels.kl_div_logits(torch.randn(2, 8), torch.randn(2, 8))
+    assert kernels.stats()["reasons"].get("backend=fallback") == 1
+
+
+def test_forced_backend_refuses_cpu_tensors_loudly():
+    kernels.set_backend("hip")
+    with pytest.raises(RuntimeError, match="forced"):
+        kernels.rms_norm(torch.randn(4, 8), torch.randn(8), 1e-6)
+
+
+def test_stats_are_not_touched_while_tracing():
+    # reference tests/test_kernels.py:188-199
+    kernels.reset_stats()
+    w, x = torch.randn(8), torch.randn(4, 8)
+    fn = torch.compile(lambda t: kernels.rms_norm(t, w, 1e-6), backend="aot_eager", fullgraph=True)
+    before = kernels.stats()
+    out = fn(x)
+    assert kernels.stats() == before
+    assert torch.allclose(out, F.rms_norm(x, (8,), w, 1e-6), atol=2e-6)
+
+
+def test_ops_are_registered_and_dispatch_flag_works():
+    # reference tests/test_kernel_ops.py:112-117, 168-175
+    names = {n for n in dir(torch.ops.forgemind) if not n.startswith("_")}
+    for op in ("rms_norm", "add_rms_norm"):
+        assert op in names and f"{op}_backward" in names
+    assert _ops.wanted() is False
+    assert _ops.use_custom_ops(True) is True and _ops.wanted() is True
+    assert _ops.use_custom_ops(False) is False
+    assert _ops.use_custom_ops(None) is False
+    assert _ops.available() is True
+
+
+def test_op_path_is_not_entered_when_the_kernel_cannot_run():
+    # reference tests/test_kernel_ops.py:187-199
+    kernels.set_backend("fallback")
+    _ops.use_custom_ops(True)
+    x, w = torch.randn(4, 8), torch.randn(8)
+    kernels.reset_stats()
+    y = kernels.rms_norm(x, w, 1e-6)
+    assert torch.allclose(y, F.rms_norm(x, (8,), w, 1e-6), atol=2e-6)
+    assert kernels.stats()["fallback"] == 1
+
+
+def test_fake_impls_have_the_real_shapes_and_dtypes():
+    # reference tests/test_kernel_ops.py:156-165, without running a kernel
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    with FakeTensorMode() as mode:
+        x = mode.from_tensor(torch.empty(3, 5, 16, dtype=torch.bfloat16))
+        w = mode.from_tensor(torch.empty(16, dtype=torch.float32))
+        y, rstd = torch.ops.forgemind.rms_norm(x, w, 1e-6)
+        assert y.shape == x.shape and y.dtype == x.dtype
+        assert rstd.shape == (15,) and rstd.dtype == torch.float32
+        xn, y2, r2 = torch.ops.forgemind.add_rms_norm(x, x, w, 1e-6)
+        assert xn.shape == x.shape and y2.dtype == x.dtype and r2.shape == (15,)
+        dx, dw = torch.ops.forgemind.rms_norm_backward(x, w, rstd, x)
+        assert dx.shape == x.shape and dw.shape == w.shape and dw.dtype == w.dtype
+        dx, dd, dw = torch.ops.forgemind.add_rms_norm_backward(x, w, rstd, x, x)
+        assert dd.shape == x.shape and dw.dtype == torch.float32
+
+
+# ------------------------------------------------------------------ torch path == oracle
+@pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16, torch.float64])
+def test_rms_norm_torch_path_matches_oracle(dt):
+    torch.manual_seed(0)
+    x = torch.randn(6, 24).to(dt).requires_grad_(True)
+    w = torch.randn(24).to(dt).requires_grad_(True)
+    g = torch.randn(6, 24).to(dt)
+    y = kernels.rms_norm(x, w, 1e-6)
+    y.backward(g)
+    acc = torch.float64 if dt == torch.float64 else torch.float32
+    oy, _ = O.rms_norm(x.detach(), w.detach(), 1e-6, acc)
+    odx, odw = O.rms_norm_bwd(x.detach(), w.detach(), g, 1e-6, acc)
+    tol = dict(atol=3e-2, rtol=2e-2) if dt == torch.bfloat16 else dict(atol=2e-6, rtol=1e-5)
+    assert y.dtype == dt and torch.allclose(y.float(), oy.float(), **tol)
+    assert torch.allclose(x.grad.float(), odx.float(), **tol)
+    assert torch.allclose(w.grad.float(), odw.float(), atol=1e-1 if dt == torch.bfloat16 else 1e-5)
+
+
+def test_add_rms_norm_torch_path():
+    torch.manual_seed(0)
+    x, d, w = torch.randn(4, 8), torch.randn(4, 8), torch.randn(8)
+    xn, y = kernels.add_rms_norm(x, d, w)
+    oxn, oy, _ = O.add_rms_norm(x, d, w)
+    assert torch.equal(xn, oxn) and torch.allclose(y, oy, atol=2e-6)
+    # mismatching shapes never reach a kernel (reference norm.py:1272)
+    xn2, _ = kernels.add_rms_norm(x, d[:1], w)
+    assert xn2.shape == x.shape
+
+
+def test_kl_surface():
+    torch.manual_seed(0)
+    s, t = torch.randn(6, 40), torch.randn(6, 40)
+    for red in ("mean", "sum", "none"):
+        got = kernels.kl_div_logits(s, t, red)
+        exp, _ = O.kl_div(s, t, red)
+        assert torch.allclose(got, exp, rtol=1e-5, atol=1e-6)
+    s2 = s.clone().requires_grad_(True)
+    kernels.kl_div_logits(s2, t, "mean", temperature=2.0).backward()
+    assert torch.allclose(s2.grad, O.kl_div(s, t, "mean", 2.0)[1], atol=1e-6)
+    with pytest.raises(ValueError, match="reduction must be"):
+        kernels.kl_div_logits(s, t, "avg")
+    assert kernels.kl_div is kernels.kl_div_logits and kernels.distill_kl is kernels.kl_distill_loss
+    keep = s.clone()
+    kernels.kl_div_logits(s.requires_grad_(True), t).backward()       # inputs are never mutated
+    assert torch.equal(s.detach(), keep)
+
+
+def test_kl_distill_chunking_is_transparent():
+    # reference tests/test_kernels.py:143-156
+    torch.manual_seed(0)
+    n, d, v = 8, 4, 24
+    hs, ht, w, wt = torch.randn(n, d), torch.randn(n, d), torch.randn(v, d), torch.randn(v, d)
+    head = lambda z: z @ wt.t()
+    full = kernels.kl_distill_loss(hs, ht, w, head, chunk=1000)
+    chunked = kernels.kl_distill_loss(hs, ht, w, head, chunk=3)
+    exp, _ = O.kl_div(hs @ w.t(), ht @ wt.t(), "mean")
+    assert full.item() == pytest.approx(exp.item(), rel=1e-5)
+    assert chunked.item() == pytest.approx(exp.item(), rel=1e-5)
+    wt_p = wt.clone().requires_grad_(True)
+    hs_p = hs.clone().requires_grad_(True)
+    kernels.kl_distill_loss(hs_p, ht, w, lambda z: z @ wt_p.t()).backward()
+    assert wt_p.grad is None and hs_p.grad is not None              # the teacher is not trained
+
+
+def test_topk_surface_and_errors():
+    # reference tests/test_topk.py:68-124
+    v, idx = kernels.topk(torch.tensor([[1.0, 3.0, 3.0, 2.0, 3.0]]), 3)
+    assert idx[0].tolist() == [1, 2, 4] and idx.dtype == torch.int64
+    v, idx = kernels.topk(torch.tensor([[float("nan"), 1.0, 2.0, float("nan"), 0.0]]), 3)
+    assert idx[0].tolist() == [0, 3, 2] and math.isnan(v[0, 0]) and v[0, 2].item() == 2.0
+    x = torch.randn(4, 8)
+    for bad in (9, 0):
+        with pytest.raises(RuntimeError, match="selected index k out of range"):
+            kernels.topk(x, bad)
+    with pytest.raises(ValueError, match="ndim"):
+        kernels.topk(torch.tensor(3.0), 1)
+    tv, ti = torch.topk(x, 2, dim=0)
+    v, i = kernels.topk(x, 2, dim=0)
+    assert torch.equal(v, tv) and torch.equal(i, ti)
+    xg = torch.randn(3, 128, requires_grad=True)
+    v, idx = kernels.topk(xg, 10)
+    assert not idx.requires_grad
+    (v * 2).sum().backward()
+    assert int((xg.grad != 0).sum()) == 30
+    ov, oi = O.topk(xg.detach(), 10)
+    assert torch.equal(idx, oi) and torch.equal(v.detach(), ov)
+    kernels.reset_stats()
+    kernels.topk(torch.randint(0, 100, (4, 64)), 8)
+    assert kernels.stats()["fallback"] >= 1
+
+
+def test_softmax_surface():
+    # reference tests/test_softmax.py
+    x = torch.randn(4, 64, requires_grad=True)
+    y = kernels.softmax(x)
+    assert torch.allclose(y, torch.softmax(x, -1), atol=1e-6)
+    assert torch.allclose(kernels.softmax(x, dim=0), torch.softmax(x, 0))
+    with pytest.raises(ValueError, match="ndim"):
+        kernels.softmax(torch.tensor(1.0))
+    yb = kernels.softmax(x, dtype=torch.bfloat16)
+    assert yb.dtype == torch.bfloat16
+    yb.float().sum().backward()
+    assert x.grad is not None and x.grad.dtype == torch.float32
+
+
+def test_cross_entropy_surface_and_edge_cases():
+    torch.manual_seed(0)
+    lg = torch.randn(9, 16, requires_grad=True)
+    y = torch.randint(0, 16, (9,))
+    y[2] = -100
+    loss = kernels.cross_entropy(lg, y)
+    loss.backward()
+    ol, og = O.cross_entropy(lg.detach(), y)
+    assert loss.dtype == torch.float32 and loss.item() == pytest.approx(ol.item(), rel=1e-6)
+    assert torch.allclose(lg.grad, og, atol=1e-7)
+    s = kernels.cross_entropy(lg.detach(), y, reduction="sum")
+    assert s.item() == pytest.approx(ol.item() * 8, rel=1e-6)
+    with pytest.raises(ValueError):
+        kernels.cross_entropy(lg, y, reduction="none")
+    with pytest.raises(ValueError):
+        kernels.cross_entropy(lg, y[:3])
+
+
+def test_loss_module_edge_cases():
+    # reference tests/test_edge_cases.py:21-56
+    h = torch.randn(6, 8, requires_grad=True)
+    w = torch.randn(16, 8, requires_grad=True)
+    loss = chunked_cross_entropy(h, w, torch.full((6,), -100), chunk=4)
+    assert loss.item() == 0.0
+    loss.backward()
+    assert h.grad is not None
+    assert chunked_cross_entropy(torch.randn(0, 8, requires_grad=True), w,
+                                 torch.zeros(0, dtype=torch.long)).item() == 0.0
+    torch.manual_seed(0)
+    h, w, y = torch.randn(9, 8), torch.randn(16, 8), torch.randint(0, 16, (9,))
+    y[2] = -100
+    exp = F.cross_entropy(h @ w.t(), y, ignore_index=-100, reduction="mean")
+    assert chunked_cross_entropy(h, w, y, chunk=4).item() == pytest.approx(exp.item(), rel=1e-5)
+    lg, y3 = torch.randn(2, 5, 16), torch.randint(0, 16, (2, 5))
+    full = logits_cross_entropy(lg, y3)
+    assert full.item() == pytest.approx(logits_cross_entropy(lg, y3, chunk=3).item(), rel=1e-6)
+    assert full.item() == pytest.approx(F.cross_entropy(lg.reshape(10, 16), y3.reshape(10)).item(), rel=1e-5)
+
+
+def test_moe_route_torch_path_matches_oracle():
+    torch.manual_seed(0)
+    logits = torch.round(torch.randn(200, 16) * 16) / 16
+    r = kernels.moe_route(logits, 2)
+    idx, w, counts, slot, order = O.router(logits, 2)
+    assert torch.equal(r.idx.long(), idx) and torch.allclose(r.weights, w, rtol=1e-6)
+    assert torch.equal(r.counts.long(), counts)
+    assert torch.equal(r.slot.long(), slot) and torch.equal(r.order.long(), order)
+    assert r.idx.dtype == torch.int32 and r.order.dtype == torch.int32
+    with pytest.raises(RuntimeError, match="selected index k out of range"):
+        kernels.moe_route(logits, 17)
+    with pytest.raises(ValueError):
+        kernels.moe_route(logits[0], 2)
+
+
+def test_router_module_matches_the_reference_expression():
+    # forgemind/moe.py:86-96 written out
+    torch.manual_seed(0)
+    router = fm.moe.Router(32, 8, 2)
+    x = torch.randn(50, 32)
+    w, idx, aux, z = router(x)
+    logits = router.gate(x).float()
+    probs = logits.softmax(-1)
+    tw, _ = probs.topk(2, dim=-1)
+    assert torch.allclose(w, tw / tw.sum(-1, keepdim=True), rtol=1e-5)
+    oa, oz = O.router_aux(logits.detach(), idx)
+    assert aux.item() == pytest.approx(oa.item(), rel=1e-5) and z.item() == pytest.approx(oz.item(), rel=1e-5)
+    plan = router.last_plan
+    assert torch.equal(plan.order, torch.sort(idx.reshape(-1), stable=True).indices)
+    assert torch.equal(plan.tok, plan.order // 2)
+    assert torch.equal(plan.offsets.long(), plan.counts.cumsum(0))
+    (w.sum() + aux + z).backward()
+    assert router.gate.weight.grad is not None
+
+
+# ------------------------------------------------------------------ modules and patching
+def test_nn_rmsnorm_is_a_drop_in():
+    # reference tests/test_nn_blocks.py:40-114
+    torch.manual_seed(0)
+    ours, theirs = fm.nn.RMSNorm(16, eps=1e-5), nn.RMSNorm(16, eps=1e-5)
+    theirs.load_state_dict(ours.state_dict())
+    x = torch.randn(3, 5, 16)
+    assert torch.allclose(ours(x), theirs(x), atol=2e-6)
+    normed, res = ours.forward_with_residual(x, x)
+    assert torch.equal(res, x + x) and torch.allclose(normed, theirs(x + x), atol=2e-6)
+    n0, r0 = ours.forward_with_residual(x)
+    assert torch.equal(r0, x) and torch.allclose(n0, ours(x), atol=2e-6)
+    with pytest.raises(ValueError):
+        ours(torch.randn(3, 8))
+    with pytest.raises(ValueError):
+        ours.forward_with_residual(x, x[:1])
+    with pytest.raises(ValueError):
+        fm.nn.RMSNorm(0)
+    xd = x.double().requires_grad_(True)
+    m = fm.nn.RMSNorm(16).double()
+    assert torch.autograd.gradcheck(lambda t: m(t), (xd,), atol=1e-6)
+
+
+def test_patch_enable_revert():
+    # reference tests/test_nn_blocks.py:160-236
+    torch.manual_seed(0)
+
+    class MLP(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.w1, self.w2, self.w3 = nn.Linear(16, 32), nn.Linear(32, 16), nn.Linear(16, 32)
+
+        def forward(self, x):
+            return self.w2(F.silu(self.w1(x)) * self.w3(x))
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.norm, self.mlp = nn.RMSNorm(16), MLP()
+
+        def forward(self, x):
+            return x + self.mlp(self.norm(x))
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a, self.b = Block(), Block()
+
+        def forward(self, x):
+            return self.b(self.a(x))
+
+    net = Net()
+    x = torch.randn(4, 16)
+    ref = net(x)
+    kernels.enable(net)
+    assert net._fm_fused == {"norm": 2, "mlp": 2}
+    assert torch.allclose(net(x), ref, atol=1e-5)
+    kernels.enable(net)
+    assert net._fm_fused == {"norm": 0, "mlp": 0}                     # idempotent
+    kernels.revert(net)
+    assert net._fm_fused_reverted["restored"] == 4 and torch.allclose(net(x), ref, atol=1e-6)
+    assert kernels.patch(nn.LayerNorm(16)) is False
+    assert kernels.patch(nn.RMSNorm(16)) is True
+    m = nn.RMSNorm(16)                                                # eps=None -> finfo eps
+    exp = m(x)
+    kernels.patch(m)
+    assert torch.allclose(m(x), exp, atol=2e-6)
+    with pytest.raises(TypeError):
+        kernels.patch(nn.Linear(4, 4), kind="norm")
+    with pytest.raises(ValueError):
+        kernels.patch(nn.RMSNorm(4), kind="attention")
+
+
+def test_out_of_path_names_keep_their_torch_expression():
+    g, u = torch.randn(33), torch.randn(33)
+    assert torch.allclose(kernels.swiglu(g, u), F.silu(g) * u, atol=2e-6)
+    x = torch.randn(7, 16)
+    assert torch.allclose(kernels.swiglu_split(x), F.silu(x[..., :8]) * x[..., 8:], atol=2e-6)
+    with pytest.raises(ValueError):
+        kernels.swiglu_split(torch.randn(3, 7))
+    q = kernels.qk_norm_rope(torch.randn(2, 5, 3, 8), torch.randn(8), torch.randn(5, 4), torch.randn(5, 4))
+    assert q.shape == (2, 5, 3, 8)
+    o = kernels.newton_schulz(torch.randn(8, 16))
+    assert o.shape == (8, 16)
