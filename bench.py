@@ -315,6 +315,23 @@ def measure(torch, w, steps, warmup):
     return out
 
 
+def stream_ceiling(torch, L, dev):
+    """What a plain read sweep and a plain copy reach on this GPU (1 GiB, min of 10)."""
+    n = 1 << 30
+    src = torch.empty(n, device=dev, dtype=torch.uint8).fill_(1)
+    dst = torch.empty_like(src)
+    sink = torch.zeros(1, device=dev, dtype=torch.int32)
+    st = torch.cuda.current_stream().cuda_stream
+    out = {}
+    for mode, name, moved in ((0, "read_gbps", n), (1, "copy_gbps", 2 * n)):
+        fn = lambda: _check(L.fm_stream_probe(src.data_ptr(), dst.data_ptr(), sink.data_ptr(), n, mode, st),
+                            "fm_stream_probe")
+        _, best, _ = time_kernel_events(torch, fn, 12)
+        out[name] = round(moved / best / 1e6, 1)
+    out["note"] = "fm_stream_probe, 16-byte non-temporal accesses, one 64 KiB chunk per workgroup"
+    return out
+
+
 # ---------------------------------------------------------------------------- CPU baseline
 def cpu_baseline(torch):
     """The CPU oracle's CE forward + backward on a bounded sample of the headline workload."""
@@ -357,13 +374,16 @@ def main():
     torch.cuda.set_device(dev)
 
     if a.copy_probe:
+        # one plain copy of known size per step: what FETCH_SIZE / WRITE_SIZE are calibrated on
         n = a.copy_probe << 20
         src = torch.empty(n, device=dev, dtype=torch.uint8).fill_(1)
         dst = torch.empty_like(src)
+        st = torch.cuda.current_stream().cuda_stream
         for _ in range(max(a.steps, 1)):
-            dst.copy_(src)
+            _check(L.fm_stream_probe(src.data_ptr(), dst.data_ptr(), None, n, 1, st), "fm_stream_probe")
         torch.cuda.synchronize()
-        print(json.dumps({"copy_probe_bytes_read": n, "copy_probe_bytes_written": n, "launches": max(a.steps, 1)}))
+        print(json.dumps({"copy_probe_bytes_read": n, "copy_probe_bytes_written": n,
+                          "launches": max(a.steps, 1)}))
         return 0
 
     head = make_workload(a.workload, torch, L, dev)
@@ -401,6 +421,7 @@ def main():
             del wl
             torch.cuda.empty_cache()
         line["workloads"] = extras
+    line["hbm_ceiling_measured"] = stream_ceiling(torch, L, dev)
     line["cpu_baseline"] = None if a.no_cpu else cpu_baseline(torch)
     print(json.dumps(line))
     return 0

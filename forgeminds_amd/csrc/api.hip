@@ -15,6 +15,7 @@ const char* const kParamNames[fm_host::P_COUNT] = {
     "norm_bwd_blocks_per_cu",
     "vocab_threads",
     "norm_tpr",
+    "topk_variant",
 };
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cus[kMaxDevices];

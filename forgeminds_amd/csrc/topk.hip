@@ -334,7 +334,9 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
   const dim3 grid((unsigned)n);
 #define GO(TH, IT)                                                                               \
   hipLaunchKernelGGL((topk_kernel<T, TH, IT>), grid, dim3(TH), 0, st, xp, vp, i32, i64, v, k, vec_ok)
-  if (v <= kCap || nvec <= 256 * 4) GO(256, 4);
+  const int variant = fm_host::get_param(fm_host::P_TOPK_VARIANT);
+  if (variant == 1 && v > kCap) GO(1024, 0);
+  else if (v <= kCap || nvec <= 256 * 4) GO(256, 4);
   else if (nvec <= 1024 * 4) GO(1024, 4);
   else if (nvec <= 1024 * 16) GO(1024, 16);
   else GO(1024, 0);

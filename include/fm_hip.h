@@ -51,6 +51,14 @@ const char* fm_last_error(void);
  * value <= 0 restores the built-in heuristic. Not part of the reference surface. */
 int fm_set_param(const char* name, int value);
 
+/* STREAM-style probe with the kernels' own access pattern (16-byte non-temporal accesses, one
+ * 64 KiB chunk per workgroup): mode 0 reads `bytes` from src (sink: one uint32 on device, never
+ * written for ordinary data), mode 1 copies src to dst. Used by bench.py to report the HBM
+ * ceiling this GPU reaches and to calibrate profiler byte counters against a known transfer.
+ * No counterpart in the reference. bytes must be a multiple of 16. */
+int fm_stream_probe(const void* src, void* dst, uint32_t* sink, size_t bytes, int mode,
+                    fm_stream_t stream);
+
 /* ------------------------------------------------------------------ RMSNorm
  * Replaces _launch_rms_fwd / _rms_layernorm_forward (forgemind/kernels/norm.py:1095-1101,
  * 133-175); semantics of _fallback.rms_norm (forgemind/kernels/_fallback.py:26-30):
