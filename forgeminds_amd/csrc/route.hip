@@ -10,8 +10,9 @@
 //   route_kernel    one wave per row, experts spread over the lanes (lane l owns experts
 //                   l, l+64, ...). Wave max / sum give the softmax; each of the k picks is a
 //                   wave max over order-preserving integer keys followed by a wave min over
-//                   the tied expert indices. Each workgroup owns a contiguous tile of rows
-//                   and leaves its expert histogram in `hist[tile][e]`.
+//                   the tied expert indices. A wave keeps four rows in flight so that their
+//                   dependent reduction chains overlap. Each 16-wave workgroup owns a
+//                   contiguous tile of rows and leaves its expert histogram in `hist[tile][e]`.
 //   permute_kernel  every workgroup sums the histograms of the tiles before it (and of all
 //                   tiles, for the expert bases), then walks its own tile in ascending flat
 //                   position and gives each assignment the slot
@@ -34,86 +35,121 @@ __device__ __forceinline__ uint32_t key_of(float f) {
   return b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);
 }
 
+constexpr int kRouteThreads = 1024;   // 16 waves per tile
+constexpr int kRowsAtOnce = 4;        // rows a wave works on together (independent chains)
+
 template <typename T, int EPL>
-__global__ __launch_bounds__(256) void route_kernel(const T* __restrict__ logits,
-                                                     int32_t* __restrict__ idx,
-                                                     float* __restrict__ weights,
-                                                     int32_t* __restrict__ hist, int64_t n, int e,
-                                                     int k, int tile_rows) {
+__global__ __launch_bounds__(kRouteThreads) void route_kernel(const T* __restrict__ logits,
+                                                               int32_t* __restrict__ idx,
+                                                               float* __restrict__ weights,
+                                                               int32_t* __restrict__ hist, int64_t n,
+                                                               int e, int k, int tile_rows) {
+  constexpr int R = kRowsAtOnce;
+  constexpr int NW = kRouteThreads / 64;
   __shared__ int lh[kMaxE];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  for (int i = tid; i < e; i += 256) lh[i] = 0;
+  for (int i = tid; i < e; i += kRouteThreads) lh[i] = 0;
   __syncthreads();
   const int64_t row0 = (int64_t)blockIdx.x * tile_rows;
   const int64_t row1 = row0 + tile_rows < n ? row0 + tile_rows : n;
-  for (int64_t row = row0 + wave; row < row1; row += 4) {
-    float z[EPL];
-    float m = -INFINITY;
+  // wave w owns rows row0 + w, + NW, ...; R of them are in flight at once so that the
+  // dependent DPP / readlane chains of different rows overlap
+  for (int64_t rb = row0 + wave; rb < row1; rb += (int64_t)NW * R) {
+    float p[R][EPL];
+    uint32_t key[R][EPL];
+    bool live[R];
 #pragma unroll
-    for (int q = 0; q < EPL; ++q) {
-      const int ex = lane + 64 * q;
-      z[q] = ex < e ? Elem<T>::load1(logits + row * (int64_t)e + ex) : -INFINITY;
-      m = fmaxf(m, z[q]);
-    }
-    m = wave_max(m);
-    float p[EPL];
-    float s = 0.f;
+    for (int r = 0; r < R; ++r) {
+      const int64_t row = rb + (int64_t)r * NW;
+      live[r] = row < row1;
 #pragma unroll
-    for (int q = 0; q < EPL; ++q) {
-      p[q] = fast_exp2((z[q] - m) * kLog2e);
-      s += p[q];
+      for (int q = 0; q < EPL; ++q) {
+        const int ex = lane + 64 * q;
+        p[r][q] = (live[r] && ex < e) ? Elem<T>::load1(logits + row * (int64_t)e + ex) : -INFINITY;
+      }
     }
-    s = wave_sum(s);
-    uint32_t key[EPL];
+    float m[R], s[R];
 #pragma unroll
-    for (int q = 0; q < EPL; ++q) {
-      p[q] = p[q] / s;
-      key[q] = (lane + 64 * q) < e ? key_of(p[q]) : 0u;   // 0 is below every real key
+    for (int r = 0; r < R; ++r) {
+      m[r] = p[r][0];
+#pragma unroll
+      for (int q = 1; q < EPL; ++q) m[r] = fmaxf(m[r], p[r][q]);
     }
-    int sel_i[kMaxK];
-    float sel_p[kMaxK];
-    float wsum = 0.f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) m[r] = wave_max(m[r]);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      s[r] = 0.f;
+#pragma unroll
+      for (int q = 0; q < EPL; ++q) {
+        p[r][q] = fast_exp2((p[r][q] - m[r]) * kLog2e);
+        s[r] += p[r][q];
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) s[r] = wave_sum(s[r]);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+#pragma unroll
+      for (int q = 0; q < EPL; ++q) {
+        p[r][q] = p[r][q] / s[r];
+        key[r][q] = (lane + 64 * q) < e ? key_of(p[r][q]) : 0u;   // 0 is below every real key
+      }
+    }
+    int my_i[R];
+    float my_p[R], wsum[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) { my_i[r] = 0; my_p[r] = 0.f; wsum[r] = 0.f; }
 #pragma unroll
     for (int j = 0; j < kMaxK; ++j) {
       if (j < k) {
-        uint32_t bk = key[0];
-        int bq = 0;
+        uint32_t bk[R];
+        int bq[R], wi[R];
 #pragma unroll
-        for (int q = 1; q < EPL; ++q) {
-          if (key[q] > bk) { bk = key[q]; bq = q; }
+        for (int r = 0; r < R; ++r) {
+          bk[r] = key[r][0];
+          bq[r] = 0;
+#pragma unroll
+          for (int q = 1; q < EPL; ++q) {
+            if (key[r][q] > bk[r]) { bk[r] = key[r][q]; bq[r] = q; }
+          }
         }
-        const uint32_t wk = wave_max_u(bk);
-        const int cand = (bk == wk) ? lane + 64 * bq : 0x7fffffff;
-        const int wi = wave_min_i(cand);
-        const int wq = wi >> 6, wl = wi & 63;
-        float pv = p[0];
+        uint32_t wk[R];
 #pragma unroll
-        for (int q = 1; q < EPL; ++q) pv = (q == wq) ? p[q] : pv;
-        pv = __shfl(pv, wl, 64);
+        for (int r = 0; r < R; ++r) wk[r] = wave_max_u(bk[r]);
 #pragma unroll
-        for (int q = 0; q < EPL; ++q) {
-          if (lane == wl && q == wq) key[q] = 0u;
+        for (int r = 0; r < R; ++r) wi[r] = wave_min_i((bk[r] == wk[r]) ? lane + 64 * bq[r] : 0x7fffffff);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const int wq = wi[r] >> 6, wl = wi[r] & 63;
+          float pv = p[r][0];
+#pragma unroll
+          for (int q = 1; q < EPL; ++q) pv = (q == wq) ? p[r][q] : pv;
+          pv = __shfl(pv, wl, 64);
+#pragma unroll
+          for (int q = 0; q < EPL; ++q) {
+            if (lane == wl && q == wq) key[r][q] = 0u;
+          }
+          wsum[r] += pv;
+          if (lane == j) { my_i[r] = wi[r]; my_p[r] = pv; }
         }
-        sel_i[j] = wi;
-        sel_p[j] = pv;
-        wsum += pv;
       }
     }
-    int my_i = 0;
-    float my_p = 0.f;
 #pragma unroll
-    for (int j = 0; j < kMaxK; ++j) {
-      if (j < k && lane == j) { my_i = sel_i[j]; my_p = sel_p[j]; }
-    }
-    if (lane < k) {
-      idx[row * (int64_t)k + lane] = my_i;
-      weights[row * (int64_t)k + lane] = my_p / wsum;
-      atomicAdd(&lh[my_i], 1);
+    for (int r = 0; r < R; ++r) {
+      const int64_t row = rb + (int64_t)r * NW;
+      if (live[r] && lane < k) {
+        idx[row * (int64_t)k + lane] = my_i[r];
+        weights[row * (int64_t)k + lane] = my_p[r] / wsum[r];
+        atomicAdd(&lh[my_i[r]], 1);
+      }
     }
   }
   __syncthreads();
-  for (int i = tid; i < e; i += 256) hist[(int64_t)blockIdx.x * e + i] = lh[i];
+  for (int i = tid; i < e; i += kRouteThreads) hist[(int64_t)blockIdx.x * e + i] = lh[i];
 }
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(256) void permute_kernel(const int32_t* __restrict__ idx,
                                                        const int32_t* __restrict__ hist,
@@ -121,51 +157,106 @@ __global__ __launch_bounds__(256) void permute_kernel(const int32_t* __restrict_
                                                        int32_t* __restrict__ slot,
                                                        int32_t* __restrict__ order, int64_t n, int e,
                                                        int k, int tile_rows, int ntiles, int emit) {
-  __shared__ int part_b[4][kMaxE];
-  __shared__ int part_t[4][kMaxE];
+  // partial sums of the tile histograms: [group][expert], "before my tile" and "all tiles"
+  __shared__ int part_b[4 * kMaxE];   // flat [group][e]; groups * e <= 4 * kMaxE on every path
+  __shared__ int part_t[4 * kMaxE];
   __shared__ int total[kMaxE];
   __shared__ int offs[kMaxE];      // next free slot of each expert for this tile
   __shared__ int wcnt[4][kMaxE];   // per-wave assignment counts of the current chunk
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int me = blockIdx.x;
 
-  for (int c0 = 0; c0 < e; c0 += 64) {
-    const int col = c0 + lane;
-    int bef = 0, tot = 0;
-    if (col < e) {
-      for (int t = wave; t < ntiles; t += 4) {
-        const int h = hist[(int64_t)t * e + col];
-        tot += h;
-        bef += t < me ? h : 0;
+  // the first chunk of this tile's assignments is fetched now, under the histogram loads
+  const int64_t p0 = (int64_t)me * tile_rows * k;
+  int64_t p1 = p0 + (int64_t)tile_rows * k;
+  const int64_t pend = n * (int64_t)k;
+  if (p1 > pend) p1 = pend;
+  int ex_next = (emit && p0 + tid < p1) ? idx[p0 + tid] : -1;
+
+  const int e4 = e >> 2;
+  int groups;
+  if ((e & 3) == 0 && e4 <= 256 && (e4 & (e4 - 1)) == 0) {
+    // 16-byte loads: a thread keeps four neighbouring experts and walks tiles g, g+groups, ...
+    groups = 256 / e4;
+    if (groups > 16) groups = 16;
+    const int col4 = tid % e4, g = tid / e4;
+    i32x4 bef = {0, 0, 0, 0}, tot = {0, 0, 0, 0};
+    if (g < groups) {
+      const i32x4* h4 = reinterpret_cast<const i32x4*>(hist);
+      int t = g;
+      for (; t + 7 * groups < ntiles; t += 8 * groups) {
+        i32x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = h4[(int64_t)(t + u * groups) * e4 + col4];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          tot += v[u];
+          if (t + u * groups < me) bef += v[u];
+        }
       }
-      part_b[wave][col] = bef;
-      part_t[wave][col] = tot;
+      for (; t < ntiles; t += groups) {
+        const i32x4 v = h4[(int64_t)t * e4 + col4];
+        tot += v;
+        if (t < me) bef += v;
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        part_b[g * e + col4 * 4 + c] = bef[c];
+        part_t[g * e + col4 * 4 + c] = tot[c];
+      }
+    }
+  } else {
+    groups = 4;
+    for (int c0 = 0; c0 < e; c0 += 64) {
+      const int col = c0 + lane;
+      int bef = 0, tot = 0;
+      if (col < e) {
+        for (int t = wave; t < ntiles; t += 4) {
+          const int h = hist[(int64_t)t * e + col];
+          tot += h;
+          bef += t < me ? h : 0;
+        }
+        part_b[wave * e + col] = bef;
+        part_t[wave * e + col] = tot;
+      }
     }
   }
   for (int i = tid; i < 4 * kMaxE; i += 256) (&wcnt[0][0])[i] = 0;
   __syncthreads();
   for (int col = tid; col < e; col += 256) {
-    total[col] = (part_t[0][col] + part_t[1][col]) + (part_t[2][col] + part_t[3][col]);
-    part_b[0][col] = (part_b[0][col] + part_b[1][col]) + (part_b[2][col] + part_b[3][col]);
+    int tb = 0, tt = 0;
+    for (int g = 0; g < groups; ++g) { tb += part_b[g * e + col]; tt += part_t[g * e + col]; }
+    total[col] = tt;
+    offs[col] = tb;
   }
   __syncthreads();
-  for (int col = tid; col < e; col += 256) {
-    int base = 0;
-    for (int c = 0; c < col; ++c) base += total[c];
-    offs[col] = base + part_b[0][col];
-    if (me == 0) counts[col] = total[col];
+  // exclusive prefix of the expert totals: wave scan per 64 experts, chunks chained in order
+  {
+    int carry = 0;
+    for (int c0 = 0; c0 < e; c0 += 64) {          // every wave walks all chunks (e <= 512)
+      const int col = c0 + lane;
+      const int v = col < e ? total[col] : 0;
+      int inc = v;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(inc, o, 64);
+        if (lane >= o) inc += up;
+      }
+      if (wave == 0 && col < e) {
+        offs[col] += carry + inc - v;
+        if (me == 0) counts[col] = v;
+      }
+      carry += __builtin_amdgcn_readlane(inc, 63);
+    }
   }
   __syncthreads();
   if (!emit) return;
 
-  const int64_t p0 = (int64_t)me * tile_rows * k;
-  int64_t p1 = p0 + (int64_t)tile_rows * k;
-  const int64_t pend = n * (int64_t)k;
-  if (p1 > pend) p1 = pend;
   for (int64_t c0 = p0; c0 < p1; c0 += 256) {
     const int64_t p = c0 + tid;
     const bool act = p < p1;
-    const int ex = act ? idx[p] : -1;
+    const int ex = ex_next;
+    ex_next = (p + 256 < p1) ? idx[p + 256] : -1;
     // rank among equal experts inside the wave, in lane (= flat position) order
     int rank = 0;
     unsigned long long todo = __ballot(act);
@@ -205,7 +296,7 @@ Tiling make_tiling(int64_t n) {
   Tiling t;
   int64_t rows = 64;
   if ((n + rows - 1) / rows > kMaxTiles) rows = (n + kMaxTiles - 1) / kMaxTiles;
-  rows = (rows + 3) / 4 * 4;
+  rows = (rows + 15) / 16 * 16;
   t.tile_rows = (int)rows;
   t.ntiles = (int)((n + rows - 1) / rows);
   if (t.ntiles < 1) t.ntiles = 1;
@@ -216,7 +307,7 @@ template <typename T>
 int launch_route(const void* logits, int32_t* idx, float* weights, int32_t* hist, int64_t n, int e,
                  int k, const Tiling& tl, hipStream_t st) {
   const T* lp = static_cast<const T*>(logits);
-  const dim3 grid((unsigned)tl.ntiles), block(256);
+  const dim3 grid((unsigned)tl.ntiles), block(kRouteThreads);
 #define GO(EPL) \
   hipLaunchKernelGGL((route_kernel<T, EPL>), grid, block, 0, st, lp, idx, weights, hist, n, e, k, tl.tile_rows)
   if (e <= 64) GO(1);

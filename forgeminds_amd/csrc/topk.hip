@@ -4,19 +4,24 @@
 // descending, index ascending inside ties; at the k-th value the smallest indices win; NaN is
 // the largest value and the original NaN is what lands in `values`; -0.0 ties with +0.0.
 //
-// One workgroup per row. The row is read from HBM once and kept in registers (packed, 16
-// bytes per vector) while three cheap phases run over it:
-//   A  every thread takes the maximum of its share of the row ("group maximum");
+// One workgroup per row, one streaming read of the row from HBM:
+//   A  every thread folds each 16-byte vector it reads to one maximum and keeps those vector
+//      maxima (not the data) in registers; their maximum is the thread's "group maximum";
 //   T  each wave finds the ceil(k / waves)-th largest of its 64 group maxima with a ballot
 //      search; the minimum over the waves, tau, can never be above the true k-th value,
 //      because at least k group maxima are >= tau;
-//   B  every element >= tau becomes a candidate (key, index) in LDS -- normally a few
-//      hundred out of 128k -- and candidates are ranked by counting how many others beat them
-//      under (key descending, index ascending); rank r < k is output slot r.
+//   B  only vectors whose maximum is >= tau can hold candidates -- a few hundred out of
+//      16k -- so their indices go to a work list, the workgroup re-reads just those vectors
+//      (one parallel round trip, served by cache) and every element >= tau becomes a
+//      candidate (key, index) in LDS; candidates are ranked by counting how many others beat
+//      them under (key descending, index ascending); rank r < k is output slot r.
+// Keeping maxima instead of the row keeps the kernel at 64 registers, so two 1024-thread
+// workgroups share a compute unit and one streams while the other selects.
 // Rows with too many candidates (long runs of equal values) take an exact path instead: a
 // bitwise search for the k-th key over the whole row, then an index-ordered scan that admits
-// the first (k - #greater) ties. Keys are order-preserving integer images of the fp32 value,
-// so no float is ever summed and the result is bit-reproducible.
+// the first (k - #greater) ties. Rows wider than the register budget make two full passes.
+// Keys are order-preserving integer images of the fp32 value, so no float is ever summed and
+// the result is bit-reproducible.
 #include "fm_vocab.cuh"
 
 using namespace fm;
@@ -70,21 +75,22 @@ __device__ __forceinline__ int block_excl_scan(int v, int* smem, int nw, int* to
   return before + inc - v;
 }
 
+constexpr int kWorkCap = 2048;  // vectors that may be revisited in phase B
+
 template <typename T, int THREADS, int ITERS>
-__global__ __launch_bounds__(THREADS) void topk_kernel(const T* __restrict__ x,
-                                                        T* __restrict__ values,
-                                                        int32_t* __restrict__ idx32,
-                                                        int64_t* __restrict__ idx64, int v, int k,
-                                                        bool vec_ok) {
+__global__ __launch_bounds__(THREADS, (ITERS > 0 && ITERS <= 16 && THREADS == 1024) ? 8 : 1)
+void topk_kernel(const T* __restrict__ x, T* __restrict__ values, int32_t* __restrict__ idx32,
+                 int64_t* __restrict__ idx64, int v, int k, bool vec_ok) {
   constexpr int EPV = Elem<T>::kVec;
   constexpr int NW = THREADS / 64;
-  constexpr bool REGS = ITERS > 0;
+  constexpr bool VMAX = ITERS > 0;   // vector maxima live in registers
   constexpr uint32_t KMASK = sizeof(T) == 2 ? 0xFFFF0000u : 0xFFFFFFFFu;
   __shared__ unsigned long long ccomp[kCap];  // (key << 32) | ~index : larger is better
   __shared__ int crank[kCap];
+  __shared__ int work[VMAX ? kWorkCap : 1];
   __shared__ int s_int[NW];
   __shared__ uint32_t s_tau[NW];
-  __shared__ int s_count;
+  __shared__ int s_count, s_nwork;
 
   const int64_t row = blockIdx.x;
   const T* rp = x + row * (int64_t)v;
@@ -92,9 +98,21 @@ __global__ __launch_bounds__(THREADS) void topk_kernel(const T* __restrict__ x,
   const int lane = tid & 63, wave = tid >> 6;
   const RowSplit sp = split_row<EPV>(row, v, vec_ok);
   const int ne = edge_count(sp, v);
-  u32x4 regs[REGS ? ITERS : 1];
+  float vmax[VMAX ? ITERS : 1];
+
+  // maximum of one vector; NaN if the vector holds a NaN (NaN outranks everything)
+  auto fold = [&](const u32x4& raw) {
+    float f[EPV];
+    Elem<T>::unpack(raw, f);
+    float m = f[0];
+    bool bad = f[0] != f[0];
+#pragma unroll
+    for (int e = 1; e < EPV; ++e) { m = fmaxf(m, f[e]); bad |= (f[e] != f[e]); }
+    return bad ? __builtin_nanf("") : m;
+  };
 
   int C = 0;
+  bool overflow = false;
   if (v <= kCap) {
     // short row: every element is a candidate
     for (int j = tid; j < v; j += THREADS)
@@ -102,28 +120,33 @@ __global__ __launch_bounds__(THREADS) void topk_kernel(const T* __restrict__ x,
     C = v;
     __syncthreads();
   } else {
-    // ---- phase A: group maxima
+    // ---- phase A: vector maxima and the thread's group maximum
     float fm = -INFINITY;
     bool has_nan = false;
+    if constexpr (VMAX) {
 #pragma unroll
-    for (int i = 0; i < (REGS ? ITERS : 1); ++i) {
-      if constexpr (REGS) {
-        const int c = i * THREADS + tid;
-        if (c < sp.nvec) {
-          regs[i] = load16_stream(rp + sp.head + (int64_t)c * EPV);
-          float f[EPV];
-          Elem<T>::unpack(regs[i], f);
+      for (int i0 = 0; i0 < ITERS; i0 += 4) {
+        u32x4 raw[4];
 #pragma unroll
-          for (int e = 0; e < EPV; ++e) { fm = fmaxf(fm, f[e]); has_nan |= (f[e] != f[e]); }
+        for (int u = 0; u < 4; ++u) {
+          const int c = (i0 + u) * THREADS + tid;
+          if (c < sp.nvec) raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int c = (i0 + u) * THREADS + tid;
+          float m = -INFINITY;
+          if (c < sp.nvec) m = fold(raw[u]);
+          vmax[i0 + u] = m;
+          fm = fmaxf(fm, m);
+          has_nan |= (m != m);
         }
       }
-    }
-    if constexpr (!REGS) {
+    } else {
       for (int c = tid; c < sp.nvec; c += THREADS) {
-        float f[EPV];
-        Elem<T>::unpack(load16(rp + sp.head + (int64_t)c * EPV), f);
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) { fm = fmaxf(fm, f[e]); has_nan |= (f[e] != f[e]); }
+        const float m = fold(load16(rp + sp.head + (int64_t)c * EPV));
+        fm = fmaxf(fm, m);
+        has_nan |= (m != m);
       }
     }
     for (int e = tid; e < ne; e += THREADS) {
@@ -145,7 +168,7 @@ __global__ __launch_bounds__(THREADS) void topk_kernel(const T* __restrict__ x,
       }
     }
     if (lane == 0) s_tau[wave] = tw;
-    if (tid == 0) s_count = 0;
+    if (tid == 0) { s_count = 0; s_nwork = 0; }
     __syncthreads();
     uint32_t tau = s_tau[0];
 #pragma unroll
@@ -154,11 +177,11 @@ __global__ __launch_bounds__(THREADS) void topk_kernel(const T* __restrict__ x,
     const float tau_f = tau <= 0x007FFFFFu ? -INFINITY
                                            : (tau == 0xFFFFFFFFu ? __builtin_nanf("") : float_of_key(tau));
     const bool only_nan = tau == 0xFFFFFFFFu;
+    auto take_of = [&](float f) { return only_nan ? (f != f) : !(f < tau_f); };
 
     // ---- phase B: candidates
     auto consider = [&](float f, int col) {
-      const bool take = only_nan ? (f != f) : !(f < tau_f);
-      if (take) {
+      if (take_of(f)) {
         const int slot = atomicAdd(&s_count, 1);
         if (slot < kCap) ccomp[slot] = ((unsigned long long)key_of(f) << 32) | (uint32_t)(~col);
       }
@@ -168,17 +191,31 @@ __global__ __launch_bounds__(THREADS) void topk_kernel(const T* __restrict__ x,
       Elem<T>::unpack(raw, f);
       bool any = false;
 #pragma unroll
-      for (int e = 0; e < EPV; ++e) any |= only_nan ? (f[e] != f[e]) : !(f[e] < tau_f);
+      for (int e = 0; e < EPV; ++e) any |= take_of(f[e]);
       if (any) {
 #pragma unroll
         for (int e = 0; e < EPV; ++e) consider(f[e], sp.head + c * EPV + e);
       }
     };
-    if constexpr (REGS) {
+    if constexpr (VMAX) {
+      // B1: vectors that can hold a candidate go to the work list
 #pragma unroll
       for (int i = 0; i < ITERS; ++i) {
         const int c = i * THREADS + tid;
-        if (c < sp.nvec) scan_vec(regs[i], c);
+        if (c < sp.nvec && take_of(vmax[i])) {
+          const int slot = atomicAdd(&s_nwork, 1);
+          if (slot < kWorkCap) work[slot] = c;
+        }
+      }
+      __syncthreads();
+      const int nwork = s_nwork;
+      overflow = nwork > kWorkCap;
+      // B2: revisit only those vectors, spread over the whole workgroup
+      if (!overflow) {
+        for (int w = tid; w < nwork; w += THREADS) {
+          const int c = work[w];
+          scan_vec(load16(rp + sp.head + (int64_t)c * EPV), c);
+        }
       }
     } else {
       for (int c = tid; c < sp.nvec; c += THREADS) scan_vec(load16(rp + sp.head + (int64_t)c * EPV), c);
@@ -190,6 +227,7 @@ __global__ __launch_bounds__(THREADS) void topk_kernel(const T* __restrict__ x,
     __syncthreads();
     C = s_count;
     __syncthreads();
+    if (overflow) C = kCap + 1;
 
     if (C > kCap) {
       // ---- exact path: k-th key by bitwise search over the whole row
@@ -339,6 +377,7 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
   else if (v <= kCap || nvec <= 256 * 4) GO(256, 4);
   else if (nvec <= 1024 * 4) GO(1024, 4);
   else if (nvec <= 1024 * 16) GO(1024, 16);
+  else if (nvec <= 1024 * 32) GO(1024, 32);
   else GO(1024, 0);
 #undef GO
   return FM_OK;
