@@ -120,7 +120,7 @@ def make_workload(name, torch, L, dev):
 
         w.step, w.warm_step = step, warm_step
         w.dominant_launch = lambda: bwd(state["i"])
-        w.dominant = "norm_bwd_kernel<bf16,f32,64,2> + colsum"
+        w.dominant = "norm_bwd_kernel<bf16,f32,64,2> + colsum_kernel"
         w.dominant_bytes = n * d * 6
         w.bytes = n * d * 10
         w.desc = f"RMSNorm fwd+bwd x bf16 [{n},{d}], w fp32, eps 1e-6 (rotating {sets} buffer sets)"
@@ -157,7 +157,7 @@ def make_workload(name, torch, L, dev):
 
         w.step = step
         w.dominant_launch = bwd
-        w.dominant = "norm_bwd_kernel<bf16,f32,512,2> + colsum"
+        w.dominant = "norm_bwd_kernel<bf16,f32,512,2> + colsum_kernel"
         w.dominant_bytes = n * d * 8
         w.bytes = n * d * 16
         w.desc = f"add-RMSNorm fwd+bwd x,delta bf16 [{n},{d}], w fp32, eps 1e-5, with residual grad"
@@ -188,7 +188,7 @@ def make_workload(name, torch, L, dev):
 
         w.step = step
         w.dominant_launch = bwd
-        w.dominant = "ce_bwd_kernel<bf16,512,4>"
+        w.dominant = "ce_bwd_kernel<bf16,1024,4>"
         w.dominant_bytes = n * v * 4
         w.bytes = n * v * 6
         w.desc = (f"fused CE fwd+bwd logits bf16 [{n},{v}], 5% ignore_index, mean; "
@@ -234,7 +234,7 @@ def make_workload(name, torch, L, dev):
 
         w.step = step
         w.dominant_launch = bwd
-        w.dominant = "kl_bwd_kernel<bf16,bf16,1024,2>"
+        w.dominant = "kl_bwd_kernel<bf16,bf16,1024,8>"
         w.dominant_bytes = n * v * 6
         w.bytes = n * v * 10
         w.desc = f"KL(teacher||student) fwd+bwd bf16 [{n},{v}], T=2, mean"

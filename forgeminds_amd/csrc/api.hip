@@ -16,7 +16,7 @@ const char* const kParamNames[fm_host::P_COUNT] = {
     "vocab_threads",
     "norm_tpr",
     "topk_variant",
-    "debug_stop",
+    "vocab_unroll",
 };
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cus[kMaxDevices];

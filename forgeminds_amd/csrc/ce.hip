@@ -173,17 +173,13 @@ template <typename T>
 int launch_fwd(const void* logits, const int64_t* labels, float* lse, float* row_loss, int64_t n,
                int v, int64_t ignore_index, bool vec_ok, hipStream_t st) {
   const T* lp = static_cast<const T*>(logits);
-  const int threads = fm_host::vocab_threads(v, sizeof(T));
+  const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 512, 4);
   const dim3 grid((unsigned)n);
-  if (threads == 1024)
-    hipLaunchKernelGGL((ce_fwd_kernel<T, 1024, 4>), grid, dim3(1024), 0, st, lp, labels, lse,
-                       row_loss, v, ignore_index, vec_ok);
-  else if (threads == 512)
-    hipLaunchKernelGGL((ce_fwd_kernel<T, 512, 4>), grid, dim3(512), 0, st, lp, labels, lse, row_loss,
-                       v, ignore_index, vec_ok);
-  else
-    hipLaunchKernelGGL((ce_fwd_kernel<T, 256, 4>), grid, dim3(256), 0, st, lp, labels, lse, row_loss,
-                       v, ignore_index, vec_ok);
+#define LAUNCH(TH, UN)                                                                          \
+  hipLaunchKernelGGL((ce_fwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, lp, labels, lse, row_loss, \
+                     v, ignore_index, vec_ok)
+  FM_VOCAB_DISPATCH(sh, LAUNCH);
+#undef LAUNCH
   return FM_OK;
 }
 
@@ -193,17 +189,13 @@ int launch_bwd(const void* logits, const int64_t* labels, const float* lse, cons
                bool vec_ok, hipStream_t st) {
   const T* lp = static_cast<const T*>(logits);
   T* gp = static_cast<T*>(dlogits);
-  const int threads = fm_host::vocab_threads(v, sizeof(T));
+  const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 4);
   const dim3 grid((unsigned)n);
-  if (threads == 1024)
-    hipLaunchKernelGGL((ce_bwd_kernel<T, 1024, 4>), grid, dim3(1024), 0, st, lp, labels, lse,
-                       n_valid, grad_out, gp, v, ignore_index, vec_ok);
-  else if (threads == 512)
-    hipLaunchKernelGGL((ce_bwd_kernel<T, 512, 4>), grid, dim3(512), 0, st, lp, labels, lse, n_valid,
-                       grad_out, gp, v, ignore_index, vec_ok);
-  else
-    hipLaunchKernelGGL((ce_bwd_kernel<T, 256, 4>), grid, dim3(256), 0, st, lp, labels, lse, n_valid,
-                       grad_out, gp, v, ignore_index, vec_ok);
+#define LAUNCH(TH, UN)                                                                         \
+  hipLaunchKernelGGL((ce_bwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, lp, labels, lse, n_valid, \
+                     grad_out, gp, v, ignore_index, vec_ok)
+  FM_VOCAB_DISPATCH(sh, LAUNCH);
+#undef LAUNCH
   return FM_OK;
 }
 

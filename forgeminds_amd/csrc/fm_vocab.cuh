@@ -102,14 +102,33 @@ __device__ __forceinline__ float block_max(float v, float* smem) {
 }  // namespace fm
 
 namespace fm_host {
-// Threads per row for the vocabulary kernels: wide rows get more waves so that one row's
-// loads are spread over more outstanding requests.
-inline int vocab_threads(int64_t v, int esize) {
-  int t = get_param(P_VOCAB_THREADS);
-  if (t == 256 || t == 512 || t == 1024) return t;
+// Launch shape of the vocabulary kernels: threads per row and 16-byte vectors a thread has
+// in flight. `pref_threads` is the per-kernel default (read-only kernels do best with 512
+// threads on 64 KB rows, kernels that also write with 1024); both can be overridden for sweeps.
+struct VocabShape { int threads, unroll; };
+inline VocabShape vocab_shape(int64_t v, int esize, int pref_threads, int pref_unroll) {
+  VocabShape s{pref_threads, pref_unroll};
   const int64_t bytes = v * esize;
-  if (bytes >= 128 * 1024) return 1024;
-  if (bytes >= 32 * 1024) return 512;
-  return 256;
+  if (bytes < 16 * 1024) s.threads = 256;
+  else if (bytes < 48 * 1024 && s.threads > 512) s.threads = 512;
+  const int t = get_param(P_VOCAB_THREADS);
+  if (t == 256 || t == 512 || t == 1024) s.threads = t;
+  const int u = get_param(P_VOCAB_UNROLL);
+  if (u == 2 || u == 4 || u == 8) s.unroll = u;
+  return s;
 }
 }  // namespace fm_host
+
+// Dispatch a kernel template over (threads, unroll): FM_VOCAB_DISPATCH(shape, LAUNCH) expands
+// LAUNCH(TH, UN) for the selected pair.
+#define FM_VOCAB_DISPATCH(shape, LAUNCH)                              \
+  do {                                                                \
+    const int th__ = (shape).threads, un__ = (shape).unroll;          \
+    if (th__ == 1024) {                                               \
+      if (un__ == 2) { LAUNCH(1024, 2); } else if (un__ == 8) { LAUNCH(1024, 8); } else { LAUNCH(1024, 4); } \
+    } else if (th__ == 512) {                                         \
+      if (un__ == 2) { LAUNCH(512, 2); } else if (un__ == 8) { LAUNCH(512, 8); } else { LAUNCH(512, 4); }    \
+    } else {                                                          \
+      if (un__ == 2) { LAUNCH(256, 2); } else if (un__ == 8) { LAUNCH(256, 8); } else { LAUNCH(256, 4); }    \
+    }                                                                 \
+  } while (0)

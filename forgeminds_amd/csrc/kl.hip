@@ -218,17 +218,13 @@ void launch_fwd(const void* s, const void* t, float* lse_s, float* lse_t, float*
                 int v, float inv_temp, bool vec_ok, hipStream_t st) {
   const T* sp = static_cast<const T*>(s);
   const T* tp = static_cast<const T*>(t);
-  const int threads = fm_host::vocab_threads(v, sizeof(T));
+  const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 512, 2);
   const dim3 grid((unsigned)n);
-  if (threads == 1024)
-    hipLaunchKernelGGL((kl_fwd_kernel<T, 1024, 2>), grid, dim3(1024), 0, st, sp, tp, lse_s, lse_t,
-                       row_kl, v, inv_temp, vec_ok);
-  else if (threads == 512)
-    hipLaunchKernelGGL((kl_fwd_kernel<T, 512, 2>), grid, dim3(512), 0, st, sp, tp, lse_s, lse_t,
-                       row_kl, v, inv_temp, vec_ok);
-  else
-    hipLaunchKernelGGL((kl_fwd_kernel<T, 256, 2>), grid, dim3(256), 0, st, sp, tp, lse_s, lse_t,
-                       row_kl, v, inv_temp, vec_ok);
+#define LAUNCH(TH, UN)                                                                            \
+  hipLaunchKernelGGL((kl_fwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, sp, tp, lse_s, lse_t, row_kl, \
+                     v, inv_temp, vec_ok)
+  FM_VOCAB_DISPATCH(sh, LAUNCH);
+#undef LAUNCH
 }
 
 template <typename T, typename GT>
@@ -238,17 +234,13 @@ void launch_bwd(const void* s, const void* t, const float* lse_s, const float* l
   const T* sp = static_cast<const T*>(s);
   const T* tp = static_cast<const T*>(t);
   GT* gp = static_cast<GT*>(ds);
-  const int threads = fm_host::vocab_threads(v, sizeof(T));
+  const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 8);
   const dim3 grid((unsigned)n);
-  if (threads == 1024)
-    hipLaunchKernelGGL((kl_bwd_kernel<T, GT, 1024, 2>), grid, dim3(1024), 0, st, sp, tp, lse_s, lse_t,
-                       grad_out, grad_per_row, gp, v, inv_temp, scale, vec_ok);
-  else if (threads == 512)
-    hipLaunchKernelGGL((kl_bwd_kernel<T, GT, 512, 2>), grid, dim3(512), 0, st, sp, tp, lse_s, lse_t,
-                       grad_out, grad_per_row, gp, v, inv_temp, scale, vec_ok);
-  else
-    hipLaunchKernelGGL((kl_bwd_kernel<T, GT, 256, 2>), grid, dim3(256), 0, st, sp, tp, lse_s, lse_t,
-                       grad_out, grad_per_row, gp, v, inv_temp, scale, vec_ok);
+#define LAUNCH(TH, UN)                                                                           \
+  hipLaunchKernelGGL((kl_bwd_kernel<T, GT, TH, UN>), grid, dim3(TH), 0, st, sp, tp, lse_s, lse_t, \
+                     grad_out, grad_per_row, gp, v, inv_temp, scale, vec_ok)
+  FM_VOCAB_DISPATCH(sh, LAUNCH);
+#undef LAUNCH
 }
 
 int check_shape(const char* what, int64_t n, int64_t v, int dtype) {

@@ -17,6 +17,10 @@ using namespace fm;
 namespace {
 
 constexpr int kMinBlock = 256;
+// The backward always runs 16-wave workgroups: many rows per workgroup are folded through
+// LDS, so the number of fp32 partial rows (one per workgroup) stays at the CU count while
+// each SIMD still has four waves to hide load latency.
+constexpr int kBwdBlock = 1024;
 
 template <int TPR> struct BlockOf { static constexpr int value = TPR > kMinBlock ? TPR : kMinBlock; };
 
@@ -98,12 +102,12 @@ __global__ __launch_bounds__(BlockOf<TPR>::value) void norm_fwd_kernel(
 // ---------------------------------------------------------------- backward (vector path)
 // grid-persistent; `partial` is [gridDim.x, d] fp32 (or NULL when dW is not wanted).
 template <typename T, typename WT, int TPR, int ITERS>
-__global__ __launch_bounds__(BlockOf<TPR>::value) void norm_bwd_kernel(
+__global__ __launch_bounds__(kBwdBlock) void norm_bwd_kernel(
     const T* __restrict__ x, const WT* __restrict__ w, const float* __restrict__ rstd,
     const T* __restrict__ dy, const T* __restrict__ gxn, T* __restrict__ dx,
     T* __restrict__ dd, float* __restrict__ partial, int64_t n, int d, int64_t tiles) {
   constexpr int EPV = Elem<T>::kVec;
-  constexpr int BLOCK = BlockOf<TPR>::value;
+  constexpr int BLOCK = kBwdBlock;
   constexpr int RPB = BLOCK / TPR;
   constexpr int COVER = TPR * ITERS * EPV;   // columns covered by one row's threads
   __shared__ float red[RPB * (TPR > 64 ? TPR / 64 : 1)];
@@ -217,27 +221,61 @@ __global__ __launch_bounds__(BlockOf<TPR>::value) void norm_bwd_kernel(
   }
 }
 
-// Column sum of `p` partial rows, [p, d] fp32 -> dw[d] in WT. One workgroup owns 64
-// columns; wave g sums rows g, g+16, ... in ascending order, then the 16 wave results are
-// added in wave order. The order depends only on (p, d), never on timing.
+// Column sum of `p` partial rows, [p, d] fp32 -> dw[d] in WT. One workgroup owns 64 columns
+// as 16 quads; thread (g, q) adds rows g, g+64, ... of quad q with 16-byte loads, then the 64
+// row-group results are added in group order. The order depends only on (p, d), never on
+// timing. Requires d % 4 == 0 (the register path guarantees it); otherwise colsum_scalar.
 template <typename WT>
 __global__ __launch_bounds__(1024) void colsum_kernel(const float* __restrict__ partial,
                                                        WT* __restrict__ dw, int p, int d) {
+  __shared__ float s[64][64 + 4];
+  const int q = threadIdx.x & 15;
+  const int g = threadIdx.x >> 4;
+  const int col = blockIdx.x * 64 + q * 4;
+  float a[4] = {0.f, 0.f, 0.f, 0.f};
+  if (col < d) {
+    int r = g;
+    for (; r + 192 < p; r += 256) {
+      float v[4][4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) Elem<float>::unpack(load16(partial + (int64_t)(r + 64 * u) * d + col), v[u]);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) a[c] += v[u][c];
+      }
+    }
+    for (; r < p; r += 64) {
+      float v[4];
+      Elem<float>::unpack(load16(partial + (int64_t)r * d + col), v);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) a[c] += v[c];
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) s[g][q * 4 + c] = a[c];
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    const int cc = blockIdx.x * 64 + threadIdx.x;
+    if (cc < d) {
+      float tot = s[0][threadIdx.x];
+#pragma unroll 8
+      for (int i = 1; i < 64; ++i) tot += s[i][threadIdx.x];
+      Elem<WT>::store1(dw + cc, tot);
+    }
+  }
+}
+
+template <typename WT>
+__global__ __launch_bounds__(1024) void colsum_scalar_kernel(const float* __restrict__ partial,
+                                                              WT* __restrict__ dw, int p, int d) {
   __shared__ float s[16][64];
   const int lane = threadIdx.x & 63;
   const int g = threadIdx.x >> 6;
   const int col = blockIdx.x * 64 + lane;
   float a = 0.f;
   if (col < d) {
-    int r = g;
-    for (; r + 48 < p; r += 64) {
-      const float v0 = partial[(int64_t)r * d + col];
-      const float v1 = partial[(int64_t)(r + 16) * d + col];
-      const float v2 = partial[(int64_t)(r + 32) * d + col];
-      const float v3 = partial[(int64_t)(r + 48) * d + col];
-      a += v0; a += v1; a += v2; a += v3;
-    }
-    for (; r < p; r += 16) a += partial[(int64_t)r * d + col];
+    for (int r = g; r < p; r += 16) a += partial[(int64_t)r * d + col];
   }
   s[g][lane] = a;
   __syncthreads();
@@ -344,7 +382,8 @@ struct Plan {
   bool vec;        // register-resident vector path
   int tpr, iters;  // threads per row, 16-byte vectors per thread
   int rpb;         // rows per workgroup
-  int64_t tiles;   // row tiles (vector path)
+  int64_t tiles;   // row tiles of the forward (vector path)
+  int64_t bwd_tiles;  // row tiles of the backward
   int bwd_blocks;  // persistent grid of the backward == partial rows
   int64_t rows_per_chunk;  // any-width path
 };
@@ -376,10 +415,11 @@ Plan make_plan(int64_t n, int64_t d, int x_dtype, bool aligned) {
     const int block = p.tpr > kMinBlock ? p.tpr : kMinBlock;
     p.rpb = block / p.tpr;
     p.tiles = (n + p.rpb - 1) / p.rpb;
+    p.bwd_tiles = (n + (kBwdBlock / p.tpr) - 1) / (kBwdBlock / p.tpr);
     int per_cu = fm_host::get_param(fm_host::P_NORM_BWD_BLOCKS_PER_CU);
-    if (per_cu <= 0) per_cu = block >= 1024 ? 1 : (block >= 512 ? 2 : 4);
+    if (per_cu <= 0) per_cu = 1;
     int64_t blocks = (int64_t)fm_host::num_cus() * per_cu;
-    if (blocks > p.tiles) blocks = p.tiles;
+    if (blocks > p.bwd_tiles) blocks = p.bwd_tiles;
     if (blocks < 1) blocks = 1;
     p.bwd_blocks = (int)blocks;
   } else {
@@ -446,8 +486,8 @@ int launch_bwd(const Plan& p, const void* x, const void* w, const float* rstd, c
 #define X(TPR_, IT_)                                                                           \
   if (!done && p.tpr == TPR_ && p.iters == IT_) {                                              \
     hipLaunchKernelGGL((norm_bwd_kernel<T, WT, TPR_, IT_>), dim3((unsigned)p.bwd_blocks),      \
-                       dim3(BlockOf<TPR_>::value), 0, st, xp, wp, rstd, dyp, gp, dxp, ddp,     \
-                       partial, n, (int)d, p.tiles);                                           \
+                       dim3(kBwdBlock), 0, st, xp, wp, rstd, dyp, gp, dxp, ddp,                \
+                       partial, n, (int)d, p.bwd_tiles);                                       \
     done = true;                                                                               \
   }
     FM_FOR_EACH_SHAPE(X)
@@ -458,8 +498,12 @@ int launch_bwd(const Plan& p, const void* x, const void* w, const float* rstd, c
     }
   }
   if (partial != nullptr) {
-    hipLaunchKernelGGL((colsum_kernel<WT>), dim3((unsigned)((d + 63) / 64)), dim3(1024), 0, st,
-                       partial, static_cast<WT*>(dw), p.bwd_blocks, (int)d);
+    if (d % 4 == 0)
+      hipLaunchKernelGGL((colsum_kernel<WT>), dim3((unsigned)((d + 63) / 64)), dim3(1024), 0, st,
+                         partial, static_cast<WT*>(dw), p.bwd_blocks, (int)d);
+    else
+      hipLaunchKernelGGL((colsum_scalar_kernel<WT>), dim3((unsigned)((d + 63) / 64)), dim3(1024), 0,
+                         st, partial, static_cast<WT*>(dw), p.bwd_blocks, (int)d);
   }
   return FM_OK;
 }

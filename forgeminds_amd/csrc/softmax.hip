@@ -80,14 +80,12 @@ template <typename T>
 void launch(const void* x, void* y, int64_t n, int v, bool vec_ok, hipStream_t st) {
   const T* xp = static_cast<const T*>(x);
   T* yp = static_cast<T*>(y);
-  const int threads = fm_host::vocab_threads(v, sizeof(T));
+  const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 4);
   const dim3 grid((unsigned)n);
-  if (threads == 1024)
-    hipLaunchKernelGGL((softmax_kernel<T, 1024, 4>), grid, dim3(1024), 0, st, xp, yp, v, vec_ok);
-  else if (threads == 512)
-    hipLaunchKernelGGL((softmax_kernel<T, 512, 4>), grid, dim3(512), 0, st, xp, yp, v, vec_ok);
-  else
-    hipLaunchKernelGGL((softmax_kernel<T, 256, 2>), grid, dim3(256), 0, st, xp, yp, v, vec_ok);
+#define LAUNCH(TH, UN) \
+  hipLaunchKernelGGL((softmax_kernel<T, TH, UN>), grid, dim3(TH), 0, st, xp, yp, v, vec_ok)
+  FM_VOCAB_DISPATCH(sh, LAUNCH);
+#undef LAUNCH
 }
 
 }  // namespace
