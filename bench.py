@@ -35,9 +35,11 @@ METRIC = "HBM GB/s & % roofline: RMSNorm, CE/KL fwd+bwd; MoE top-k rows/s"
 
 # HBM bytes per launch of the dominant kernels, from `rocprofv3 --pmc FETCH_SIZE` and
 # `--pmc WRITE_SIZE` runs of this file (summaries under profiles/), each scaled by what the
-# same counter reads for a copy of known size; None until measured.
+# same counter reads for a copy of known size; None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "ce": None,
+    # ce_bwd_kernel: FETCH_SIZE 244172.5 KiB x 2.00000 + WRITE_SIZE 512204.4 KiB x 0.99915
+    # (profiles/ce_fwd_bwd_hbm_traffic_pmc.txt)
+    "ce": 1024108600,
 }
 
 
