@@ -7,6 +7,8 @@
     loss = fm.kernels.kl_div_logits(student, teacher)    # KL(teacher || student)
     v, i = fm.kernels.topk(x, 64)                        # canonical, deterministic order
     r = fm.kernels.moe_route(router_logits, k=2)         # idx, weights, counts, slot, order
+    xs = fm.kernels.moe_gather(x, r.order, 2, r.slot)    # tokens grouped by expert
+    out = fm.kernels.moe_combine(ys, r.weights, r.slot, r.order)   # weighted return to tokens
 
     fm.kernels.enable(model)              # patch RMSNorm / SwiGLU modules in place
     fm.kernels.set_backend("fallback")    # force the torch expressions (A/B, debugging)
@@ -23,6 +25,7 @@ from ._common import HAS_TRITON, get_backend, reset_stats, set_backend, stats
 from ._ops import use_custom_ops
 from .apply import enable, patch, revert
 from .ce import cross_entropy
+from .dispatch import moe_combine, moe_gather
 from .extras import newton_schulz, qk_norm_rope, swiglu, swiglu_split
 from .kl import distill_kl, kl_distill_loss, kl_div, kl_div_logits
 from .norm import add_rms_norm, rms_norm
@@ -35,6 +38,7 @@ __all__ = [
     "rms_norm", "add_rms_norm", "qk_norm_rope", "swiglu", "swiglu_split",
     "kl_div_logits", "kl_div", "kl_distill_loss", "distill_kl",
     "newton_schulz", "topk", "softmax", "cross_entropy", "moe_route", "Routing",
+    "moe_gather", "moe_combine",
     "enable", "patch", "revert", "available", "use_custom_ops",
 ]
 

@@ -46,6 +46,9 @@ SIGNATURES = {
     "fm_topk": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _int, _vp]),
     "fm_softmax_fwd": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "fm_route_workspace": (_sz, [_i64, _int, _int]),
+    "fm_moe_gather": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
+    "fm_moe_combine": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
+    "fm_moe_combine_dw": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "fm_route": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _int, _int, _int, _vp]),
 }
 
@@ -294,3 +297,37 @@ def route(logits2, k: int, want_permutation: bool = True):
                               _ptr(order), _ptr(ws), nbytes, n, e, int(k),
                               dtype_code(logits2.dtype), _stream(logits2)), "fm_route")
     return idx, wts, counts, slot, order
+
+
+# ------------------------------------------------------------------ token moves around the permutation
+def moe_gather(x2, order, k: int, scale_flat=None):
+    """x2 [n, d], order int32 [n*k] -> xs [n*k, d] = scale * x2[order // k]."""
+    _dense(x2, order, scale_flat)
+    n, d = x2.shape
+    xs = torch.empty((n * k, d), device=x2.device, dtype=x2.dtype)
+    with torch.cuda.device(x2.device):
+        _check(lib().fm_moe_gather(_ptr(x2), _ptr(order), _ptr(scale_flat), _ptr(xs), n, d, int(k),
+                                   dtype_code(x2.dtype), _stream(x2)), "fm_moe_gather")
+    return xs
+
+
+def moe_combine(ys, weights, slot, n: int, k: int):
+    """ys [n*k, d], weights fp32 [n, k] or None, slot int32 [n*k] -> out [n, d]."""
+    _dense(ys, weights, slot)
+    d = ys.shape[1]
+    out = torch.empty((n, d), device=ys.device, dtype=ys.dtype)
+    with torch.cuda.device(ys.device):
+        _check(lib().fm_moe_combine(_ptr(ys), _ptr(weights), _ptr(slot), _ptr(out), n, d, int(k),
+                                    dtype_code(ys.dtype), _stream(ys)), "fm_moe_combine")
+    return out
+
+
+def moe_combine_dw(ys, dout, slot, n: int, k: int):
+    """-> dweights fp32 [n, k] = <ys[slot[t*k+j]], dout[t]>."""
+    _dense(ys, dout, slot)
+    d = ys.shape[1]
+    dw = torch.empty((n, k), device=ys.device, dtype=torch.float32)
+    with torch.cuda.device(ys.device):
+        _check(lib().fm_moe_combine_dw(_ptr(ys), _ptr(dout), _ptr(slot), _ptr(dw), n, d, int(k),
+                                       dtype_code(ys.dtype), _stream(ys)), "fm_moe_combine_dw")
+    return dw

@@ -11,9 +11,9 @@ from typing import NamedTuple
 import torch
 import torch.nn as nn
 
-from .kernels import moe_route
+from .kernels import moe_combine, moe_gather, moe_route
 
-__all__ = ["Router", "Dispatch", "dispatch_plan"]
+__all__ = ["Router", "Dispatch", "dispatch_plan", "Experts", "MoE"]
 
 
 class Dispatch(NamedTuple):
@@ -23,6 +23,8 @@ class Dispatch(NamedTuple):
     idx: torch.Tensor       # [n, k] int64
     order: torch.Tensor     # [n*k] int64: flat assignments grouped by expert (stable)
     tok: torch.Tensor       # [n*k] int64: order // k, the token of each grouped assignment
+    slot: torch.Tensor      # [n*k] int32: inverse of `order`
+    order32: torch.Tensor   # [n*k] int32 copy of `order` for the token-move kernels
     counts: torch.Tensor    # [e] int64
     offsets: torch.Tensor   # [e] int32 inclusive cumsum of counts (torch._grouped_mm offsets)
     aux: torch.Tensor       # load-balance loss
@@ -40,7 +42,7 @@ def dispatch_plan(logits: torch.Tensor, top_k: int, out_dtype=None) -> Dispatch:
     order = r.order.long()
     counts = r.counts.long()
     w = r.weights if out_dtype is None else r.weights.to(out_dtype)
-    return Dispatch(w, r.idx.long(), order, order // top_k, counts,
+    return Dispatch(w, r.idx.long(), order, order // top_k, r.slot, r.order, counts,
                     counts.cumsum(0).to(torch.int32), aux, z)
 
 
@@ -59,3 +61,52 @@ class Router(nn.Module):
         plan = dispatch_plan(logits, self.top_k, x.dtype)
         self.last_plan = plan       # MoE.forward reuses order / counts instead of re-sorting
         return plan.weights, plan.idx, plan.aux, plan.z
+
+
+class Experts(nn.Module):
+    """Stacked SwiGLU experts run as a per-expert loop over contiguous token groups -- the
+    eager path of the reference's ``Experts`` (``forgemind/moe.py:99-164``). The grouped GEMM
+    and expert parallelism of the reference are outside this build."""
+
+    def __init__(self, dim: int, hidden: int, n_experts: int):
+        super().__init__()
+        scale = dim ** -0.5
+        self.w1 = nn.Parameter(torch.randn(n_experts, dim, hidden) * scale)
+        self.w3 = nn.Parameter(torch.randn(n_experts, dim, hidden) * scale)
+        self.w2 = nn.Parameter(torch.randn(n_experts, hidden, dim) * hidden ** -0.5)
+
+    def forward(self, xs: torch.Tensor, counts) -> torch.Tensor:
+        out = torch.empty_like(xs)
+        lo = 0
+        for e, c in enumerate(counts):
+            if c:
+                seg = xs[lo:lo + c]
+                out[lo:lo + c] = (torch.nn.functional.silu(seg @ self.w1[e]) * (seg @ self.w3[e])) @ self.w2[e]
+            lo += c
+        return out
+
+
+class MoE(nn.Module):
+    """Single-device mixture of experts with the forward of the reference's ``MoE.forward``
+    (``forgemind/moe.py:227-251``, ``ep_size == 1``): route, gather tokens by expert, run the
+    experts on contiguous groups, return the weighted outputs to their tokens. Routing and
+    both token moves are fused kernels; ``last_aux`` carries the auxiliary losses."""
+
+    def __init__(self, dim: int, hidden: int, n_experts: int, top_k: int, aux_coef: float = 0.01,
+                 z_coef: float = 1e-3):
+        super().__init__()
+        self.router = Router(dim, n_experts, top_k)
+        self.experts = Experts(dim, hidden, n_experts)
+        self.top_k, self.aux_coef, self.z_coef = int(top_k), aux_coef, z_coef
+        self.last_aux = None
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1])
+        w, _idx, aux, z = self.router(x2)
+        plan = self.router.last_plan
+        self.last_aux = self.aux_coef * aux + self.z_coef * z
+        xs = moe_gather(x2, plan.order32, self.top_k, plan.slot)
+        ys = self.experts(xs, plan.counts.tolist())          # the one host sync of the eager path
+        out = moe_combine(ys, w, plan.slot, plan.order32)
+        return out.reshape(shape)

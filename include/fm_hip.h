@@ -171,6 +171,26 @@ int fm_route(const void* logits, int32_t* idx, float* weights, int32_t* counts, 
              int32_t* order, void* workspace, size_t workspace_bytes, int64_t n, int e, int k,
              int dtype, fm_stream_t stream);
 
+/* ------------------------------------------------------------------ token moves around the permutation
+ * Replaces `xs = x[order // k]` (forgemind/moe.py:234-235): xs[s, :] = scale * x[order[s] / k, :]
+ * with scale = scale_flat[order[s]] when scale_flat (fp32 [n*k], indexed by flat assignment)
+ * is given, 1 otherwise. x: [n, d]; xs: [n*k, d]; order: [n*k] int32 from fm_route.
+ * With a scale it is also the backward of fm_moe_combine wrt ys (x = dout, scale = weights). */
+int fm_moe_gather(const void* x, const int32_t* order, const float* scale_flat, void* xs, int64_t n,
+                  int64_t d, int k, int dtype, fm_stream_t stream);
+
+/* Replaces `ys * w[order]` + `zeros.index_add_(0, order // k, ys)` (moe.py:247-248) by a gather
+ * per token through the slot array of fm_route:
+ *   out[t, :] = sum_j weights[t, j] * ys[slot[t*k + j], :]   (fp32 sum in j order, one rounding)
+ * weights: fp32 [n, k] or NULL for unit weights (then it is the backward of fm_moe_gather).
+ * ys: [n*k, d]; out: [n, d]. No atomics: every output row is written once, deterministically. */
+int fm_moe_combine(const void* ys, const float* weights, const int32_t* slot, void* out, int64_t n,
+                   int64_t d, int k, int dtype, fm_stream_t stream);
+
+/* Backward of fm_moe_combine wrt the weights: dweights[t, j] = <ys[slot[t*k+j], :], dout[t, :]>. */
+int fm_moe_combine_dw(const void* ys, const void* dout, const int32_t* slot, float* dweights,
+                      int64_t n, int64_t d, int k, int dtype, fm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

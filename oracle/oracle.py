@@ -205,3 +205,19 @@ def router_aux(logits, idx):
     aux = e * (frac * probs.mean(dim=0)).sum()
     z = torch.logsumexp(lf, dim=-1).pow(2).mean()
     return aux, z
+
+
+# ------------------------------------------------------------------ token moves around the permutation
+def moe_gather(x, order, k):
+    """xs = x[order // k]. Reference forgemind/moe.py:234-235 (tok = order // top_k; xs = x[tok])."""
+    return x[(order // k).long()]
+
+
+def moe_combine(ys, weights, order, k, n):
+    """out [n, d]. Reference forgemind/moe.py:247-248, rounding points included:
+    ys = ys * w.reshape(-1)[order].unsqueeze(-1)   (product in ys' dtype, w in the activation dtype)
+    out = zeros_like(x).index_add_(0, order // k, ys)   (accumulated in the activation dtype)."""
+    w = weights.to(ys.dtype).reshape(-1)[order.long()].unsqueeze(-1)
+    scaled = ys * w
+    out = torch.zeros(n, ys.shape[1], dtype=ys.dtype)
+    return out.index_add_(0, (order // k).long(), scaled)

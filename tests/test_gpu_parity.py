@@ -37,7 +37,7 @@ def rel_max(got, ref):
     return ((got - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item()
 
 
-def assert_close_lowp(got, ref, dt, what, ulps=2.0, cancel=0.0):
+def assert_close_lowp(got, ref, dt, what, ulps=2.0, cancel=0.0, cancel_lowp=0.0):
     """<= 1e-2 of the tensor's scale, and elementwise within a few ulps of the dtype.
 
     `cancel` is the magnitude of the fp32 terms the result is a difference of (g - xh*c in the
@@ -51,7 +51,9 @@ def assert_close_lowp(got, ref, dt, what, ulps=2.0, cancel=0.0):
     assert ((got - ref).abs().max() / scale).item() <= 1e-2, what
     eps = {BF16: 2.0 ** -8, F16: 2.0 ** -11, F32: 2.0 ** -20}[dt]
     quantum = {BF16: 0.0, F16: 2.0 ** -24, F32: 0.0}[dt]      # fp16 subnormal spacing
-    bound = ulps * eps * ref.abs() + 1e-6 * scale + 8 * 2.0 ** -23 * cancel + quantum
+    # cancel_lowp: same idea when the *reference* rounds its intermediate terms to the storage dtype
+    bound = (ulps * eps * ref.abs() + 1e-6 * scale + 8 * 2.0 ** -23 * cancel + quantum
+             + ulps * eps * float(cancel_lowp))
     bad = ((got - ref).abs() > bound)
     assert not bad.any(), f"{what}: {int(bad.sum())} elements beyond {ulps} ulp"
 
@@ -363,3 +365,35 @@ def test_route_half_precision_logits_and_all_equal_rows():
     assert counts.cpu().tolist() == [130, 130] + [0] * 62
     assert torch.allclose(w.cpu(), torch.full((130, 2), 0.5))
     assert order.cpu().tolist() == list(range(0, 260, 2)) + list(range(1, 260, 2))
+
+
+# ------------------------------------------------------------------ gather / combine around the permutation
+@pytest.mark.parametrize("n,e,k,d,dt", [(1000, 8, 2, 1024, BF16), (257, 16, 4, 100, F32), (64, 4, 1, 7, F16),
+                                         (2048, 64, 2, 4096, BF16), (33, 8, 8, 256, F32)])
+def test_moe_gather_and_combine(n, e, k, d, dt):
+    g = gen(1007)
+    lg = router_inputs(n, e, 77)
+    idx, w, counts, slot, order = O.router(lg, k)
+    x = torch.randn(n, d, generator=g).to(dt)
+    ys = torch.randn(n * k, d, generator=g).to(dt)
+    o32, s32 = order.to(torch.int32).to(DEV), slot.to(torch.int32).to(DEV)
+    xs = _hip.moe_gather(x.to(DEV), o32, k)
+    assert torch.equal(xs.cpu(), O.moe_gather(x, order, k))                    # a pure copy: bit-exact
+    out = _hip.moe_combine(ys.to(DEV), w.to(DEV), s32, n, k)
+    ref = O.moe_combine(ys, w, order, k, n)
+    # the reference rounds each w*y product and each partial sum to the activation dtype
+    assert_close_lowp(out, ref, dt, "combine", ulps=2.0, cancel_lowp=k * float(ys.float().abs().max()))
+    # unit weights undo the gather: k copies of each token (exact for k <= 2: x and 2x need no rounding)
+    back = _hip.moe_combine(xs, None, s32, n, k)
+    if k <= 2:
+        assert torch.equal(back.float().cpu(), (x.float() * k).to(dt).float())
+    else:
+        assert torch.allclose(back.float().cpu(), x.float() * k, rtol=2.0 ** -7 if dt != F32 else 1e-6)
+    # the two backward uses: weighted gather and the weight gradient
+    dout = torch.randn(n, d, generator=g).to(dt)
+    dys = _hip.moe_gather(dout.to(DEV), o32, k, w.reshape(-1).to(DEV))
+    want = (dout.float()[(order // k)] * w.reshape(-1)[order][:, None]).to(dt)
+    assert_close_lowp(dys, want, dt, "combine backward wrt ys", ulps=2.0)
+    dw = _hip.moe_combine_dw(ys.to(DEV), dout.to(DEV), s32, n, k)
+    want_dw = (ys.float()[slot].view(n, k, d) * dout.float()[:, None, :]).sum(-1)
+    assert torch.allclose(dw.cpu(), want_dw, rtol=1e-4, atol=1e-4 * float(want_dw.abs().max()))

@@ -370,3 +370,22 @@ def test_out_of_path_names_keep_their_torch_expression():
     assert q.shape == (2, 5, 3, 8)
     o = kernels.newton_schulz(torch.randn(8, 16))
     assert o.shape == (8, 16)
+
+
+def test_moe_gather_combine_torch_path_and_grads():
+    g = torch.Generator().manual_seed(3)
+    n, k, e, d = 33, 2, 8, 16
+    x = torch.randn(n, d, generator=g, requires_grad=True)
+    r = kernels.moe_route(torch.randn(n, e, generator=g), k)
+    xs = kernels.moe_gather(x, r.order, k, r.slot)
+    assert torch.equal(xs, O.moe_gather(x.detach(), r.order.long(), k))
+    ys = (xs * 2.0)
+    w = r.weights.clone().requires_grad_(True)
+    out = kernels.moe_combine(ys, w, r.slot, r.order)
+    assert torch.allclose(out, O.moe_combine(ys.detach(), w.detach(), r.order.long(), k, n), atol=1e-6)
+    out.square().sum().backward()
+    assert x.grad is not None and w.grad is not None
+    with pytest.raises(ValueError):
+        kernels.moe_gather(x, r.order[:-1], k)
+    with pytest.raises(ValueError):
+        kernels.moe_combine(ys, w, r.slot[:-1])

@@ -317,3 +317,23 @@ def test_router_aux_matches_the_reference_expression():
     c = torch.zeros(8, dtype=torch.int64).scatter_add_(0, idx.reshape(-1), torch.ones(128, dtype=torch.int64))
     assert aux.item() == pytest.approx((8 * ((c / 128) * probs.mean(0)).sum()).item(), rel=1e-6)
     assert z.item() == pytest.approx(logits.logsumexp(-1).pow(2).mean().item(), rel=1e-6)
+
+
+# ------------------------------------------------------------------ gather / combine
+def test_moe_gather_combine_brute_force():
+    g = torch.Generator().manual_seed(9)
+    n, k, e, d = 7, 2, 4, 5
+    x = torch.randn(n, d, generator=g)
+    idx, w, counts, slot, order = O.router(torch.randn(n, e, generator=g), k)
+    xs = O.moe_gather(x, order, k)
+    flat = idx.reshape(-1)
+    for s in range(n * k):                       # grouped position s holds the token of assignment order[s]
+        assert torch.equal(xs[s], x[order[s] // k])
+        assert flat[order[s]] == torch.sort(flat).values[s]
+    ys = torch.randn(n * k, d, generator=g)
+    out = O.moe_combine(ys, w, order, k, n)
+    for t in range(n):
+        want = sum(w[t, j] * ys[slot[t * k + j]] for j in range(k))
+        assert torch.allclose(out[t], want, atol=1e-6)
+    # unit weights after a gather return k copies of every token
+    assert torch.allclose(O.moe_combine(xs, torch.ones(n, k), order, k, n), k * x, atol=1e-6)
