@@ -257,7 +257,7 @@ def make_workload(name, torch, L, dev):
 
         def step():
             _check(L.fm_route(lg.data_ptr(), idx.data_ptr(), wt.data_ptr(), cnt.data_ptr(), sl.data_ptr(),
-                              od.data_ptr(), ws.data_ptr(), nb, n, e, k, F32c, st), "fm_route")
+                              od.data_ptr(), None, ws.data_ptr(), nb, n, e, k, F32c, st), "fm_route")
 
         w.step = step
         w.dominant_launch = step

@@ -42,11 +42,18 @@ template <typename T, int EPL>
 __global__ __launch_bounds__(kRouteThreads) void route_kernel(const T* __restrict__ logits,
                                                                int32_t* __restrict__ idx,
                                                                float* __restrict__ weights,
-                                                               int32_t* __restrict__ hist, int64_t n,
+                                                               int32_t* __restrict__ hist,
+                                                               float* __restrict__ fstat, int64_t n,
                                                                int e, int k, int tile_rows) {
   constexpr int R = kRowsAtOnce;
   constexpr int NW = kRouteThreads / 64;
   __shared__ int lh[kMaxE];
+  __shared__ float wstat[NW][EPL * 64];   // per-wave column sums of the probabilities
+  __shared__ float wz[NW];                // per-wave sums of logsumexp^2
+  float psum[EPL];
+  float zsum = 0.f;
+#pragma unroll
+  for (int q = 0; q < EPL; ++q) psum[q] = 0.f;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int i = tid; i < e; i += kRouteThreads) lh[i] = 0;
   __syncthreads();
@@ -94,6 +101,11 @@ __global__ __launch_bounds__(kRouteThreads) void route_kernel(const T* __restric
       for (int q = 0; q < EPL; ++q) {
         p[r][q] = p[r][q] / s[r];
         key[r][q] = (lane + 64 * q) < e ? key_of(p[r][q]) : 0u;   // 0 is below every real key
+        if (live[r] && (lane + 64 * q) < e) psum[q] += p[r][q];    // rows in ascending order
+      }
+      if (live[r]) {
+        const float lse = m[r] + fast_log2(s[r]) * kLn2;
+        zsum += lse * lse;
       }
     }
     int my_i[R];
@@ -145,8 +157,48 @@ __global__ __launch_bounds__(kRouteThreads) void route_kernel(const T* __restric
       }
     }
   }
+  if (fstat != nullptr) {
+#pragma unroll
+    for (int q = 0; q < EPL; ++q) wstat[wave][lane + 64 * q] = psum[q];
+    if (lane == 0) wz[wave] = zsum;
+  }
   __syncthreads();
   for (int i = tid; i < e; i += kRouteThreads) hist[(int64_t)blockIdx.x * e + i] = lh[i];
+  if (fstat != nullptr) {   // fold the waves in wave order: one fp32 partial row per tile
+    float* out = fstat + (int64_t)blockIdx.x * (e + 1);
+    for (int i = tid; i < e; i += kRouteThreads) {
+      float a = wstat[0][i];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) a += wstat[w][i];
+      out[i] = a;
+    }
+    if (tid == 0) {
+      float a = wz[0];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) a += wz[w];
+      out[e] = a;
+    }
+  }
+}
+
+// Sums the per-tile partial rows [ntiles, e+1] in tile order: stats[0..e) = column sums of the
+// probabilities, stats[e] = sum of logsumexp^2. One workgroup; thread c owns column c.
+__global__ __launch_bounds__(1024) void route_stats_kernel(const float* __restrict__ fstat,
+                                                            float* __restrict__ stats, int e,
+                                                            int ntiles) {
+  const int c = threadIdx.x;
+  if (c > e) return;
+  float a = 0.f;
+  int t = 0;
+  for (; t + 7 < ntiles; t += 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = fstat[(int64_t)(t + u) * (e + 1) + c];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) a += v[u];
+  }
+  for (; t < ntiles; ++t) a += fstat[(int64_t)t * (e + 1) + c];
+  stats[c] = a;
 }
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
@@ -304,12 +356,12 @@ Tiling make_tiling(int64_t n) {
 }
 
 template <typename T>
-int launch_route(const void* logits, int32_t* idx, float* weights, int32_t* hist, int64_t n, int e,
-                 int k, const Tiling& tl, hipStream_t st) {
+int launch_route(const void* logits, int32_t* idx, float* weights, int32_t* hist, float* fstat,
+                 int64_t n, int e, int k, const Tiling& tl, hipStream_t st) {
   const T* lp = static_cast<const T*>(logits);
   const dim3 grid((unsigned)tl.ntiles), block(kRouteThreads);
 #define GO(EPL) \
-  hipLaunchKernelGGL((route_kernel<T, EPL>), grid, block, 0, st, lp, idx, weights, hist, n, e, k, tl.tile_rows)
+  hipLaunchKernelGGL((route_kernel<T, EPL>), grid, block, 0, st, lp, idx, weights, hist, fstat, n, e, k, tl.tile_rows)
   if (e <= 64) GO(1);
   else if (e <= 128) GO(2);
   else if (e <= 256) GO(4);
@@ -324,14 +376,15 @@ extern "C" {
 
 size_t fm_route_workspace(int64_t n, int e, int k) {
   (void)k;
-  if (n <= 0 || e <= 0) return 0;
+  if (n < 0 || e <= 0) return 0;
   const Tiling tl = make_tiling(n);
-  return (size_t)tl.ntiles * (size_t)e * sizeof(int32_t);
+  // [ntiles, e] int32 histograms, then [ntiles, e+1] fp32 statistics partials
+  return (size_t)tl.ntiles * ((size_t)e * sizeof(int32_t) + (size_t)(e + 1) * sizeof(float));
 }
 
 int fm_route(const void* logits, int32_t* idx, float* weights, int32_t* counts, int32_t* slot,
-             int32_t* order, void* workspace, size_t workspace_bytes, int64_t n, int e, int k,
-             int dtype, fm_stream_t stream) {
+             int32_t* order, float* stats, void* workspace, size_t workspace_bytes, int64_t n, int e,
+             int k, int dtype, fm_stream_t stream) {
   FM_CHECK_ARG(n >= 0 && e > 0 && k >= 1, "fm_route: bad shape n=%lld e=%d k=%d", (long long)n, e, k);
   FM_CHECK_ARG(dtype == FM_F32 || dtype == FM_F16 || dtype == FM_BF16, "fm_route: bad dtype %d", dtype);
   FM_CHECK_ARG(k <= e, "fm_route: selected index k out of range (got %d vs %d)", k, e);
@@ -343,18 +396,26 @@ int fm_route(const void* logits, int32_t* idx, float* weights, int32_t* counts, 
   FM_CHECK_ARG(counts != nullptr, "fm_route: NULL counts");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const Tiling tl = make_tiling(n);
-  const size_t need = (size_t)tl.ntiles * (size_t)e * sizeof(int32_t);
+  const size_t hist_bytes = (size_t)tl.ntiles * (size_t)e * sizeof(int32_t);
+  const size_t need = hist_bytes + (size_t)tl.ntiles * (size_t)(e + 1) * sizeof(float);
   if (workspace == nullptr || workspace_bytes < need) {
     fm_host::set_error("fm_route: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
     return FM_ERR_WORKSPACE;
   }
   FM_CHECK_ARG(n == 0 || (logits && idx && weights), "fm_route: NULL pointer");
   int32_t* hist = static_cast<int32_t*>(workspace);
-  // with n == 0 the single tile has no rows and leaves an all-zero histogram
-  if (dtype == FM_F32) launch_route<float>(logits, idx, weights, hist, n, e, k, tl, st);
-  else if (dtype == FM_BF16) launch_route<bf16_t>(logits, idx, weights, hist, n, e, k, tl, st);
-  else launch_route<f16_t>(logits, idx, weights, hist, n, e, k, tl, st);
+  float* fstat = stats != nullptr
+                     ? reinterpret_cast<float*>(static_cast<char*>(workspace) + hist_bytes)
+                     : nullptr;
+  // with n == 0 the single tile has no rows and leaves all-zero partials
+  if (dtype == FM_F32) launch_route<float>(logits, idx, weights, hist, fstat, n, e, k, tl, st);
+  else if (dtype == FM_BF16) launch_route<bf16_t>(logits, idx, weights, hist, fstat, n, e, k, tl, st);
+  else launch_route<f16_t>(logits, idx, weights, hist, fstat, n, e, k, tl, st);
   FM_CHECK_LAUNCH("fm_route");
+  if (stats != nullptr) {
+    hipLaunchKernelGGL(route_stats_kernel, dim3(1), dim3(1024), 0, st, fstat, stats, e, tl.ntiles);
+    FM_CHECK_LAUNCH("fm_route(stats)");
+  }
   const int emit = (slot != nullptr || order != nullptr) && n > 0 ? 1 : 0;
   hipLaunchKernelGGL(permute_kernel, dim3(emit ? (unsigned)tl.ntiles : 1u), dim3(256), 0, st, idx, hist,
                      counts, slot, order, n, e, k, tl.tile_rows, tl.ntiles, emit);

@@ -49,7 +49,7 @@ SIGNATURES = {
     "fm_moe_gather": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "fm_moe_combine": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "fm_moe_combine_dw": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
-    "fm_route": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _int, _int, _int, _vp]),
+    "fm_route": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _int, _int, _int, _vp]),
 }
 
 
@@ -280,8 +280,9 @@ def softmax_fwd(x2):
     return y
 
 
-def route(logits2, k: int, want_permutation: bool = True):
-    """-> (idx int32 [n, k], weights fp32 [n, k], counts int32 [e], slot, order int32 [n*k])."""
+def route(logits2, k: int, want_permutation: bool = True, want_stats: bool = False):
+    """-> (idx int32 [n, k], weights fp32 [n, k], counts int32 [e], slot, order int32 [n*k])
+    and, with want_stats, a sixth item: fp32 [e+1] = column sums of probs, then sum(lse^2)."""
     _dense(logits2)
     n, e = logits2.shape
     dev = logits2.device
@@ -290,12 +291,15 @@ def route(logits2, k: int, want_permutation: bool = True):
     counts = torch.empty(e, device=dev, dtype=torch.int32)
     slot = torch.empty(n * k, device=dev, dtype=torch.int32) if want_permutation else None
     order = torch.empty(n * k, device=dev, dtype=torch.int32) if want_permutation else None
+    stats = torch.empty(e + 1, device=dev, dtype=torch.float32) if want_stats else None
     with torch.cuda.device(dev):
         nbytes = int(lib().fm_route_workspace(n, e, k))
         ws = torch.empty(max(nbytes, 16), device=dev, dtype=torch.uint8)
         _check(lib().fm_route(_ptr(logits2), _ptr(idx), _ptr(wts), _ptr(counts), _ptr(slot),
-                              _ptr(order), _ptr(ws), nbytes, n, e, int(k),
+                              _ptr(order), _ptr(stats), _ptr(ws), nbytes, n, e, int(k),
                               dtype_code(logits2.dtype), _stream(logits2)), "fm_route")
+    if want_stats:
+        return idx, wts, counts, slot, order, stats
     return idx, wts, counts, slot, order
 
 

@@ -30,9 +30,11 @@ class Routing(NamedTuple):
     counts: torch.Tensor    # [e] int32 assignments per expert
     slot: torch.Tensor      # [n*k] int32 position of flat assignment p after the stable sort
     order: torch.Tensor     # [n*k] int32 inverse: order[slot[p]] == p (== stable argsort of idx.flat)
+    aux: "torch.Tensor | None" = None   # load-balance loss E * sum(frac * mean(probs)) (with_aux=True)
+    z: "torch.Tensor | None" = None     # router z-loss mean(logsumexp(logits)^2)     (with_aux=True)
 
 
-def _torch_route(logits: torch.Tensor, k: int) -> Routing:
+def _torch_route(logits: torch.Tensor, k: int, with_aux: bool = False) -> Routing:
     """The same result from torch ops (CPU tensors, float64, oversize shapes)."""
     probs = torch.softmax(logits.float(), dim=-1)
     top_p, idx = fb.topk_canonical(probs, k)
@@ -44,39 +46,73 @@ def _torch_route(logits: torch.Tensor, k: int) -> Routing:
     order = torch.sort(flat, stable=True).indices
     slot = torch.empty_like(order)
     slot[order] = torch.arange(order.numel(), device=order.device)
+    aux = z = None
+    if with_aux:
+        frac = counts.to(torch.float32) / max(flat.numel(), 1)
+        aux = e * (frac * probs.mean(dim=0)).sum()
+        z = torch.logsumexp(logits.float(), dim=-1).pow(2).mean()
     return Routing(idx.to(torch.int32), weights, counts.to(torch.int32), slot.to(torch.int32),
-                   order.to(torch.int32))
+                   order.to(torch.int32), aux, z)
+
+
+def _aux_z(counts, stats, n: int, k: int, e: int):
+    """aux = E * sum(frac * mean_rows(probs)), z = mean(logsumexp^2) (reference moe.py:92-95)."""
+    frac = counts.to(torch.float32) / max(n * k, 1)
+    aux = e * (frac * (stats[:e] / max(n, 1))).sum()
+    z = stats[e] / max(n, 1)
+    return aux, z
 
 
 class _RouteFn(torch.autograd.Function):
-    """Weights are differentiable wrt the logits; every integer output is not."""
+    """Weights and the two auxiliary losses are differentiable wrt the logits; every integer
+    output is not. The backward recomputes softmax on the small [n, e] tensor with tensor ops."""
 
     @staticmethod
-    def forward(ctx, logits, k):
-        idx, w, counts, slot, order = _hip.route(logits.contiguous(), k, True)
-        ctx.save_for_backward(logits, idx)
+    def forward(ctx, logits, k, with_aux):
+        n, e = logits.shape
+        if with_aux:
+            idx, w, counts, slot, order, stats = _hip.route(logits.contiguous(), k, True, True)
+            aux, z = _aux_z(counts, stats, n, k, e)
+        else:
+            idx, w, counts, slot, order = _hip.route(logits.contiguous(), k, True)
+            aux = z = logits.new_zeros((), dtype=torch.float32)
+        ctx.save_for_backward(logits, idx, counts)
+        ctx.k, ctx.with_aux = k, with_aux
         ctx.mark_non_differentiable(idx, counts, slot, order)
-        return idx, w, counts, slot, order
+        return idx, w, counts, slot, order, aux, z
 
     @staticmethod
-    def backward(ctx, _gi, gw, _gc, _gs, _go):
-        logits, idx = ctx.saved_tensors
-        if gw is None:
-            return None, None
-        # d/dlogits of (p_top / sum p_top) with p = softmax(logits): recomputed on the tiny
-        # [n, e] tensor with tensor ops
-        p = torch.softmax(logits.float(), dim=-1)
-        pk = torch.gather(p, 1, idx.long())
-        s = pk.sum(dim=-1, keepdim=True)
-        w = pk / s
-        g_pk = (gw - (gw * w).sum(dim=-1, keepdim=True)) / s          # through the renormalise
-        g_p = torch.zeros_like(p).scatter_(1, idx.long(), g_pk)      # through the gather
-        g_logits = (g_p - (g_p * p).sum(dim=-1, keepdim=True)) * p    # through the softmax
-        return g_logits.to(logits.dtype), None
+    def backward(ctx, _gi, gw, _gc, _gs, _go, g_aux, g_z):
+        logits, idx, counts = ctx.saved_tensors
+        n, e = logits.shape
+        lf = logits.float()
+        lse = torch.logsumexp(lf, dim=-1, keepdim=True)
+        p = torch.exp(lf - lse)
+        g_p = torch.zeros_like(p)
+        if gw is not None:
+            # through the renormalise and the gather: w = p_top / sum(p_top)
+            pk = torch.gather(p, 1, idx.long())
+            s = pk.sum(dim=-1, keepdim=True)
+            w = pk / s
+            g_pk = (gw - (gw * w).sum(dim=-1, keepdim=True)) / s
+            g_p.scatter_(1, idx.long(), g_pk)
+        g_logits = None
+        if ctx.with_aux and g_aux is not None:
+            # aux = E * sum_e frac_e * mean_rows(p)_e, with frac a constant (no_grad in moe.py:92-93)
+            frac = counts.to(torch.float32) / max(n * ctx.k, 1)
+            g_p = g_p + g_aux * (e / max(n, 1)) * frac
+        g_logits = (g_p - (g_p * p).sum(dim=-1, keepdim=True)) * p          # through the softmax
+        if ctx.with_aux and g_z is not None:
+            g_logits = g_logits + g_z * (2.0 / max(n, 1)) * lse * p          # d mean(lse^2) / dlogits
+        return g_logits.to(logits.dtype), None, None
 
 
-def moe_route(logits: torch.Tensor, k: int) -> Routing:
+def moe_route(logits: torch.Tensor, k: int, with_aux: bool = False) -> Routing:
     """Route ``n`` tokens over ``e`` experts: ``logits`` is ``[n, e]``.
+
+    ``with_aux=True`` also returns the two auxiliary router losses of the reference
+    (``moe.py:92-95``), computed from sums the routing kernel accumulates on the way, so the
+    logits are read once; both are differentiable wrt ``logits``.
 
     Returns a :class:`Routing`. ``flat[p] = idx[p // k, p % k]`` is the expert of flat
     assignment ``p``; ``order`` lists the flat assignments grouped by expert, ascending ``p``
@@ -90,10 +126,11 @@ def moe_route(logits: torch.Tensor, k: int) -> Routing:
         raise RuntimeError(f"selected index k out of range (got {k} vs {e})")
     if e > MAX_EXPERTS or k > MAX_TOP_K or n * k >= 2 ** 31 - 1:
         _note("route shape")
-        return _torch_route(logits, k)
+        return _torch_route(logits, k, with_aux)
     if not fast_ok(logits):
-        return _torch_route(logits, k)
-    return Routing(*_RouteFn.apply(logits, k))
+        return _torch_route(logits, k, with_aux)
+    out = _RouteFn.apply(logits, k, bool(with_aux))
+    return Routing(*out) if with_aux else Routing(*out[:5])
 
 
 __all__ = ["moe_route", "Routing", "MAX_EXPERTS", "MAX_TOP_K"]

@@ -33,12 +33,8 @@ class Dispatch(NamedTuple):
 
 def dispatch_plan(logits: torch.Tensor, top_k: int, out_dtype=None) -> Dispatch:
     """Everything the expert layer needs from ``[n, e]`` router logits."""
-    e = logits.shape[-1]
-    r = moe_route(logits, top_k)
-    probs_mean = torch.softmax(logits.float(), dim=-1).mean(dim=0)
-    frac = r.counts.to(torch.float32) / max(r.idx.numel(), 1)
-    aux = e * (frac.detach() * probs_mean).sum()
-    z = torch.logsumexp(logits.float(), dim=-1).pow(2).mean()
+    r = moe_route(logits, top_k, with_aux=True)
+    aux, z = r.aux, r.z
     order = r.order.long()
     counts = r.counts.long()
     w = r.weights if out_dtype is None else r.weights.to(out_dtype)

@@ -165,11 +165,14 @@ int fm_softmax_fwd(const void* x, void* y, int64_t n, int64_t v, int dtype, fm_s
  *   order[slot[p]] = p  (== torch.sort(flat, stable=True).indices).
  * logits: [n, e] of dtype (fp32 math inside); idx: [n, k] int32; weights: [n, k] fp32;
  * counts: [e] int32; slot, order: [n*k] int32 (either may be NULL: then only routing and
- * counts are produced when both are NULL). 1 <= k <= 8, k <= e <= 512, n*k < 2^31. */
+ * counts are produced when both are NULL). stats: fp32 [e+1] or NULL; receives what the
+ * auxiliary losses of moe.py:92-95 need without another pass over the logits:
+ *   stats[j] = sum_rows probs[:, j] (j < e),  stats[e] = sum_rows logsumexp(logits)^2,
+ * summed in a fixed order. 1 <= k <= 8, k <= e <= 512, n*k < 2^31. */
 size_t fm_route_workspace(int64_t n, int e, int k);
 int fm_route(const void* logits, int32_t* idx, float* weights, int32_t* counts, int32_t* slot,
-             int32_t* order, void* workspace, size_t workspace_bytes, int64_t n, int e, int k,
-             int dtype, fm_stream_t stream);
+             int32_t* order, float* stats, void* workspace, size_t workspace_bytes, int64_t n,
+             int e, int k, int dtype, fm_stream_t stream);
 
 /* ------------------------------------------------------------------ token moves around the permutation
  * Replaces `xs = x[order // k]` (forgemind/moe.py:234-235): xs[s, :] = scale * x[order[s] / k, :]

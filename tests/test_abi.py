@@ -62,8 +62,8 @@ def test_argument_validation_happens_before_any_launch(lib):
     assert lib.fm_topk(None, None, None, 4, 4096, 600, 0, 32, None) == 2             # k > 512
     assert lib.fm_kl_fwd(None, None, None, None, None, None, 4, 8, 2, 1.0, 9, None) == 1
     assert lib.fm_ce_fwd(None, None, None, None, None, None, 4, 8, 2, -100, 0, None) == 1
-    assert lib.fm_route(None, None, None, None, None, None, None, 0, 4, 8, 9, 0, None) == 1
-    assert lib.fm_route(None, None, None, None, None, None, None, 0, 4, 1024, 2, 0, None) == 2
+    assert lib.fm_route(None, None, None, None, None, None, None, None, 0, 4, 8, 9, 0, None) == 1
+    assert lib.fm_route(None, None, None, None, None, None, None, None, 0, 4, 1024, 2, 0, None) == 2
     # empty problems are a no-op that succeeds
     assert lib.fm_rmsnorm_fwd(None, None, None, None, 0, 8, 2, 2, 1e-6, None) == 0
     assert lib.fm_softmax_fwd(None, None, 0, 8, 2, None) == 0

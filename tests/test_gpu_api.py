@@ -259,6 +259,20 @@ def test_router_module_and_route_backward():
     assert torch.allclose(lg.grad, lr.grad, rtol=1e-4, atol=1e-7)
     (w.sum() + aux + z).backward()
     assert router.gate.weight.grad is not None
+    # auxiliary losses and their gradients against the reference expression (moe.py:92-95)
+    la = logits.detach().clone().requires_grad_(True)
+    ra = kernels.moe_route(la, 2, with_aux=True)
+    (3.0 * ra.aux + 0.5 * ra.z + (ra.weights * gw).sum()).backward()
+    lb = logits.detach().clone().requires_grad_(True)
+    pb = lb.softmax(-1)
+    pkb = pb.gather(1, ra.idx.long())
+    wb = pkb / pkb.sum(-1, keepdim=True)
+    frac = ra.counts.float() / ra.idx.numel()
+    aux_b = 16 * (frac * pb.mean(0)).sum()
+    z_b = lb.logsumexp(-1).pow(2).mean()
+    (3.0 * aux_b + 0.5 * z_b + (wb * gw).sum()).backward()
+    assert ra.aux.item() == pytest.approx(aux_b.item(), rel=1e-5) and ra.z.item() == pytest.approx(z_b.item(), rel=1e-5)
+    assert torch.allclose(la.grad, lb.grad, rtol=1e-4, atol=1e-7)
 
 
 def test_modules_on_gpu():

@@ -352,6 +352,15 @@ def test_route_is_bit_exact(n, e, k):
     assert torch.allclose(w.cpu(), ow, rtol=1e-5, atol=0)
     i2, w2, c2, none_a, none_b = _hip.route(lg.to(DEV), k, want_permutation=False)
     assert none_a is None and none_b is None and torch.equal(i2, idx) and torch.equal(c2, counts)
+    # the sums behind the auxiliary losses (forgemind/moe.py:92-95), from the same pass
+    *_, stats = _hip.route(lg.to(DEV), k, want_stats=True)
+    probs = torch.softmax(lg.double(), -1)
+    assert torch.allclose(stats[:e].cpu().double(), probs.sum(0), rtol=1e-4, atol=1e-6)
+    lse2 = torch.logsumexp(lg.double(), -1).pow(2).sum()
+    assert stats[e].item() == pytest.approx(lse2.item(), rel=1e-4)
+    aux, z = O.router_aux(lg, oi)
+    got_aux = e * ((counts.cpu().float() / (n * k)) * (stats[:e].cpu() / n)).sum()
+    assert got_aux.item() == pytest.approx(aux.item(), rel=1e-4) and (stats[e] / n).item() == pytest.approx(z.item(), rel=1e-4)
 
 
 def test_route_half_precision_logits_and_all_equal_rows():
