@@ -49,6 +49,10 @@ SIGNATURES = {
     "fm_moe_gather": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "fm_moe_combine": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "fm_moe_combine_dw": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
+    "fm_swiglu_fwd": (_int, [_vp, _vp, _vp, _i64, _int, _vp]),
+    "fm_swiglu_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _vp]),
+    "fm_swiglu_split_fwd": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
+    "fm_swiglu_split_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _vp]),
     "fm_route": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _int, _int, _int, _vp]),
 }
 
@@ -335,3 +339,43 @@ def moe_combine_dw(ys, dout, slot, n: int, k: int):
         _check(lib().fm_moe_combine_dw(_ptr(ys), _ptr(dout), _ptr(slot), _ptr(dw), n, d, int(k),
                                        dtype_code(ys.dtype), _stream(ys)), "fm_moe_combine_dw")
     return dw
+
+
+# ------------------------------------------------------------------ SwiGLU epilogues
+def swiglu_fwd(gate, up):
+    _dense(gate, up)
+    y = torch.empty_like(gate)
+    with torch.cuda.device(gate.device):
+        _check(lib().fm_swiglu_fwd(_ptr(gate), _ptr(up), _ptr(y), gate.numel(), dtype_code(gate.dtype),
+                                   _stream(gate)), "fm_swiglu_fwd")
+    return y
+
+
+def swiglu_bwd(gate, up, dy):
+    _dense(gate, up, dy)
+    dg, du = torch.empty_like(gate), torch.empty_like(up)
+    with torch.cuda.device(gate.device):
+        _check(lib().fm_swiglu_bwd(_ptr(gate), _ptr(up), _ptr(dy), _ptr(dg), _ptr(du), gate.numel(),
+                                   dtype_code(gate.dtype), _stream(gate)), "fm_swiglu_bwd")
+    return dg, du
+
+
+def swiglu_split_fwd(x2):
+    """x2 [rows, 2h] -> y [rows, h]."""
+    _dense(x2)
+    rows, w = x2.shape
+    y = torch.empty((rows, w // 2), device=x2.device, dtype=x2.dtype)
+    with torch.cuda.device(x2.device):
+        _check(lib().fm_swiglu_split_fwd(_ptr(x2), _ptr(y), rows, w // 2, dtype_code(x2.dtype),
+                                         _stream(x2)), "fm_swiglu_split_fwd")
+    return y
+
+
+def swiglu_split_bwd(x2, dy2):
+    _dense(x2, dy2)
+    rows, w = x2.shape
+    dx = torch.empty_like(x2)
+    with torch.cuda.device(x2.device):
+        _check(lib().fm_swiglu_split_bwd(_ptr(x2), _ptr(dy2), _ptr(dx), rows, w // 2,
+                                         dtype_code(x2.dtype), _stream(x2)), "fm_swiglu_split_bwd")
+    return dx

@@ -12,7 +12,7 @@ import types
 import torch
 import torch.nn as nn
 
-from .extras import swiglu, swiglu_split
+from .swiglu import swiglu, swiglu_split
 from .norm import rms_norm
 
 

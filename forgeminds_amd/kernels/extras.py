@@ -1,8 +1,7 @@
 """Surface names of the reference's kernel package that are outside the packed hot path.
 
-``swiglu``, ``swiglu_split``, ``qk_norm_rope`` and ``newton_schulz`` are elementwise or
-GEMM-bound utilities (reference ``forgemind/kernels/{swiglu,rope,ns}.py``); they keep their
-torch expression here so code written against ``fm.kernels`` imports and runs unchanged.
+``qk_norm_rope`` and ``newton_schulz`` (reference ``forgemind/kernels/{rope,ns}.py``) keep
+their torch expression here so code written against ``fm.kernels`` imports and runs unchanged.
 """
 
 from __future__ import annotations
@@ -10,20 +9,6 @@ from __future__ import annotations
 import torch
 
 from . import _fallback as fb
-
-
-def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
-    """``F.silu(gate) * up`` with fp32 math for half inputs (reference ``swiglu.py:291-298``)."""
-    if gate.shape != up.shape:
-        raise ValueError(f"swiglu: gate {tuple(gate.shape)} and up {tuple(up.shape)} differ")
-    return fb.swiglu(gate, up)
-
-
-def swiglu_split(gate_up: torch.Tensor) -> torch.Tensor:
-    """``silu(x[..., :h]) * x[..., h:]`` for a fused gate|up projection (``swiglu.py:301-309``)."""
-    if gate_up.shape[-1] % 2 != 0:
-        raise ValueError(f"swiglu_split needs an even last dim, got {gate_up.shape[-1]}")
-    return fb.swiglu_split(gate_up)
 
 
 def qk_norm_rope(x, w, cos, sin, eps: float = 1e-6):
@@ -49,4 +34,4 @@ def newton_schulz(g: torch.Tensor, steps: int = 5, eps: float = 1e-7) -> torch.T
     return x.to(g.dtype)
 
 
-__all__ = ["swiglu", "swiglu_split", "qk_norm_rope", "newton_schulz"]
+__all__ = ["qk_norm_rope", "newton_schulz"]

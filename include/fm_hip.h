@@ -194,6 +194,18 @@ int fm_moe_combine(const void* ys, const float* weights, const int32_t* slot, vo
 int fm_moe_combine_dw(const void* ys, const void* dout, const int32_t* slot, float* dweights,
                       int64_t n, int64_t d, int k, int dtype, fm_stream_t stream);
 
+/* ------------------------------------------------------------------ SwiGLU epilogues
+ * Replace _swiglu_fwd_kernel / _swiglu_bwd_kernel and the split variants
+ * (forgemind/kernels/swiglu.py:48-120); semantics of _fallback.swiglu (_fallback.py:48-49):
+ * y = silu(gate) * up in fp32, one rounding. n counts elements; the split form reads a fused
+ * projection x [rows, 2h] (gate = x[:, :h], up = x[:, h:]) and writes y [rows, h] / dx [rows, 2h]. */
+int fm_swiglu_fwd(const void* gate, const void* up, void* y, int64_t n, int dtype, fm_stream_t stream);
+int fm_swiglu_bwd(const void* gate, const void* up, const void* dy, void* dgate, void* dup, int64_t n,
+                  int dtype, fm_stream_t stream);
+int fm_swiglu_split_fwd(const void* x, void* y, int64_t rows, int64_t h, int dtype, fm_stream_t stream);
+int fm_swiglu_split_bwd(const void* x, const void* dy, void* dx, int64_t rows, int64_t h, int dtype,
+                        fm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

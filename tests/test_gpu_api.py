@@ -113,7 +113,9 @@ def test_op_path_equals_eager_path_bit_for_bit():
         return out.detach().clone(), [t.grad.clone() for t in ins if t.grad is not None]
 
     for fn in (lambda t: kernels.rms_norm(t[0], t[2], 1e-6),
-               lambda t: sum(kernels.add_rms_norm(t[0], t[1], t[2], 1e-6))):
+               lambda t: sum(kernels.add_rms_norm(t[0], t[1], t[2], 1e-6)),
+               lambda t: kernels.swiglu(t[0], t[1]) * t[2],
+               lambda t: kernels.swiglu_split(t[0]) * t[2][:32] + t[1][:, :32]):
         ye, ge = run(False, fn)
         yo, go = run(True, fn)
         assert torch.equal(ye, yo) and len(ge) == len(go)

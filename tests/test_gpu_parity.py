@@ -406,3 +406,34 @@ def test_moe_gather_and_combine(n, e, k, d, dt):
     dw = _hip.moe_combine_dw(ys.to(DEV), dout.to(DEV), s32, n, k)
     want_dw = (ys.float()[slot].view(n, k, d) * dout.float()[:, None, :]).sum(-1)
     assert torch.allclose(dw.cpu(), want_dw, rtol=1e-4, atol=1e-4 * float(want_dw.abs().max()))
+
+
+# ------------------------------------------------------------------ SwiGLU epilogues
+@pytest.mark.parametrize("shape,dt", [((37,), F32), ((4096,), F32), ((300, 11008), BF16), ((7, 33), F16),
+                                       ((2, 5, 64), BF16)])
+def test_swiglu_fwd_bwd(shape, dt):
+    g = gen(31)
+    a, b, dy = (torch.randn(*shape, generator=g).to(dt) for _ in range(3))
+    ar, br = a.float().requires_grad_(True), b.float().requires_grad_(True)
+    ref = torch.nn.functional.silu(ar) * br
+    ref.backward(dy.float())
+    y = _hip.swiglu_fwd(a.to(DEV), b.to(DEV))
+    da, db = _hip.swiglu_bwd(a.to(DEV), b.to(DEV), dy.to(DEV))
+    assert_close_lowp(y, ref.detach(), dt, "swiglu", ulps=2.0)
+    assert_close_lowp(da, ar.grad, dt, "dgate", ulps=3.0, cancel=float(dy.float().abs().max() * b.float().abs().max()))
+    assert_close_lowp(db, br.grad, dt, "dup", ulps=3.0)
+
+
+@pytest.mark.parametrize("rows,h,dt", [(6, 8, F32), (5, 6, F32), (3, 32, BF16), (200, 11008, BF16), (9, 1, F32),
+                                        (4, 100, F16)])
+def test_swiglu_split_fwd_bwd(rows, h, dt):
+    g = gen(32)
+    x = torch.randn(rows, 2 * h, generator=g).to(dt)
+    dy = torch.randn(rows, h, generator=g).to(dt)
+    xr = x.float().requires_grad_(True)
+    ref = torch.nn.functional.silu(xr[:, :h]) * xr[:, h:]
+    ref.backward(dy.float())
+    y = _hip.swiglu_split_fwd(x.to(DEV))
+    dx = _hip.swiglu_split_bwd(x.to(DEV), dy.to(DEV))
+    assert_close_lowp(y, ref.detach(), dt, "swiglu_split", ulps=2.0)
+    assert_close_lowp(dx, xr.grad, dt, "dx", ulps=3.0, cancel=float(dy.float().abs().max() * x.float().abs().max()))
