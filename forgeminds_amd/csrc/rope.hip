@@ -1,0 +1,249 @@
+// Per-head RMSNorm followed by half-split RoPE, forward and backward, for gfx950.
+//
+// Reference semantics: forgemind/kernels/_fallback.py:38-45 and forgemind/kernels/rope.py:46-120:
+// x is [B, T, H, D]; per head r = rsqrt(mean(x^2) + eps), y = x * r * w, then with the halves
+// (y1, y2) and cos/sin [T, D/2]:  out = (y1*cos - y2*sin, y1*sin + y2*cos), one rounding.
+// Backward: rotate the incoming gradient back (dy1 = do1*cos + do2*sin, dy2 = -do1*sin + do2*cos),
+// then the RMSNorm backward of norm.hip; dw = sum over heads of dy * xhat in fp32, written as
+// one partial row per workgroup and summed in a fixed order.
+//
+// Heads are short (64-256 elements), so a head is owned by a group of G lanes; a lane holds up
+// to four consecutive elements of each half, which keeps both rotation partners in one thread.
+#include "fm_common.cuh"
+
+using namespace fm;
+
+namespace {
+
+constexpr int kEH = 4;        // elements per lane per half
+constexpr int kBlock = 256;
+
+template <typename T, typename WT, int G, bool BWD>
+__global__ __launch_bounds__(kBlock) void rope_kernel(const T* __restrict__ x, const WT* __restrict__ w,
+                                                       const float* __restrict__ cosv,
+                                                       const float* __restrict__ sinv,
+                                                       const T* __restrict__ dout, float* __restrict__ rstd,
+                                                       T* __restrict__ out, float* __restrict__ partial,
+                                                       int64_t rows, int t_len, int heads, int d, float eps,
+                                                       int64_t tiles) {
+  constexpr int RPB = kBlock / G;
+  __shared__ float fold[BWD ? RPB * G * 2 * kEH : 1];
+  const int tid = threadIdx.x, rib = tid / G, l = tid % G;
+  const int half = d / 2;
+  float wv1[kEH], wv2[kEH], a1[kEH], a2[kEH];
+#pragma unroll
+  for (int e = 0; e < kEH; ++e) {
+    const int j = l * kEH + e;
+    wv1[e] = j < half ? Elem<WT>::load1(w + j) : 0.f;
+    wv2[e] = j < half ? Elem<WT>::load1(w + half + j) : 0.f;
+    a1[e] = 0.f; a2[e] = 0.f;
+  }
+  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    const int64_t row = tile * RPB + rib;
+    const bool valid = row < rows;
+    const int t = valid ? (int)((row / heads) % t_len) : 0;
+    const T* xp = x + row * (int64_t)d;
+    float x1[kEH], x2[kEH], c[kEH], s[kEH];
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < kEH; ++e) {
+      const int j = l * kEH + e;
+      const bool on = valid && j < half;
+      x1[e] = on ? Elem<T>::load1(xp + j) : 0.f;
+      x2[e] = on ? Elem<T>::load1(xp + half + j) : 0.f;
+      c[e] = on ? cosv[(int64_t)t * half + j] : 0.f;
+      s[e] = on ? sinv[(int64_t)t * half + j] : 0.f;
+      ss += x1[e] * x1[e] + x2[e] * x2[e];
+    }
+    if constexpr (!BWD) {
+      ss = group_reduce<G, OpSum>(ss);
+      const float r = rsqrtf(ss / (float)d + eps);
+      if (valid && l == 0) rstd[row] = r;
+      T* op = out + row * (int64_t)d;
+#pragma unroll
+      for (int e = 0; e < kEH; ++e) {
+        const int j = l * kEH + e;
+        if (valid && j < half) {
+          const float y1 = (x1[e] * r) * wv1[e], y2 = (x2[e] * r) * wv2[e];
+          Elem<T>::store1(op + j, y1 * c[e] - y2 * s[e]);
+          Elem<T>::store1(op + half + j, y1 * s[e] + y2 * c[e]);
+        }
+      }
+    } else {
+      const float r = valid ? rstd[row] : 0.f;
+      const T* gp = dout + row * (int64_t)d;
+      float g1[kEH], g2[kEH];
+      float dot = 0.f;
+#pragma unroll
+      for (int e = 0; e < kEH; ++e) {
+        const int j = l * kEH + e;
+        const bool on = valid && j < half;
+        const float o1 = on ? Elem<T>::load1(gp + j) : 0.f;
+        const float o2 = on ? Elem<T>::load1(gp + half + j) : 0.f;
+        const float dy1 = o1 * c[e] + o2 * s[e], dy2 = o2 * c[e] - o1 * s[e];
+        x1[e] *= r; x2[e] *= r;                       // xhat
+        a1[e] += dy1 * x1[e]; a2[e] += dy2 * x2[e];
+        g1[e] = dy1 * wv1[e]; g2[e] = dy2 * wv2[e];
+        dot += g1[e] * x1[e] + g2[e] * x2[e];
+      }
+      dot = group_reduce<G, OpSum>(dot);
+      const float cm = dot / (float)d;
+      T* op = out + row * (int64_t)d;
+#pragma unroll
+      for (int e = 0; e < kEH; ++e) {
+        const int j = l * kEH + e;
+        if (valid && j < half) {
+          Elem<T>::store1(op + j, (g1[e] - x1[e] * cm) * r);
+          Elem<T>::store1(op + half + j, (g2[e] - x2[e] * cm) * r);
+        }
+      }
+    }
+  }
+  if constexpr (BWD) {
+    if (partial == nullptr) return;
+    // fold the rows of this workgroup in row order, then write one partial row
+#pragma unroll
+    for (int e = 0; e < kEH; ++e) {
+      fold[(rib * 2 + 0) * G * kEH + l * kEH + e] = a1[e];
+      fold[(rib * 2 + 1) * G * kEH + l * kEH + e] = a2[e];
+    }
+    __syncthreads();
+    float* prow = partial + (int64_t)blockIdx.x * d;
+    for (int j = tid; j < d; j += kBlock) {
+      const int hsel = j >= half ? 1 : 0, jj = j - hsel * half;
+      float acc = 0.f;
+      for (int rr = 0; rr < RPB; ++rr) acc += fold[(rr * 2 + hsel) * G * kEH + jj];
+      prow[j] = acc;
+    }
+  }
+}
+
+template <typename WT>
+__global__ __launch_bounds__(256) void rope_colsum_kernel(const float* __restrict__ partial,
+                                                           WT* __restrict__ dw, int p, int d) {
+  const int col = blockIdx.x * 256 + threadIdx.x;
+  if (col >= d) return;
+  float a = 0.f;
+  for (int r = 0; r < p; ++r) a += partial[(int64_t)r * d + col];
+  Elem<WT>::store1(dw + col, a);
+}
+
+struct Shape { int g; int64_t tiles; int blocks; };
+
+bool make_shape(int64_t rows, int64_t d, Shape* s) {
+  if (d < 2 || d % 2 != 0) return false;
+  const int64_t half = d / 2;
+  int g = 1;
+  while ((int64_t)g * kEH < half) g *= 2;
+  if (g > 64) return false;
+  s->g = g;
+  const int rpb = kBlock / g;
+  s->tiles = (rows + rpb - 1) / rpb;
+  int64_t blocks = (int64_t)fm_host::num_cus() * 4;
+  if (blocks > s->tiles) blocks = s->tiles;
+  s->blocks = (int)(blocks < 1 ? 1 : blocks);
+  return true;
+}
+
+template <typename T, typename WT, bool BWD>
+int launch(const Shape& sh, const void* x, const void* w, const float* c, const float* s, const void* dout,
+           float* rstd, void* out, float* partial, int64_t rows, int t_len, int heads, int d, float eps,
+           hipStream_t st) {
+  const int64_t blocks = BWD ? sh.blocks : sh.tiles;
+#define GO(G)                                                                                         \
+  hipLaunchKernelGGL((rope_kernel<T, WT, G, BWD>), dim3((unsigned)blocks), dim3(kBlock), 0, st,       \
+                     static_cast<const T*>(x), static_cast<const WT*>(w), c, s,                       \
+                     static_cast<const T*>(dout), rstd, static_cast<T*>(out), partial, rows, t_len,   \
+                     heads, d, eps, sh.tiles)
+  switch (sh.g) {
+    case 1: GO(1); break;
+    case 2: GO(2); break;
+    case 4: GO(4); break;
+    case 8: GO(8); break;
+    case 16: GO(16); break;
+    case 32: GO(32); break;
+    default: GO(64); break;
+  }
+#undef GO
+  return FM_OK;
+}
+
+int check(const char* what, int64_t b, int64_t t, int64_t h, int64_t d, int x_dtype, int w_dtype, Shape* sh) {
+  FM_CHECK_ARG(b >= 0 && t > 0 && h > 0 && d > 0, "%s: bad shape", what);
+  FM_CHECK_ARG(x_dtype == FM_F32 || x_dtype == FM_F16 || x_dtype == FM_BF16, "%s: bad x_dtype %d", what, x_dtype);
+  FM_CHECK_ARG(w_dtype == x_dtype || w_dtype == FM_F32, "%s: w_dtype must equal x_dtype or be fp32", what);
+  if (b * t * h > 0x7fffffffLL || !make_shape(b * t * h, d, sh)) {
+    fm_host::set_error("%s: head dim must be even and <= 512, rows < 2^31 (d=%lld)", what, (long long)d);
+    return FM_ERR_UNSUPPORTED;
+  }
+  return FM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t fm_qk_norm_rope_bwd_workspace(int64_t b, int64_t t, int64_t h, int64_t d) {
+  Shape sh;
+  if (b <= 0 || t <= 0 || h <= 0 || !make_shape(b * t * h, d, &sh)) return 0;
+  return (size_t)sh.blocks * (size_t)d * sizeof(float);
+}
+
+int fm_qk_norm_rope_fwd(const void* x, const void* w, const float* cosv, const float* sinv, void* out,
+                        float* rstd, int64_t b, int64_t t, int64_t h, int64_t d, int x_dtype, int w_dtype,
+                        float eps, fm_stream_t stream) {
+  Shape sh;
+  int rc = check("fm_qk_norm_rope_fwd", b, t, h, d, x_dtype, w_dtype, &sh);
+  if (rc != FM_OK) return rc;
+  if (b == 0) return FM_OK;
+  FM_CHECK_ARG(x && w && cosv && sinv && out && rstd, "fm_qk_norm_rope_fwd: NULL pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t rows = b * t * h;
+#define CALL(T, WT) launch<T, WT, false>(sh, x, w, cosv, sinv, nullptr, rstd, out, nullptr, rows, (int)t, (int)h, (int)d, eps, st)
+  if (x_dtype == FM_F32) CALL(float, float);
+  else if (x_dtype == FM_BF16 && w_dtype == FM_BF16) CALL(bf16_t, bf16_t);
+  else if (x_dtype == FM_BF16) CALL(bf16_t, float);
+  else if (w_dtype == FM_F16) CALL(f16_t, f16_t);
+  else CALL(f16_t, float);
+#undef CALL
+  FM_CHECK_LAUNCH("fm_qk_norm_rope_fwd");
+  return FM_OK;
+}
+
+int fm_qk_norm_rope_bwd(const void* x, const void* w, const float* cosv, const float* sinv,
+                        const float* rstd, const void* dout, void* dx, void* dw, void* workspace,
+                        size_t workspace_bytes, int64_t b, int64_t t, int64_t h, int64_t d, int x_dtype,
+                        int w_dtype, fm_stream_t stream) {
+  Shape sh;
+  int rc = check("fm_qk_norm_rope_bwd", b, t, h, d, x_dtype, w_dtype, &sh);
+  if (rc != FM_OK) return rc;
+  FM_CHECK_ARG(b > 0, "fm_qk_norm_rope_bwd: empty batch");
+  FM_CHECK_ARG(x && w && cosv && sinv && rstd && dout && dx, "fm_qk_norm_rope_bwd: NULL pointer");
+  float* partial = nullptr;
+  if (dw != nullptr) {
+    const size_t need = (size_t)sh.blocks * (size_t)d * sizeof(float);
+    if (workspace == nullptr || workspace_bytes < need) {
+      fm_host::set_error("fm_qk_norm_rope_bwd: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+      return FM_ERR_WORKSPACE;
+    }
+    partial = static_cast<float*>(workspace);
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t rows = b * t * h;
+#define CALL(T, WT)                                                                                    \
+  launch<T, WT, true>(sh, x, w, cosv, sinv, dout, const_cast<float*>(rstd), dx, partial, rows, (int)t,  \
+                      (int)h, (int)d, 0.f, st);                                                        \
+  if (partial != nullptr)                                                                              \
+    hipLaunchKernelGGL((rope_colsum_kernel<WT>), dim3((unsigned)((d + 255) / 256)), dim3(256), 0, st,   \
+                       partial, static_cast<WT*>(dw), sh.blocks, (int)d)
+  if (x_dtype == FM_F32) { CALL(float, float); }
+  else if (x_dtype == FM_BF16 && w_dtype == FM_BF16) { CALL(bf16_t, bf16_t); }
+  else if (x_dtype == FM_BF16) { CALL(bf16_t, float); }
+  else if (w_dtype == FM_F16) { CALL(f16_t, f16_t); }
+  else { CALL(f16_t, float); }
+#undef CALL
+  FM_CHECK_LAUNCH("fm_qk_norm_rope_bwd");
+  return FM_OK;
+}
+
+}  // extern "C"

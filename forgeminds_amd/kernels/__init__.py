@@ -26,9 +26,10 @@ from ._ops import use_custom_ops
 from .apply import enable, patch, revert
 from .ce import cross_entropy
 from .dispatch import moe_combine, moe_gather
-from .extras import newton_schulz, qk_norm_rope
+from .extras import newton_schulz
 from .kl import distill_kl, kl_distill_loss, kl_div, kl_div_logits
 from .norm import add_rms_norm, rms_norm
+from .rope import qk_norm_rope
 from .route import Routing, moe_route
 from .softmax import softmax
 from .swiglu import swiglu, swiglu_split

@@ -53,6 +53,10 @@ SIGNATURES = {
     "fm_swiglu_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _vp]),
     "fm_swiglu_split_fwd": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "fm_swiglu_split_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _vp]),
+    "fm_qk_norm_rope_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _int, _int, _f32, _vp]),
+    "fm_qk_norm_rope_bwd_workspace": (_sz, [_i64, _i64, _i64, _i64]),
+    "fm_qk_norm_rope_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64, _i64, _i64,
+                                   _int, _int, _vp]),
     "fm_route": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _int, _int, _int, _vp]),
 }
 
@@ -379,3 +383,32 @@ def swiglu_split_bwd(x2, dy2):
         _check(lib().fm_swiglu_split_bwd(_ptr(x2), _ptr(dy2), _ptr(dx), rows, w // 2,
                                          dtype_code(x2.dtype), _stream(x2)), "fm_swiglu_split_bwd")
     return dx
+
+
+# ------------------------------------------------------------------ per-head RMSNorm + RoPE
+def qk_norm_rope_fwd(x4, w, cos, sin, eps: float):
+    """x4 [b, t, h, d], cos/sin fp32 [t, d/2] -> (out like x4, rstd fp32 [b*t*h])."""
+    _dense(x4, w, cos, sin)
+    b, t, h, d = x4.shape
+    out = torch.empty_like(x4)
+    rstd = torch.empty(b * t * h, device=x4.device, dtype=torch.float32)
+    with torch.cuda.device(x4.device):
+        _check(lib().fm_qk_norm_rope_fwd(_ptr(x4), _ptr(w), _ptr(cos), _ptr(sin), _ptr(out), _ptr(rstd),
+                                         b, t, h, d, dtype_code(x4.dtype), dtype_code(w.dtype), float(eps),
+                                         _stream(x4)), "fm_qk_norm_rope_fwd")
+    return out, rstd
+
+
+def qk_norm_rope_bwd(x4, w, cos, sin, rstd, dout, want_dw: bool = True):
+    _dense(x4, w, cos, sin, rstd, dout)
+    b, t, h, d = x4.shape
+    dx = torch.empty_like(x4)
+    dw = torch.empty_like(w) if want_dw else None
+    with torch.cuda.device(x4.device):
+        nbytes = int(lib().fm_qk_norm_rope_bwd_workspace(b, t, h, d)) if want_dw else 0
+        ws = torch.empty(max(nbytes, 16), device=x4.device, dtype=torch.uint8) if want_dw else None
+        _check(lib().fm_qk_norm_rope_bwd(_ptr(x4), _ptr(w), _ptr(cos), _ptr(sin), _ptr(rstd), _ptr(dout),
+                                         _ptr(dx), _ptr(dw), _ptr(ws), nbytes, b, t, h, d,
+                                         dtype_code(x4.dtype), dtype_code(w.dtype), _stream(x4)),
+               "fm_qk_norm_rope_bwd")
+    return dx, dw

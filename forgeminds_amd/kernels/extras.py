@@ -1,21 +1,13 @@
 """Surface names of the reference's kernel package that are outside the packed hot path.
 
-``qk_norm_rope`` and ``newton_schulz`` (reference ``forgemind/kernels/{rope,ns}.py``) keep
-their torch expression here so code written against ``fm.kernels`` imports and runs unchanged.
+``newton_schulz`` (reference ``forgemind/kernels/ns.py``) is GEMM-bound optimizer plumbing; it
+keeps its torch expression here so code written against ``fm.kernels`` imports and runs unchanged.
 """
 
 from __future__ import annotations
 
 import torch
 
-from . import _fallback as fb
-
-
-def qk_norm_rope(x, w, cos, sin, eps: float = 1e-6):
-    """Per-head RMSNorm + half-split RoPE for ``x [B, T, H, D]``, ``cos``/``sin`` ``[T, D/2]``
-    (reference ``rope.py:227-244``)."""
-    t, half = cos.shape[-2], cos.shape[-1]
-    return fb.qk_norm_rope(x, w, cos.reshape(1, t, 1, half), sin.reshape(1, t, 1, half), eps)
 
 
 def newton_schulz(g: torch.Tensor, steps: int = 5, eps: float = 1e-7) -> torch.Tensor:
@@ -34,4 +26,4 @@ def newton_schulz(g: torch.Tensor, steps: int = 5, eps: float = 1e-7) -> torch.T
     return x.to(g.dtype)
 
 
-__all__ = ["qk_norm_rope", "newton_schulz"]
+__all__ = ["newton_schulz"]

@@ -206,6 +206,20 @@ int fm_swiglu_split_fwd(const void* x, void* y, int64_t rows, int64_t h, int dty
 int fm_swiglu_split_bwd(const void* x, const void* dy, void* dx, int64_t rows, int64_t h, int dtype,
                         fm_stream_t stream);
 
+/* ------------------------------------------------------------------ per-head RMSNorm + RoPE
+ * Replace _qknorm_rope_fwd / _qknorm_rope_bwd (forgemind/kernels/rope.py:46-120); semantics of
+ * _fallback.qk_norm_rope (_fallback.py:38-45). x, out, dout, dx: [b, t, h, d] of x_dtype (d even,
+ * <= 512); w: [d] of w_dtype; cos, sin: fp32 [t, d/2]; rstd: fp32 [b*t*h]. dw ([d], w_dtype)
+ * may be NULL; otherwise workspace of fm_qk_norm_rope_bwd_workspace bytes is needed. */
+int fm_qk_norm_rope_fwd(const void* x, const void* w, const float* cosv, const float* sinv, void* out,
+                        float* rstd, int64_t b, int64_t t, int64_t h, int64_t d, int x_dtype, int w_dtype,
+                        float eps, fm_stream_t stream);
+size_t fm_qk_norm_rope_bwd_workspace(int64_t b, int64_t t, int64_t h, int64_t d);
+int fm_qk_norm_rope_bwd(const void* x, const void* w, const float* cosv, const float* sinv,
+                        const float* rstd, const void* dout, void* dx, void* dw, void* workspace,
+                        size_t workspace_bytes, int64_t b, int64_t t, int64_t h, int64_t d, int x_dtype,
+                        int w_dtype, fm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -366,3 +366,26 @@ def test_moe_layer_matches_the_reference_expression():
     assert torch.allclose(out, ref, rtol=1e-4, atol=1e-5)
     assert torch.allclose(gx, xr.grad, rtol=1e-3, atol=1e-5)
     assert torch.allclose(gate_g, layer.router.gate.weight.grad, rtol=1e-3, atol=1e-5)
+
+
+def test_qk_norm_rope_surface_and_op_path():
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(2, 9, 4, 64, generator=g).to(DEV)
+    w = torch.randn(64, generator=g).to(DEV)
+    cos, sin = torch.randn(9, 32, generator=g).to(DEV), torch.randn(9, 32, generator=g).to(DEV)
+
+    def run(mode):
+        _ops.use_custom_ops(mode)
+        xi, wi = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+        out = kernels.qk_norm_rope(xi, wi, cos, sin, 1e-6)
+        out.square().sum().backward()
+        return out.detach(), xi.grad, wi.grad
+
+    eager, op = run(False), run(True)
+    assert all(torch.equal(a, b) for a, b in zip(eager, op))
+    kernels.set_backend("fallback")
+    ref = run(False)
+    kernels.set_backend("auto")
+    assert all(torch.allclose(a, b, rtol=1e-4, atol=1e-4) for a, b in zip(eager, ref))
+    with pytest.raises(ValueError):
+        kernels.qk_norm_rope(x[0], w, cos, sin)

@@ -416,6 +416,7 @@ def test_swiglu_fwd_bwd(shape, dt):
     a, b, dy = (torch.randn(*shape, generator=g).to(dt) for _ in range(3))
     ar, br = a.float().requires_grad_(True), b.float().requires_grad_(True)
     ref = torch.nn.functional.silu(ar) * br
+    b = b.detach()
     ref.backward(dy.float())
     y = _hip.swiglu_fwd(a.to(DEV), b.to(DEV))
     da, db = _hip.swiglu_bwd(a.to(DEV), b.to(DEV), dy.to(DEV))
@@ -437,3 +438,29 @@ def test_swiglu_split_fwd_bwd(rows, h, dt):
     dx = _hip.swiglu_split_bwd(x.to(DEV), dy.to(DEV))
     assert_close_lowp(y, ref.detach(), dt, "swiglu_split", ulps=2.0)
     assert_close_lowp(dx, xr.grad, dt, "dx", ulps=3.0, cancel=float(dy.float().abs().max() * x.float().abs().max()))
+
+
+# ------------------------------------------------------------------ per-head RMSNorm + RoPE
+@pytest.mark.parametrize("b,t,h,hd,dt,wdt", [(2, 5, 3, 4, F32, F32), (1, 7, 2, 8, F32, F32), (2, 3, 4, 6, F32, F32),
+                                              (2, 64, 8, 64, BF16, F32), (1, 33, 4, 32, F16, F16), (2, 16, 2, 256, BF16, BF16)])
+def test_qk_norm_rope_fwd_bwd(b, t, h, hd, dt, wdt):
+    # shapes of reference tests/kernel_interp_check.py:82-89, then realistic head sizes
+    g = gen(41)
+    d = 2 * hd
+    x = torch.randn(b, t, h, d, generator=g).to(dt)
+    w = (1 + 0.1 * torch.randn(d, generator=g)).to(wdt)
+    cos, sin = torch.randn(t, hd, generator=g), torch.randn(t, hd, generator=g)
+    do = torch.randn(b, t, h, d, generator=g).to(dt)
+    xr, wr = x.float().requires_grad_(True), w.float().requires_grad_(True)
+    r = torch.rsqrt(xr.pow(2).mean(-1, keepdim=True) + 1e-6)
+    y = xr * r * wr
+    y1, y2 = y.chunk(2, -1)
+    c, s = cos.view(1, t, 1, hd), sin.view(1, t, 1, hd)
+    ref = torch.cat((y1 * c - y2 * s, y1 * s + y2 * c), -1)
+    ref.backward(do.float())
+    out, rstd = _hip.qk_norm_rope_fwd(x.to(DEV), w.to(DEV), cos.to(DEV), sin.to(DEV), 1e-6)
+    dx, dw = _hip.qk_norm_rope_bwd(x.to(DEV), w.to(DEV), cos.to(DEV), sin.to(DEV), rstd, do.to(DEV))
+    scale = float(ref.detach().abs().max())
+    assert_close_lowp(out, ref.detach(), dt, "qk_norm_rope", ulps=3.0, cancel=scale)
+    assert_close_lowp(dx, xr.grad, dt, "dx", ulps=4.0, cancel=float(xr.grad.abs().max()) * 4)
+    assert rel_max(dw, wr.grad) <= (1e-2 if wdt != F32 else 1e-4)

@@ -70,7 +70,7 @@ def test_stats_are_not_touched_while_tracing():
 def test_ops_are_registered_and_dispatch_flag_works():
     # reference tests/test_kernel_ops.py:112-117, 168-175
     names = {n for n in dir(torch.ops.forgemind) if not n.startswith("_")}
-    for op in ("rms_norm", "add_rms_norm", "swiglu", "swiglu_split"):
+    for op in ("rms_norm", "add_rms_norm", "swiglu", "swiglu_split", "qk_norm_rope"):
         assert op in names and f"{op}_backward" in names
     assert _ops.wanted() is False
     assert _ops.use_custom_ops(True) is True and _ops.wanted() is True
