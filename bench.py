@@ -49,7 +49,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="ce",
-                    choices=["ce", "rmsnorm", "add_rmsnorm", "kl", "topk", "route", "moe_dispatch"])
+                    choices=["ce", "rmsnorm", "add_rmsnorm", "kl", "kl_topk", "topk", "route", "moe_dispatch"])
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
@@ -199,7 +199,7 @@ def make_workload(name, torch, L, dev):
         w.tensors = (lg, y)
         return w
 
-    if name in ("kl", "topk"):
+    if name in ("kl", "kl_topk", "topk"):
         n, v = 4096, 128256
         g.manual_seed(1005)
         s = (3 * torch.randn(n, v, device=dev, generator=g)).bfloat16()
@@ -230,6 +230,15 @@ def make_workload(name, torch, L, dev):
             _check(L.fm_kl_bwd(s.data_ptr(), t.data_ptr(), b3[0].data_ptr(), b3[1].data_ptr(), None, 0,
                                gs.data_ptr(), n, v, BF, BF, 0.5, 1.0 / n, st), "fm_kl_bwd")
 
+        if name == "kl_topk":
+            idx = torch.empty(n, 64, device=dev, dtype=torch.int32)
+            pr = torch.empty(n, 64, device=dev)
+
+            def fwd():  # noqa: F811 -- the fused forward replaces the plain one
+                _check(L.fm_kl_fwd_topk(s.data_ptr(), t.data_ptr(), b3[0].data_ptr(), b3[1].data_ptr(),
+                                        b3[2].data_ptr(), ls.data_ptr(), None, idx.data_ptr(),
+                                        pr.data_ptr(), n, v, 64, BF, 32, 0.5, 2, st), "fm_kl_fwd_topk")
+
         def step():
             fwd()
             bwd()
@@ -240,6 +249,8 @@ def make_workload(name, torch, L, dev):
         w.dominant_bytes = n * v * 6
         w.bytes = n * v * 10
         w.desc = f"KL(teacher||student) fwd+bwd bf16 [{n},{v}], T=2, mean"
+        if name == "kl_topk":
+            w.desc += "; the forward also returns the teacher's top-64 (int32 indices, fp32 probabilities)"
         w.rows = n
         return w
 
@@ -484,7 +495,7 @@ def main():
     torch.cuda.empty_cache()
     if not a.no_extras:
         extras = {a.workload: res}
-        for name in ["rmsnorm", "add_rmsnorm", "ce", "kl", "topk", "route", "moe_dispatch"]:
+        for name in ["rmsnorm", "add_rmsnorm", "ce", "kl", "kl_topk", "topk", "route", "moe_dispatch"]:
             if name == a.workload:
                 continue
             wl = make_workload(name, torch, L, dev)

@@ -9,15 +9,110 @@
 // a thread carries (m_s, d_s, m_t, d_t, A) and rescales d_t and A whenever its teacher
 // maximum moves. The backward recomputes both softmaxes from the saved lse values.
 // All exponentials run in the base-2 domain; the temperature is folded into the scale.
-#include "fm_vocab.cuh"
+#include "fm_topk.cuh"
 
 using namespace fm;
 
 namespace {
 
+// widest row (in 16-byte vectors) the fused KL + top-k kernel keeps key prefixes for
+constexpr int kFusedMaxVec = 20480;
+
 struct KLState {
   float ms, ds, mt, dt, a;
 };
+
+// Folds UNROLL vectors of student / teacher logits (vector u is column c_first + u * stride,
+// live when that is below nvec) into the running state.
+template <typename T, int UNROLL>
+__device__ __forceinline__ void kl_update(KLState& k, const u32x4 (&rs)[UNROLL],
+                                          const u32x4 (&rt)[UNROLL], int c_first, int stride,
+                                          int nvec, float c1) {
+  constexpr int EPV = Elem<T>::kVec;
+  float zs[UNROLL][EPV], zt[UNROLL][EPV];
+  float cms = k.ms, cmt = k.mt;
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const int c = c_first + u * stride;
+    if (c < nvec) {
+      Elem<T>::unpack(rs[u], zs[u]);
+      Elem<T>::unpack(rt[u], zt[u]);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        zs[u][e] *= c1;
+        zt[u][e] *= c1;
+        cms = fmaxf(cms, zs[u][e]);
+        cmt = fmaxf(cmt, zt[u][e]);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) { zs[u][e] = -INFINITY; zt[u][e] = -INFINITY; }
+    }
+  }
+  float ds = k.ds * fast_exp2(k.ms - cms);
+  const float ft = fast_exp2(k.mt - cmt);
+  float dt = k.dt * ft;
+  float a = k.a * ft;
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const int c = c_first + u * stride;
+    if (c < nvec) {   // uniform per vector; keeps (-inf) - (-inf) out of the A term
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        ds += fast_exp2(zs[u][e] - cms);
+        const float et = fast_exp2(zt[u][e] - cmt);
+        dt += et;
+        a += et * (zt[u][e] - zs[u][e]);
+      }
+    }
+  }
+  k.ms = cms; k.ds = ds; k.mt = cmt; k.dt = dt; k.a = a;
+}
+
+// One scalar column.
+__device__ __forceinline__ void kl_update1(KLState& k, float zs, float zt) {
+  const float cms = fmaxf(k.ms, zs), cmt = fmaxf(k.mt, zt);
+  k.ds = k.ds * fast_exp2(k.ms - cms) + fast_exp2(zs - cms);
+  const float ft = fast_exp2(k.mt - cmt);
+  const float et = fast_exp2(zt - cmt);
+  k.dt = k.dt * ft + et;
+  k.a = k.a * ft + et * (zt - zs);
+  k.ms = cms; k.mt = cmt;
+}
+
+// Workgroup merge: maxima first (exact), then rescaled sums in lane / wave order. Every thread
+// returns the row's base-2 log-sum-exps and KL (in bits); smem holds 5 * NW floats.
+template <int NW>
+__device__ __forceinline__ void kl_merge(const KLState& k, float* smem, float* l2s, float* l2t,
+                                         float* kl2) {
+  const int tid = threadIdx.x;
+  const float wms = wave_max(k.ms), wmt = wave_max(k.mt);
+  const float fs = fast_exp2(k.ms - wms), ft = fast_exp2(k.mt - wmt);
+  float wds = wave_sum(k.ds * fs), wdt = wave_sum(k.dt * ft), wa = wave_sum(k.a * ft);
+  float Ms = wms, Mt = wmt, Ds = wds, Dt = wdt, A = wa;
+  if constexpr (NW > 1) {
+    const int lane = tid & 63, wave = tid >> 6;
+    if (lane == 0) {
+      smem[wave] = wms; smem[NW + wave] = wmt; smem[2 * NW + wave] = wds;
+      smem[3 * NW + wave] = wdt; smem[4 * NW + wave] = wa;
+    }
+    __syncthreads();
+    Ms = smem[0]; Mt = smem[NW];
+#pragma unroll
+    for (int i = 1; i < NW; ++i) { Ms = fmaxf(Ms, smem[i]); Mt = fmaxf(Mt, smem[NW + i]); }
+    Ds = 0.f; Dt = 0.f; A = 0.f;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      const float gs = fast_exp2(smem[i] - Ms), gt = fast_exp2(smem[NW + i] - Mt);
+      Ds += smem[2 * NW + i] * gs;
+      Dt += smem[3 * NW + i] * gt;
+      A += smem[4 * NW + i] * gt;
+    }
+  }
+  *l2s = Ms + fast_log2(Ds);
+  *l2t = Mt + fast_log2(Dt);
+  *kl2 = A / Dt - *l2t + *l2s;
+}
 
 template <typename T, int THREADS, int UNROLL>
 __global__ __launch_bounds__(THREADS) void kl_fwd_kernel(const T* __restrict__ student,
@@ -47,89 +142,94 @@ __global__ __launch_bounds__(THREADS) void kl_fwd_kernel(const T* __restrict__ s
         rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
       }
     }
-    float zs[UNROLL][EPV], zt[UNROLL][EPV];
-    float cms = k.ms, cmt = k.mt;
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) {
-        Elem<T>::unpack(rs[u], zs[u]);
-        Elem<T>::unpack(rt[u], zt[u]);
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) {
-          zs[u][e] *= c1;
-          zt[u][e] *= c1;
-          cms = fmaxf(cms, zs[u][e]);
-          cmt = fmaxf(cmt, zt[u][e]);
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) { zs[u][e] = -INFINITY; zt[u][e] = -INFINITY; }
-      }
-    }
-    float ds = k.ds * fast_exp2(k.ms - cms);
-    const float ft = fast_exp2(k.mt - cmt);
-    float dt = k.dt * ft;
-    float a = k.a * ft;
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) {   // uniform per vector; keeps (-inf) - (-inf) out of the A term
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) {
-          ds += fast_exp2(zs[u][e] - cms);
-          const float et = fast_exp2(zt[u][e] - cmt);
-          dt += et;
-          a += et * (zt[u][e] - zs[u][e]);
-        }
-      }
-    }
-    k.ms = cms; k.ds = ds; k.mt = cmt; k.dt = dt; k.a = a;
+    kl_update<T, UNROLL>(k, rs, rt, c0 + tid, THREADS, sp.nvec, c1);
   }
   const int ne = edge_count(sp, v);
   for (int e = tid; e < ne; e += THREADS) {
     const int col = edge_col(sp, e);
-    const float zs = Elem<T>::load1(sp_ + col) * c1;
-    const float zt = Elem<T>::load1(tp_ + col) * c1;
-    const float cms = fmaxf(k.ms, zs), cmt = fmaxf(k.mt, zt);
-    k.ds = k.ds * fast_exp2(k.ms - cms) + fast_exp2(zs - cms);
-    const float ft = fast_exp2(k.mt - cmt);
-    const float et = fast_exp2(zt - cmt);
-    k.dt = k.dt * ft + et;
-    k.a = k.a * ft + et * (zt - zs);
-    k.ms = cms; k.mt = cmt;
+    kl_update1(k, Elem<T>::load1(sp_ + col) * c1, Elem<T>::load1(tp_ + col) * c1);
   }
 
-  // workgroup merge: maxima first (exact), then rescaled sums in lane / wave order
-  const float wms = wave_max(k.ms), wmt = wave_max(k.mt);
-  const float fs = fast_exp2(k.ms - wms), ft = fast_exp2(k.mt - wmt);
-  float wds = wave_sum(k.ds * fs), wdt = wave_sum(k.dt * ft), wa = wave_sum(k.a * ft);
-  float Ms = wms, Mt = wmt, Ds = wds, Dt = wdt, A = wa;
-  if constexpr (NW > 1) {
-    const int lane = tid & 63, wave = tid >> 6;
-    if (lane == 0) {
-      smem[wave] = wms; smem[NW + wave] = wmt; smem[2 * NW + wave] = wds;
-      smem[3 * NW + wave] = wdt; smem[4 * NW + wave] = wa;
-    }
-    __syncthreads();
-    Ms = smem[0]; Mt = smem[NW];
-#pragma unroll
-    for (int i = 1; i < NW; ++i) { Ms = fmaxf(Ms, smem[i]); Mt = fmaxf(Mt, smem[NW + i]); }
-    Ds = 0.f; Dt = 0.f; A = 0.f;
-#pragma unroll
-    for (int i = 0; i < NW; ++i) {
-      const float gs = fast_exp2(smem[i] - Ms), gt = fast_exp2(smem[NW + i] - Mt);
-      Ds += smem[2 * NW + i] * gs;
-      Dt += smem[3 * NW + i] * gt;
-      A += smem[4 * NW + i] * gt;
-    }
-  }
+  float l2s, l2t, kl2;
+  kl_merge<NW>(k, smem, &l2s, &l2t, &kl2);
   if (tid == 0) {
-    const float l2s = Ms + fast_log2(Ds), l2t = Mt + fast_log2(Dt);
     lse_s[row] = l2s * kLn2;
     lse_t[row] = l2t * kLn2;
-    row_kl[row] = (A / Dt - l2t + l2s) * kLn2;
+    row_kl[row] = kl2 * kLn2;
   }
+}
+
+// The same forward, also returning the exact top-k of the teacher row (raw logits; softmax and
+// the temperature are monotone, so the order is that of the probabilities). The streaming pass
+// leaves a 16-bit key prefix of every teacher vector's maximum in LDS (2 bytes per 16 bytes of
+// row), so the selection revisits only the few vectors that can hold a winner.
+template <typename T, int THREADS, int UNROLL>
+__global__ __launch_bounds__(THREADS) void kl_fwd_topk_kernel(
+    const T* __restrict__ student, const T* __restrict__ teacher, float* __restrict__ lse_s,
+    float* __restrict__ lse_t, float* __restrict__ row_kl, T* __restrict__ tk_values,
+    int32_t* __restrict__ tk_idx32, int64_t* __restrict__ tk_idx64, float* __restrict__ tk_probs,
+    int v, int k, float inv_temp, bool vec_ok) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int NW = THREADS / 64;
+  __shared__ float smem[5 * NW];
+  __shared__ TopkShared<THREADS, kVecMaxLds> sh;
+  extern __shared__ __align__(16) uint16_t vhi[];
+  const int64_t row = blockIdx.x;
+  const T* sp_ = student + row * (int64_t)v;
+  const T* tp_ = teacher + row * (int64_t)v;
+  const RowSplit sp = split_row<EPV>(row, v, vec_ok);
+  const int tid = threadIdx.x;
+  const float c1 = kLog2e * inv_temp;
+
+  KLState st{kNegBig, 0.f, kNegBig, 0.f, 0.f};
+  float fm = -INFINITY;
+  bool has_nan = false;
+  {  // zero the padding of the last quad of prefixes
+    const int p = ((sp.nvec + 3) & ~3) - 1 - tid;
+    if (tid < 3 && p >= sp.nvec) vhi[p] = 0;
+  }
+  __syncthreads();
+  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+    u32x4 rs[UNROLL], rt[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) {
+        rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
+        rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
+      }
+    }
+    kl_update<T, UNROLL>(st, rs, rt, c0 + tid, THREADS, sp.nvec, c1);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) {
+        const float m = fold_vector_max<T>(rt[u]);
+        const bool bad = m != m;
+        vhi[c] = (uint16_t)(bad ? 0xFFFFu : key_prefix(key_of(m)));
+        fm = fmaxf(fm, m);
+        has_nan |= bad;
+      }
+    }
+  }
+  const int ne = edge_count(sp, v);
+  for (int e = tid; e < ne; e += THREADS) {
+    const int col = edge_col(sp, e);
+    const float t = Elem<T>::load1(tp_ + col);
+    kl_update1(st, Elem<T>::load1(sp_ + col) * c1, t * c1);
+    fm = fmaxf(fm, t);
+    has_nan |= (t != t);
+  }
+  float l2s, l2t, kl2;
+  kl_merge<NW>(st, smem, &l2s, &l2t, &kl2);
+  if (tid == 0) {
+    lse_s[row] = l2s * kLn2;
+    lse_t[row] = l2t * kLn2;
+    row_kl[row] = kl2 * kLn2;
+  }
+  const float none[1] = {0.f};
+  topk_finish<T, THREADS, 1, kVecMaxLds>(tp_, sp, v, k, none, vhi, fm, has_nan, sh, row, tk_values,
+                                         tk_idx32, tk_idx64, tk_probs, c1, l2t);
 }
 
 // loss = sum(row_kl) * scale in a fixed order (thread i adds rows i, i+1024, ...).
@@ -278,6 +378,62 @@ int fm_kl_fwd(const void* student, const void* teacher, float* lse_s, float* lse
     const float scale = (reduction == FM_REDUCE_MEAN && n > 0) ? 1.f / (float)n : 1.f;
     hipLaunchKernelGGL(kl_finalize_kernel, dim3(1), dim3(1024), 0, st, row_kl, n, scale, loss);
     FM_CHECK_LAUNCH("fm_kl_fwd(finalize)");
+  }
+  return FM_OK;
+}
+
+int fm_kl_fwd_topk(const void* student, const void* teacher, float* lse_s, float* lse_t,
+                   float* row_kl, float* loss, void* topk_values, void* topk_indices,
+                   float* topk_probs, int64_t n, int64_t v, int k, int dtype, int index_bits,
+                   float inv_temperature, int reduction, fm_stream_t stream) {
+  int rc = check_shape("fm_kl_fwd_topk", n, v, dtype);
+  if (rc != FM_OK) return rc;
+  FM_CHECK_ARG(reduction == FM_REDUCE_NONE || reduction == FM_REDUCE_SUM || reduction == FM_REDUCE_MEAN,
+               "fm_kl_fwd_topk: bad reduction %d", reduction);
+  FM_CHECK_ARG(index_bits == 32 || index_bits == 64, "fm_kl_fwd_topk: index_bits must be 32 or 64");
+  FM_CHECK_ARG(k >= 1 && k <= v, "fm_kl_fwd_topk: selected index k out of range (k=%d, v=%lld)", k,
+               (long long)v);
+  FM_CHECK_ARG(inv_temperature > 0.f, "fm_kl_fwd_topk: the temperature must be positive");
+  const int esize = dtype == FM_F32 ? 4 : 2;
+  const int64_t nvec_max = v / (16 / esize);
+  if (k > kMaxK || nvec_max > kFusedMaxVec) {
+    fm_host::set_error("fm_kl_fwd_topk: k <= %d and rows of at most %d bytes are fused (k=%d, v=%lld); "
+                       "call fm_kl_fwd and fm_topk instead", kMaxK, kFusedMaxVec * 16, k, (long long)v);
+    return FM_ERR_UNSUPPORTED;
+  }
+  FM_CHECK_ARG(n == 0 || (student && teacher && lse_s && lse_t && row_kl && topk_indices),
+               "fm_kl_fwd_topk: NULL pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (n > 0) {
+    const bool vec_ok = fm_host::aligned16(student) && fm_host::aligned16(teacher);
+    int32_t* i32 = index_bits == 32 ? static_cast<int32_t*>(topk_indices) : nullptr;
+    int64_t* i64 = index_bits == 64 ? static_cast<int64_t*>(topk_indices) : nullptr;
+    int threads = fm_host::get_param(fm_host::P_VOCAB_THREADS);
+    if (threads != 256 && threads != 1024) threads = 512;
+    const size_t lds = (size_t)((nvec_max + 3) / 4 * 4 + 4) * sizeof(uint16_t);
+    const dim3 grid((unsigned)n);
+#define LAUNCH(T, TH)                                                                              \
+  hipLaunchKernelGGL((kl_fwd_topk_kernel<T, TH, 2>), grid, dim3(TH), lds, st,                      \
+                     static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t, \
+                     row_kl, static_cast<T*>(topk_values), i32, i64, topk_probs, (int)v, k,        \
+                     inv_temperature, vec_ok)
+#define BY_THREADS(T)                      \
+  do {                                     \
+    if (threads == 256) LAUNCH(T, 256);    \
+    else if (threads == 512) LAUNCH(T, 512); \
+    else LAUNCH(T, 1024);                  \
+  } while (0)
+    if (dtype == FM_F32) BY_THREADS(float);
+    else if (dtype == FM_BF16) BY_THREADS(bf16_t);
+    else BY_THREADS(f16_t);
+#undef BY_THREADS
+#undef LAUNCH
+    FM_CHECK_LAUNCH("fm_kl_fwd_topk");
+  }
+  if (reduction != FM_REDUCE_NONE && loss != nullptr) {
+    const float scale = (reduction == FM_REDUCE_MEAN && n > 0) ? 1.f / (float)n : 1.f;
+    hipLaunchKernelGGL(kl_finalize_kernel, dim3(1), dim3(1024), 0, st, row_kl, n, scale, loss);
+    FM_CHECK_LAUNCH("fm_kl_fwd_topk(finalize)");
   }
   return FM_OK;
 }

@@ -46,6 +46,43 @@ class _KLDivFn(torch.autograd.Function):
         return grad.view(shape), None, None, None, None
 
 
+class _KLDivTopkFn(torch.autograd.Function):
+    """KL forward that also hands back the teacher's top-k (indices and probabilities)."""
+
+    @staticmethod
+    def forward(ctx, student, teacher, k, reduction, grad_dtype, temperature, index_dtype):
+        v = student.shape[-1]
+        s2 = student.contiguous().view(-1, v)
+        t2 = teacher.contiguous().view(-1, v)
+        inv_t = 1.0 / float(temperature)
+        out = _hip.kl_fwd_topk(s2, t2, k, inv_t, reduction, index_dtype)
+        if out is None:   # row too wide for the fused kernel: two launches, same results
+            loss, rows, lse_s, lse_t = _hip.kl_fwd(s2, t2, inv_t, reduction)
+            vals, idx = _hip.topk(t2, k, index_dtype)
+            probs = torch.exp(vals.float() * inv_t - lse_t[:, None])
+        else:
+            loss, rows, lse_s, lse_t, _, idx, probs = out
+        ctx.save_for_backward(s2, t2, lse_s, lse_t)
+        ctx.meta = (student.shape, reduction, grad_dtype or student.dtype, inv_t)
+        lead = student.shape[:-1]
+        probs = probs.view(*lead, k)
+        idx = idx.view(*lead, k)
+        ctx.mark_non_differentiable(probs, idx)
+        if reduction == "none":
+            return rows.clone().view(lead), probs, idx
+        return loss, probs, idx
+
+    @staticmethod
+    def backward(ctx, g, _gp, _gi):
+        s2, t2, lse_s, lse_t = ctx.saved_tensors
+        shape, reduction, gdt, inv_t = ctx.meta
+        n = s2.shape[0]
+        g32 = g.detach().to(torch.float32).contiguous().view(-1)
+        scale = 1.0 / n if reduction == "mean" else 1.0
+        grad = _hip.kl_bwd(s2, t2, lse_s, lse_t, g32, reduction == "none", gdt, inv_t, scale)
+        return grad.view(shape), None, None, None, None, None, None
+
+
 def _kernel_ok(*tensors) -> bool:
     if any(t.numel() >= 2 ** 31 * 4 for t in tensors):
         _note("kl numel")
@@ -77,6 +114,41 @@ def kl_div_logits(student: torch.Tensor, teacher: torch.Tensor, reduction: str =
     return _KLDivFn.apply(student, teacher, reduction, grad_dtype, float(temperature))
 
 
+def kl_div_logits_topk(student: torch.Tensor, teacher: torch.Tensor, k: int,
+                       reduction: str = "mean", grad_dtype: "torch.dtype | None" = None,
+                       temperature: float = 1.0, index_dtype: torch.dtype = torch.int64):
+    """``kl_div_logits`` plus the teacher's exact top-``k`` from the same pass over the logits.
+
+    Returns ``(loss, probs, idx)``: ``idx [..., k]`` are the columns ``topk(teacher, k)`` would
+    return (value descending, lowest index first among equals; reference
+    ``forgemind/kernels/topk.py:13-19``) and ``probs [..., k]`` (fp32) are
+    ``softmax(teacher / T)`` at those columns. The reference reads the teacher twice for this
+    (``kernels/kl.py:194-207`` then ``kernels/topk.py:273-297``); the kernel reads it once.
+    """
+    if reduction not in _REDUCTIONS:
+        raise ValueError(f"reduction must be mean|sum|none, got {reduction!r}")
+    if temperature <= 0:
+        raise ValueError(f"temperature must be positive, got {temperature}")
+    if index_dtype not in (torch.int64, torch.int32):
+        raise ValueError("index_dtype must be torch.int64 or torch.int32")
+    if student.dim() < 1 or not 1 <= k <= max(student.shape[-1], 1):
+        raise RuntimeError("selected index k out of range")
+    ok = (student.shape == teacher.shape and student.shape[-1] > 0 and student.numel() > 0
+          and student.dtype == teacher.dtype and k <= 512
+          and grad_dtype in (None, student.dtype, torch.float32))
+    if not ok or not _kernel_ok(student, teacher):
+        if ok is False:
+            _note("kl operands")
+        loss = fb.kl_div_logits(student, teacher, reduction, temperature)
+        with torch.no_grad():
+            _, idx = fb.topk_canonical(teacher, k)
+            logp = torch.log_softmax(teacher.float() / temperature, dim=-1)
+            probs = torch.gather(logp, -1, idx).exp()
+        return loss, probs, idx.to(index_dtype)
+    return _KLDivTopkFn.apply(student, teacher, int(k), reduction, grad_dtype, float(temperature),
+                              index_dtype)
+
+
 def kl_distill_loss(hs: torch.Tensor, ht: torch.Tensor, w: torch.Tensor, teacher_head,
                     chunk: int = 4096) -> torch.Tensor:
     """Mean forward KL of ``softmax(teacher_head(ht)) || softmax(hs @ w.T)`` in row chunks.
@@ -104,4 +176,4 @@ def kl_distill_loss(hs: torch.Tensor, ht: torch.Tensor, w: torch.Tensor, teacher
 kl_div = kl_div_logits
 distill_kl = kl_distill_loss
 
-__all__ = ["kl_div_logits", "kl_div", "kl_distill_loss", "distill_kl"]
+__all__ = ["kl_div_logits", "kl_div_logits_topk", "kl_div", "kl_distill_loss", "distill_kl"]

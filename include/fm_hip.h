@@ -132,6 +132,19 @@ int fm_kl_fwd(const void* student, const void* teacher, float* lse_s, float* lse
               float* row_kl, float* loss, int64_t n, int64_t v, int dtype,
               float inv_temperature, int reduction, fm_stream_t stream);
 
+/* fm_kl_fwd that also returns the exact top-k of every teacher row from the same pass over
+ * the logits. The reference has no fused form: a distillation step calls kl_div_logits
+ * (kernels/kl.py:194-232) and topk (kernels/topk.py:273-297) one after the other, reading the
+ * teacher twice. Selection follows topk.py:13-19 on the raw teacher logits (softmax and a
+ * positive temperature keep the order): topk_values [n, k] (row dtype, may be NULL),
+ * topk_indices [n, k] (int32 or int64 by index_bits), topk_probs [n, k] fp32 (may be NULL) =
+ * softmax(teacher * inv_temperature) at the selected columns. Rows wider than 320 KiB or
+ * k > 512 return FM_ERR_UNSUPPORTED; the caller then uses fm_kl_fwd + fm_topk. */
+int fm_kl_fwd_topk(const void* student, const void* teacher, float* lse_s, float* lse_t,
+                   float* row_kl, float* loss, void* topk_values, void* topk_indices,
+                   float* topk_probs, int64_t n, int64_t v, int k, int dtype, int index_bits,
+                   float inv_temperature, int reduction, fm_stream_t stream);
+
 /* Gradient wrt the (unscaled) student logits, recomputed from the saved lse values
  * (the reference stores it from the forward, kl.py:112-134, and rescales it in
  * _KLDivFn.backward, kl.py:181-191):

@@ -389,3 +389,29 @@ def test_qk_norm_rope_surface_and_op_path():
     assert all(torch.allclose(a, b, rtol=1e-4, atol=1e-4) for a, b in zip(eager, ref))
     with pytest.raises(ValueError):
         kernels.qk_norm_rope(x[0], w, cos, sin)
+
+
+def test_kl_div_logits_topk_autograd_and_wide_rows():
+    g = torch.Generator().manual_seed(77)
+    s = (3 * torch.randn(6, 5000, generator=g)).bfloat16()
+    t = (s.float() + 0.5 * torch.randn(6, 5000, generator=g)).bfloat16()
+    sd = s.to("cuda").requires_grad_(True)
+    loss, probs, idx = kernels.kl_div_logits_topk(sd, t.to("cuda"), 16, temperature=2.0, index_dtype=torch.int32)
+    loss.backward()
+    sr = s.to("cuda").requires_grad_(True)
+    ref = kernels.kl_div_logits(sr, t.to("cuda"), temperature=2.0)
+    ref.backward()
+    assert loss.item() == pytest.approx(ref.item(), rel=1e-6)
+    assert torch.allclose(sd.grad.float(), sr.grad.float(), rtol=1e-2, atol=1e-9)
+    assert not probs.requires_grad and idx.dtype == torch.int32
+    assert torch.equal(idx.cpu().long(), O.topk(t, 16)[1])
+    # a row wider than the fused kernel takes goes through the two kernels, same results
+    s = torch.randn(1, 32 * 1024 * 4 + 40, generator=g)
+    t = torch.randn(1, 32 * 1024 * 4 + 40, generator=g)
+    loss, probs, idx = kernels.kl_div_logits_topk(s.to("cuda"), t.to("cuda"), 8, reduction="sum")
+    assert torch.equal(idx.cpu(), O.topk(t, 8)[1])
+    want = torch.gather(torch.softmax(t.double(), -1), -1, idx.cpu())
+    assert torch.allclose(probs.cpu().double(), want, rtol=1e-4)
+    assert loss.item() == pytest.approx(O.kl_div(s, t, "sum", 1.0, acc=torch.float64)[0].item(), rel=1e-4)
+    with pytest.raises(RuntimeError):
+        kernels.kl_div_logits_topk(s.to("cuda"), t.to("cuda"), 0)

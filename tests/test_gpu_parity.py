@@ -244,6 +244,67 @@ def test_kl_known_answers_on_gpu():
     assert torch.equal(s, keep)
 
 
+# ------------------------------------------------------------------ KL + teacher top-k, one pass
+KLTOPK_CASES = [(16, 128256, 64, BF16, 2.0), (6, 32000, 64, BF16, 1.0), (4, 50257, 33, BF16, 2.0),
+                (3, 4096, 8, F32, 1.0), (2, 80000, 64, F32, 2.0), (5, 20000, 100, F16, 1.0),
+                (3, 700, 5, BF16, 1.0), (2, 1025, 512, BF16, 2.0), (4, 1, 1, F32, 1.0),
+                (2, 9000, 512, F32, 1.0)]
+
+
+@pytest.mark.parametrize("n,v,k,dt,T", KLTOPK_CASES)
+def test_kl_fwd_topk_matches_the_two_kernels(n, v, k, dt, T):
+    g = gen(1015)
+    s = (3 * torch.randn(n, v, generator=g)).to(dt)
+    t = (s.float() + 0.5 * torch.randn(n, v, generator=g)).to(dt)
+    o64, _ = O.kl_div(s, t, "mean", T, acc=torch.float64)
+    orow, _ = O.kl_div(s, t, "none", T, acc=torch.float64)
+    ov, oi = O.topk(t, k)
+    sd, td = s.to(DEV), t.to(DEV)
+    for bits in (torch.int32, torch.int64):
+        out = _hip.kl_fwd_topk(sd, td, k, 1.0 / T, "mean", bits, want_values=True, want_probs=True)
+        assert out is not None
+        loss, rows, ls, lt, vals, idx, probs = out
+        loss2, rows2, ls2, lt2 = _hip.kl_fwd(sd, td, 1.0 / T, "mean")
+        torch.cuda.synchronize()
+        assert idx.dtype == bits and torch.equal(idx.cpu().long(), oi)      # bit-exact selection
+        assert torch.equal(vals.cpu(), ov)
+        assert loss.item() == pytest.approx(o64.item(), rel=1e-4, abs=2e-7)
+        assert torch.allclose(rows.cpu().double(), orow, rtol=2e-4, atol=2e-6)
+        assert torch.allclose(rows, rows2, rtol=2e-4, atol=2e-6)
+        assert torch.allclose(ls, ls2, rtol=1e-6, atol=2e-6) and torch.allclose(lt, lt2, rtol=1e-6, atol=2e-6)
+        want = torch.gather(torch.softmax(t.double() / T, -1), -1, oi)
+        assert torch.allclose(probs.cpu().double(), want, rtol=1e-4, atol=1e-9)
+
+
+def test_kl_fwd_topk_ties_unaligned_and_unsupported():
+    g = gen(1016)
+    # three distinct teacher values: the exact path runs inside the fused kernel
+    t = torch.randint(0, 3, (4, 40000), generator=g).to(BF16)
+    s = torch.randn(4, 40000, generator=g).to(BF16)
+    out = _hip.kl_fwd_topk(s.to(DEV), t.to(DEV), 300, 1.0, "none", torch.int32)
+    assert torch.equal(out[5].cpu().long(), O.topk(t, 300)[1])
+    orow, _ = O.kl_div(s, t, "none", 1.0, acc=torch.float64)
+    assert torch.allclose(out[1].cpu().double(), orow, rtol=2e-4, atol=2e-6)
+    # rows that start off a 16-byte boundary
+    base_s = (3 * torch.randn(3 * 9001 + 1, generator=g)).bfloat16().to(DEV)
+    base_t = (3 * torch.randn(3 * 9001 + 1, generator=g)).bfloat16().to(DEV)
+    s2, t2 = base_s[1:].view(3, 9001), base_t[1:].view(3, 9001)
+    out = _hip.kl_fwd_topk(s2, t2, 20, 0.5, "none", torch.int64)
+    assert torch.equal(out[5].cpu(), O.topk(t2.cpu(), 20)[1])
+    orow, _ = O.kl_div(s2.cpu(), t2.cpu(), "none", 2.0, acc=torch.float64)
+    assert torch.allclose(out[1].cpu().double(), orow, rtol=2e-4, atol=2e-6)
+    # NaN in the teacher: selected first, KL of that row is NaN, other rows untouched
+    t3 = torch.randn(2, 5000, generator=g)
+    t3[0, 77] = float("nan")
+    s3 = torch.randn(2, 5000, generator=g)
+    out = _hip.kl_fwd_topk(s3.to(DEV), t3.to(DEV), 4, 1.0, "none", torch.int64)
+    assert torch.equal(out[5].cpu(), O.topk(t3, 4)[1]) and out[5][0, 0].item() == 77
+    assert math.isnan(out[1][0].item()) and math.isfinite(out[1][1].item())
+    # rows wider than the fused kernel's register budget: the binding says so
+    wide = torch.zeros(1, 32 * 1024 * 8 + 8, dtype=BF16, device=DEV)
+    assert _hip.kl_fwd_topk(wide, wide, 4, 1.0, "none", torch.int64) is None
+
+
 # ------------------------------------------------------------------ top-k
 TOPK_CASES = [(32, 128256, 64, BF16), (8, 4096, 64, F32), (4, 64, 8, F32), (3, 5000, 512, BF16),
               (4, 20000, 100, F16), (2, 300000, 17, BF16), (3, 9000, 5, F32), (2, 100, 99, F32),
