@@ -213,7 +213,7 @@ def make_workload(name, torch, L, dev):
 
             w.step = step
             w.dominant_launch = step
-            w.dominant = "topk_kernel<bf16,1024,16>"
+            w.dominant = "topk_lds_kernel<bf16,1024,4>"
             w.dominant_bytes = w.bytes = n * v * 2
             w.desc = f"top-64 of teacher logits bf16 [{n},{v}], int32 indices (separate launch)"
             w.rows = n

@@ -141,17 +141,21 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
     const bool has = tid < sp.nvec || tid < ne;
     const uint32_t mykey = !has ? 0u : (has_nan ? 0xFFFFFFFFu : key_of(fm));
 
-    // ---- phase T: per-wave j-th largest group maximum, then the minimum over waves
-    const int j = (k + NW - 1) / NW;
+    // ---- phase T: per-wave j-th largest group maximum, then the minimum over waves.
+    // Only waves whose 64 lanes all hold data vote: nfull of them with j maxima each bound
+    // at least k elements from below; a part-filled wave would drag tau to the bottom.
+    const int active = (sp.nvec > ne ? sp.nvec : ne) < THREADS ? (sp.nvec > ne ? sp.nvec : ne) : THREADS;
+    const int nfull = active >> 6;
+    const int j = nfull > 0 ? (k + nfull - 1) / nfull : 65;
     uint32_t tw = 0u;
-    if (j <= 64) {
+    if (j <= 64 && wave < nfull) {
       for (int bit = 31; bit >= 0; --bit) {
         const uint32_t trial = tw | (1u << bit);
         const int cnt = __builtin_popcountll(__ballot(mykey >= trial));
         if (cnt >= j) tw = trial;
       }
     }
-    if (lane == 0) s_tau[wave] = tw;
+    if (lane == 0) s_tau[wave] = (wave < nfull || j > 64) ? tw : 0xFFFFFFFFu;
     if (tid == 0) { s_count = 0; s_nwork = 0; }
     __syncthreads();
     uint32_t tau = s_tau[0];

@@ -5,21 +5,23 @@
 // the largest value and the original NaN is what lands in `values`; -0.0 ties with +0.0.
 //
 // One workgroup per row, one streaming read of the row from HBM:
-//   A  every thread folds each 16-byte vector it reads to one maximum and keeps those vector
-//      maxima (not the data) in registers; their maximum is the thread's "group maximum";
-//   T  each wave finds the ceil(k / waves)-th largest of its 64 group maxima with a ballot
-//      search; the minimum over the waves, tau, can never be above the true k-th value,
-//      because at least k group maxima are >= tau;
-//   B  only vectors whose maximum is >= tau can hold candidates -- a few hundred out of
+//   A  every thread folds each 16-byte vector it reads to one maximum and leaves a 16-bit
+//      prefix of that maximum's key in LDS (2 bytes per 16 bytes of row); the maximum over
+//      its vectors is the thread's "group maximum";
+//   T  each full wave finds the ceil(k / waves)-th largest of its 64 group maxima with a
+//      ballot search; the minimum over the waves, tau, can never be above the true k-th
+//      value, because at least k group maxima are >= tau;
+//   B  only vectors whose prefix reaches tau's can hold candidates -- a few hundred out of
 //      16k -- so their indices go to a work list, the workgroup re-reads just those vectors
 //      (one parallel round trip, served by cache) and every element >= tau becomes a
 //      candidate (key, index) in LDS; candidates are ranked by counting how many others beat
 //      them under (key descending, index ascending); rank r < k is output slot r.
-// Keeping maxima instead of the row keeps the kernel at 64 registers, so two 1024-thread
-// workgroups share a compute unit and one streams while the other selects.
+// Keeping prefixes instead of the row keeps registers and LDS small, so several workgroups
+// share a compute unit and one streams while another selects.
 // Rows with too many candidates (long runs of equal values) take an exact path instead: a
 // bitwise search for the k-th key over the whole row, then an index-ordered scan that admits
-// the first (k - #greater) ties. Rows wider than the register budget make two full passes.
+// the first (k - #greater) ties. Rows wider than the LDS budget keep the vector maxima in
+// registers (up to 32 per thread) or make two full passes.
 // Keys are order-preserving integer images of the fp32 value, so no float is ever summed and
 // the result is bit-reproducible.
 #include "fm_topk.cuh"
@@ -87,6 +89,62 @@ void topk_kernel(const T* __restrict__ x, T* __restrict__ values, int32_t* __res
                                                                 row, values, idx32, idx64, nullptr, 0.f, 0.f);
 }
 
+// Variant that leaves a 16-bit key prefix of every vector's maximum in LDS instead of the
+// maxima in registers: few registers, so several workgroups share a compute unit and one
+// row's selection overlaps the next row's streaming read.
+template <typename T, int THREADS, int UNROLL>
+__global__ __launch_bounds__(THREADS) void topk_lds_kernel(const T* __restrict__ x, T* __restrict__ values,
+                                                           int32_t* __restrict__ idx32,
+                                                           int64_t* __restrict__ idx64, int v, int k,
+                                                           bool vec_ok) {
+  constexpr int EPV = Elem<T>::kVec;
+  __shared__ TopkShared<THREADS, kVecMaxLds> sh;
+  extern __shared__ __align__(16) uint16_t vhi[];
+  const int64_t row = blockIdx.x;
+  const T* rp = x + row * (int64_t)v;
+  const int tid = threadIdx.x;
+  const RowSplit sp = split_row<EPV>(row, v, vec_ok);
+  float fm = -INFINITY;
+  bool has_nan = false;
+  if (v > kCap) {
+    {  // zero the padding of the last quad of prefixes
+      const int p = ((sp.nvec + 3) & ~3) - 1 - tid;
+      if (tid < 3 && p >= sp.nvec) vhi[p] = 0;
+    }
+    for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+      u32x4 raw[UNROLL];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const int c = c0 + u * THREADS + tid;
+        if (c < sp.nvec) raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
+      }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const int c = c0 + u * THREADS + tid;
+        if (c < sp.nvec) {
+          const float m = fold_vector_max<T>(raw[u]);
+          const bool bad = m != m;
+          vhi[c] = (uint16_t)(bad ? 0xFFFFu : key_prefix(key_of(m)));
+          fm = fmaxf(fm, m);
+          has_nan |= bad;
+        }
+      }
+    }
+    const int ne = edge_count(sp, v);
+    for (int e = tid; e < ne; e += THREADS) {
+      const float f = Elem<T>::load1(rp + edge_col(sp, e));
+      fm = fmaxf(fm, f);
+      has_nan |= (f != f);
+    }
+  }
+  const float none[1] = {0.f};
+  topk_finish<T, THREADS, 1, kVecMaxLds>(rp, sp, v, k, none, vhi, fm, has_nan, sh, row, values, idx32, idx64,
+                                         nullptr, 0.f, 0.f);
+}
+
+// widest row (in 16-byte vectors) whose key prefixes fit the LDS budget
+constexpr int kLdsMaxVec = 20480;
+
 template <typename T>
 int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, int index_bits,
            bool vec_ok, hipStream_t st) {
@@ -99,14 +157,20 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
   const dim3 grid((unsigned)n);
 #define GO(TH, IT)                                                                               \
   hipLaunchKernelGGL((topk_kernel<T, TH, IT>), grid, dim3(TH), 0, st, xp, vp, i32, i64, v, k, vec_ok)
-  const int variant = fm_host::get_param(fm_host::P_TOPK_VARIANT);
-  if (variant == 1 && v > kCap) GO(1024, 0);
-  else if (v <= kCap || nvec <= 256 * 4) GO(256, 4);
-  else if (nvec <= 1024 * 4) GO(1024, 4);
-  else if (nvec <= 1024 * 16) GO(1024, 16);
-  else if (nvec <= 1024 * 32) GO(1024, 32);
-  else GO(1024, 0);
+#define GOL(TH, UN)                                                                              \
+  hipLaunchKernelGGL((topk_lds_kernel<T, TH, UN>), grid, dim3(TH), (size_t)(nvec + 8) * 2, st, xp, vp, i32, \
+                     i64, v, k, vec_ok)
+  int variant = fm_host::get_param(fm_host::P_TOPK_VARIANT);
+  if (variant == 0) variant = nvec <= 3072 ? 1 : (nvec <= 12288 ? 2 : 3);
+  if (v <= kCap) GOL(256, 4);             // every element is a candidate; no prefixes used
+  else if (nvec > kLdsMaxVec) {
+    if (nvec <= 1024 * 32) GO(1024, 32);
+    else GO(1024, 0);
+  } else if (variant == 1) GOL(256, 4);
+  else if (variant == 2) GOL(512, 4);
+  else GOL(1024, 4);
 #undef GO
+#undef GOL
   return FM_OK;
 }
 
