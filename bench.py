@@ -49,7 +49,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="ce",
-                    choices=["ce", "rmsnorm", "add_rmsnorm", "kl", "kl_topk", "topk", "route", "moe_dispatch"])
+                    choices=["ce", "ce_one_pass", "rmsnorm", "add_rmsnorm", "kl", "kl_topk", "topk", "route", "moe_dispatch"])
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
@@ -166,7 +166,7 @@ def make_workload(name, torch, L, dev):
         w.rows = n
         return w
 
-    if name == "ce":
+    if name in ("ce", "ce_one_pass"):
         n, v = 8192, 32000
         g.manual_seed(1002)
         lg = (2 * torch.randn(n, v, device=dev, generator=g)).bfloat16()
@@ -183,6 +183,29 @@ def make_workload(name, torch, L, dev):
         def bwd():
             _check(L.fm_ce_bwd(lg.data_ptr(), y.data_ptr(), lse.data_ptr(), sc.data_ptr() + 4, None,
                                dlg.data_ptr(), n, v, BF, -100, st), "fm_ce_bwd")
+
+        if name == "ce_one_pass":
+            one = torch.ones((), device=dev)
+
+            def both():
+                _check(L.fm_ce_loss_grad(lg.data_ptr(), y.data_ptr(), lse.data_ptr(), rl.data_ptr(),
+                                         sc.data_ptr(), sc.data_ptr() + 4, dlg.data_ptr(), n, v, BF, -100, 2,
+                                         st), "fm_ce_loss_grad")
+
+            def step():
+                both()      # forward: loss and gradient from one read of the logits
+                _check(L.fm_scale_inplace(dlg.data_ptr(), one.data_ptr(), n * v, BF, st),
+                       "fm_scale_inplace")   # backward: upstream gradient 1, nothing to move
+
+            w.step = step
+            w.dominant_launch = both
+            w.dominant = "ce_loss_grad_kernel<bf16,512,8>"
+            w.dominant_bytes = w.bytes = n * v * 4
+            w.desc = (f"fused CE loss + gradient in one pass, logits bf16 [{n},{v}], 5% ignore_index, mean; "
+                      "dataflow read + write = 4 B/logit")
+            w.rows = n
+            w.tensors = (lg, y)
+            return w
 
         def step():
             fwd()
@@ -495,7 +518,7 @@ def main():
     torch.cuda.empty_cache()
     if not a.no_extras:
         extras = {a.workload: res}
-        for name in ["rmsnorm", "add_rmsnorm", "ce", "kl", "kl_topk", "topk", "route", "moe_dispatch"]:
+        for name in ["rmsnorm", "add_rmsnorm", "ce", "ce_one_pass", "kl", "kl_topk", "topk", "route", "moe_dispatch"]:
             if name == a.workload:
                 continue
             wl = make_workload(name, torch, L, dev)

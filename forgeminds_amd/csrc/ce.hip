@@ -169,6 +169,156 @@ __global__ __launch_bounds__(THREADS) void ce_bwd_kernel(const T* __restrict__ l
   }
 }
 
+// Number of rows whose label is not ignore_index, as the float the gradient is divided by
+// (at least 1). One workgroup; runs ahead of ce_loss_grad_kernel, which needs the count.
+__global__ __launch_bounds__(1024) void ce_count_kernel(const int64_t* __restrict__ labels, int64_t n,
+                                                        int64_t ignore_index,
+                                                        float* __restrict__ n_valid) {
+  __shared__ int si[16];
+  int cnt = 0;
+  for (int64_t i = threadIdx.x; i < n; i += 1024) cnt += labels[i] != ignore_index ? 1 : 0;
+  cnt = wave_sum_i(cnt);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) si[wave] = cnt;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int c = si[0];
+    for (int i = 1; i < 16; ++i) c += si[i];
+    *n_valid = c > 0 ? (float)c : 1.f;
+  }
+}
+
+// Loss and gradient from ONE read of the logits: the row stays in registers (ITERS 16-byte
+// vectors per thread) between the log-sum-exp and the gradient store, so the whole
+// forward + backward of a training step moves 2 + 2 bytes per bf16 logit instead of 2 + 2 + 2.
+// dlogits may be the logits buffer itself: every element is read by the thread that later
+// writes it. The gradient is (softmax - onehot) * scale, scale = 1 / n_valid for the mean.
+template <typename T, int THREADS, int ITERS>
+__global__ __launch_bounds__(THREADS) void ce_loss_grad_kernel(const T* logits,
+                                                                const int64_t* __restrict__ labels,
+                                                                const float* __restrict__ n_valid,
+                                                                float* __restrict__ lse,
+                                                                float* __restrict__ row_loss,
+                                                                T* dlogits, int v,
+                                                                int64_t ignore_index) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int NW = THREADS / 64;
+  __shared__ float smem[2 * NW];
+  const int64_t row = blockIdx.x;
+  const T* rp = logits + row * (int64_t)v;
+  T* gp = dlogits + row * (int64_t)v;
+  const RowSplit sp = split_row<EPV>(row, v, true);
+  const int tid = threadIdx.x;
+  const int ne = edge_count(sp, v);
+  const int64_t y64 = labels[row];
+
+  if (y64 == ignore_index) {  // ignored row: zeros, and the logits are never read
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = i * THREADS + tid;
+      if (c < sp.nvec) store16_stream(gp + sp.head + (int64_t)c * EPV, zero);
+    }
+    for (int e = tid; e < ne; e += THREADS) Elem<T>::store1(gp + edge_col(sp, e), 0.f);
+    if (tid == 0) {
+      row_loss[row] = 0.f;
+      if (lse != nullptr) lse[row] = 0.f;
+    }
+    return;
+  }
+  const int y = (y64 >= 0 && y64 < v) ? (int)y64 : -1;
+
+  u32x4 raw[ITERS];
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * THREADS + tid;
+    if (c < sp.nvec) raw[i] = load16_stream(rp + sp.head + (int64_t)c * EPV);
+  }
+  // the unaligned ends of the row (at most EPV - 1 elements each): thread e keeps edge e
+  float edge = -INFINITY;
+  int edge_at = -1;
+  if (tid < ne) {
+    edge_at = edge_col(sp, tid);
+    edge = Elem<T>::load1(rp + edge_at) * kLog2e;
+  }
+  // maximum first, then the sum: the data sits in registers, a second sweep costs no traffic
+  float mz = fmaxf(edge, kNegBig);
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * THREADS + tid;
+    if (c < sp.nvec) {
+      float z[EPV];
+      Elem<T>::unpack(raw[i], z);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) mz = fmaxf(mz, z[e] * kLog2e);
+    }
+  }
+  float ssum = edge_at >= 0 ? fast_exp2(edge - mz) : 0.f;
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * THREADS + tid;
+    if (c < sp.nvec) {
+      float z[EPV];
+      Elem<T>::unpack(raw[i], z);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) ssum += fast_exp2(z[e] * kLog2e - mz);
+    }
+  }
+  const MaxSum tot = block_merge<NW>(MaxSum{mz, ssum}, smem);
+  const float l2 = tot.m + fast_log2(tot.s);
+  const float scale = 1.f / (n_valid != nullptr ? *n_valid : 1.f);
+  if (tid == 0) {
+    const float l = l2 * kLn2;
+    if (lse != nullptr) lse[row] = l;
+    row_loss[row] = y >= 0 ? l - Elem<T>::load1(rp + y) : __builtin_nanf("");
+  }
+  __syncthreads();   // the label logit is read before any thread overwrites it in place
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * THREADS + tid;
+    if (c < sp.nvec) {
+      float z[EPV], o[EPV];
+      Elem<T>::unpack(raw[i], z);
+      const int col0 = sp.head + c * EPV;
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) o[e] = fast_exp2(z[e] * kLog2e - l2);
+      if (y >= col0 && y < col0 + EPV) {
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] -= (col0 + e == y) ? 1.f : 0.f;
+      }
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) o[e] *= scale;
+      store16_stream(gp + col0, Elem<T>::pack(o));
+    }
+  }
+  if (edge_at >= 0) {
+    float p = fast_exp2(edge - l2);
+    if (edge_at == y) p -= 1.f;
+    Elem<T>::store1(gp + edge_at, p * scale);
+  }
+}
+
+// x *= *factor in place, skipped altogether when the factor is exactly 1 (the usual upstream
+// gradient of a loss): the gradient written by ce_loss_grad_kernel then costs no second pass.
+template <typename T>
+__global__ __launch_bounds__(1024) void scale_inplace_kernel(T* x, const float* __restrict__ factor,
+                                                             int64_t count, bool vec_ok) {
+  constexpr int EPV = Elem<T>::kVec;
+  const float f = *factor;
+  if (f == 1.f) return;
+  const int64_t nvec = vec_ok ? count / EPV : 0;
+  const int64_t stride = (int64_t)gridDim.x * 1024;
+  for (int64_t c = (int64_t)blockIdx.x * 1024 + threadIdx.x; c < nvec; c += stride) {
+    float z[EPV];
+    Elem<T>::unpack(load16_stream(x + c * EPV), z);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) z[e] *= f;
+    store16_stream(x + c * EPV, Elem<T>::pack(z));
+  }
+  for (int64_t i = nvec * EPV + (int64_t)blockIdx.x * 1024 + threadIdx.x; i < count; i += stride)
+    Elem<T>::store1(x + i, Elem<T>::load1(x + i) * f);
+}
+
 template <typename T>
 int launch_fwd(const void* logits, const int64_t* labels, float* lse, float* row_loss, int64_t n,
                int v, int64_t ignore_index, bool vec_ok, hipStream_t st) {
@@ -250,6 +400,99 @@ int fm_ce_bwd(const void* logits, const int64_t* labels, const float* lse, const
   else if (dtype == FM_BF16) launch_bwd<bf16_t>(logits, labels, lse, n_valid, grad_out, dlogits, n, (int)v, ignore_index, vec_ok, st);
   else launch_bwd<f16_t>(logits, labels, lse, n_valid, grad_out, dlogits, n, (int)v, ignore_index, vec_ok, st);
   FM_CHECK_LAUNCH("fm_ce_bwd");
+  return FM_OK;
+}
+
+int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float* row_loss,
+                    float* loss, float* n_valid, void* dlogits, int64_t n, int64_t v, int dtype,
+                    int64_t ignore_index, int reduction, fm_stream_t stream) {
+  int rc = check_shape("fm_ce_loss_grad", n, v, dtype);
+  if (rc != FM_OK) return rc;
+  FM_CHECK_ARG(reduction == FM_REDUCE_SUM || reduction == FM_REDUCE_MEAN,
+               "fm_ce_loss_grad: reduction must be sum or mean (got %d)", reduction);
+  FM_CHECK_ARG(loss && n_valid, "fm_ce_loss_grad: NULL scalar output");
+  FM_CHECK_ARG(n == 0 || (logits && labels && row_loss && dlogits), "fm_ce_loss_grad: NULL pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int esize = dtype == FM_F32 ? 4 : 2;
+  const int64_t nvec = v / (16 / esize);
+  const bool one_pass = n > 0 && fm_host::aligned16(logits) && fm_host::aligned16(dlogits) &&
+                        nvec <= 8 * 1024;
+  if (!one_pass) {
+    // rows too wide for the register file (or unaligned buffers): the two-pass kernels,
+    // which give the same outputs; lse is then needed as scratch
+    if (n > 0 && lse == nullptr) {
+      fm_host::set_error("fm_ce_loss_grad: lse is required for rows of more than %d bytes or unaligned buffers",
+                         8 * 1024 * 16);
+      return FM_ERR_INVALID;
+    }
+    rc = fm_ce_fwd(logits, labels, lse, row_loss, loss, n_valid, n, v, dtype, ignore_index, reduction, stream);
+    if (rc != FM_OK) return rc;
+    return fm_ce_bwd(logits, labels, lse, reduction == FM_REDUCE_MEAN ? n_valid : nullptr, nullptr, dlogits,
+                     n, v, dtype, ignore_index, stream);
+  }
+  const bool mean = reduction == FM_REDUCE_MEAN;
+  const int pref = fm_host::get_param(fm_host::P_VOCAB_THREADS);
+  if (mean) {
+    hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(1024), 0, st, labels, n, ignore_index, n_valid);
+    FM_CHECK_LAUNCH("fm_ce_loss_grad(count)");
+  }
+  const float* nv = mean ? n_valid : nullptr;
+  const dim3 grid((unsigned)n);
+#define LAUNCH(T, TH, IT)                                                                        \
+  hipLaunchKernelGGL((ce_loss_grad_kernel<T, TH, IT>), grid, dim3(TH), 0, st,                    \
+                     static_cast<const T*>(logits), labels, nv, lse, row_loss,                   \
+                     static_cast<T*>(dlogits), (int)v, ignore_index)
+#define BY_ITERS(T, TH)                        \
+  do {                                         \
+    if (iters == 2) LAUNCH(T, TH, 2);          \
+    else if (iters == 4) LAUNCH(T, TH, 4);     \
+    else if (iters == 8) LAUNCH(T, TH, 8);     \
+    else LAUNCH(T, TH, 16);                    \
+  } while (0)
+#define BY_SHAPE(T)                            \
+  do {                                         \
+    if (threads == 256) BY_ITERS(T, 256);      \
+    else if (threads == 512) BY_ITERS(T, 512); \
+    else if (iters == 2) LAUNCH(T, 1024, 2);   \
+    else if (iters == 4) LAUNCH(T, 1024, 4);   \
+    else LAUNCH(T, 1024, 8);                   \
+  } while (0)
+  // the fewest threads that hold the row in at most 8 vectors each: small workgroups keep
+  // several rows per compute unit in different phases (loading, reducing, storing)
+  int threads = pref == 256 || pref == 512 || pref == 1024 ? pref : 256;
+  while (threads < 1024 && nvec > (int64_t)threads * 8) threads *= 2;
+  int iters = 2;
+  while ((int64_t)threads * iters < nvec) iters *= 2;
+  if (dtype == FM_F32) BY_SHAPE(float);
+  else if (dtype == FM_BF16) BY_SHAPE(bf16_t);
+  else BY_SHAPE(f16_t);
+#undef BY_ITERS
+#undef BY_SHAPE
+#undef LAUNCH
+  FM_CHECK_LAUNCH("fm_ce_loss_grad");
+  hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, st, row_loss, labels, n,
+                     ignore_index, mean ? 1 : 0, loss, n_valid);
+  FM_CHECK_LAUNCH("fm_ce_loss_grad(finalize)");
+  return FM_OK;
+}
+
+int fm_scale_inplace(void* x, const float* factor, int64_t count, int dtype, fm_stream_t stream) {
+  FM_CHECK_ARG(count >= 0, "fm_scale_inplace: bad count %lld", (long long)count);
+  FM_CHECK_ARG(dtype == FM_F32 || dtype == FM_F16 || dtype == FM_BF16, "fm_scale_inplace: bad dtype %d",
+               dtype);
+  if (count == 0) return FM_OK;
+  FM_CHECK_ARG(x && factor, "fm_scale_inplace: NULL pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool vec_ok = fm_host::aligned16(x);
+  const int64_t per_block = 1024 * 8 * 4;   // elements a workgroup covers per sweep, roughly
+  int64_t blocks = (count + per_block - 1) / per_block;
+  const int64_t cap = (int64_t)fm_host::num_cus() * 8;
+  if (blocks > cap) blocks = cap;
+  const dim3 grid((unsigned)blocks);
+  if (dtype == FM_F32) hipLaunchKernelGGL(scale_inplace_kernel<float>, grid, dim3(1024), 0, st, static_cast<float*>(x), factor, count, vec_ok);
+  else if (dtype == FM_BF16) hipLaunchKernelGGL(scale_inplace_kernel<bf16_t>, grid, dim3(1024), 0, st, static_cast<bf16_t*>(x), factor, count, vec_ok);
+  else hipLaunchKernelGGL(scale_inplace_kernel<f16_t>, grid, dim3(1024), 0, st, static_cast<f16_t*>(x), factor, count, vec_ok);
+  FM_CHECK_LAUNCH("fm_scale_inplace");
   return FM_OK;
 }
 

@@ -41,6 +41,8 @@ SIGNATURES = {
                                   _int, _int, _vp]),
     "fm_ce_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _i64, _int, _vp]),
     "fm_ce_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _i64, _vp]),
+    "fm_ce_loss_grad": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _i64, _int, _vp]),
+    "fm_scale_inplace": (_int, [_vp, _vp, _i64, _int, _vp]),
     "fm_kl_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _f32, _int, _vp]),
     "fm_kl_fwd_topk": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _int,
                               _f32, _int, _vp]),
@@ -225,6 +227,32 @@ def ce_fwd(logits2, labels, ignore_index: int, reduction: str):
                                dtype_code(logits2.dtype), int(ignore_index), REDUCE[reduction],
                                _stream(logits2)), "fm_ce_fwd")
     return scal[0], lse, scal[1], row_loss
+
+
+def ce_loss_grad(logits2, labels, ignore_index: int, reduction: str, inplace: bool = False):
+    """-> (loss fp32 scalar, dlogits [n, v], n_valid, row_loss); the gradient is for an upstream
+    gradient of 1 and lands in ``logits2`` itself when ``inplace``."""
+    _dense(logits2, labels)
+    n, v = logits2.shape
+    dev = logits2.device
+    buf = torch.empty(2, max(n, 1), device=dev, dtype=torch.float32)
+    scalars = torch.empty(2, device=dev, dtype=torch.float32)
+    dl = logits2 if inplace else torch.empty_like(logits2)
+    with torch.cuda.device(dev):
+        _check(lib().fm_ce_loss_grad(_ptr(logits2), _ptr(labels), buf[0].data_ptr(), buf[1].data_ptr(),
+                                     scalars[0:].data_ptr(), scalars[1:].data_ptr(), _ptr(dl), n, v,
+                                     dtype_code(logits2.dtype), int(ignore_index), REDUCE[reduction],
+                                     _stream(logits2)), "fm_ce_loss_grad")
+    return scalars[0], dl, scalars[1], buf[1][:n]
+
+
+def scale_inplace(x, factor):
+    """x *= factor (fp32 device scalar), skipped on the device when the factor is exactly 1."""
+    _dense(x, factor)
+    with torch.cuda.device(x.device):
+        _check(lib().fm_scale_inplace(_ptr(x), _ptr(factor), x.numel(), dtype_code(x.dtype), _stream(x)),
+               "fm_scale_inplace")
+    return x
 
 
 def ce_bwd(logits2, labels, lse, n_valid, grad_out, ignore_index: int):

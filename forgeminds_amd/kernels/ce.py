@@ -2,8 +2,11 @@
 
 Stands in for the ``F.cross_entropy(..., reduction="sum") / n`` pattern of the reference's
 ``forgemind/loss.py:54-70`` (there is no fused CE kernel in the reference; its path is
-aten ``log_softmax`` + ``nll_loss``). One read of the logits in the forward (online
-max / sum-exp, per-row ``lse`` saved), softmax recomputed from ``lse`` in the backward.
+aten ``log_softmax`` + ``nll_loss``). When the logits need a gradient the forward produces it
+in the same pass (each row stays in registers between the log-sum-exp and the gradient store),
+the way the reference's KL writes its gradient in the forward (``kernels/kl.py:143-191``); the
+backward multiplies by the upstream gradient in place, which the kernel skips when that is 1.
+Without a gradient the forward is one read of the logits (online max / sum-exp).
 
 The loss is fp32 math on the logits' values; a bf16 input does not yield a bf16-rounded
 loss the way the literal ``F.cross_entropy(bf16)`` call does.
@@ -20,26 +23,35 @@ from ._common import _note, fast_ok
 
 class _CrossEntropyFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, logits, labels, ignore_index, reduction):
+    def forward(ctx, logits, labels, ignore_index, reduction, inplace):
         lg2 = logits.contiguous().view(-1, logits.shape[-1])
         y = labels.contiguous().view(-1)
-        loss, lse, n_valid, _rows = _hip.ce_fwd(lg2, y, ignore_index, reduction)
-        ctx.save_for_backward(lg2, y, lse, n_valid)
-        ctx.ignore_index = ignore_index
-        ctx.mean = reduction == "mean"
         ctx.shape = logits.shape
-        return loss.clone()     # `loss` is a view into a 2-element scratch tensor
+        ctx.spent = False
+        if not ctx.needs_input_grad[0]:
+            loss, _lse, _n_valid, _rows = _hip.ce_fwd(lg2, y, ignore_index, reduction)
+            return loss.clone()     # `loss` is a view into a 2-element scratch tensor
+        # writing into the caller's storage is only done when asked for and when lg2 is that
+        # storage (contiguous() did not copy)
+        own = inplace and lg2.data_ptr() == logits.data_ptr()
+        loss, dl, _n_valid, _rows = _hip.ce_loss_grad(lg2.detach(), y, ignore_index, reduction, own)
+        ctx.save_for_backward(dl)
+        return loss.clone()
 
     @staticmethod
     def backward(ctx, g):
-        lg2, y, lse, n_valid = ctx.saved_tensors
+        (dl,) = ctx.saved_tensors
+        if ctx.spent:
+            raise RuntimeError("cross_entropy: the gradient buffer written in the forward was already "
+                               "consumed by a backward pass; run the forward again")
+        ctx.spent = True
         g32 = g.detach().to(torch.float32).contiguous()
-        dl = _hip.ce_bwd(lg2, y, lse, n_valid if ctx.mean else None, g32, ctx.ignore_index)
-        return dl.view(ctx.shape), None, None, None
+        _hip.scale_inplace(dl, g32)
+        return dl.view(ctx.shape), None, None, None, None
 
 
 def cross_entropy(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int = -100,
-                  reduction: str = "mean") -> torch.Tensor:
+                  reduction: str = "mean", inplace: bool = False) -> torch.Tensor:
     """fp32 scalar CE over the last dim of ``logits``.
 
     ``reduction="mean"`` divides the sum over valid rows by ``max(1, #valid)`` (all-ignored
@@ -47,6 +59,10 @@ def cross_entropy(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int 
     ``tests/test_edge_cases.py:21-36``); ``"sum"`` returns the plain sum, which is what one
     chunk of ``chunked_cross_entropy`` contributes. Labels are int64; rows whose label equals
     ``ignore_index`` contribute nothing and receive a zero gradient.
+
+    ``inplace=True`` lets the kernel write the gradient over ``logits`` (only for a tensor the
+    caller owns and no longer reads, e.g. the output of the head projection): no second
+    ``[N, V]`` buffer exists. The gradient buffer serves one backward pass.
     """
     if reduction not in ("mean", "sum"):
         raise ValueError(f"reduction must be mean|sum, got {reduction!r}")
@@ -58,7 +74,7 @@ def cross_entropy(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int 
         return fb.cross_entropy(logits, labels, ignore_index, reduction)
     if not fast_ok(logits):
         return fb.cross_entropy(logits, labels, ignore_index, reduction)
-    return _CrossEntropyFn.apply(logits, labels, int(ignore_index), reduction)
+    return _CrossEntropyFn.apply(logits, labels, int(ignore_index), reduction, bool(inplace))
 
 
 __all__ = ["cross_entropy"]

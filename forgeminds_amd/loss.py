@@ -35,7 +35,8 @@ def chunked_cross_entropy(h, weight, labels, chunk: int = 4096, ignore_index: in
     w = weight if weight.dtype == h.dtype else weight.to(h.dtype)
 
     def piece(hc, yc):
-        return cross_entropy(F.linear(hc, w), yc, ignore_index, "sum")
+        # the chunk's logits are a temporary nobody else reads: the gradient may overwrite them
+        return cross_entropy(F.linear(hc, w), yc, ignore_index, "sum", inplace=True)
 
     total = None
     for lo in range(0, h.size(0), chunk):

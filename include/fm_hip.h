@@ -120,6 +120,25 @@ int fm_ce_bwd(const void* logits, const int64_t* labels, const float* lse, const
               const float* grad_out, void* dlogits, int64_t n, int64_t v, int dtype,
               int64_t ignore_index, fm_stream_t stream);
 
+/* Loss AND gradient of loss.py:54-70 from one read of the logits: fm_ce_fwd's outputs plus
+ *   dlogits[i,j] = (softmax(logits[i,:])[j] - [j == labels[i]]) / n_valid   (FM_REDUCE_MEAN)
+ * i.e. fm_ce_bwd with grad_out = 1, written in the same pass (a training step whose loss is
+ * the last node has exactly that upstream gradient; fm_scale_inplace applies any other one).
+ * Rows stay in registers between the log-sum-exp and the store, so the step moves 2 + 2
+ * bytes per 16-bit logit instead of 2 + 2 + 2. dlogits may be the logits buffer itself
+ * (the way the reference's KL writes its gradient into an owned student tensor,
+ * kernels/kl.py:146-150, 157-160). lse may be NULL when rows are at most 128 KiB and both
+ * buffers are 16-byte aligned; wider rows run fm_ce_fwd + fm_ce_bwd internally and need it.
+ * lse of ignored rows is written as 0 by the one-pass form (those rows are not read). */
+int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float* row_loss,
+                    float* loss, float* n_valid, void* dlogits, int64_t n, int64_t v, int dtype,
+                    int64_t ignore_index, int reduction, fm_stream_t stream);
+
+/* x[i] *= *factor for count elements of dtype, in place; a factor of exactly 1 returns
+ * without touching x. Stands in for `grad * g` in the backward of a loss whose gradient was
+ * produced in the forward (kernels/kl.py:181-191 does that multiply unconditionally). */
+int fm_scale_inplace(void* x, const float* factor, int64_t count, int dtype, fm_stream_t stream);
+
 /* ------------------------------------------------------------------ distillation KL
  * Replaces _kl_fwd_bwd_kernel's loss half (forgemind/kernels/kl.py:73-135, 143-179);
  * semantics of _fallback.kl_div_logits (_fallback.py:52-69) on logits scaled by

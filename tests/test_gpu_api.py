@@ -163,6 +163,17 @@ def test_cross_entropy_autograd_and_callers():
     (loss * 3.0).backward()
     assert loss.dtype == torch.float32 and loss.item() == pytest.approx(ol.item(), rel=1e-4)
     assert close(lgd.grad, og.float() * 3.0)
+    # the gradient written over an owned logits tensor; one backward per forward
+    owned = lg.to(DEV)
+    leaf = owned.clone().requires_grad_(True)
+    tmp = leaf * 1.0                                   # a temporary that only the loss reads
+    l_in = kernels.cross_entropy(tmp, y.to(DEV), inplace=True)
+    l_in.backward(retain_graph=True)
+    assert l_in.item() == loss.item() and close(leaf.grad, og.float())
+    with pytest.raises(RuntimeError, match="already consumed"):
+        l_in.backward()
+    with torch.no_grad():                              # no gradient wanted: plain forward
+        assert kernels.cross_entropy(owned, y.to(DEV)).item() == pytest.approx(ol.item(), rel=1e-4)
     # logits_cross_entropy on [B, T, V] (reference tests/test_edge_cases.py:50-56)
     l3 = logits_cross_entropy(lg.to(DEV).view(3, 100, 4000), y.to(DEV).view(3, 100))
     assert l3.item() == pytest.approx(ol.item(), rel=1e-4)

@@ -181,6 +181,68 @@ def test_ce_fwd_bwd(n, v, dt):
     assert torch.allclose(lse.cpu().double(), lse_ref, rtol=1e-5, atol=1e-5)
 
 
+CE1_CASES = CE_CASES + [(5, 140000, BF16), (3, 70000, F32), (4, 600, BF16), (3, 9000, F16)]
+
+
+@pytest.mark.parametrize("n,v,dt", CE1_CASES)
+@pytest.mark.parametrize("reduction", ["mean", "sum"])
+def test_ce_loss_and_gradient_in_one_pass(n, v, dt, reduction):
+    g = gen(1012)
+    lg = (2 * torch.randn(n, v, generator=g)).to(dt)
+    y = torch.randint(0, v, (n,), generator=g)
+    y[torch.rand(n, generator=g) < 0.2] = -100
+    o64, _ = O.cross_entropy(lg, y, acc=torch.float64)
+    _, ograd = O.cross_entropy(lg, y)
+    n_valid = max(1, int((y != -100).sum()))
+    if reduction == "sum":
+        o64, ograd = o64 * n_valid, ograd.float() * n_valid
+    lgd, yd = lg.to(DEV), y.to(DEV)
+    keep = lgd.clone()
+    loss, dl, nv, rows = _hip.ce_loss_grad(lgd, yd, -100, reduction)
+    torch.cuda.synchronize()
+    assert torch.equal(lgd, keep), "the input is left alone unless in-place is asked for"
+    assert nv.item() == n_valid
+    assert loss.item() == pytest.approx(o64.item(), rel=1e-4, abs=1e-6)
+    cancel = 1.0 / n_valid if reduction == "mean" else 1.0
+    assert_close_lowp(dl, ograd.float(), dt, "dlogits", ulps=3.0, cancel=cancel)
+    ign = (y == -100)
+    assert not dl.cpu()[ign].any() and not rows.cpu()[ign].any()
+    # the same call writing over the logits gives the same bits
+    loss2, dl2, _, _ = _hip.ce_loss_grad(lgd, yd, -100, reduction, inplace=True)
+    torch.cuda.synchronize()
+    assert dl2.data_ptr() == lgd.data_ptr()
+    assert torch.equal(dl2, dl) and loss2.item() == loss.item()
+    # and it agrees with the two-pass kernels to the last bit of the loss and a rounding of the grad
+    loss3, lse, nv3, _ = _hip.ce_fwd(keep, yd, -100, reduction)
+    dl3 = _hip.ce_bwd(keep, yd, lse, nv3 if reduction == "mean" else None, None, -100)
+    assert loss3.item() == pytest.approx(loss.item(), rel=1e-6, abs=1e-7)
+    assert_close_lowp(dl, dl3.float().cpu(), dt, "vs two-pass", ulps=2.0, cancel=cancel)
+
+
+def test_ce_loss_grad_unaligned_and_scale_inplace():
+    g = gen(1013)
+    base = (2 * torch.randn(5 * 3001 + 1, generator=g)).bfloat16().to(DEV)
+    lg = base[1:].view(5, 3001)                                      # base pointer off by 2 bytes
+    y = torch.randint(0, 3001, (5,), generator=g).to(DEV)
+    loss, dl, nv, _ = _hip.ce_loss_grad(lg, y, -100, "mean")
+    o64, _ = O.cross_entropy(lg.cpu(), y.cpu(), acc=torch.float64)
+    _, ograd = O.cross_entropy(lg.cpu(), y.cpu())
+    assert loss.item() == pytest.approx(o64.item(), rel=1e-4)
+    assert_close_lowp(dl, ograd.float(), BF16, "dlogits", ulps=3.0, cancel=0.2)
+    # scale_inplace: a factor of 1 leaves every bit alone, any other factor multiplies once
+    for dt, cnt in ((BF16, 100003), (F32, 4099), (F16, 7)):
+        x = torch.randn(cnt, generator=g).to(dt).to(DEV)
+        before = x.clone()
+        _hip.scale_inplace(x, torch.tensor(1.0, device=DEV))
+        assert torch.equal(x, before)
+        _hip.scale_inplace(x, torch.tensor(0.375, device=DEV))
+        assert torch.equal(x, (before.float() * 0.375).to(dt))
+    x = torch.randn(33, device=DEV)[1:]                              # unaligned start
+    before = x.clone()
+    _hip.scale_inplace(x, torch.tensor(-2.0, device=DEV))
+    assert torch.equal(x, before * -2.0)
+
+
 def test_ce_known_answers_on_gpu():
     # all ignored -> 0.0 and a zero gradient; reference tests/test_edge_cases.py:21-28
     lg = torch.randn(6, 16, device=DEV)
