@@ -425,6 +425,11 @@ int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float
                          8 * 1024 * 16);
       return FM_ERR_INVALID;
     }
+    if (n > 0 && dlogits == logits) {
+      fm_host::set_error("fm_ce_loss_grad: the gradient can overwrite the logits only for aligned rows of "
+                         "at most %d bytes", 8 * 1024 * 16);
+      return FM_ERR_UNSUPPORTED;
+    }
     rc = fm_ce_fwd(logits, labels, lse, row_loss, loss, n_valid, n, v, dtype, ignore_index, reduction, stream);
     if (rc != FM_OK) return rc;
     return fm_ce_bwd(logits, labels, lse, reduction == FM_REDUCE_MEAN ? n_valid : nullptr, nullptr, dlogits,

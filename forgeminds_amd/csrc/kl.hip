@@ -18,6 +18,9 @@ namespace {
 // widest row (in 16-byte vectors) the fused KL + top-k kernel keeps key prefixes for
 constexpr int kFusedMaxVec = 20480;
 
+// widest row (in 16-byte vectors) that the one-pass loss + gradient kernel keeps in registers
+constexpr int kOnePassMaxVec = 4096;
+
 struct KLState {
   float ms, ds, mt, dt, a;
 };
@@ -313,6 +316,118 @@ __global__ __launch_bounds__(THREADS) void kl_bwd_kernel(const T* __restrict__ s
   }
 }
 
+// KL and its gradient from ONE read of both rows: student and teacher stay in registers
+// (ITERS 16-byte vectors each per thread) between the log-sum-exps and the gradient store,
+// the dataflow of the reference's kernel (kl.py:73-135) without its second read. The gradient
+// is for an upstream gradient of 1: (p_s - p_t) * mul, mul = inv_temp * (1/n for the mean).
+// dstudent may be the student buffer itself when both have the same dtype: every element
+// is read by the thread that later writes it.
+template <typename T, typename GT, int THREADS, int ITERS>
+__global__ __launch_bounds__(THREADS) void kl_loss_grad_kernel(const T* student,
+                                                                const T* __restrict__ teacher,
+                                                                float* __restrict__ lse_s,
+                                                                float* __restrict__ lse_t,
+                                                                float* __restrict__ row_kl,
+                                                                GT* dstudent, int v, float inv_temp,
+                                                                float mul) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int NW = THREADS / 64;
+  __shared__ float smem[5 * NW];
+  const int64_t row = blockIdx.x;
+  const T* sp_ = student + row * (int64_t)v;
+  const T* tp_ = teacher + row * (int64_t)v;
+  GT* gp = dstudent + row * (int64_t)v;
+  const RowSplit sp = split_row<EPV>(row, v, true);
+  const int tid = threadIdx.x;
+  const int ne = edge_count(sp, v);
+  const float c1 = kLog2e * inv_temp;
+
+  u32x4 rs[ITERS], rt[ITERS];
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * THREADS + tid;
+    if (c < sp.nvec) {
+      rs[i] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
+      rt[i] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
+    }
+  }
+  // the unaligned ends of the row (at most EPV - 1 elements each): thread e keeps edge e
+  int edge_at = -1;
+  float es = -INFINITY, et = -INFINITY;
+  if (tid < ne) {
+    edge_at = edge_col(sp, tid);
+    es = Elem<T>::load1(sp_ + edge_at) * c1;
+    et = Elem<T>::load1(tp_ + edge_at) * c1;
+  }
+  KLState k{fmaxf(es, kNegBig), 0.f, fmaxf(et, kNegBig), 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * THREADS + tid;
+    if (c < sp.nvec) {
+      float zs[EPV], zt[EPV];
+      Elem<T>::unpack(rs[i], zs);
+      Elem<T>::unpack(rt[i], zt);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        k.ms = fmaxf(k.ms, zs[e] * c1);
+        k.mt = fmaxf(k.mt, zt[e] * c1);
+      }
+    }
+  }
+  if (edge_at >= 0) {
+    const float w = fast_exp2(et - k.mt);
+    k.ds = fast_exp2(es - k.ms);
+    k.dt = w;
+    k.a = w * (et - es);
+  }
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * THREADS + tid;
+    if (c < sp.nvec) {
+      float zs[EPV], zt[EPV];
+      Elem<T>::unpack(rs[i], zs);
+      Elem<T>::unpack(rt[i], zt);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        const float a = zs[e] * c1, b = zt[e] * c1;
+        k.ds += fast_exp2(a - k.ms);
+        const float w = fast_exp2(b - k.mt);
+        k.dt += w;
+        k.a += w * (b - a);
+      }
+    }
+  }
+  float l2s, l2t, kl2;
+  kl_merge<NW>(k, smem, &l2s, &l2t, &kl2);
+  if (tid == 0) {
+    if (lse_s != nullptr) lse_s[row] = l2s * kLn2;
+    if (lse_t != nullptr) lse_t[row] = l2t * kLn2;
+    row_kl[row] = kl2 * kLn2;
+  }
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * THREADS + tid;
+    if (c < sp.nvec) {
+      float zs[EPV], zt[EPV], o[EPV];
+      Elem<T>::unpack(rs[i], zs);
+      Elem<T>::unpack(rt[i], zt);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e)
+        o[e] = (fast_exp2(zs[e] * c1 - l2s) - fast_exp2(zt[e] * c1 - l2t)) * mul;
+      GT* dst = gp + sp.head + (int64_t)c * EPV;
+      if constexpr (sizeof(GT) == sizeof(T)) {
+        store16_stream(dst, Elem<GT>::pack(o));
+      } else {  // fp32 gradient next to 16-bit logits: two 16-byte stores
+        static_assert(sizeof(GT) == 4 && EPV == 8, "gradient is the logits' dtype or fp32");
+        float lo[4] = {o[0], o[1], o[2], o[3]}, hi[4] = {o[4], o[5], o[6], o[7]};
+        store16_stream(dst, Elem<float>::pack(lo));
+        store16_stream(dst + 4, Elem<float>::pack(hi));
+      }
+    }
+  }
+  if (edge_at >= 0) Elem<GT>::store1(gp + edge_at, (fast_exp2(es - l2s) - fast_exp2(et - l2t)) * mul);
+}
+
 template <typename T>
 void launch_fwd(const void* s, const void* t, float* lse_s, float* lse_t, float* row_kl, int64_t n,
                 int v, float inv_temp, bool vec_ok, hipStream_t st) {
@@ -461,6 +576,81 @@ int fm_kl_bwd(const void* student, const void* teacher, const float* lse_s, cons
   else CALL(f16_t, float);
 #undef CALL
   FM_CHECK_LAUNCH("fm_kl_bwd");
+  return FM_OK;
+}
+
+int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, float* lse_t,
+                    float* row_kl, float* loss, void* dstudent, int64_t n, int64_t v, int dtype,
+                    int grad_dtype, float inv_temperature, int reduction, fm_stream_t stream) {
+  int rc = check_shape("fm_kl_loss_grad", n, v, dtype);
+  if (rc != FM_OK) return rc;
+  FM_CHECK_ARG(reduction == FM_REDUCE_SUM || reduction == FM_REDUCE_MEAN,
+               "fm_kl_loss_grad: reduction must be sum or mean (got %d)", reduction);
+  FM_CHECK_ARG(grad_dtype == dtype || grad_dtype == FM_F32,
+               "fm_kl_loss_grad: grad_dtype must equal dtype or be fp32 (dtype=%d grad_dtype=%d)", dtype,
+               grad_dtype);
+  FM_CHECK_ARG(n == 0 || (student && teacher && row_kl && dstudent), "fm_kl_loss_grad: NULL pointer");
+  FM_CHECK_ARG(dstudent != student || grad_dtype == dtype,
+               "fm_kl_loss_grad: the gradient can overwrite the student only in the student's dtype");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const float scale = (reduction == FM_REDUCE_MEAN && n > 0) ? 1.f / (float)n : 1.f;
+  const int esize = dtype == FM_F32 ? 4 : 2;
+  const int64_t nvec = v / (16 / esize);
+  const bool one_pass = n > 0 && fm_host::aligned16(student) && fm_host::aligned16(teacher) &&
+                        fm_host::aligned16(dstudent) && nvec <= kOnePassMaxVec;
+  if (!one_pass) {
+    if (n > 0 && dstudent == student) {
+      fm_host::set_error("fm_kl_loss_grad: the gradient can overwrite the student only for aligned rows "
+                         "of at most %d bytes", kOnePassMaxVec * 16);
+      return FM_ERR_UNSUPPORTED;
+    }
+    if (n > 0 && (lse_s == nullptr || lse_t == nullptr)) {
+      fm_host::set_error("fm_kl_loss_grad: lse_s and lse_t are required for rows of more than %d bytes or "
+                         "unaligned buffers", kOnePassMaxVec * 16);
+      return FM_ERR_INVALID;
+    }
+    rc = fm_kl_fwd(student, teacher, lse_s, lse_t, row_kl, loss, n, v, dtype, inv_temperature, reduction,
+                   stream);
+    if (rc != FM_OK) return rc;
+    return fm_kl_bwd(student, teacher, lse_s, lse_t, nullptr, 0, dstudent, n, v, dtype, grad_dtype,
+                     inv_temperature, scale, stream);
+  }
+  // the fewest threads that hold both rows in at most 4 vectors each per thread
+  int threads = 256;
+  while (threads < 1024 && nvec > (int64_t)threads * 4) threads *= 2;
+  int iters = 1;
+  while ((int64_t)threads * iters < nvec) iters *= 2;
+  const float mul = inv_temperature * scale;
+  const dim3 grid((unsigned)n);
+#define LAUNCH(T, GT, TH, IT)                                                                      \
+  hipLaunchKernelGGL((kl_loss_grad_kernel<T, GT, TH, IT>), grid, dim3(TH), 0, st,                  \
+                     static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t, \
+                     row_kl, static_cast<GT*>(dstudent), (int)v, inv_temperature, mul)
+#define BY_ITERS(T, GT, TH)                       \
+  do {                                            \
+    if (iters == 1) LAUNCH(T, GT, TH, 1);         \
+    else if (iters == 2) LAUNCH(T, GT, TH, 2);    \
+    else LAUNCH(T, GT, TH, 4);                    \
+  } while (0)
+#define BY_SHAPE(T, GT)                               \
+  do {                                                \
+    if (threads == 256) BY_ITERS(T, GT, 256);         \
+    else if (threads == 512) BY_ITERS(T, GT, 512);    \
+    else BY_ITERS(T, GT, 1024);                       \
+  } while (0)
+  if (dtype == FM_F32) BY_SHAPE(float, float);
+  else if (dtype == FM_BF16 && grad_dtype == FM_BF16) BY_SHAPE(bf16_t, bf16_t);
+  else if (dtype == FM_BF16) BY_SHAPE(bf16_t, float);
+  else if (grad_dtype == FM_F16) BY_SHAPE(f16_t, f16_t);
+  else BY_SHAPE(f16_t, float);
+#undef BY_SHAPE
+#undef BY_ITERS
+#undef LAUNCH
+  FM_CHECK_LAUNCH("fm_kl_loss_grad");
+  if (loss != nullptr) {
+    hipLaunchKernelGGL(kl_finalize_kernel, dim3(1), dim3(1024), 0, st, row_kl, n, scale, loss);
+    FM_CHECK_LAUNCH("fm_kl_loss_grad(finalize)");
+  }
   return FM_OK;
 }
 

@@ -2,9 +2,12 @@
 
 Call surface of the reference's ``forgemind/kernels/kl.py:194-238``. The reference kernel
 writes dKL/dlogits during the forward and multiplies it by the upstream gradient in the
-backward (``kl.py:143-191``); here the forward is a single pass that keeps only the two
-per-row log-sum-exps, and the backward recomputes both softmaxes -- one pass fewer over the
-``[N, V]`` tensors and no ``[N, V]`` buffer held between forward and backward.
+backward (``kl.py:143-191``). Here rows of up to 64 KiB do the same from ONE read of both
+tensors (they stay in registers between the log-sum-exps and the gradient store) and the
+backward's multiply is skipped on the device when the upstream gradient is 1. Wider rows, and
+``reduction="none"``, keep a single-pass forward that saves only the two per-row
+log-sum-exps and a backward that recomputes both softmaxes: no ``[N, V]`` buffer is held
+between forward and backward.
 
 ``temperature`` (not in the reference) divides both logit tensors before the softmax; the
 gradient is wrt the undivided student logits, with no T**2 factor.
@@ -23,27 +26,46 @@ _REDUCTIONS = ("mean", "sum", "none")
 
 class _KLDivFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, student, teacher, reduction, grad_dtype, temperature):
+    def forward(ctx, student, teacher, reduction, grad_dtype, temperature, reuse):
         v = student.shape[-1]
         s2 = student.contiguous().view(-1, v)
         t2 = teacher.contiguous().view(-1, v)
         inv_t = 1.0 / float(temperature)
+        gdt = grad_dtype or student.dtype
+        ctx.meta = (student.shape, reduction, gdt, inv_t)
+        ctx.in_forward = False
+        ctx.spent = False
+        if reduction != "none" and ctx.needs_input_grad[0]:
+            # gradient written in the forward (reference kl.py:143-176); `reuse` lets it land in
+            # the student's own storage when that is the tensor the caller handed in
+            own = reuse and s2.data_ptr() == student.data_ptr()
+            loss, grad, _rows = _hip.kl_loss_grad(s2.detach(), t2, inv_t, reduction, gdt, own)
+            ctx.in_forward = True
+            ctx.save_for_backward(grad)
+            return loss
         loss, rows, lse_s, lse_t = _hip.kl_fwd(s2, t2, inv_t, reduction)
         ctx.save_for_backward(s2, t2, lse_s, lse_t)
-        ctx.meta = (student.shape, reduction, grad_dtype or student.dtype, inv_t)
         if reduction == "none":
             return rows.clone().view(student.shape[:-1])
         return loss
 
     @staticmethod
     def backward(ctx, g):
-        s2, t2, lse_s, lse_t = ctx.saved_tensors
         shape, reduction, gdt, inv_t = ctx.meta
+        if ctx.in_forward:
+            (grad,) = ctx.saved_tensors
+            if ctx.spent:
+                raise RuntimeError("kl_div_logits: the gradient buffer written in the forward was "
+                                   "already consumed by a backward pass; run the forward again")
+            ctx.spent = True
+            _hip.scale_inplace(grad, g.detach().to(torch.float32).contiguous())
+            return grad.view(shape), None, None, None, None, None
+        s2, t2, lse_s, lse_t = ctx.saved_tensors
         n = s2.shape[0]
         g32 = g.detach().to(torch.float32).contiguous().view(-1)
         scale = 1.0 / n if reduction == "mean" else 1.0
         grad = _hip.kl_bwd(s2, t2, lse_s, lse_t, g32, reduction == "none", gdt, inv_t, scale)
-        return grad.view(shape), None, None, None, None
+        return grad.view(shape), None, None, None, None, None
 
 
 class _KLDivTopkFn(torch.autograd.Function):
@@ -92,13 +114,14 @@ def _kernel_ok(*tensors) -> bool:
 
 def kl_div_logits(student: torch.Tensor, teacher: torch.Tensor, reduction: str = "mean",
                   grad_dtype: "torch.dtype | None" = None,
-                  temperature: float = 1.0) -> torch.Tensor:
+                  temperature: float = 1.0, reuse: bool = False) -> torch.Tensor:
     """``KL(softmax(teacher / T) || softmax(student / T))`` over the last dim.
 
     ``mean`` divides by the number of rows (there is no ignore mask, reference
     ``_fallback.py:64-67``); ``none`` returns the per-row values. The teacher is a constant.
     ``grad_dtype`` (the student's dtype by default, or ``torch.float32``) is the dtype the
-    kernel writes the student gradient in.
+    kernel writes the student gradient in. ``reuse=True`` (reference ``kl.py:146-150``) lets
+    the gradient overwrite ``student``: only for a tensor the caller owns and no longer reads.
     """
     if reduction not in _REDUCTIONS:
         raise ValueError(f"reduction must be mean|sum|none, got {reduction!r}")
@@ -111,7 +134,7 @@ def kl_div_logits(student: torch.Tensor, teacher: torch.Tensor, reduction: str =
         return fb.kl_div_logits(student, teacher, reduction, temperature)
     if not _kernel_ok(student, teacher):
         return fb.kl_div_logits(student, teacher, reduction, temperature)
-    return _KLDivFn.apply(student, teacher, reduction, grad_dtype, float(temperature))
+    return _KLDivFn.apply(student, teacher, reduction, grad_dtype, float(temperature), bool(reuse))
 
 
 def kl_div_logits_topk(student: torch.Tensor, teacher: torch.Tensor, k: int,
@@ -154,8 +177,8 @@ def kl_distill_loss(hs: torch.Tensor, ht: torch.Tensor, w: torch.Tensor, teacher
     """Mean forward KL of ``softmax(teacher_head(ht)) || softmax(hs @ w.T)`` in row chunks.
 
     Same structure as the reference's ``kl.py:209-233``: the teacher head runs under
-    ``no_grad``; one chunk of student logits exists at a time in the forward. The chunk's
-    logits (not its gradient) are what is kept for the backward.
+    ``no_grad``; one chunk of student logits exists at a time in the forward, and its gradient
+    is written over it (``reuse=True``, as in the reference) when the rows are narrow enough.
     """
     hs2 = hs.reshape(-1, hs.shape[-1])
     ht2 = ht.reshape(-1, ht.shape[-1])
@@ -166,7 +189,8 @@ def kl_distill_loss(hs: torch.Tensor, ht: torch.Tensor, w: torch.Tensor, teacher
         with torch.no_grad():
             t_log = teacher_head(ht2[lo:hi]).detach()
         s_log = hs2[lo:hi] @ w.t()
-        piece = kl_div_logits(s_log, t_log.to(s_log.dtype), "sum")
+        # the chunk's student logits are a temporary of this loop: the gradient may overwrite them
+        piece = kl_div_logits(s_log, t_log.to(s_log.dtype), "sum", reuse=True)
         total = piece if total is None else total + piece
     if total is None:
         return hs2.new_zeros((), dtype=torch.float32)

@@ -194,6 +194,31 @@ def test_cross_entropy_autograd_and_callers():
     assert z.item() == 0.0 and h2.grad is not None and not h2.grad.any()
 
 
+def test_kl_gradient_in_forward_reuse_and_second_backward():
+    g = torch.Generator().manual_seed(41)
+    s = (3 * torch.randn(12, 3000, generator=g)).bfloat16()
+    t = (s.float() + 0.5 * torch.randn(12, 3000, generator=g)).bfloat16()
+    _, og = O.kl_div(s, t, "mean", 1.0)
+    leaf = s.to(DEV).requires_grad_(True)
+    tmp = leaf * 1.0                                   # a temporary that only the loss reads
+    loss = kernels.kl_div_logits(tmp, t.to(DEV), reuse=True)
+    (loss * 2.0).backward(retain_graph=True)
+    assert close(leaf.grad, og.float() * 2.0)
+    with pytest.raises(RuntimeError, match="already consumed"):
+        loss.backward()
+    # distillation loop: chunk logits overwritten by their gradient, both operands train
+    hs = torch.randn(40, 32, generator=g).to(DEV).requires_grad_(True)
+    w = torch.randn(700, 32, generator=g).to(DEV).requires_grad_(True)
+    ht = torch.randn(40, 32, generator=g).to(DEV)
+    head = nn.Linear(32, 700, bias=False).to(DEV)
+    out = kernels.kl_distill_loss(hs, ht, w, head, chunk=16)
+    out.backward()
+    ref = F.kl_div(torch.log_softmax(hs.detach() @ w.detach().t(), -1), torch.softmax(head(ht).detach(), -1),
+                   reduction="sum") / 40
+    assert out.item() == pytest.approx(ref.item(), rel=1e-4)
+    assert hs.grad is not None and w.grad is not None and hs.grad.abs().sum() > 0
+
+
 def test_kl_autograd_reductions_and_temperature():
     g = torch.Generator().manual_seed(4)
     s = (3 * torch.randn(20, 3000, generator=g)).bfloat16()

@@ -210,7 +210,8 @@ def test_ce_loss_and_gradient_in_one_pass(n, v, dt, reduction):
     # the same call writing over the logits gives the same bits
     loss2, dl2, _, _ = _hip.ce_loss_grad(lgd, yd, -100, reduction, inplace=True)
     torch.cuda.synchronize()
-    assert dl2.data_ptr() == lgd.data_ptr()
+    wide = v * lg.element_size() > 8 * 1024 * 16        # such rows get a buffer of their own
+    assert (dl2.data_ptr() == lgd.data_ptr()) == (not wide)
     assert torch.equal(dl2, dl) and loss2.item() == loss.item()
     # and it agrees with the two-pass kernels to the last bit of the loss and a rounding of the grad
     loss3, lse, nv3, _ = _hip.ce_fwd(keep, yd, -100, reduction)
@@ -292,6 +293,43 @@ def test_kl_fwd_bwd(n, v, dt, T):
     want = g_none * up[:, None]
     tol = (1e-2 if dt != F32 else 1e-4) * want.abs().max().item() + 1e-6 / T
     assert (gs32.cpu() - want).abs().max().item() <= tol
+
+
+KL1_CASES = [(64, 32000, BF16, 2.0, BF16), (6, 5000, F32, 1.0, F32), (3, 1, F32, 1.0, F32),
+             (5, 32768, BF16, 1.0, F32), (4, 7, F32, 1.0, F32), (9, 32000, F16, 1.5, F16),
+             (7, 4099, BF16, 1.0, BF16), (3, 50257, BF16, 1.0, BF16), (4, 16000, F32, 4.0, F32),
+             (5, 600, F16, 1.0, F32), (6, 2048, BF16, 2.0, BF16)]
+
+
+@pytest.mark.parametrize("n,v,dt,T,gdt", KL1_CASES)
+@pytest.mark.parametrize("reduction", ["mean", "sum"])
+def test_kl_loss_and_gradient_in_one_pass(n, v, dt, T, gdt, reduction):
+    g = gen(1025)
+    s = (3 * torch.randn(n, v, generator=g)).to(dt)
+    t = (s.float() + 0.5 * torch.randn(n, v, generator=g)).to(dt)
+    o64, _ = O.kl_div(s, t, reduction, T, acc=torch.float64)
+    orow, _ = O.kl_div(s, t, "none", T, acc=torch.float64)
+    _, ograd = O.kl_div(s.float() if gdt == F32 else s, t.float() if gdt == F32 else t, reduction, T)
+    sd, td = s.to(DEV), t.to(DEV)
+    keep = sd.clone()
+    loss, grad, rows = _hip.kl_loss_grad(sd, td, 1.0 / T, reduction, gdt)
+    torch.cuda.synchronize()
+    assert torch.equal(sd, keep) and grad.dtype == gdt
+    assert loss.item() == pytest.approx(o64.item(), rel=1e-4, abs=2e-6 if reduction == "sum" else 2e-7)
+    assert torch.allclose(rows.cpu().double(), orow, rtol=2e-4, atol=2e-6)
+    cancel = 1.0 / (T * n) if reduction == "mean" else 1.0 / T
+    assert_close_lowp(grad, ograd.float(), gdt, "dstudent", ulps=3.0, cancel=cancel)
+    # against the two-pass kernels
+    loss2, rows2, ls, lt = _hip.kl_fwd(sd, td, 1.0 / T, reduction)
+    g2 = _hip.kl_bwd(sd, td, ls, lt, None, False, gdt, 1.0 / T, 1.0 / n if reduction == "mean" else 1.0)
+    assert loss2.item() == pytest.approx(loss.item(), rel=2e-5, abs=1e-7)
+    assert_close_lowp(grad, g2.float().cpu(), gdt, "vs two-pass", ulps=2.0, cancel=cancel)
+    # written over the student when the dtypes agree and the row fits the register file
+    loss3, g3, _ = _hip.kl_loss_grad(sd, td, 1.0 / T, reduction, gdt, inplace=True)
+    torch.cuda.synchronize()
+    fits = v * s.element_size() <= 4096 * 16
+    assert (g3.data_ptr() == sd.data_ptr()) == (fits and gdt == dt)
+    assert torch.equal(g3, grad) and loss3.item() == loss.item()
 
 
 def test_kl_known_answers_on_gpu():
