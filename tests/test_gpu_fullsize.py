@@ -59,6 +59,12 @@ def test_config2_cross_entropy_8192x32000():
     sums = dl[~ign].float().sum(-1)
     assert sums.abs().max().item() < 0.05 / n_all             # softmax - onehot sums to zero per row
     assert nv.item() == n_all
+    # loss and gradient from one read of the logits: same loss, the same gradient up to a rounding
+    loss1, dl1, nv1, _ = _hip.ce_loss_grad(lgd, yd, -100, "mean")
+    assert nv1.item() == n_all and loss1.item() == pytest.approx(loss.item(), rel=1e-6)
+    assert not dl1[ign].any()
+    assert lowp_close(dl1, dl, 2.0, cancel=1.0 / n_all)
+    assert dl1[~ign].float().sum(-1).abs().max().item() < 0.05 / n_all
 
 
 def test_config3_router_16384x64():
@@ -147,3 +153,11 @@ def test_config5_kl_and_topk_4096x128256():
         first_left = torch.where(left, pos, torch.full_like(pos, v)).min(-1).values
         last_taken = torch.where(chosen & (xf == k_lo), pos, torch.full_like(pos, -1)).max(-1).values
         assert (last_taken < first_left).all()                 # ... all sit after the taken ones
+    # the KL forward that selects the teacher's top-64 in the same pass: identical selection
+    out = _hip.kl_fwd_topk(sd, td, 64, 1.0 / T, "mean", torch.int32, want_values=True, want_probs=True)
+    loss_f, rows_f, ls_f, lt_f, vals_f, idx_f, probs_f = out
+    assert torch.equal(idx_f, idx) and torch.equal(vals_f, vals)
+    assert loss_f.item() == pytest.approx(loss.item(), rel=1e-5)
+    assert torch.allclose(rows_f, rows, rtol=2e-4, atol=1e-7) and torch.allclose(lt_f, lt, rtol=1e-6, atol=2e-6)
+    want = torch.exp(vals.double() / T - lt.double()[:, None])
+    assert torch.allclose(probs_f.double(), want, rtol=1e-5, atol=1e-12)
