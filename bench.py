@@ -49,7 +49,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="ce",
-                    choices=["ce", "ce_one_pass", "rmsnorm", "add_rmsnorm", "kl", "kl_topk", "topk", "route", "moe_dispatch"])
+                    choices=["ce", "ce_one_pass", "rmsnorm", "add_rmsnorm", "add_layernorm", "kl", "kl_topk", "topk", "route", "moe_dispatch"])
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
@@ -163,6 +163,44 @@ def make_workload(name, torch, L, dev):
         w.dominant_bytes = n * d * 8
         w.bytes = n * d * 16
         w.desc = f"add-RMSNorm fwd+bwd x,delta bf16 [{n},{d}], w fp32, eps 1e-5, with residual grad"
+        w.rows = n
+        return w
+
+    if name == "add_layernorm":
+        n, d = 16384, 8192
+        g.manual_seed(1034)
+        x = torch.randn(n, d, device=dev, generator=g).bfloat16()
+        dl = torch.randn(n, d, device=dev, generator=g).bfloat16()
+        gy = torch.randn(n, d, device=dev, generator=g).bfloat16()
+        gxn = torch.randn(n, d, device=dev, generator=g).bfloat16()
+        wt = (1 + 0.02 * torch.randn(d, device=dev, generator=g))
+        bs = 0.1 * torch.randn(d, device=dev, generator=g)
+        xn, y, dx = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+        mean, rstd = torch.empty(n, device=dev), torch.empty(n, device=dev)
+        dw, db = torch.empty_like(wt), torch.empty_like(wt)
+        nb = L.fm_layernorm_bwd_workspace(n, d, BF)
+        ws = torch.empty(nb, device=dev, dtype=torch.uint8)
+
+        def fwd():
+            _check(L.fm_add_layernorm_fwd(x.data_ptr(), dl.data_ptr(), wt.data_ptr(), bs.data_ptr(),
+                                          xn.data_ptr(), y.data_ptr(), mean.data_ptr(), rstd.data_ptr(), n, d,
+                                          BF, F32c, 1e-5, st), "fm_add_layernorm_fwd")
+
+        def bwd():
+            _check(L.fm_layernorm_bwd(xn.data_ptr(), wt.data_ptr(), mean.data_ptr(), rstd.data_ptr(),
+                                      gy.data_ptr(), gxn.data_ptr(), dx.data_ptr(), dw.data_ptr(), db.data_ptr(),
+                                      ws.data_ptr(), nb, n, d, BF, F32c, st), "fm_layernorm_bwd")
+
+        def step():
+            fwd()
+            bwd()
+
+        w.step = step
+        w.dominant_launch = bwd
+        w.dominant = "norm_bwd_kernel<bf16,f32,512,2,LN> + 2 colsum_kernel"
+        w.dominant_bytes = n * d * 8
+        w.bytes = n * d * 16
+        w.desc = f"add-LayerNorm fwd+bwd x,delta bf16 [{n},{d}], w,b fp32, eps 1e-5, with residual grad"
         w.rows = n
         return w
 
@@ -518,7 +556,7 @@ def main():
     torch.cuda.empty_cache()
     if not a.no_extras:
         extras = {a.workload: res}
-        for name in ["rmsnorm", "add_rmsnorm", "ce", "ce_one_pass", "kl", "kl_topk", "topk", "route", "moe_dispatch"]:
+        for name in ["rmsnorm", "add_rmsnorm", "add_layernorm", "ce", "ce_one_pass", "kl", "kl_topk", "topk", "route", "moe_dispatch"]:
             if name == a.workload:
                 continue
             wl = make_workload(name, torch, L, dev)

@@ -2,631 +2,41 @@
 //
 // Reference semantics: forgemind/kernels/_fallback.py:26-35 (forward, rounding points),
 // forgemind/kernels/norm.py:179-231 (backward row math), norm.py:571-593 (fixed-order
-// column sum of the fp32 weight-gradient partials).
-//
-// Layout: rows are dense, row-major. A row is owned by TPR threads (a lane group, a wave or
-// several waves of one workgroup); each thread keeps ITERS 16-byte vectors of the row in
-// registers between the reduction and the store, so every tensor is read exactly once.
-// The backward is persistent: a fixed grid walks the row tiles, each thread accumulates its
-// columns of dW in fp32 registers, the workgroup folds its rows through LDS and writes one
-// partial row; a second kernel sums the partial rows in a fixed order.
-#include "fm_common.cuh"
-
-using namespace fm;
-
-namespace {
-
-constexpr int kMinBlock = 256;
-// The backward always runs 16-wave workgroups: many rows per workgroup are folded through
-// LDS, so the number of fp32 partial rows (one per workgroup) stays at the CU count while
-// each SIMD still has four waves to hide load latency.
-constexpr int kBwdBlock = 1024;
-
-template <int TPR> struct BlockOf { static constexpr int value = TPR > kMinBlock ? TPR : kMinBlock; };
-
-// Load the EPV weights that line up with one 16-byte vector of the activations.
-template <typename T, typename WT>
-__device__ __forceinline__ void load_w(const WT* w, int col, float (&o)[Elem<T>::kVec]) {
-  constexpr int EPV = Elem<T>::kVec;
-  if constexpr (sizeof(WT) == sizeof(T)) {
-    Elem<WT>::unpack(load16(w + col), o);
-  } else {  // fp32 weights next to 16-bit activations: two 16-byte loads
-    static_assert(sizeof(WT) == 4 && EPV == 8, "weights are either x's dtype or fp32");
-    float a[4], b[4];
-    Elem<float>::unpack(load16(w + col), a);
-    Elem<float>::unpack(load16(w + col + 4), b);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) { o[i] = a[i]; o[4 + i] = b[i]; }
-  }
-}
-
-// ---------------------------------------------------------------- forward (vector path)
-template <typename T, typename WT, int TPR, int ITERS, bool ADD>
-__global__ __launch_bounds__(BlockOf<TPR>::value) void norm_fwd_kernel(
-    const T* __restrict__ x, const T* __restrict__ delta, const WT* __restrict__ w,
-    T* __restrict__ xn, T* __restrict__ y, float* __restrict__ rstd, int64_t n, int d, float eps) {
-  constexpr int EPV = Elem<T>::kVec;
-  constexpr int BLOCK = BlockOf<TPR>::value;
-  constexpr int RPB = BLOCK / TPR;
-  __shared__ float smem[RPB * (TPR > 64 ? TPR / 64 : 1)];
-
-  const int tid = threadIdx.x;
-  const int rib = tid / TPR;
-  const int t = tid % TPR;
-  const int64_t row = (int64_t)blockIdx.x * RPB + rib;
-  const bool valid = row < n;
-  const int nvec = d / EPV;
-  const int64_t base = row * (int64_t)d;
-
-  float v[ITERS][EPV];
-  float ss = 0.f;
-#pragma unroll
-  for (int i = 0; i < ITERS; ++i) {
-    const int c = i * TPR + t;
-    if (valid && c < nvec) {
-      u32x4 rx = load16_stream(x + base + (int64_t)c * EPV);
-      Elem<T>::unpack(rx, v[i]);
-      if constexpr (ADD) {
-        float dv[EPV];
-        Elem<T>::unpack(load16_stream(delta + base + (int64_t)c * EPV), dv);
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) v[i][e] += dv[e];
-        // statistics come from the value a tensor add would have stored
-        u32x4 packed = Elem<T>::pack(v[i]);
-        store16(xn + base + (int64_t)c * EPV, packed);
-        Elem<T>::unpack(packed, v[i]);
-      }
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) ss += v[i][e] * v[i][e];
-    } else {
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) v[i][e] = 0.f;
-    }
-  }
-  ss = row_reduce<TPR, OpSum>(ss, smem, rib, t);
-  const float r = rsqrtf(ss / (float)d + eps);
-  if (valid && t == 0) rstd[row] = r;
-#pragma unroll
-  for (int i = 0; i < ITERS; ++i) {
-    const int c = i * TPR + t;
-    if (valid && c < nvec) {
-      float wv[EPV], o[EPV];
-      load_w<T, WT>(w, c * EPV, wv);
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) o[e] = (v[i][e] * r) * wv[e];
-      store16_stream(y + base + (int64_t)c * EPV, Elem<T>::pack(o));
-    }
-  }
-}
-
-// ---------------------------------------------------------------- backward (vector path)
-// grid-persistent; `partial` is [gridDim.x, d] fp32 (or NULL when dW is not wanted).
-template <typename T, typename WT, int TPR, int ITERS>
-__global__ __launch_bounds__(kBwdBlock) void norm_bwd_kernel(
-    const T* __restrict__ x, const WT* __restrict__ w, const float* __restrict__ rstd,
-    const T* __restrict__ dy, const T* __restrict__ gxn, T* __restrict__ dx,
-    T* __restrict__ dd, float* __restrict__ partial, int64_t n, int d, int64_t tiles) {
-  constexpr int EPV = Elem<T>::kVec;
-  constexpr int BLOCK = kBwdBlock;
-  constexpr int RPB = BLOCK / TPR;
-  constexpr int COVER = TPR * ITERS * EPV;   // columns covered by one row's threads
-  __shared__ float red[RPB * (TPR > 64 ? TPR / 64 : 1)];
-  __shared__ float fold[RPB > 1 ? RPB * COVER : 1];
-
-  const int tid = threadIdx.x;
-  const int rib = tid / TPR;
-  const int t = tid % TPR;
-  const int nvec = d / EPV;
-  const float inv_d = 1.f / (float)d;
-
-  float wv[ITERS][EPV];
-  float acc[ITERS][EPV];
-#pragma unroll
-  for (int i = 0; i < ITERS; ++i) {
-    const int c = i * TPR + t;
-    if (c < nvec) {
-      load_w<T, WT>(w, c * EPV, wv[i]);
-    } else {
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) wv[i][e] = 0.f;
-    }
-#pragma unroll
-    for (int e = 0; e < EPV; ++e) acc[i][e] = 0.f;
-  }
-
-  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-    const int64_t row = tile * RPB + rib;
-    const bool valid = row < n;
-    const int64_t base = row * (int64_t)d;
-    // x and dy stay packed in registers between the two sweeps (half the footprint of fp32)
-    u32x4 rx[ITERS], rg[ITERS];
-    const float r = valid ? rstd[row] : 0.f;
-    float dot = 0.f;
-#pragma unroll
-    for (int i = 0; i < ITERS; ++i) {
-      const int c = i * TPR + t;
-      if (valid && c < nvec) {
-        rx[i] = load16_stream(x + base + (int64_t)c * EPV);
-        rg[i] = load16_stream(dy + base + (int64_t)c * EPV);
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < ITERS; ++i) {
-      const int c = i * TPR + t;
-      if (valid && c < nvec) {
-        float xv[EPV], gv[EPV];
-        Elem<T>::unpack(rx[i], xv);
-        Elem<T>::unpack(rg[i], gv);
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) {
-          const float xh = xv[e] * r;
-          acc[i][e] += gv[e] * xh;
-          dot += (gv[e] * wv[i][e]) * xh;
-        }
-      }
-    }
-    dot = row_reduce<TPR, OpSum>(dot, red, rib, t);
-    const float cmean = dot * inv_d;
-#pragma unroll
-    for (int i = 0; i < ITERS; ++i) {
-      const int c = i * TPR + t;
-      if (valid && c < nvec) {
-        float xv[EPV], gv[EPV], o[EPV];
-        Elem<T>::unpack(rx[i], xv);
-        Elem<T>::unpack(rg[i], gv);
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) o[e] = (gv[e] * wv[i][e] - (xv[e] * r) * cmean) * r;
-        if (gxn != nullptr) {
-          float rv[EPV];
-          Elem<T>::unpack(load16_stream(gxn + base + (int64_t)c * EPV), rv);
-#pragma unroll
-          for (int e = 0; e < EPV; ++e) o[e] += rv[e];
-        }
-        const u32x4 packed = Elem<T>::pack(o);
-        store16_stream(dx + base + (int64_t)c * EPV, packed);
-        if (dd != nullptr) store16_stream(dd + base + (int64_t)c * EPV, packed);
-      }
-    }
-  }
-
-  if (partial == nullptr) return;
-  float* prow = partial + (int64_t)blockIdx.x * d;
-  if constexpr (RPB == 1) {
-#pragma unroll
-    for (int i = 0; i < ITERS; ++i) {
-      const int c = i * TPR + t;
-      if (c < nvec) {
-#pragma unroll
-        for (int q = 0; q < EPV / 4; ++q) {
-          float o4[4] = {acc[i][4 * q], acc[i][4 * q + 1], acc[i][4 * q + 2], acc[i][4 * q + 3]};
-          store16(prow + c * EPV + 4 * q, Elem<float>::pack(o4));
-        }
-      }
-    }
-  } else {
-    // fold the RPB rows of this workgroup in row order, then write one partial row
-#pragma unroll
-    for (int i = 0; i < ITERS; ++i) {
-      const int c = i * TPR + t;
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) fold[rib * COVER + c * EPV + e] = acc[i][e];
-    }
-    __syncthreads();
-    for (int j = tid; j < d; j += BLOCK) {
-      float s = fold[j];
-#pragma unroll
-      for (int rr = 1; rr < RPB; ++rr) s += fold[rr * COVER + j];
-      prow[j] = s;
-    }
-  }
-}
-
-// Column sum of `p` partial rows, [p, d] fp32 -> dw[d] in WT. One workgroup owns 64 columns
-// as 16 quads; thread (g, q) adds rows g, g+64, ... of quad q with 16-byte loads, then the 64
-// row-group results are added in group order. The order depends only on (p, d), never on
-// timing. Requires d % 4 == 0 (the register path guarantees it); otherwise colsum_scalar.
-template <typename WT>
-__global__ __launch_bounds__(1024) void colsum_kernel(const float* __restrict__ partial,
-                                                       WT* __restrict__ dw, int p, int d) {
-  __shared__ float s[64][64 + 4];
-  const int q = threadIdx.x & 15;
-  const int g = threadIdx.x >> 4;
-  const int col = blockIdx.x * 64 + q * 4;
-  float a[4] = {0.f, 0.f, 0.f, 0.f};
-  if (col < d) {
-    int r = g;
-    for (; r + 192 < p; r += 256) {
-      float v[4][4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) Elem<float>::unpack(load16(partial + (int64_t)(r + 64 * u) * d + col), v[u]);
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) a[c] += v[u][c];
-      }
-    }
-    for (; r < p; r += 64) {
-      float v[4];
-      Elem<float>::unpack(load16(partial + (int64_t)r * d + col), v);
-#pragma unroll
-      for (int c = 0; c < 4; ++c) a[c] += v[c];
-    }
-  }
-#pragma unroll
-  for (int c = 0; c < 4; ++c) s[g][q * 4 + c] = a[c];
-  __syncthreads();
-  if (threadIdx.x < 64) {
-    const int cc = blockIdx.x * 64 + threadIdx.x;
-    if (cc < d) {
-      float tot = s[0][threadIdx.x];
-#pragma unroll 8
-      for (int i = 1; i < 64; ++i) tot += s[i][threadIdx.x];
-      Elem<WT>::store1(dw + cc, tot);
-    }
-  }
-}
-
-template <typename WT>
-__global__ __launch_bounds__(1024) void colsum_scalar_kernel(const float* __restrict__ partial,
-                                                              WT* __restrict__ dw, int p, int d) {
-  __shared__ float s[16][64];
-  const int lane = threadIdx.x & 63;
-  const int g = threadIdx.x >> 6;
-  const int col = blockIdx.x * 64 + lane;
-  float a = 0.f;
-  if (col < d) {
-    for (int r = g; r < p; r += 16) a += partial[(int64_t)r * d + col];
-  }
-  s[g][lane] = a;
-  __syncthreads();
-  if (g == 0 && col < d) {
-    float tot = s[0][lane];
-#pragma unroll
-    for (int i = 1; i < 16; ++i) tot += s[i][lane];
-    Elem<WT>::store1(dw + col, tot);
-  }
-}
-
-// ---------------------------------------------------------------- any-width path
-// One 256-thread workgroup per row, two passes over the row (the second one hits cache).
-// Used when d is not a multiple of the 16-byte vector width, a pointer is not 16-byte
-// aligned, or the row is wider than the register path covers.
-template <typename T, typename WT, bool ADD>
-__global__ __launch_bounds__(256) void norm_fwd_generic(
-    const T* __restrict__ x, const T* __restrict__ delta, const WT* __restrict__ w,
-    T* __restrict__ xn, T* __restrict__ y, float* __restrict__ rstd, int64_t d, float eps) {
-  __shared__ float smem[4];
-  const int64_t base = (int64_t)blockIdx.x * d;
-  float ss = 0.f;
-  for (int64_t j = threadIdx.x; j < d; j += 256) {
-    float v = Elem<T>::load1(x + base + j);
-    if constexpr (ADD) {
-      v = Elem<T>::round(v + Elem<T>::load1(delta + base + j));
-      Elem<T>::store1(xn + base + j, v);
-    }
-    ss += v * v;
-  }
-  ss = row_reduce<256, OpSum>(ss, smem, 0, threadIdx.x);
-  const float r = rsqrtf(ss / (float)d + eps);
-  if (threadIdx.x == 0) rstd[blockIdx.x] = r;
-  for (int64_t j = threadIdx.x; j < d; j += 256) {
-    float v;
-    if constexpr (ADD) {
-      v = Elem<T>::round(Elem<T>::load1(x + base + j) + Elem<T>::load1(delta + base + j));
-    } else {
-      v = Elem<T>::load1(x + base + j);
-    }
-    Elem<T>::store1(y + base + j, (v * r) * Elem<WT>::load1(w + j));
-  }
-}
-
-template <typename T, typename WT>
-__global__ __launch_bounds__(256) void norm_bwd_generic(
-    const T* __restrict__ x, const WT* __restrict__ w, const float* __restrict__ rstd,
-    const T* __restrict__ dy, const T* __restrict__ gxn, T* __restrict__ dx,
-    T* __restrict__ dd, int64_t d) {
-  __shared__ float smem[4];
-  const int64_t base = (int64_t)blockIdx.x * d;
-  const float r = rstd[blockIdx.x];
-  float dot = 0.f;
-  for (int64_t j = threadIdx.x; j < d; j += 256) {
-    const float xh = Elem<T>::load1(x + base + j) * r;
-    dot += (Elem<T>::load1(dy + base + j) * Elem<WT>::load1(w + j)) * xh;
-  }
-  dot = row_reduce<256, OpSum>(dot, smem, 0, threadIdx.x);
-  const float cmean = dot / (float)d;
-  for (int64_t j = threadIdx.x; j < d; j += 256) {
-    const float xh = Elem<T>::load1(x + base + j) * r;
-    const float g = Elem<T>::load1(dy + base + j) * Elem<WT>::load1(w + j);
-    float o = (g - xh * cmean) * r;
-    if (gxn != nullptr) o += Elem<T>::load1(gxn + base + j);
-    Elem<T>::store1(dx + base + j, o);
-    if (dd != nullptr) Elem<T>::store1(dd + base + j, o);
-  }
-}
-
-// dW partials for the any-width path: grid (ceil(d/64), chunks); chunk c owns rows
-// [c*rows_per_chunk, ...); 4 row lanes x 64 columns per workgroup.
-template <typename T>
-__global__ __launch_bounds__(256) void dw_generic(const T* __restrict__ x,
-                                                   const float* __restrict__ rstd,
-                                                   const T* __restrict__ dy,
-                                                   float* __restrict__ partial, int64_t n,
-                                                   int64_t d, int64_t rows_per_chunk) {
-  __shared__ float s[4][64];
-  const int lane = threadIdx.x & 63;
-  const int g = threadIdx.x >> 6;
-  const int64_t col = (int64_t)blockIdx.x * 64 + lane;
-  const int64_t r0 = (int64_t)blockIdx.y * rows_per_chunk;
-  const int64_t r1 = (r0 + rows_per_chunk < n) ? r0 + rows_per_chunk : n;
-  float a = 0.f;
-  if (col < d) {
-    for (int64_t r = r0 + g; r < r1; r += 4) {
-      a += Elem<T>::load1(dy + r * d + col) * (Elem<T>::load1(x + r * d + col) * rstd[r]);
-    }
-  }
-  s[g][lane] = a;
-  __syncthreads();
-  if (g == 0 && col < d) {
-    partial[(int64_t)blockIdx.y * d + col] = (s[0][lane] + s[1][lane]) + (s[2][lane] + s[3][lane]);
-  }
-}
-
-__global__ void zero_u16_kernel(uint16_t* p, int64_t n) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) p[i] = 0;
-}
-
-// ---------------------------------------------------------------- host: plan + dispatch
-struct Plan {
-  bool vec;        // register-resident vector path
-  int tpr, iters;  // threads per row, 16-byte vectors per thread
-  int rpb;         // rows per workgroup
-  int64_t tiles;   // row tiles of the forward (vector path)
-  int64_t bwd_tiles;  // row tiles of the backward
-  int bwd_blocks;  // persistent grid of the backward == partial rows
-  int64_t rows_per_chunk;  // any-width path
-};
-
-int elem_size(int dt) { return dt == FM_F32 ? 4 : 2; }
-
-Plan make_plan(int64_t n, int64_t d, int x_dtype, bool aligned) {
-  Plan p{};
-  const int epv = 16 / elem_size(x_dtype);
-  const int64_t nvec = d / epv;
-  p.vec = aligned && (d % epv == 0) && nvec <= 4096;
-  if (p.vec) {
-    if (nvec <= 64) {
-      int t = 4;
-      while (t < nvec) t *= 2;
-      p.tpr = t; p.iters = 1;
-    } else {
-      static const int kPairs[][3] = {{128, 64, 2},   {192, 64, 3},    {256, 128, 2},  {384, 128, 3},
-                                      {512, 256, 2},  {768, 256, 3},   {1024, 512, 2}, {1536, 512, 3},
-                                      {2048, 1024, 2}, {3072, 1024, 3}, {4096, 1024, 4}};
-      for (auto& pr : kPairs) {
-        if (nvec <= pr[0]) { p.tpr = pr[1]; p.iters = pr[2]; break; }
-      }
-      // experiment hook: trade threads per row against vectors per thread
-      const int want = fm_host::get_param(fm_host::P_NORM_TPR);
-      if (want == 256 && nvec > 768 && nvec <= 1024) { p.tpr = 256; p.iters = 4; }
-      if (want == 128 && nvec > 64 && nvec <= 128) { p.tpr = 128; p.iters = 1; }
-    }
-    const int block = p.tpr > kMinBlock ? p.tpr : kMinBlock;
-    p.rpb = block / p.tpr;
-    p.tiles = (n + p.rpb - 1) / p.rpb;
-    p.bwd_tiles = (n + (kBwdBlock / p.tpr) - 1) / (kBwdBlock / p.tpr);
-    int per_cu = fm_host::get_param(fm_host::P_NORM_BWD_BLOCKS_PER_CU);
-    if (per_cu <= 0) per_cu = 1;
-    int64_t blocks = (int64_t)fm_host::num_cus() * per_cu;
-    if (blocks > p.bwd_tiles) blocks = p.bwd_tiles;
-    if (blocks < 1) blocks = 1;
-    p.bwd_blocks = (int)blocks;
-  } else {
-    int64_t chunks = n < 256 ? n : 256;
-    if (chunks < 1) chunks = 1;
-    p.rows_per_chunk = (n + chunks - 1) / chunks;
-    p.bwd_blocks = (int)((n + p.rows_per_chunk - 1) / (p.rows_per_chunk > 0 ? p.rows_per_chunk : 1));
-    if (p.bwd_blocks < 1) p.bwd_blocks = 1;
-  }
-  return p;
-}
-
-#define FM_FOR_EACH_SHAPE(X) \
-  X(4, 1) X(8, 1) X(16, 1) X(32, 1) X(64, 1) X(128, 1) X(64, 2) X(64, 3) X(128, 2) X(128, 3)    \
-  X(256, 2) X(256, 3) X(256, 4) X(512, 2) X(512, 3) X(1024, 2) X(1024, 3) X(1024, 4)
-
-template <typename T, typename WT, bool ADD>
-int launch_fwd(const Plan& p, const void* x, const void* delta, const void* w, void* xn, void* y,
-               float* rstd, int64_t n, int64_t d, float eps, hipStream_t st) {
-  const T* xp = static_cast<const T*>(x);
-  const T* dp = static_cast<const T*>(delta);
-  const WT* wp = static_cast<const WT*>(w);
-  T* xnp = static_cast<T*>(xn);
-  T* yp = static_cast<T*>(y);
-  if (!p.vec) {
-    hipLaunchKernelGGL((norm_fwd_generic<T, WT, ADD>), dim3((unsigned)n), dim3(256), 0, st, xp, dp,
-                       wp, xnp, yp, rstd, d, eps);
-    return FM_OK;
-  }
-#define X(TPR_, IT_)                                                                          \
-  if (p.tpr == TPR_ && p.iters == IT_) {                                                      \
-    hipLaunchKernelGGL((norm_fwd_kernel<T, WT, TPR_, IT_, ADD>), dim3((unsigned)p.tiles),     \
-                       dim3(BlockOf<TPR_>::value), 0, st, xp, dp, wp, xnp, yp, rstd, n, (int)d, \
-                       eps);                                                                  \
-    return FM_OK;                                                                             \
-  }
-  FM_FOR_EACH_SHAPE(X)
-#undef X
-  fm_host::set_error("rmsnorm: no kernel for tpr=%d iters=%d", p.tpr, p.iters);
-  return FM_ERR_UNSUPPORTED;
-}
-
-template <typename T, typename WT>
-int launch_bwd(const Plan& p, const void* x, const void* w, const float* rstd, const void* dy,
-               const void* gxn, void* dx, void* dd, void* dw, float* partial, int64_t n, int64_t d,
-               hipStream_t st) {
-  const T* xp = static_cast<const T*>(x);
-  const WT* wp = static_cast<const WT*>(w);
-  const T* dyp = static_cast<const T*>(dy);
-  const T* gp = static_cast<const T*>(gxn);
-  T* dxp = static_cast<T*>(dx);
-  T* ddp = static_cast<T*>(dd);
-  if (dw == nullptr) partial = nullptr;
-  if (!p.vec) {
-    hipLaunchKernelGGL((norm_bwd_generic<T, WT>), dim3((unsigned)n), dim3(256), 0, st, xp, wp, rstd,
-                       dyp, gp, dxp, ddp, d);
-    if (partial != nullptr) {
-      dim3 grid((unsigned)((d + 63) / 64), (unsigned)p.bwd_blocks);
-      hipLaunchKernelGGL((dw_generic<T>), grid, dim3(256), 0, st, xp, rstd, dyp, partial, n, d,
-                         p.rows_per_chunk);
-    }
-  } else {
-    bool done = false;
-#define X(TPR_, IT_)                                                                           \
-  if (!done && p.tpr == TPR_ && p.iters == IT_) {                                              \
-    hipLaunchKernelGGL((norm_bwd_kernel<T, WT, TPR_, IT_>), dim3((unsigned)p.bwd_blocks),      \
-                       dim3(kBwdBlock), 0, st, xp, wp, rstd, dyp, gp, dxp, ddp,                \
-                       partial, n, (int)d, p.bwd_tiles);                                       \
-    done = true;                                                                               \
-  }
-    FM_FOR_EACH_SHAPE(X)
-#undef X
-    if (!done) {
-      fm_host::set_error("rmsnorm_bwd: no kernel for tpr=%d iters=%d", p.tpr, p.iters);
-      return FM_ERR_UNSUPPORTED;
-    }
-  }
-  if (partial != nullptr) {
-    if (d % 4 == 0)
-      hipLaunchKernelGGL((colsum_kernel<WT>), dim3((unsigned)((d + 63) / 64)), dim3(1024), 0, st,
-                         partial, static_cast<WT*>(dw), p.bwd_blocks, (int)d);
-    else
-      hipLaunchKernelGGL((colsum_scalar_kernel<WT>), dim3((unsigned)((d + 63) / 64)), dim3(1024), 0,
-                         st, partial, static_cast<WT*>(dw), p.bwd_blocks, (int)d);
-  }
-  return FM_OK;
-}
-
-int check_common(const char* what, int64_t n, int64_t d, int x_dtype, int w_dtype) {
-  FM_CHECK_ARG(n >= 0 && d > 0, "%s: bad shape n=%lld d=%lld", what, (long long)n, (long long)d);
-  FM_CHECK_ARG(x_dtype == FM_F32 || x_dtype == FM_F16 || x_dtype == FM_BF16, "%s: bad x_dtype %d",
-               what, x_dtype);
-  FM_CHECK_ARG(w_dtype == x_dtype || w_dtype == FM_F32,
-               "%s: w_dtype must equal x_dtype or be fp32 (got x=%d w=%d)", what, x_dtype, w_dtype);
-  if (n > 0x7fffffffLL || d > 0x7fffffffLL) {
-    fm_host::set_error("%s: n and d must be below 2^31", what);
-    return FM_ERR_UNSUPPORTED;
-  }
-  return FM_OK;
-}
-
-template <bool ADD>
-int fwd_entry(const char* what, const void* x, const void* delta, const void* w, void* xn, void* y,
-              float* rstd, int64_t n, int64_t d, int x_dtype, int w_dtype, float eps,
-              fm_stream_t stream) {
-  int rc = check_common(what, n, d, x_dtype, w_dtype);
-  if (rc != FM_OK) return rc;
-  if (n == 0) return FM_OK;
-  FM_CHECK_ARG(x && w && y && rstd && (!ADD || (delta && xn)), "%s: NULL pointer", what);
-  bool al = fm_host::aligned16(x) && fm_host::aligned16(w) && fm_host::aligned16(y);
-  if (ADD) al = al && fm_host::aligned16(delta) && fm_host::aligned16(xn);
-  const Plan p = make_plan(n, d, x_dtype, al);
-  hipStream_t st = static_cast<hipStream_t>(stream);
-#define CALL(T, WT) rc = launch_fwd<T, WT, ADD>(p, x, delta, w, xn, y, rstd, n, d, eps, st)
-  if (x_dtype == FM_F32) CALL(float, float);
-  else if (x_dtype == FM_BF16 && w_dtype == FM_BF16) CALL(bf16_t, bf16_t);
-  else if (x_dtype == FM_BF16) CALL(bf16_t, float);
-  else if (w_dtype == FM_F16) CALL(f16_t, f16_t);
-  else CALL(f16_t, float);
-#undef CALL
-  if (rc != FM_OK) return rc;
-  FM_CHECK_LAUNCH(what);
-  return FM_OK;
-}
-
-int bwd_entry(const char* what, const void* x, const void* w, const float* rstd, const void* dy,
-              const void* gxn, void* dx, void* dd, void* dw, void* workspace, size_t workspace_bytes,
-              int64_t n, int64_t d, int x_dtype, int w_dtype, fm_stream_t stream) {
-  int rc = check_common(what, n, d, x_dtype, w_dtype);
-  if (rc != FM_OK) return rc;
-  FM_CHECK_ARG(w != nullptr, "%s: NULL weight", what);
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  if (n == 0) {
-    if (dw != nullptr) {  // empty batch: the weight gradient is exactly zero
-      // a fill kernel rather than a memset node, so the call stays safe under graph capture
-      const int64_t words = ((int64_t)d * elem_size(w_dtype) + 1) / 2;
-      hipLaunchKernelGGL(zero_u16_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, st,
-                         static_cast<uint16_t*>(dw), words);
-      FM_CHECK_LAUNCH(what);
-    }
-    return FM_OK;
-  }
-  FM_CHECK_ARG(x && rstd && dy && dx, "%s: NULL pointer", what);
-  if (dd == dx) dd = nullptr;
-  bool al = fm_host::aligned16(x) && fm_host::aligned16(w) && fm_host::aligned16(dy) &&
-            fm_host::aligned16(dx) && fm_host::aligned16(gxn) && fm_host::aligned16(dd) &&
-            fm_host::aligned16(workspace);
-  const Plan p = make_plan(n, d, x_dtype, al);
-  if (dw != nullptr) {
-    const size_t need = (size_t)p.bwd_blocks * (size_t)d * sizeof(float);
-    if (workspace == nullptr || workspace_bytes < need) {
-      fm_host::set_error("%s: workspace of %zu bytes needed, %zu given", what, need, workspace_bytes);
-      return FM_ERR_WORKSPACE;
-    }
-  }
-  float* partial = static_cast<float*>(workspace);
-#define CALL(T, WT) rc = launch_bwd<T, WT>(p, x, w, rstd, dy, gxn, dx, dd, dw, partial, n, d, st)
-  if (x_dtype == FM_F32) CALL(float, float);
-  else if (x_dtype == FM_BF16 && w_dtype == FM_BF16) CALL(bf16_t, bf16_t);
-  else if (x_dtype == FM_BF16) CALL(bf16_t, float);
-  else if (w_dtype == FM_F16) CALL(f16_t, f16_t);
-  else CALL(f16_t, float);
-#undef CALL
-  if (rc != FM_OK) return rc;
-  FM_CHECK_LAUNCH(what);
-  return FM_OK;
-}
-
-}  // namespace
+// column sum of the fp32 weight-gradient partials). Kernels: fm_norm.cuh with LN = false.
+#include "fm_norm.cuh"
 
 extern "C" {
 
 int fm_rmsnorm_fwd(const void* x, const void* w, void* y, float* rstd, int64_t n, int64_t d,
                    int x_dtype, int w_dtype, float eps, fm_stream_t stream) {
-  return fwd_entry<false>("fm_rmsnorm_fwd", x, nullptr, w, nullptr, y, rstd, n, d, x_dtype, w_dtype,
-                          eps, stream);
+  return fwd_entry<false, false>("fm_rmsnorm_fwd", x, nullptr, w, nullptr, nullptr, y, nullptr, rstd, n, d,
+                                 x_dtype, w_dtype, eps, stream);
 }
 
 int fm_add_rmsnorm_fwd(const void* x, const void* delta, const void* w, void* xn, void* y,
                        float* rstd, int64_t n, int64_t d, int x_dtype, int w_dtype, float eps,
                        fm_stream_t stream) {
-  return fwd_entry<true>("fm_add_rmsnorm_fwd", x, delta, w, xn, y, rstd, n, d, x_dtype, w_dtype, eps,
-                         stream);
+  return fwd_entry<true, false>("fm_add_rmsnorm_fwd", x, delta, w, nullptr, xn, y, nullptr, rstd, n, d,
+                                x_dtype, w_dtype, eps, stream);
 }
 
 size_t fm_rmsnorm_bwd_workspace(int64_t n, int64_t d, int x_dtype) {
-  if (n <= 0 || d <= 0) return 0;
-  // the larger of the two paths, so the answer does not depend on pointer alignment
-  const Plan a = make_plan(n, d, x_dtype, true);
-  const Plan b = make_plan(n, d, x_dtype, false);
-  const int p = a.bwd_blocks > b.bwd_blocks ? a.bwd_blocks : b.bwd_blocks;
-  return (size_t)p * (size_t)d * sizeof(float);
+  return bwd_workspace_bytes(n, d, x_dtype, false);
 }
 
 int fm_rmsnorm_bwd(const void* x, const void* w, const float* rstd, const void* dy, void* dx,
                    void* dw, void* workspace, size_t workspace_bytes, int64_t n, int64_t d,
                    int x_dtype, int w_dtype, fm_stream_t stream) {
-  return bwd_entry("fm_rmsnorm_bwd", x, w, rstd, dy, nullptr, dx, nullptr, dw, workspace,
-                   workspace_bytes, n, d, x_dtype, w_dtype, stream);
+  return bwd_entry<false>("fm_rmsnorm_bwd", x, w, nullptr, rstd, dy, nullptr, dx, nullptr, dw, nullptr,
+                          workspace, workspace_bytes, n, d, x_dtype, w_dtype, stream);
 }
 
 int fm_add_rmsnorm_bwd(const void* xn, const void* w, const float* rstd, const void* gy,
                        const void* gxn, void* dx, void* ddelta, void* dw, void* workspace,
                        size_t workspace_bytes, int64_t n, int64_t d, int x_dtype, int w_dtype,
                        fm_stream_t stream) {
-  return bwd_entry("fm_add_rmsnorm_bwd", xn, w, rstd, gy, gxn, dx, ddelta, dw, workspace,
-                   workspace_bytes, n, d, x_dtype, w_dtype, stream);
+  return bwd_entry<false>("fm_add_rmsnorm_bwd", xn, w, nullptr, rstd, gy, gxn, dx, ddelta, dw, nullptr,
+                          workspace, workspace_bytes, n, d, x_dtype, w_dtype, stream);
 }
 
 }  // extern "C"

@@ -28,6 +28,7 @@ from .ce import cross_entropy
 from .dispatch import moe_combine, moe_gather
 from .extras import newton_schulz
 from .kl import distill_kl, kl_distill_loss, kl_div, kl_div_logits, kl_div_logits_topk
+from .layernorm import add_layer_norm, layer_norm
 from .norm import add_rms_norm, rms_norm
 from .rope import qk_norm_rope
 from .route import Routing, moe_route
@@ -38,7 +39,7 @@ from .topk import topk
 __all__ = [
     "HAS_TRITON", "set_backend", "get_backend", "stats", "reset_stats",
     "rms_norm", "add_rms_norm", "qk_norm_rope", "swiglu", "swiglu_split",
-    "kl_div_logits", "kl_div_logits_topk", "kl_div", "kl_distill_loss", "distill_kl",
+    "layer_norm", "add_layer_norm", "kl_div_logits", "kl_div_logits_topk", "kl_div", "kl_distill_loss", "distill_kl",
     "newton_schulz", "topk", "softmax", "cross_entropy", "moe_route", "Routing",
     "moe_gather", "moe_combine",
     "enable", "patch", "revert", "available", "use_custom_ops",

@@ -30,6 +30,20 @@ def add_rms_norm(x, delta, w, eps: float = 1e-6):
     return summed, rms_norm(summed, w, eps)
 
 
+def layer_norm(x, w, b=None, eps: float = 1e-5):
+    """``F.layer_norm`` in the wide dtype, one rounding (the rule of ``rms_norm`` above)."""
+    xw = _wide(x)
+    out = torch.nn.functional.layer_norm(xw, (x.shape[-1],), _wide(w).to(xw.dtype),
+                                         None if b is None else _wide(b).to(xw.dtype), eps)
+    return out.to(x.dtype)
+
+
+def add_layer_norm(x, delta, w, b=None, eps: float = 1e-5):
+    """The sum is rounded to x's dtype before it is normalised."""
+    summed = x + delta
+    return summed, layer_norm(summed, w, b, eps)
+
+
 def kl_div_logits(student, teacher, reduction: str = "mean", temperature: float = 1.0):
     """KL(teacher || student) over the last dim (reference ``_fallback.py:52-69``).
 

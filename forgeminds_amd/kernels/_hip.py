@@ -39,6 +39,11 @@ SIGNATURES = {
     "fm_add_rmsnorm_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _f32, _vp]),
     "fm_add_rmsnorm_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64,
                                   _int, _int, _vp]),
+    "fm_layernorm_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _f32, _vp]),
+    "fm_add_layernorm_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _f32, _vp]),
+    "fm_layernorm_bwd_workspace": (_sz, [_i64, _i64, _int]),
+    "fm_layernorm_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64, _int, _int,
+                                _vp]),
     "fm_ce_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _i64, _int, _vp]),
     "fm_ce_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _i64, _vp]),
     "fm_ce_loss_grad": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _i64, _int, _vp]),
@@ -211,6 +216,45 @@ def add_rmsnorm_bwd(xn2, w, rstd, gy2, gxn2, want_dw: bool = True):
                                         dtype_code(xn2.dtype), dtype_code(w.dtype),
                                         _stream(xn2)), "fm_add_rmsnorm_bwd")
     return dx, dw
+
+
+def layernorm_fwd(x2, w, b, eps: float, delta2=None):
+    """-> (xn or None, y [n, d], mean [n], rstd [n]); with ``delta2`` the residual-add form."""
+    _dense(x2, w, b, delta2)
+    n, d = x2.shape
+    y = torch.empty_like(x2)
+    stats = torch.empty(2, n, device=x2.device, dtype=torch.float32)
+    xn = torch.empty_like(x2) if delta2 is not None else None
+    with torch.cuda.device(x2.device):
+        if delta2 is None:
+            _check(lib().fm_layernorm_fwd(_ptr(x2), _ptr(w), _ptr(b), _ptr(y), stats[0].data_ptr(),
+                                          stats[1].data_ptr(), n, d, dtype_code(x2.dtype),
+                                          dtype_code(w.dtype), float(eps), _stream(x2)), "fm_layernorm_fwd")
+        else:
+            _check(lib().fm_add_layernorm_fwd(_ptr(x2), _ptr(delta2), _ptr(w), _ptr(b), _ptr(xn), _ptr(y),
+                                              stats[0].data_ptr(), stats[1].data_ptr(), n, d,
+                                              dtype_code(x2.dtype), dtype_code(w.dtype), float(eps),
+                                              _stream(x2)), "fm_add_layernorm_fwd")
+    return xn, y, stats[0], stats[1]
+
+
+def layernorm_bwd(x2, w, mean, rstd, dy2, gxn2=None, want_dw: bool = True, want_db: bool = True):
+    """-> (dx [n, d], dw or None, db or None); ``x2`` is the normalised input (xn of the add form)."""
+    _dense(x2, w, mean, rstd, dy2, gxn2)
+    n, d = x2.shape
+    dx = torch.empty_like(x2)
+    dw = torch.empty_like(w) if want_dw else None
+    db = torch.empty_like(w) if want_db else None
+    with torch.cuda.device(x2.device):
+        ws, nbytes = None, 0
+        if want_dw or want_db:
+            nbytes = int(lib().fm_layernorm_bwd_workspace(n, d, dtype_code(x2.dtype)))
+            ws = torch.empty(max(nbytes, 16), device=x2.device, dtype=torch.uint8)
+        _check(lib().fm_layernorm_bwd(_ptr(x2), _ptr(w), _ptr(mean), _ptr(rstd), _ptr(dy2), _ptr(gxn2),
+                                      _ptr(dx), _ptr(dw), _ptr(db), _ptr(ws), nbytes, n, d,
+                                      dtype_code(x2.dtype), dtype_code(w.dtype), _stream(x2)),
+               "fm_layernorm_bwd")
+    return dx, dw, db
 
 
 # ------------------------------------------------------------------ cross entropy

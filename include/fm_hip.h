@@ -97,6 +97,35 @@ int fm_add_rmsnorm_bwd(const void* xn, const void* w, const float* rstd, const v
                        size_t workspace_bytes, int64_t n, int64_t d, int x_dtype, int w_dtype,
                        fm_stream_t stream);
 
+/* ------------------------------------------------------------------ LayerNorm
+ * No kernel of this name exists in the reference (its norm kernels are the RMS pair,
+ * kernels/norm.py:133-316); these follow the same contract and rounding rule as the RMSNorm
+ * entry points above (_fallback.py:15-35: fp32 math on the stored values, one rounding) with
+ * torch.nn.functional.layer_norm's arithmetic:
+ *   mean = sum(x)/d;  rstd = rsqrt(sum((x-mean)^2)/d + eps);  y = ((x-mean)*rstd)*w + bias.
+ * bias may be NULL. mean, rstd: [n] fp32, kept for the backward. */
+int fm_layernorm_fwd(const void* x, const void* w, const void* bias, void* y, float* mean,
+                     float* rstd, int64_t n, int64_t d, int x_dtype, int w_dtype, float eps,
+                     fm_stream_t stream);
+
+/* xn = x + delta rounded to x's dtype; y = layer_norm(xn) computed from the rounded xn
+ * (the residual-add form of fm_add_rmsnorm_fwd). */
+int fm_add_layernorm_fwd(const void* x, const void* delta, const void* w, const void* bias,
+                         void* xn, void* y, float* mean, float* rstd, int64_t n, int64_t d,
+                         int x_dtype, int w_dtype, float eps, fm_stream_t stream);
+
+/* Bytes of scratch fm_layernorm_bwd needs (fp32 partial rows for dw and db). */
+size_t fm_layernorm_bwd_workspace(int64_t n, int64_t d, int x_dtype);
+
+/* g = dy*w; xh = (x-mean)*rstd; dx = rstd * ((g - mean(g)) - xh*mean(g*xh)) [+ gxn];
+ * dw = sum_rows dy*xh; db = sum_rows dy. x is the normalised input (xn of the add form);
+ * gxn (gradient of the residual output of the add form) may be NULL; dw and db may be NULL
+ * (no workspace is needed when both are). */
+int fm_layernorm_bwd(const void* x, const void* w, const float* mean, const float* rstd,
+                     const void* dy, const void* gxn, void* dx, void* dw, void* db,
+                     void* workspace, size_t workspace_bytes, int64_t n, int64_t d, int x_dtype,
+                     int w_dtype, fm_stream_t stream);
+
 /* ------------------------------------------------------------------ cross entropy
  * Replaces the F.cross_entropy(reduction="sum") / n reduction of logits_cross_entropy and
  * chunked_cross_entropy (forgemind/loss.py:54-70, 23-51):

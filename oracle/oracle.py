@@ -82,6 +82,48 @@ def add_rms_norm_bwd(xn, w, gy, gxn, eps=1e-6, acc=torch.float32):
     return dx.to(xn.dtype), dw.to(w.dtype)
 
 
+# ------------------------------------------------------------------ LayerNorm
+def layer_norm(x, w, b=None, eps=1e-5, acc=torch.float32):
+    """y, mean, rstd. torch.nn.functional.layer_norm's arithmetic in `acc` on the stored
+    values, one rounding to x's dtype -- the rounding rule the reference applies to its norm
+    fallback (forgemind/kernels/_fallback.py:15-35); the reference has no LayerNorm of its own.
+    Biased variance of the centred values, as F.layer_norm."""
+    xf, wf = _up(x, acc), _up(w, acc)
+    mean = xf.mean(dim=-1, keepdim=True)
+    xc = xf - mean
+    rstd = torch.rsqrt((xc * xc).mean(dim=-1, keepdim=True) + eps)
+    y = (xc * rstd) * wf
+    if b is not None:
+        y = y + _up(b, acc)
+    return y.to(x.dtype), mean.squeeze(-1), rstd.squeeze(-1)
+
+
+def layer_norm_bwd(x, w, dy, eps=1e-5, gxn=None, acc=torch.float32):
+    """dx (x.dtype), dw, db (w.dtype): g = dy*w, xh = (x-mean)*rstd,
+    dx = rstd*((g - mean(g)) - xh*mean(g*xh)) [+ gxn]; dw = sum_rows dy*xh; db = sum_rows dy."""
+    xf, wf, gf = _up(x, acc), _up(w, acc), _up(dy, acc)
+    d = x.shape[-1]
+    mean = xf.mean(dim=-1, keepdim=True)
+    xc = xf - mean
+    rstd = torch.rsqrt((xc * xc).mean(dim=-1, keepdim=True) + eps)
+    xh = xc * rstd
+    g = gf * wf
+    dx = ((g - g.mean(dim=-1, keepdim=True)) - xh * (g * xh).mean(dim=-1, keepdim=True)) * rstd
+    if gxn is not None:
+        dx = dx + _up(gxn, acc)
+    dw = (gf * xh).reshape(-1, d).sum(dim=0)
+    db = gf.reshape(-1, d).sum(dim=0)
+    return dx.to(x.dtype), dw.to(w.dtype), db.to(w.dtype)
+
+
+def add_layer_norm(x, delta, w, b=None, eps=1e-5, acc=torch.float32):
+    """xn, y, mean, rstd: the sum is a tensor add in x's dtype (rounded for bf16/fp16, as
+    forgemind/kernels/_fallback.py:33-35 does for RMSNorm), the norm is taken of the rounded sum."""
+    xn = x + delta
+    y, mean, rstd = layer_norm(xn, w, b, eps, acc)
+    return xn, y, mean, rstd
+
+
 # ------------------------------------------------------------------ cross entropy
 def cross_entropy(logits, labels, ignore_index=-100, acc=torch.float32):
     """loss (0-d, `acc`), dlogits (logits.dtype) for upstream gradient 1.

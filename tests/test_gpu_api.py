@@ -451,3 +451,44 @@ def test_kl_div_logits_topk_autograd_and_wide_rows():
     assert loss.item() == pytest.approx(O.kl_div(s, t, "sum", 1.0, acc=torch.float64)[0].item(), rel=1e-4)
     with pytest.raises(RuntimeError):
         kernels.kl_div_logits_topk(s.to("cuda"), t.to("cuda"), 0)
+
+
+def test_layer_norm_autograd_module_and_op_path():
+    g = torch.Generator().manual_seed(51)
+    x = (0.5 + torch.randn(4, 50, 768, generator=g)).bfloat16()
+    w, b = 1 + 0.02 * torch.randn(768, generator=g), 0.1 * torch.randn(768, generator=g)
+    dy = torch.randn(4, 50, 768, generator=g).bfloat16()
+    odx, odw, odb = O.layer_norm_bwd(x, w, dy, 1e-5)
+    xd = x.to(DEV).requires_grad_(True)
+    wd, bd = w.to(DEV).requires_grad_(True), b.to(DEV).requires_grad_(True)
+    kernels.reset_stats()
+    y = kernels.layer_norm(xd, wd, bd, 1e-5)
+    y.backward(dy.to(DEV))
+    assert kernels.stats()["fast"] == 1 and kernels.stats()["fallback"] == 0
+    assert close(y, O.layer_norm(x, w, b, 1e-5)[0]) and close(xd.grad, odx)
+    assert close(wd.grad, odw, 1e-3) and close(bd.grad, odb, 1e-3)
+    # the op path gives the same bits as the eager path
+    x2 = x.to(DEV).requires_grad_(True)
+    _ops.use_custom_ops(True)
+    y2 = kernels.layer_norm(x2, wd.detach(), bd.detach(), 1e-5)
+    y2.backward(dy.to(DEV))
+    _ops.use_custom_ops(None)
+    assert torch.equal(y2, y) and torch.equal(x2.grad, xd.grad)
+    # residual form through the module, against torch.nn.LayerNorm
+    m = fm.nn.LayerNorm(768).to(DEV)
+    ref = nn.LayerNorm(768).to(DEV)
+    with torch.no_grad():
+        m.weight.copy_(w); m.bias.copy_(b); ref.weight.copy_(w); ref.bias.copy_(b)
+    h = torch.randn(6, 768, device=DEV, requires_grad=True)
+    r = torch.randn(6, 768, device=DEV)
+    normed, res = m.forward_with_residual(h, r)
+    (normed.sum() + res.sum()).backward()
+    h2 = h.detach().clone().requires_grad_(True)
+    s2 = h2 + r
+    (ref(s2).sum() + s2.sum()).backward()
+    assert torch.equal(res, h.detach() + r) and torch.allclose(normed, ref(h.detach() + r), atol=1e-5)
+    assert torch.allclose(h.grad, h2.grad, atol=1e-4) and torch.allclose(m.bias.grad, ref.bias.grad, atol=1e-5)
+    assert torch.allclose(m.weight.grad, ref.weight.grad, atol=1e-4)
+    fn = torch.compile(lambda t: kernels.layer_norm(t, wd.detach(), bd.detach()).float().sum(), fullgraph=True,
+                       backend="eager")
+    assert torch.isfinite(fn(x.to(DEV)))

@@ -148,6 +148,92 @@ def test_add_rmsnorm_fwd_bwd(n, d, dt, wdt, eps):
     assert rel_max(rstd, orstd) < 1e-5
 
 
+# ------------------------------------------------------------------ LayerNorm
+LN_CASES = [
+    (512, 1024, BF16, F32, 1e-5, True), (64, 8192, BF16, BF16, 1e-5, True), (33, 768, F16, F16, 1e-5, False),
+    (17, 100, F32, F32, 1e-6, True), (5, 7, BF16, F32, 1e-5, True), (300, 5120, BF16, F32, 1e-5, False),
+    (16, 64, BF16, BF16, 1e-5, True), (3, 1, F32, F32, 1e-5, True), (6, 8, F32, F32, 1e-5, True),
+    (9, 16384, BF16, F32, 1e-5, True), (4, 40000, F16, F32, 1e-5, True), (130, 3072, F32, F32, 1e-5, True),
+    (7, 12288, BF16, BF16, 1e-5, True), (2, 24576, BF16, F32, 1e-5, False), (40, 4096, BF16, F32, 1e-5, True),
+]
+
+
+@pytest.mark.parametrize("n,d,dt,wdt,eps,bias", LN_CASES)
+def test_layernorm_fwd_bwd(n, d, dt, wdt, eps, bias):
+    g = gen(1031)
+    x = (0.5 + torch.randn(n, d, generator=g)).to(dt)           # a mean the kernel has to remove
+    w = (1 + 0.02 * torch.randn(d, generator=g)).to(wdt)
+    b = (0.1 * torch.randn(d, generator=g)).to(wdt) if bias else None
+    dy = torch.randn(n, d, generator=g).to(dt)
+    oy, omean, orstd = O.layer_norm(x, w, b, eps)
+    odx, odw, odb = O.layer_norm_bwd(x, w, dy, eps)
+    xd, wd, dyd = x.to(DEV), w.to(DEV), dy.to(DEV)
+    bd = None if b is None else b.to(DEV)
+    _, y, mean, rstd = _hip.layernorm_fwd(xd, wd, bd, eps)
+    dx, dw, db = _hip.layernorm_bwd(xd, wd, mean, rstd, dyd)
+    torch.cuda.synchronize()
+    assert y.dtype == dt and dx.dtype == dt and dw.dtype == wdt and db.dtype == wdt
+    # y = xh*w + b: where it cancels towards 0 the honest bound is a few fp32 roundings of the terms
+    yterms = 4.0 * w.float().abs().max().item() + (b.float().abs().max().item() if bias else 0.0)
+    assert_close_lowp(y, oy, dt, "y", cancel=yterms)
+    if d > 1:
+        assert torch.allclose(mean.cpu(), omean, rtol=1e-5, atol=1e-6) and rel_max(rstd, orstd) < 1e-5
+    natural = (dy.float().abs().max() * w.float().abs().max() * orstd.max()).item() * 4.0
+    assert_close_lowp(dx, odx, dt, "dx", ulps=3.0, cancel=natural)
+    _, odw64, odb64 = O.layer_norm_bwd(x, w.double(), dy, eps, acc=torch.float64)
+    tol = 1e-2 if wdt != F32 else 1e-4
+    if d > 1:                                                   # d == 1: xh is identically 0
+        assert rel_max(dw, odw64) <= tol and rel_max(dw, odw) <= 1e-2
+    assert rel_max(db, odb64) <= tol
+    # frozen parameters: no dw / db, same dx; bias gradient alone
+    dx2, none_w, none_b = _hip.layernorm_bwd(xd, wd, mean, rstd, dyd, None, False, False)
+    assert none_w is None and none_b is None and torch.equal(dx2, dx)
+    _, dw3, none_b = _hip.layernorm_bwd(xd, wd, mean, rstd, dyd, None, True, False)
+    assert none_b is None and torch.equal(dw3, dw)
+
+
+@pytest.mark.parametrize("n,d,dt,wdt", [(128, 8192, BF16, F32), (9, 24, F32, F32), (10, 33, BF16, BF16),
+                                        (40, 4096, F16, F16), (12, 2048, BF16, F32)])
+def test_add_layernorm_fwd_bwd(n, d, dt, wdt):
+    g = gen(1034)
+    x = torch.randn(n, d, generator=g).to(dt)
+    dl = (0.3 + torch.randn(n, d, generator=g)).to(dt)
+    w = (1 + 0.02 * torch.randn(d, generator=g)).to(wdt)
+    b = (0.1 * torch.randn(d, generator=g)).to(wdt)
+    gy = torch.randn(n, d, generator=g).to(dt)
+    gxn = torch.randn(n, d, generator=g).to(dt)
+    oxn, oy, omean, orstd = O.add_layer_norm(x, dl, w, b, 1e-5)
+    odx, odw, odb = O.layer_norm_bwd(oxn, w, gy, 1e-5, gxn=gxn)
+    xn, y, mean, rstd = _hip.layernorm_fwd(x.to(DEV), w.to(DEV), b.to(DEV), 1e-5, dl.to(DEV))
+    dx, dw, db = _hip.layernorm_bwd(xn, w.to(DEV), mean, rstd, gy.to(DEV), gxn.to(DEV))
+    torch.cuda.synchronize()
+    assert torch.equal(xn.cpu(), oxn), "xn must be exactly x + delta in x's dtype"
+    assert_close_lowp(y, oy, dt, "y", cancel=4.0 * w.float().abs().max().item() + b.float().abs().max().item())
+    natural = (gy.float().abs().max() * w.float().abs().max() * orstd.max()).item() * 4.0
+    assert_close_lowp(dx, odx, dt, "dx", ulps=3.0, cancel=natural)
+    assert rel_max(dw, odw) <= 1e-2 and rel_max(db, odb) <= 1e-2
+
+
+def test_layernorm_determinism_unaligned_and_empty():
+    g = gen(1035)
+    x = torch.randn(2048, 1024, generator=g).bfloat16().to(DEV)
+    w, b = torch.randn(1024, generator=g).to(DEV), torch.randn(1024, generator=g).to(DEV)
+    dy = torch.randn(2048, 1024, generator=g).bfloat16().to(DEV)
+    outs = []
+    for _ in range(2):
+        _, y, mean, rstd = _hip.layernorm_fwd(x, w, b, 1e-5)
+        outs.append((y,) + _hip.layernorm_bwd(x, w, mean, rstd, dy))
+    assert all(torch.equal(a, c) for a, c in zip(*outs))        # bit for bit
+    base = torch.randn(6 * 512 + 3, generator=g).bfloat16().to(DEV)
+    xv = base[3:].view(6, 512)                                  # 6 bytes off a 16-byte line
+    _, y, _, _ = _hip.layernorm_fwd(xv, torch.ones(512, device=DEV), None, 1e-5)
+    assert_close_lowp(y, O.layer_norm(xv.cpu(), torch.ones(512), None, 1e-5)[0], BF16, "unaligned", cancel=4.0)
+    e = torch.empty(0, 64, device=DEV)
+    _, y0, m0, _ = _hip.layernorm_fwd(e, torch.ones(64, device=DEV), None, 1e-5)
+    dx0, dw0, db0 = _hip.layernorm_bwd(e, torch.ones(64, device=DEV), m0, m0, e)
+    assert y0.shape == (0, 64) and not dw0.any() and not db0.any()
+
+
 # ------------------------------------------------------------------ cross entropy
 CE_CASES = [(512, 32000, BF16), (7, 50257, BF16), (5, 1000, F32), (4, 7, F16), (9, 16, F32),
             (3, 128256, BF16), (6, 32001, F32), (33, 4096, F16), (2, 1, F32), (64, 50257, F32)]

@@ -389,3 +389,27 @@ def test_moe_gather_combine_torch_path_and_grads():
         kernels.moe_gather(x, r.order[:-1], k)
     with pytest.raises(ValueError):
         kernels.moe_combine(ys, w, r.slot[:-1])
+
+
+def test_layer_norm_torch_path_and_module():
+    torch.manual_seed(5)
+    x = 1 + torch.randn(3, 7, 24)
+    w, b = torch.randn(24), torch.randn(24)
+    kernels.reset_stats()
+    y = kernels.layer_norm(x, w, b, 1e-5)
+    assert torch.allclose(y, F.layer_norm(x, (24,), w, b, 1e-5), atol=2e-6)
+    assert torch.equal(y, O.layer_norm(x, w, b, 1e-5)[0]) or torch.allclose(y, O.layer_norm(x, w, b, 1e-5)[0], atol=2e-6)
+    xn, yn = kernels.add_layer_norm(x.bfloat16(), x.bfloat16(), w, None, 1e-5)
+    assert torch.equal(xn, x.bfloat16() + x.bfloat16()) and yn.dtype == torch.bfloat16
+    assert kernels.stats()["fast"] == 0 and kernels.stats()["fallback"] == 2
+    m = fm.nn.LayerNorm(24)
+    ref = torch.nn.LayerNorm(24)
+    ref.load_state_dict(m.state_dict())                         # same parameter names and shapes
+    with torch.no_grad():
+        m.weight.copy_(w); m.bias.copy_(b); ref.weight.copy_(w); ref.bias.copy_(b)
+    assert torch.allclose(m(x), ref(x), atol=2e-6)
+    normed, res = m.forward_with_residual(x, 2 * x)
+    assert torch.equal(res, 3 * x) and torch.allclose(normed, ref(3 * x), atol=2e-6)
+    with pytest.raises(ValueError):
+        m(torch.randn(2, 23))
+    assert fm.nn.LayerNorm(8, bias=False).bias is None and fm.nn.LayerNorm(8, elementwise_affine=False).weight is None

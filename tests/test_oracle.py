@@ -104,6 +104,68 @@ def test_add_rms_norm_backward_is_autograd():
     assert torch.allclose(dx0, dx - gxn, atol=1e-12)
 
 
+# ------------------------------------------------------------------ layer_norm
+@pytest.mark.parametrize("d", [1, 3, 8, 100])
+@pytest.mark.parametrize("bias", [True, False])
+def test_layer_norm_is_torch_layer_norm(d, bias):
+    torch.manual_seed(d)
+    x, w = 2 + torch.randn(5, d), torch.randn(d)
+    b = torch.randn(d) if bias else None
+    y, mean, rstd = O.layer_norm(x, w, b, 1e-5)
+    assert torch.allclose(y, F.layer_norm(x, (d,), w, b, 1e-5), atol=2e-6, rtol=1e-5)
+    assert torch.allclose(mean, x.mean(-1), atol=1e-6)
+    assert torch.allclose(rstd, torch.rsqrt(x.var(-1, unbiased=False) + 1e-5), rtol=1e-5)
+
+
+def test_layer_norm_closed_forms():
+    x = 5 + torch.randn(7, 64, dtype=F64)
+    y, _, _ = O.layer_norm(x, torch.ones(64, dtype=F64), None, 0.0, acc=F64)
+    assert y.mean(-1).abs().max() < 1e-12 and torch.allclose(y.var(-1, unbiased=False),
+                                                             torch.ones(7, dtype=F64), atol=1e-12)
+    # invariant under shift and positive scaling of the input when eps == 0
+    y2, _, _ = O.layer_norm(3.0 * x - 11.0, torch.ones(64, dtype=F64), None, 0.0, acc=F64)
+    assert torch.allclose(y, y2, atol=1e-10)
+    # a constant row: zero centred values, output is the bias
+    b = torch.randn(8)
+    yc, mc, rc = O.layer_norm(torch.full((2, 8), 3.0), torch.ones(8), b, 1e-5)
+    assert torch.equal(yc, b.expand(2, 8)) and torch.equal(mc, torch.full((2,), 3.0))
+    assert torch.allclose(rc, torch.full((2,), 1e-5 ** -0.5))
+
+
+def test_layer_norm_backward_is_autograd_of_torch_layer_norm():
+    torch.manual_seed(3)
+    x = torch.randn(6, 10, dtype=F64, requires_grad=True)
+    w = torch.randn(10, dtype=F64, requires_grad=True)
+    b = torch.randn(10, dtype=F64, requires_grad=True)
+    g = torch.randn(6, 10, dtype=F64)
+    F.layer_norm(x, (10,), w, b, 1e-5).backward(g)
+    dx, dw, db = O.layer_norm_bwd(x.detach(), w.detach(), g, 1e-5, acc=F64)
+    assert torch.allclose(dx, x.grad, atol=1e-12) and torch.allclose(dw, w.grad, atol=1e-12)
+    assert torch.allclose(db, b.grad, atol=1e-12)
+    assert dx.sum(-1).abs().max() < 1e-12                       # dx has no mean component
+    dx0, _, _ = O.layer_norm_bwd(x.detach(), w.detach(), g, 0.0, acc=F64)
+    xc = x.detach() - x.detach().mean(-1, keepdim=True)
+    assert (dx0 * xc).sum(-1).abs().max() < 1e-11               # nor one along the centred row
+
+
+def test_add_layer_norm_rounding_points_and_backward():
+    torch.manual_seed(4)
+    for dt in (torch.float32, torch.bfloat16, torch.float16):
+        x, d = torch.randn(4, 8).to(dt), torch.randn(4, 8).to(dt)
+        w, b = torch.randn(8), torch.randn(8)
+        xn, y, _, _ = O.add_layer_norm(x, d, w, b)
+        assert torch.equal(xn, x + d) and torch.equal(y, O.layer_norm(x + d, w, b)[0])
+    x = torch.randn(5, 12, dtype=F64, requires_grad=True)
+    dl = torch.randn(5, 12, dtype=F64, requires_grad=True)
+    w = torch.randn(12, dtype=F64, requires_grad=True)
+    gy, gxn = torch.randn(5, 12, dtype=F64), torch.randn(5, 12, dtype=F64)
+    xn = x + dl
+    torch.autograd.backward([xn, F.layer_norm(xn, (12,), w, None, 1e-5)], [gxn, gy])
+    dx, dw, _ = O.layer_norm_bwd(xn.detach(), w.detach(), gy, 1e-5, gxn=gxn, acc=F64)
+    assert torch.allclose(dx, x.grad, atol=1e-12) and torch.allclose(dx, dl.grad, atol=1e-12)
+    assert torch.allclose(dw, w.grad, atol=1e-12)
+
+
 # ------------------------------------------------------------------ cross entropy
 def test_ce_is_torch_cross_entropy():
     # reference tests/test_edge_cases.py:39-47
