@@ -17,6 +17,7 @@ const char* const kParamNames[fm_host::P_COUNT] = {
     "norm_tpr",
     "topk_variant",
     "vocab_unroll",
+    "norm_fwd_blocks_per_cu",
 };
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cus[kMaxDevices];

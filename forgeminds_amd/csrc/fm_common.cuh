@@ -256,7 +256,8 @@ namespace fm_host {
 void set_error(const char* fmt, ...);
 int get_param(int which);
 
-enum Param { P_NORM_BWD_BLOCKS_PER_CU = 0, P_VOCAB_THREADS, P_NORM_TPR, P_TOPK_VARIANT, P_VOCAB_UNROLL, P_COUNT };
+enum Param { P_NORM_BWD_BLOCKS_PER_CU = 0, P_VOCAB_THREADS, P_NORM_TPR, P_TOPK_VARIANT, P_VOCAB_UNROLL,
+             P_NORM_FWD_BLOCKS_PER_CU, P_COUNT };
 
 int num_cus();  // compute units of the current device (cached per device)
 

@@ -42,88 +42,113 @@ __device__ __forceinline__ void load_w(const WT* w, int col, float (&o)[Elem<T>:
 }
 
 // ---------------------------------------------------------------- forward (vector path)
+// Persistent over row tiles: the grid holds a few workgroups per compute unit, each keeps its
+// columns of w (and the bias) in registers and walks tiles blockIdx.x, blockIdx.x + gridDim.x, ...
+// so the parameters are fetched once per workgroup instead of once per row.
 template <typename T, typename WT, int TPR, int ITERS, bool ADD, bool LN>
 __global__ __launch_bounds__(BlockOf<TPR>::value) void norm_fwd_kernel(
     const T* __restrict__ x, const T* __restrict__ delta, const WT* __restrict__ w,
     const WT* __restrict__ bias, T* __restrict__ xn, T* __restrict__ y, float* __restrict__ mean,
-    float* __restrict__ rstd, int64_t n, int d, float eps) {
+    float* __restrict__ rstd, int64_t n, int d, float eps, int64_t tiles) {
   constexpr int EPV = Elem<T>::kVec;
   constexpr int BLOCK = BlockOf<TPR>::value;
   constexpr int RPB = BLOCK / TPR;
+  constexpr int NB = LN ? ITERS : 1;
   __shared__ float smem[RPB * (TPR > 64 ? TPR / 64 : 1)];
 
   const int tid = threadIdx.x;
   const int rib = tid / TPR;
   const int t = tid % TPR;
-  const int64_t row = (int64_t)blockIdx.x * RPB + rib;
-  const bool valid = row < n;
   const int nvec = d / EPV;
-  const int64_t base = row * (int64_t)d;
 
-  float v[ITERS][EPV];
-  float ss = 0.f;
+  float wv[ITERS][EPV];
+  float bv[NB][EPV];
 #pragma unroll
   for (int i = 0; i < ITERS; ++i) {
     const int c = i * TPR + t;
-    if (valid && c < nvec) {
-      u32x4 rx = load16_stream(x + base + (int64_t)c * EPV);
-      Elem<T>::unpack(rx, v[i]);
-      if constexpr (ADD) {
-        float dv[EPV];
-        Elem<T>::unpack(load16_stream(delta + base + (int64_t)c * EPV), dv);
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) v[i][e] += dv[e];
-        // statistics come from the value a tensor add would have stored
-        u32x4 packed = Elem<T>::pack(v[i]);
-        store16(xn + base + (int64_t)c * EPV, packed);
-        Elem<T>::unpack(packed, v[i]);
-      }
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) ss += LN ? v[i][e] : v[i][e] * v[i][e];
+    if (c < nvec) {
+      load_w<T, WT>(w, c * EPV, wv[i]);
     } else {
 #pragma unroll
-      for (int e = 0; e < EPV; ++e) v[i][e] = 0.f;
+      for (int e = 0; e < EPV; ++e) wv[i][e] = 0.f;
     }
   }
-  ss = row_reduce<TPR, OpSum>(ss, smem, rib, t);
-  float mu = 0.f;
-  if constexpr (LN) {
-    // mean first, then the centred second moment: the row is in registers, so the second
-    // sweep is free and there is no E[x^2] - mean^2 cancellation
-    mu = ss / (float)d;
-    ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    const int c = i * TPR + t;
+    if (LN && bias != nullptr && c < nvec) {
+      load_w<T, WT>(bias, c * EPV, bv[i]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) bv[i][e] = 0.f;
+    }
+  }
+
+  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    const int64_t row = tile * RPB + rib;
+    const bool valid = row < n;
+    const int64_t base = row * (int64_t)d;
+
+    float v[ITERS][EPV];
+    float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < ITERS; ++i) {
       const int c = i * TPR + t;
       if (valid && c < nvec) {
+        u32x4 rx = load16_stream(x + base + (int64_t)c * EPV);
+        Elem<T>::unpack(rx, v[i]);
+        if constexpr (ADD) {
+          float dv[EPV];
+          Elem<T>::unpack(load16_stream(delta + base + (int64_t)c * EPV), dv);
 #pragma unroll
-        for (int e = 0; e < EPV; ++e) ss += (v[i][e] - mu) * (v[i][e] - mu);
+          for (int e = 0; e < EPV; ++e) v[i][e] += dv[e];
+          // statistics come from the value a tensor add would have stored
+          u32x4 packed = Elem<T>::pack(v[i]);
+          store16(xn + base + (int64_t)c * EPV, packed);
+          Elem<T>::unpack(packed, v[i]);
+        }
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) ss += LN ? v[i][e] : v[i][e] * v[i][e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) v[i][e] = 0.f;
       }
     }
     ss = row_reduce<TPR, OpSum>(ss, smem, rib, t);
-  }
-  const float r = rsqrtf(ss / (float)d + eps);
-  if (valid && t == 0) {
-    rstd[row] = r;
-    if constexpr (LN) mean[row] = mu;
-  }
+    float mu = 0.f;
+    if constexpr (LN) {
+      // mean first, then the centred second moment: the row is in registers, so the second
+      // sweep is free and there is no E[x^2] - mean^2 cancellation
+      mu = ss / (float)d;
+      ss = 0.f;
 #pragma unroll
-  for (int i = 0; i < ITERS; ++i) {
-    const int c = i * TPR + t;
-    if (valid && c < nvec) {
-      float wv[EPV], o[EPV];
-      load_w<T, WT>(w, c * EPV, wv);
+      for (int i = 0; i < ITERS; ++i) {
+        const int c = i * TPR + t;
+        if (valid && c < nvec) {
 #pragma unroll
-      for (int e = 0; e < EPV; ++e) o[e] = ((v[i][e] - mu) * r) * wv[e];
-      if constexpr (LN) {
-        if (bias != nullptr) {
-          float bv[EPV];
-          load_w<T, WT>(bias, c * EPV, bv);
-#pragma unroll
-          for (int e = 0; e < EPV; ++e) o[e] += bv[e];
+          for (int e = 0; e < EPV; ++e) ss += (v[i][e] - mu) * (v[i][e] - mu);
         }
       }
-      store16_stream(y + base + (int64_t)c * EPV, Elem<T>::pack(o));
+      ss = row_reduce<TPR, OpSum>(ss, smem, rib, t);
+    }
+    const float r = rsqrtf(ss / (float)d + eps);
+    if (valid && t == 0) {
+      rstd[row] = r;
+      if constexpr (LN) mean[row] = mu;
+    }
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = i * TPR + t;
+      if (valid && c < nvec) {
+        float o[EPV];
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] = ((v[i][e] - mu) * r) * wv[i][e];
+        if constexpr (LN) {
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) o[e] += bv[i][e];
+        }
+        store16_stream(y + base + (int64_t)c * EPV, Elem<T>::pack(o));
+      }
     }
   }
 }
@@ -526,6 +551,16 @@ Plan make_plan(int64_t n, int64_t d, int x_dtype, bool aligned) {
   X(4, 1) X(8, 1) X(16, 1) X(32, 1) X(64, 1) X(128, 1) X(64, 2) X(64, 3) X(128, 2) X(128, 3)    \
   X(256, 2) X(256, 3) X(256, 4) X(512, 2) X(512, 3) X(1024, 2) X(1024, 3) X(1024, 4)
 
+// Persistent grid of the forward: every workgroup slot of the device exactly once, so the
+// hardware places the same number of workgroups on every compute unit.
+inline int64_t fwd_grid(const Plan& p, int occupancy) {
+  int per_cu = fm_host::get_param(fm_host::P_NORM_FWD_BLOCKS_PER_CU);
+  if (per_cu <= 0) per_cu = occupancy;
+  int64_t g = (int64_t)fm_host::num_cus() * per_cu;
+  if (g > p.tiles) g = p.tiles;
+  return g < 1 ? 1 : g;
+}
+
 template <typename T, typename WT, bool ADD, bool LN>
 int launch_fwd(const Plan& p, const void* x, const void* delta, const void* w, const void* bias,
                void* xn, void* y, float* mean, float* rstd, int64_t n, int64_t d, float eps,
@@ -543,9 +578,18 @@ int launch_fwd(const Plan& p, const void* x, const void* delta, const void* w, c
   }
 #define X(TPR_, IT_)                                                                            \
   if (p.tpr == TPR_ && p.iters == IT_) {                                                        \
-    hipLaunchKernelGGL((norm_fwd_kernel<T, WT, TPR_, IT_, ADD, LN>), dim3((unsigned)p.tiles),   \
-                       dim3(BlockOf<TPR_>::value), 0, st, xp, dp, wp, bp, xnp, yp, mean, rstd, n, \
-                       (int)d, eps);                                                            \
+    static int occupancy = 0; /* workgroups of this kernel one compute unit holds */            \
+    if (occupancy == 0) {                                                                       \
+      int o = 0;                                                                                \
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(                                         \
+              &o, norm_fwd_kernel<T, WT, TPR_, IT_, ADD, LN>, BlockOf<TPR_>::value, 0) != hipSuccess || \
+          o < 1)                                                                                \
+        o = 2048 / BlockOf<TPR_>::value;                                                        \
+      occupancy = o;                                                                            \
+    }                                                                                           \
+    hipLaunchKernelGGL((norm_fwd_kernel<T, WT, TPR_, IT_, ADD, LN>),                            \
+                       dim3((unsigned)fwd_grid(p, occupancy)), dim3(BlockOf<TPR_>::value), 0, st, \
+                       xp, dp, wp, bp, xnp, yp, mean, rstd, n, (int)d, eps, p.tiles);           \
     return FM_OK;                                                                               \
   }
   FM_FOR_EACH_SHAPE(X)
