@@ -49,7 +49,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="ce",
-                    choices=["ce", "ce_one_pass", "rmsnorm", "add_rmsnorm", "add_layernorm", "kl", "kl_topk", "topk", "route", "moe_dispatch"])
+                    choices=["ce", "ce_one_pass", "rmsnorm", "add_rmsnorm", "add_layernorm", "kl", "kl_topk", "topk", "route", "moe_dispatch", "swiglu", "qk_norm_rope"])
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
@@ -315,6 +315,70 @@ def make_workload(name, torch, L, dev):
         w.rows = n
         return w
 
+    if name == "swiglu":
+        rows, h = 16384, 14336
+        g.manual_seed(1041)
+        x = torch.randn(rows, 2 * h, device=dev, generator=g).bfloat16()
+        dy = torch.randn(rows, h, device=dev, generator=g).bfloat16()
+        y = torch.empty(rows, h, device=dev, dtype=torch.bfloat16)
+        dx = torch.empty_like(x)
+
+        def fwd():
+            _check(L.fm_swiglu_split_fwd(x.data_ptr(), y.data_ptr(), rows, h, BF, st), "fm_swiglu_split_fwd")
+
+        def bwd():
+            _check(L.fm_swiglu_split_bwd(x.data_ptr(), dy.data_ptr(), dx.data_ptr(), rows, h, BF, st),
+                   "fm_swiglu_split_bwd")
+
+        def step():
+            fwd()
+            bwd()
+
+        w.step = step
+        w.dominant_launch = bwd
+        w.dominant = "swiglu_split_bwd_kernel<bf16>"
+        w.dominant_bytes = rows * h * 2 * 5          # gate, up, dy in; dgate, dup out
+        w.bytes = rows * h * 2 * 8                   # + gate, up in; y out
+        w.desc = f"SwiGLU on a fused projection fwd+bwd, x bf16 [{rows},{2 * h}] -> y [{rows},{h}]"
+        w.rows = rows
+        return w
+
+    if name == "qk_norm_rope":
+        b, t, hh, d = 8, 4096, 32, 128
+        g.manual_seed(1042)
+        x = torch.randn(b, t, hh, d, device=dev, generator=g).bfloat16()
+        do = torch.randn(b, t, hh, d, device=dev, generator=g).bfloat16()
+        wt = 1 + 0.02 * torch.randn(d, device=dev, generator=g)
+        ang = torch.rand(t, d // 2, device=dev, generator=g) * 6.28
+        cs, sn = torch.cos(ang), torch.sin(ang)
+        out, dx = torch.empty_like(x), torch.empty_like(x)
+        rstd = torch.empty(b * t * hh, device=dev)
+        dw = torch.empty_like(wt)
+        nb = L.fm_qk_norm_rope_bwd_workspace(b, t, hh, d)
+        ws = torch.empty(max(nb, 16), device=dev, dtype=torch.uint8)
+
+        def fwd():
+            _check(L.fm_qk_norm_rope_fwd(x.data_ptr(), wt.data_ptr(), cs.data_ptr(), sn.data_ptr(), out.data_ptr(),
+                                         rstd.data_ptr(), b, t, hh, d, BF, F32c, 1e-6, st), "fm_qk_norm_rope_fwd")
+
+        def bwd():
+            _check(L.fm_qk_norm_rope_bwd(x.data_ptr(), wt.data_ptr(), cs.data_ptr(), sn.data_ptr(), rstd.data_ptr(),
+                                         do.data_ptr(), dx.data_ptr(), dw.data_ptr(), ws.data_ptr(), nb, b, t, hh,
+                                         d, BF, F32c, st), "fm_qk_norm_rope_bwd")
+
+        def step():
+            fwd()
+            bwd()
+
+        w.step = step
+        w.dominant_launch = bwd
+        w.dominant = "qk_norm_rope_bwd_kernel<bf16,f32>"
+        w.dominant_bytes = b * t * hh * d * 2 * 3
+        w.bytes = b * t * hh * d * 2 * 5
+        w.desc = f"per-head RMSNorm + RoPE fwd+bwd, x bf16 [{b},{t},{hh},{d}], w fp32"
+        w.rows = b * t * hh
+        return w
+
     if name == "route":
         n, e, k = 16384, 64, 2
         g.manual_seed(1003)
@@ -556,7 +620,7 @@ def main():
     torch.cuda.empty_cache()
     if not a.no_extras:
         extras = {a.workload: res}
-        for name in ["rmsnorm", "add_rmsnorm", "add_layernorm", "ce", "ce_one_pass", "kl", "kl_topk", "topk", "route", "moe_dispatch"]:
+        for name in ["rmsnorm", "add_rmsnorm", "add_layernorm", "ce", "ce_one_pass", "kl", "kl_topk", "topk", "route", "moe_dispatch", "swiglu", "qk_norm_rope"]:
             if name == a.workload:
                 continue
             wl = make_workload(name, torch, L, dev)

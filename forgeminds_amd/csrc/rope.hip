@@ -7,8 +7,12 @@
 // then the RMSNorm backward of norm.hip; dw = sum over heads of dy * xhat in fp32, written as
 // one partial row per workgroup and summed in a fixed order.
 //
-// Heads are short (64-256 elements), so a head is owned by a group of G lanes; a lane holds up
-// to four consecutive elements of each half, which keeps both rotation partners in one thread.
+// Heads are short (64-256 elements), so a head is owned by a group of G lanes; a lane holds one
+// 16-byte vector of each half (the same columns of both), which keeps both rotation partners
+// in one thread and every access 16 bytes wide. Head dims that do not split into 16-byte
+// vectors per half, or unaligned buffers, use a scalar variant (four elements of each half per
+// lane). Grids are persistent: the weight columns stay in registers, cos/sin rows are shared by
+// the heads of a token and come from cache.
 #include "fm_common.cuh"
 
 using namespace fm;
@@ -118,61 +122,224 @@ __global__ __launch_bounds__(kBlock) void rope_kernel(const T* __restrict__ x, c
   }
 }
 
-template <typename WT>
-__global__ __launch_bounds__(256) void rope_colsum_kernel(const float* __restrict__ partial,
-                                                           WT* __restrict__ dw, int p, int d) {
-  const int col = blockIdx.x * 256 + threadIdx.x;
-  if (col >= d) return;
-  float a = 0.f;
-  for (int r = 0; r < p; ++r) a += partial[(int64_t)r * d + col];
-  Elem<WT>::store1(dw + col, a);
+// 16-byte loads of fp32 tables that line up with one vector of activations
+template <typename T>
+__device__ __forceinline__ void load_f32_cols(const float* p, float (&o)[Elem<T>::kVec]) {
+  constexpr int EPV = Elem<T>::kVec;
+#pragma unroll
+  for (int q = 0; q < EPV / 4; ++q) {
+    float a[4];
+    Elem<float>::unpack(load16(p + 4 * q), a);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[4 * q + i] = a[i];
+  }
 }
 
-struct Shape { int g; int64_t tiles; int blocks; };
+template <typename T, typename WT>
+__device__ __forceinline__ void load_w_cols(const WT* p, float (&o)[Elem<T>::kVec]) {
+  constexpr int EPV = Elem<T>::kVec;
+#pragma unroll
+  for (int e = 0; e < EPV; ++e) o[e] = Elem<WT>::load1(p + e);
+}
 
-bool make_shape(int64_t rows, int64_t d, Shape* s) {
+template <typename T, typename WT, int G, bool BWD>
+__global__ __launch_bounds__(kBlock) void rope_vec_kernel(const T* __restrict__ x, const WT* __restrict__ w,
+                                                           const float* __restrict__ cosv,
+                                                           const float* __restrict__ sinv,
+                                                           const T* __restrict__ dout,
+                                                           float* __restrict__ rstd, T* __restrict__ out,
+                                                           float* __restrict__ partial, int64_t rows,
+                                                           int t_len, int heads, int d, float eps,
+                                                           int64_t tiles) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int RPB = kBlock / G;
+  __shared__ float fold[BWD ? RPB * G * 2 * EPV : 1];
+  const int tid = threadIdx.x, rib = tid / G, l = tid % G;
+  const int half = d / 2;
+  const int col = l * EPV;               // this lane's columns in each half
+  const bool lane_on = col < half;
+  float wv1[EPV], wv2[EPV], a1[EPV], a2[EPV];
+#pragma unroll
+  for (int e = 0; e < EPV; ++e) { wv1[e] = 0.f; wv2[e] = 0.f; a1[e] = 0.f; a2[e] = 0.f; }
+  if (lane_on) {
+    load_w_cols<T, WT>(w + col, wv1);
+    load_w_cols<T, WT>(w + half + col, wv2);
+  }
+  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    const int64_t row = tile * RPB + rib;
+    const bool on = lane_on && row < rows;
+    const int t = row < rows ? (int)((row / heads) % t_len) : 0;
+    const T* xp = x + row * (int64_t)d;
+    float x1[EPV], x2[EPV], c[EPV], sn[EPV];
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) { x1[e] = 0.f; x2[e] = 0.f; c[e] = 0.f; sn[e] = 0.f; }
+    u32x4 r1, r2, q1, q2;
+    if (on) {
+      r1 = load16_stream(xp + col);
+      r2 = load16_stream(xp + half + col);
+      if constexpr (BWD) {
+        const T* gp = dout + row * (int64_t)d;
+        q1 = load16_stream(gp + col);
+        q2 = load16_stream(gp + half + col);
+      }
+      load_f32_cols<T>(cosv + (int64_t)t * half + col, c);
+      load_f32_cols<T>(sinv + (int64_t)t * half + col, sn);
+      Elem<T>::unpack(r1, x1);
+      Elem<T>::unpack(r2, x2);
+    }
+    if constexpr (!BWD) {
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) ss += x1[e] * x1[e] + x2[e] * x2[e];
+      ss = group_reduce<G, OpSum>(ss);
+      const float r = rsqrtf(ss / (float)d + eps);
+      if (row < rows && l == 0) rstd[row] = r;
+      if (on) {
+        float o1[EPV], o2[EPV];
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+          const float y1 = (x1[e] * r) * wv1[e], y2 = (x2[e] * r) * wv2[e];
+          o1[e] = y1 * c[e] - y2 * sn[e];
+          o2[e] = y1 * sn[e] + y2 * c[e];
+        }
+        T* op = out + row * (int64_t)d;
+        store16_stream(op + col, Elem<T>::pack(o1));
+        store16_stream(op + half + col, Elem<T>::pack(o2));
+      }
+    } else {
+      const float r = row < rows ? rstd[row] : 0.f;
+      float g1[EPV], g2[EPV];
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) { g1[e] = 0.f; g2[e] = 0.f; }
+      if (on) {
+        Elem<T>::unpack(q1, g1);
+        Elem<T>::unpack(q2, g2);
+      }
+      float dot = 0.f;
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        const float dy1 = g1[e] * c[e] + g2[e] * sn[e], dy2 = g2[e] * c[e] - g1[e] * sn[e];
+        x1[e] *= r; x2[e] *= r;                       // xhat
+        a1[e] += dy1 * x1[e]; a2[e] += dy2 * x2[e];
+        g1[e] = dy1 * wv1[e]; g2[e] = dy2 * wv2[e];
+        dot += g1[e] * x1[e] + g2[e] * x2[e];
+      }
+      dot = group_reduce<G, OpSum>(dot);
+      const float cm = dot / (float)d;
+      if (on) {
+        float o1[EPV], o2[EPV];
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+          o1[e] = (g1[e] - x1[e] * cm) * r;
+          o2[e] = (g2[e] - x2[e] * cm) * r;
+        }
+        T* op = out + row * (int64_t)d;
+        store16_stream(op + col, Elem<T>::pack(o1));
+        store16_stream(op + half + col, Elem<T>::pack(o2));
+      }
+    }
+  }
+  if constexpr (BWD) {
+    if (partial == nullptr) return;
+    // fold the rows of this workgroup in row order, then write one partial row
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) {
+      fold[(rib * 2 + 0) * G * EPV + col + e] = a1[e];
+      fold[(rib * 2 + 1) * G * EPV + col + e] = a2[e];
+    }
+    __syncthreads();
+    float* prow = partial + (int64_t)blockIdx.x * d;
+    for (int j = tid; j < d; j += kBlock) {
+      const int hsel = j >= half ? 1 : 0, jj = j - hsel * half;
+      float acc = 0.f;
+      for (int rr = 0; rr < RPB; ++rr) acc += fold[(rr * 2 + hsel) * G * EPV + jj];
+      prow[j] = acc;
+    }
+  }
+}
+
+// Column sum of the partial rows in a fixed order: 16 row groups x 64 columns per workgroup.
+template <typename WT>
+__global__ __launch_bounds__(1024) void rope_colsum_kernel(const float* __restrict__ partial,
+                                                            WT* __restrict__ dw, int p, int d) {
+  __shared__ float s[16][64];
+  const int lane = threadIdx.x & 63;
+  const int g = threadIdx.x >> 6;
+  const int col = blockIdx.x * 64 + lane;
+  float a = 0.f;
+  if (col < d) {
+    for (int r = g; r < p; r += 16) a += partial[(int64_t)r * d + col];
+  }
+  s[g][lane] = a;
+  __syncthreads();
+  if (g == 0 && col < d) {
+    float tot = s[0][lane];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) tot += s[i][lane];
+    Elem<WT>::store1(dw + col, tot);
+  }
+}
+
+struct Shape { int g; int gv; int64_t tiles; int64_t vtiles; int blocks; };
+
+// g: lanes per head of the scalar kernel; gv: of the vector kernel (0 when the head does not
+// split into 16-byte vectors per half). blocks: persistent grid, also the number of partial rows.
+bool make_shape(int64_t rows, int64_t d, int esize, Shape* s) {   // esize 0: scalar variant only
   if (d < 2 || d % 2 != 0) return false;
   const int64_t half = d / 2;
   int g = 1;
   while ((int64_t)g * kEH < half) g *= 2;
   if (g > 64) return false;
   s->g = g;
-  const int rpb = kBlock / g;
-  s->tiles = (rows + rpb - 1) / rpb;
-  int64_t blocks = (int64_t)fm_host::num_cus() * 4;
+  const int epv = esize > 0 ? 16 / esize : 1;
+  s->gv = 0;
+  if (esize > 0 && half % epv == 0) {
+    int gv = 1;
+    while ((int64_t)gv * epv < half) gv *= 2;
+    if (gv <= 64) s->gv = gv;
+  }
+  s->tiles = (rows + kBlock / g - 1) / (kBlock / g);
+  s->vtiles = s->gv ? (rows + kBlock / s->gv - 1) / (kBlock / s->gv) : 0;
+  // 8 workgroups of 256 threads per unit; the scalar variant never has fewer tiles than the
+  // vector one, so this bound holds for both and does not depend on the dtype
+  int64_t blocks = (int64_t)fm_host::num_cus() * 8;
   if (blocks > s->tiles) blocks = s->tiles;
   s->blocks = (int)(blocks < 1 ? 1 : blocks);
   return true;
 }
 
 template <typename T, typename WT, bool BWD>
-int launch(const Shape& sh, const void* x, const void* w, const float* c, const float* s, const void* dout,
-           float* rstd, void* out, float* partial, int64_t rows, int t_len, int heads, int d, float eps,
-           hipStream_t st) {
-  const int64_t blocks = BWD ? sh.blocks : sh.tiles;
-#define GO(G)                                                                                         \
-  hipLaunchKernelGGL((rope_kernel<T, WT, G, BWD>), dim3((unsigned)blocks), dim3(kBlock), 0, st,       \
+int launch(const Shape& sh, bool vec, const void* x, const void* w, const float* c, const float* s,
+           const void* dout, float* rstd, void* out, float* partial, int64_t rows, int t_len, int heads,
+           int d, float eps, hipStream_t st) {
+  const int64_t tiles = vec ? sh.vtiles : sh.tiles;
+  const int64_t blocks = sh.blocks < tiles ? sh.blocks : tiles;
+#define GO(KERNEL, G)                                                                                 \
+  hipLaunchKernelGGL((KERNEL<T, WT, G, BWD>), dim3((unsigned)blocks), dim3(kBlock), 0, st,            \
                      static_cast<const T*>(x), static_cast<const WT*>(w), c, s,                       \
                      static_cast<const T*>(dout), rstd, static_cast<T*>(out), partial, rows, t_len,   \
-                     heads, d, eps, sh.tiles)
-  switch (sh.g) {
-    case 1: GO(1); break;
-    case 2: GO(2); break;
-    case 4: GO(4); break;
-    case 8: GO(8); break;
-    case 16: GO(16); break;
-    case 32: GO(32); break;
-    default: GO(64); break;
+                     heads, d, eps, tiles)
+#define BY_G(KERNEL, g)           \
+  switch (g) {                    \
+    case 1: GO(KERNEL, 1); break; \
+    case 2: GO(KERNEL, 2); break; \
+    case 4: GO(KERNEL, 4); break; \
+    case 8: GO(KERNEL, 8); break; \
+    case 16: GO(KERNEL, 16); break; \
+    case 32: GO(KERNEL, 32); break; \
+    default: GO(KERNEL, 64); break; \
   }
+  if (vec) { BY_G(rope_vec_kernel, sh.gv) } else { BY_G(rope_kernel, sh.g) }
+#undef BY_G
 #undef GO
-  return FM_OK;
+  return (int)blocks;
 }
 
 int check(const char* what, int64_t b, int64_t t, int64_t h, int64_t d, int x_dtype, int w_dtype, Shape* sh) {
   FM_CHECK_ARG(b >= 0 && t > 0 && h > 0 && d > 0, "%s: bad shape", what);
   FM_CHECK_ARG(x_dtype == FM_F32 || x_dtype == FM_F16 || x_dtype == FM_BF16, "%s: bad x_dtype %d", what, x_dtype);
   FM_CHECK_ARG(w_dtype == x_dtype || w_dtype == FM_F32, "%s: w_dtype must equal x_dtype or be fp32", what);
-  if (b * t * h > 0x7fffffffLL || !make_shape(b * t * h, d, sh)) {
+  if (b * t * h > 0x7fffffffLL || !make_shape(b * t * h, d, x_dtype == FM_F32 ? 4 : 2, sh)) {
     fm_host::set_error("%s: head dim must be even and <= 512, rows < 2^31 (d=%lld)", what, (long long)d);
     return FM_ERR_UNSUPPORTED;
   }
@@ -185,7 +352,7 @@ extern "C" {
 
 size_t fm_qk_norm_rope_bwd_workspace(int64_t b, int64_t t, int64_t h, int64_t d) {
   Shape sh;
-  if (b <= 0 || t <= 0 || h <= 0 || !make_shape(b * t * h, d, &sh)) return 0;
+  if (b <= 0 || t <= 0 || h <= 0 || !make_shape(b * t * h, d, 0, &sh)) return 0;
   return (size_t)sh.blocks * (size_t)d * sizeof(float);
 }
 
@@ -199,7 +366,9 @@ int fm_qk_norm_rope_fwd(const void* x, const void* w, const float* cosv, const f
   FM_CHECK_ARG(x && w && cosv && sinv && out && rstd, "fm_qk_norm_rope_fwd: NULL pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int64_t rows = b * t * h;
-#define CALL(T, WT) launch<T, WT, false>(sh, x, w, cosv, sinv, nullptr, rstd, out, nullptr, rows, (int)t, (int)h, (int)d, eps, st)
+  const bool vec = sh.gv != 0 && fm_host::aligned16(x) && fm_host::aligned16(out) &&
+                   fm_host::aligned16(cosv) && fm_host::aligned16(sinv);
+#define CALL(T, WT) launch<T, WT, false>(sh, vec, x, w, cosv, sinv, nullptr, rstd, out, nullptr, rows, (int)t, (int)h, (int)d, eps, st)
   if (x_dtype == FM_F32) CALL(float, float);
   else if (x_dtype == FM_BF16 && w_dtype == FM_BF16) CALL(bf16_t, bf16_t);
   else if (x_dtype == FM_BF16) CALL(bf16_t, float);
@@ -230,12 +399,14 @@ int fm_qk_norm_rope_bwd(const void* x, const void* w, const float* cosv, const f
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int64_t rows = b * t * h;
+  const bool vec = sh.gv != 0 && fm_host::aligned16(x) && fm_host::aligned16(dx) && fm_host::aligned16(dout) &&
+                   fm_host::aligned16(cosv) && fm_host::aligned16(sinv);
 #define CALL(T, WT)                                                                                    \
-  launch<T, WT, true>(sh, x, w, cosv, sinv, dout, const_cast<float*>(rstd), dx, partial, rows, (int)t,  \
-                      (int)h, (int)d, 0.f, st);                                                        \
+  const int used = launch<T, WT, true>(sh, vec, x, w, cosv, sinv, dout, const_cast<float*>(rstd), dx,   \
+                                       partial, rows, (int)t, (int)h, (int)d, 0.f, st);                \
   if (partial != nullptr)                                                                              \
-    hipLaunchKernelGGL((rope_colsum_kernel<WT>), dim3((unsigned)((d + 255) / 256)), dim3(256), 0, st,   \
-                       partial, static_cast<WT*>(dw), sh.blocks, (int)d)
+    hipLaunchKernelGGL((rope_colsum_kernel<WT>), dim3((unsigned)((d + 63) / 64)), dim3(1024), 0, st,    \
+                       partial, static_cast<WT*>(dw), used, (int)d)
   if (x_dtype == FM_F32) { CALL(float, float); }
   else if (x_dtype == FM_BF16 && w_dtype == FM_BF16) { CALL(bf16_t, bf16_t); }
   else if (x_dtype == FM_BF16) { CALL(bf16_t, float); }
