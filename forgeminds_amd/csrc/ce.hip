@@ -27,6 +27,15 @@ __global__ __launch_bounds__(THREADS) void ce_fwd_kernel(const T* __restrict__ l
   const RowSplit sp = split_row<EPV>(row, v, vec_ok);
   const int tid = threadIdx.x;
 
+  // the label and its logit are fetched first, so the two dependent loads overlap the
+  // streaming pass instead of trailing it
+  int64_t y = 0;
+  float ylogit = 0.f;
+  if (tid == 0) {
+    y = labels[row];
+    if (y != ignore_index && y >= 0 && y < v) ylogit = Elem<T>::load1(rp + y);
+  }
+
   MaxSum st{kNegBig, 0.f};
   for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
     u32x4 raw[UNROLL];
@@ -69,11 +78,8 @@ __global__ __launch_bounds__(THREADS) void ce_fwd_kernel(const T* __restrict__ l
   if (tid == 0) {
     const float l = (tot.m + fast_log2(tot.s)) * kLn2;
     lse[row] = l;
-    const int64_t y = labels[row];
     float loss = 0.f;
-    if (y != ignore_index) {
-      loss = (y >= 0 && y < v) ? l - Elem<T>::load1(rp + y) : __builtin_nanf("");
-    }
+    if (y != ignore_index) loss = (y >= 0 && y < v) ? l - ylogit : __builtin_nanf("");
     row_loss[row] = loss;
   }
 }
@@ -227,6 +233,8 @@ __global__ __launch_bounds__(THREADS) void ce_loss_grad_kernel(const T* logits,
     return;
   }
   const int y = (y64 >= 0 && y64 < v) ? (int)y64 : -1;
+  float ylogit = 0.f;
+  if (tid == 0 && y >= 0) ylogit = Elem<T>::load1(rp + y);   // early: overlaps the row loads
 
   u32x4 raw[ITERS];
 #pragma unroll
@@ -270,9 +278,8 @@ __global__ __launch_bounds__(THREADS) void ce_loss_grad_kernel(const T* logits,
   if (tid == 0) {
     const float l = l2 * kLn2;
     if (lse != nullptr) lse[row] = l;
-    row_loss[row] = y >= 0 ? l - Elem<T>::load1(rp + y) : __builtin_nanf("");
+    row_loss[row] = y >= 0 ? l - ylogit : __builtin_nanf("");
   }
-  __syncthreads();   // the label logit is read before any thread overwrites it in place
 #pragma unroll
   for (int i = 0; i < ITERS; ++i) {
     const int c = i * THREADS + tid;
