@@ -2,8 +2,11 @@
 //
 // Reference semantics: forgemind/kernels/softmax.py:27-80 (y = exp(x - max) / sum, fp32
 // math, stored in x's dtype; NaN propagates, a row of -inf yields NaN like torch).
-// One workgroup per row: an online (max, sum-exp) pass, then a second pass over the row
-// (served by L2 for rows that fit) that writes exp2(z - m) / s.
+// Rows of up to 128 KiB whose width is a whole number of 16-byte vectors stay in registers:
+// a row is owned by TPR threads (a lane group, a wave or the waves of one workgroup, several
+// rows per workgroup when they are narrow), read once, reduced (maximum, then sum) and written.
+// Other rows take one workgroup each: an online (max, sum-exp) pass, then a second pass over
+// the row (served by L2 for rows that fit) that writes exp2(z - m) / s.
 #include "fm_vocab.cuh"
 
 using namespace fm;
@@ -76,10 +79,95 @@ __global__ __launch_bounds__(THREADS) void softmax_kernel(const T* __restrict__ 
   }
 }
 
+template <int TPR> struct RowBlock { static constexpr int value = TPR > 256 ? TPR : 256; };
+
+template <typename T, int TPR, int ITERS>
+__global__ __launch_bounds__(RowBlock<TPR>::value) void softmax_rows_kernel(const T* __restrict__ x,
+                                                                             T* __restrict__ y, int64_t n,
+                                                                             int v) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int BLOCK = RowBlock<TPR>::value;
+  constexpr int RPB = BLOCK / TPR;
+  __shared__ float smem[RPB * (TPR > 64 ? TPR / 64 : 1)];
+  const int tid = threadIdx.x;
+  const int rib = tid / TPR;
+  const int t = tid % TPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + rib;
+  const bool valid = row < n;
+  const int nvec = v / EPV;
+  const int64_t base = row * (int64_t)v;
+
+  float z[ITERS][EPV];
+  float m = kNegBig;
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * TPR + t;
+    if (valid && c < nvec) {
+      Elem<T>::unpack(load16_stream(x + base + (int64_t)c * EPV), z[i]);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) { z[i][e] *= kLog2e; m = fmaxf(m, z[i][e]); }
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) z[i][e] = -INFINITY;
+    }
+  }
+  // a NaN anywhere must reach the whole row: fmaxf drops it, so it is carried in the sum
+  m = row_reduce<TPR, OpMax>(m, smem, rib, t);
+  float ssum = 0.f;
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) {
+      z[i][e] = fast_exp2(z[i][e] - m);
+      ssum += z[i][e];
+    }
+  }
+  ssum = row_reduce<TPR, OpSum>(ssum, smem, rib, t);
+  // a row whose maximum is -inf has sum 0: 0 * inf = NaN, which is what torch returns
+  const float inv = 1.f / ssum;
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * TPR + t;
+    if (valid && c < nvec) {
+      float o[EPV];
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) o[e] = z[i][e] * inv;
+      store16_stream(y + base + (int64_t)c * EPV, Elem<T>::pack(o));
+    }
+  }
+}
+
+#define FM_SOFTMAX_SHAPES(X) \
+  X(4, 1) X(8, 1) X(16, 1) X(32, 1) X(64, 1) X(64, 2) X(128, 2) X(256, 2) X(256, 4) X(512, 4) X(512, 8) X(1024, 8)
+
+// threads per row and vectors per thread for a row of nvec 16-byte vectors; false: too wide
+bool rows_plan(int64_t nvec, int* tpr, int* iters) {
+  static const int kPlans[][3] = {{4, 4, 1},     {8, 8, 1},      {16, 16, 1},    {32, 32, 1},
+                                  {64, 64, 1},   {128, 64, 2},   {256, 128, 2},  {512, 256, 2},
+                                  {1024, 256, 4}, {2048, 512, 4}, {4096, 512, 8}, {8192, 1024, 8}};
+  for (auto& pl : kPlans) {
+    if (nvec <= pl[0]) { *tpr = pl[1]; *iters = pl[2]; return true; }
+  }
+  return false;
+}
+
 template <typename T>
 void launch(const void* x, void* y, int64_t n, int v, bool vec_ok, hipStream_t st) {
   const T* xp = static_cast<const T*>(x);
   T* yp = static_cast<T*>(y);
+  constexpr int EPV = Elem<T>::kVec;
+  int tpr = 0, iters = 0;
+  if (vec_ok && v % EPV == 0 && rows_plan(v / EPV, &tpr, &iters)) {
+#define X(TPR_, IT_)                                                                               \
+  if (tpr == TPR_ && iters == IT_) {                                                               \
+    constexpr int RPB = RowBlock<TPR_>::value / TPR_;                                              \
+    hipLaunchKernelGGL((softmax_rows_kernel<T, TPR_, IT_>), dim3((unsigned)((n + RPB - 1) / RPB)), \
+                       dim3(RowBlock<TPR_>::value), 0, st, xp, yp, n, v);                          \
+    return;                                                                                        \
+  }
+    FM_SOFTMAX_SHAPES(X)
+#undef X
+  }
   const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 4);
   const dim3 grid((unsigned)n);
 #define LAUNCH(TH, UN) \

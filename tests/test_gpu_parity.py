@@ -551,7 +551,10 @@ def test_topk_unaligned_rows():
 
 # ------------------------------------------------------------------ softmax
 @pytest.mark.parametrize("n,v,dt", [(4, 64, F32), (5, 1000, F32), (3, 4096, F32), (7, 1, F32),
-                                     (8, 50257, BF16), (6, 300, F16), (2, 128256, BF16)])
+                                     (8, 50257, BF16), (6, 300, F16), (2, 128256, BF16),
+                                     (1000, 64, F32), (77, 16, BF16), (3, 4, F32), (33, 512, BF16),
+                                     (130, 8, F16), (9, 8192, BF16), (5, 32768, F16), (3, 65536, BF16),
+                                     (257, 2048, F32), (4, 32000, BF16)])
 def test_softmax(n, v, dt):
     x = torch.randn(n, v, generator=gen(21)).to(dt)
     y = _hip.softmax_fwd(x.to(DEV))
