@@ -33,6 +33,12 @@ __device__ __forceinline__ float float_of_key(uint32_t k) {
   return __builtin_bit_cast(float, b);
 }
 
+// Bits of the key that a value of type T can set (the rest are all-zero or, for negative
+// values, all-one): bf16 keeps 16, fp16 19 (sign, fp32 exponent, 10 mantissa bits), fp32 all.
+template <typename T> struct KeyBits { static constexpr uint32_t mask = 0xFFFFFFFFu; static constexpr int low = 0; };
+template <> struct KeyBits<bf16_t> { static constexpr uint32_t mask = 0xFFFF0000u; static constexpr int low = 16; };
+template <> struct KeyBits<f16_t> { static constexpr uint32_t mask = 0xFFFFE000u; static constexpr int low = 13; };
+
 __device__ __forceinline__ int block_sum_int(int v, int* smem, int nw) {
   v = wave_sum_i(v);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -116,7 +122,7 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
   constexpr int EPV = Elem<T>::kVec;
   constexpr int NW = THREADS / 64;
   constexpr int ITERS = NV;
-  constexpr uint32_t KMASK = sizeof(T) == 2 ? 0xFFFF0000u : 0xFFFFFFFFu;
+  constexpr uint32_t KMASK = KeyBits<T>::mask;
   unsigned long long* ccomp = sh.ccomp;
   int* crank = sh.crank;
   int* work = sh.work;
@@ -246,7 +252,7 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
         return block_sum_int(cnt, s_int, NW);
       };
       uint32_t kth = 0u;
-      for (int bit = 31; bit >= (sizeof(T) == 2 ? 16 : 0); --bit) {
+      for (int bit = 31; bit >= KeyBits<T>::low; --bit) {
         const uint32_t trial = kth | (1u << bit);
         const int cnt = count_if([&](uint32_t key) { return key >= trial; });
         if (cnt >= k) kth = trial;

@@ -531,6 +531,16 @@ def test_topk_ties_nans_zeros_and_degenerate_rows():
     x[:, ::7] = float("nan")
     x[:, 5::11] = float("-inf")
     assert torch.equal(run(x, 512), O.topk(x, 512)[1])
+    # fp16 values that differ only in their last three mantissa bits, in long runs: the exact
+    # path must order them by value, not by position
+    steps = torch.randint(0, 8, (3, 6000), generator=g).float()
+    x = (1.0 + steps * 2.0 ** -10).to(F16) * torch.where(torch.rand(3, 6000, generator=g) < 0.5, 1.0, -1.0).to(F16)
+    for k in (5, 100, 512):
+        assert torch.equal(run(x, k), O.topk(x, k)[1])
+    # k close to the row width: the per-wave threshold admits everything, the exact path decides
+    for dt, v, k in ((BF16, 2048, 256), (F32, 1500, 300), (F16, 4096, 512), (BF16, 1100, 512)):
+        x = (3 * torch.randn(5, v, generator=g)).to(dt)
+        assert torch.equal(run(x, k), O.topk(x, k)[1])
     # negative NaN payloads and a row of -inf
     x = torch.full((2, 3000), float("-inf"))
     x[0, 17] = -torch.tensor(float("nan"))
