@@ -13,7 +13,7 @@
 // vectors per half, or unaligned buffers, use a scalar variant (four elements of each half per
 // lane). Grids are persistent: the weight columns stay in registers, cos/sin rows are shared by
 // the heads of a token and come from cache.
-#include "fm_common.cuh"
+#include "fm_norm.cuh"   // colsum_kernel / colsum_scalar_kernel: fixed-order column sums of partial rows
 
 using namespace fm;
 
@@ -258,28 +258,6 @@ __global__ __launch_bounds__(kBlock) void rope_vec_kernel(const T* __restrict__ 
   }
 }
 
-// Column sum of the partial rows in a fixed order: 16 row groups x 64 columns per workgroup.
-template <typename WT>
-__global__ __launch_bounds__(1024) void rope_colsum_kernel(const float* __restrict__ partial,
-                                                            WT* __restrict__ dw, int p, int d) {
-  __shared__ float s[16][64];
-  const int lane = threadIdx.x & 63;
-  const int g = threadIdx.x >> 6;
-  const int col = blockIdx.x * 64 + lane;
-  float a = 0.f;
-  if (col < d) {
-    for (int r = g; r < p; r += 16) a += partial[(int64_t)r * d + col];
-  }
-  s[g][lane] = a;
-  __syncthreads();
-  if (g == 0 && col < d) {
-    float tot = s[0][lane];
-#pragma unroll
-    for (int i = 1; i < 16; ++i) tot += s[i][lane];
-    Elem<WT>::store1(dw + col, tot);
-  }
-}
-
 struct Shape { int g; int gv; int64_t tiles; int64_t vtiles; int blocks; };
 
 // g: lanes per head of the scalar kernel; gv: of the vector kernel (0 when the head does not
@@ -404,9 +382,14 @@ int fm_qk_norm_rope_bwd(const void* x, const void* w, const float* cosv, const f
 #define CALL(T, WT)                                                                                    \
   const int used = launch<T, WT, true>(sh, vec, x, w, cosv, sinv, dout, const_cast<float*>(rstd), dx,   \
                                        partial, rows, (int)t, (int)h, (int)d, 0.f, st);                \
-  if (partial != nullptr)                                                                              \
-    hipLaunchKernelGGL((rope_colsum_kernel<WT>), dim3((unsigned)((d + 63) / 64)), dim3(1024), 0, st,    \
-                       partial, static_cast<WT*>(dw), used, (int)d)
+  if (partial != nullptr) {                                                                            \
+    if (d % 4 == 0)                                                                                    \
+      hipLaunchKernelGGL((colsum_kernel<WT>), dim3((unsigned)((d + 63) / 64)), dim3(1024), 0, st,       \
+                         partial, static_cast<WT*>(dw), used, (int)d, (int)d);                         \
+    else                                                                                               \
+      hipLaunchKernelGGL((colsum_scalar_kernel<WT>), dim3((unsigned)((d + 63) / 64)), dim3(1024), 0, st, \
+                         partial, static_cast<WT*>(dw), used, (int)d, (int)d);                         \
+  }
   if (x_dtype == FM_F32) { CALL(float, float); }
   else if (x_dtype == FM_BF16 && w_dtype == FM_BF16) { CALL(bf16_t, bf16_t); }
   else if (x_dtype == FM_BF16) { CALL(bf16_t, float); }
