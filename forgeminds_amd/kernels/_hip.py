@@ -8,6 +8,7 @@ the library's message on a non-zero status. Outputs are allocated by the callers
 
 from __future__ import annotations
 
+import contextlib
 import ctypes as C
 import os
 import threading
@@ -133,8 +134,24 @@ def _ptr(t: "torch.Tensor | None"):
     return None if t is None else t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor):
+    """The raw ``hipStream_t`` torch is currently enqueueing on for ``t``'s device."""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index if t.device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+_SAME_DEVICE = contextlib.nullcontext()
+
+
+def _guard(dev: torch.device):
+    """Make ``dev`` current for the launch; free when it already is (the usual case)."""
+    if dev.index is None or dev.index == torch.cuda.current_device():
+        return _SAME_DEVICE
+    return torch.cuda.device(dev)
 
 
 def _check(rc: int, what: str) -> None:
@@ -160,17 +177,23 @@ def rmsnorm_fwd(x2: torch.Tensor, w: torch.Tensor, eps: float):
     n, d = x2.shape
     y = torch.empty_like(x2)
     rstd = torch.empty(n, device=x2.device, dtype=torch.float32)
-    with torch.cuda.device(x2.device):
+    with _guard(x2.device):
         _check(lib().fm_rmsnorm_fwd(_ptr(x2), _ptr(w), _ptr(y), _ptr(rstd), n, d,
                                     dtype_code(x2.dtype), dtype_code(w.dtype), float(eps),
                                     _stream(x2)), "fm_rmsnorm_fwd")
     return y, rstd
 
 
+_WS_BYTES: dict = {}     # (device, rows, width, dtype) -> bytes; the answer depends on nothing else
+
+
 def _norm_ws(n: int, d: int, x: torch.Tensor, want_dw: bool):
     if not want_dw:
         return None, 0
-    nbytes = int(lib().fm_rmsnorm_bwd_workspace(n, d, dtype_code(x.dtype)))
+    key = (x.device.index, n, d, x.dtype)
+    nbytes = _WS_BYTES.get(key)
+    if nbytes is None:
+        nbytes = _WS_BYTES[key] = int(lib().fm_rmsnorm_bwd_workspace(n, d, dtype_code(x.dtype)))
     return torch.empty(max(nbytes, 16), device=x.device, dtype=torch.uint8), nbytes
 
 
@@ -180,7 +203,7 @@ def rmsnorm_bwd(x2, w, rstd, dy2, want_dw: bool = True):
     n, d = x2.shape
     dx = torch.empty_like(x2)
     dw = torch.empty_like(w) if want_dw else None
-    with torch.cuda.device(x2.device):
+    with _guard(x2.device):
         ws, nbytes = _norm_ws(n, d, x2, want_dw)
         _check(lib().fm_rmsnorm_bwd(_ptr(x2), _ptr(w), _ptr(rstd), _ptr(dy2), _ptr(dx), _ptr(dw),
                                     _ptr(ws), nbytes, n, d, dtype_code(x2.dtype),
@@ -195,7 +218,7 @@ def add_rmsnorm_fwd(x2, delta2, w, eps: float):
     xn = torch.empty_like(x2)
     y = torch.empty_like(x2)
     rstd = torch.empty(n, device=x2.device, dtype=torch.float32)
-    with torch.cuda.device(x2.device):
+    with _guard(x2.device):
         _check(lib().fm_add_rmsnorm_fwd(_ptr(x2), _ptr(delta2), _ptr(w), _ptr(xn), _ptr(y),
                                         _ptr(rstd), n, d, dtype_code(x2.dtype),
                                         dtype_code(w.dtype), float(eps), _stream(x2)),
@@ -209,7 +232,7 @@ def add_rmsnorm_bwd(xn2, w, rstd, gy2, gxn2, want_dw: bool = True):
     n, d = xn2.shape
     dx = torch.empty_like(xn2)
     dw = torch.empty_like(w) if want_dw else None
-    with torch.cuda.device(xn2.device):
+    with _guard(xn2.device):
         ws, nbytes = _norm_ws(n, d, xn2, want_dw)
         _check(lib().fm_add_rmsnorm_bwd(_ptr(xn2), _ptr(w), _ptr(rstd), _ptr(gy2), _ptr(gxn2),
                                         _ptr(dx), None, _ptr(dw), _ptr(ws), nbytes, n, d,
@@ -225,7 +248,7 @@ def layernorm_fwd(x2, w, b, eps: float, delta2=None):
     y = torch.empty_like(x2)
     stats = torch.empty(2, n, device=x2.device, dtype=torch.float32)
     xn = torch.empty_like(x2) if delta2 is not None else None
-    with torch.cuda.device(x2.device):
+    with _guard(x2.device):
         if delta2 is None:
             _check(lib().fm_layernorm_fwd(_ptr(x2), _ptr(w), _ptr(b), _ptr(y), stats[0].data_ptr(),
                                           stats[1].data_ptr(), n, d, dtype_code(x2.dtype),
@@ -245,7 +268,7 @@ def layernorm_bwd(x2, w, mean, rstd, dy2, gxn2=None, want_dw: bool = True, want_
     dx = torch.empty_like(x2)
     dw = torch.empty_like(w) if want_dw else None
     db = torch.empty_like(w) if want_db else None
-    with torch.cuda.device(x2.device):
+    with _guard(x2.device):
         ws, nbytes = None, 0
         if want_dw or want_db:
             nbytes = int(lib().fm_layernorm_bwd_workspace(n, d, dtype_code(x2.dtype)))
@@ -266,7 +289,7 @@ def ce_fwd(logits2, labels, ignore_index: int, reduction: str):
     lse = torch.empty(n, device=dev, dtype=torch.float32)
     row_loss = torch.empty(n, device=dev, dtype=torch.float32)
     scal = torch.empty(2, device=dev, dtype=torch.float32)
-    with torch.cuda.device(dev):
+    with _guard(dev):
         _check(lib().fm_ce_fwd(_ptr(logits2), _ptr(labels), _ptr(lse), _ptr(row_loss),
                                scal.data_ptr(), scal.data_ptr() + 4, n, v,
                                dtype_code(logits2.dtype), int(ignore_index), REDUCE[reduction],
@@ -283,7 +306,7 @@ def ce_loss_grad(logits2, labels, ignore_index: int, reduction: str, inplace: bo
     buf = torch.empty(2, max(n, 1), device=dev, dtype=torch.float32)
     scalars = torch.empty(2, device=dev, dtype=torch.float32)
     dl = logits2 if inplace else torch.empty_like(logits2)
-    with torch.cuda.device(dev):
+    with _guard(dev):
         def call(out):
             return lib().fm_ce_loss_grad(_ptr(logits2), _ptr(labels), buf[0].data_ptr(), buf[1].data_ptr(),
                                          scalars[0:].data_ptr(), scalars[1:].data_ptr(), _ptr(out), n, v,
@@ -300,7 +323,7 @@ def ce_loss_grad(logits2, labels, ignore_index: int, reduction: str, inplace: bo
 def scale_inplace(x, factor):
     """x *= factor (fp32 device scalar), skipped on the device when the factor is exactly 1."""
     _dense(x, factor)
-    with torch.cuda.device(x.device):
+    with _guard(x.device):
         _check(lib().fm_scale_inplace(_ptr(x), _ptr(factor), x.numel(), dtype_code(x.dtype), _stream(x)),
                "fm_scale_inplace")
     return x
@@ -311,7 +334,7 @@ def ce_bwd(logits2, labels, lse, n_valid, grad_out, ignore_index: int):
     _dense(logits2, labels, lse)
     n, v = logits2.shape
     dl = torch.empty_like(logits2)
-    with torch.cuda.device(logits2.device):
+    with _guard(logits2.device):
         _check(lib().fm_ce_bwd(_ptr(logits2), _ptr(labels), _ptr(lse), _ptr(n_valid),
                                _ptr(grad_out), _ptr(dl), n, v, dtype_code(logits2.dtype),
                                int(ignore_index), _stream(logits2)), "fm_ce_bwd")
@@ -326,7 +349,7 @@ def kl_fwd(s2, t2, inv_temperature: float, reduction: str):
     dev = s2.device
     buf = torch.empty(3, n, device=dev, dtype=torch.float32)
     loss = torch.empty((), device=dev, dtype=torch.float32) if reduction != "none" else None
-    with torch.cuda.device(dev):
+    with _guard(dev):
         _check(lib().fm_kl_fwd(_ptr(s2), _ptr(t2), buf[0].data_ptr(), buf[1].data_ptr(),
                                buf[2].data_ptr(), _ptr(loss), n, v, dtype_code(s2.dtype),
                                float(inv_temperature), REDUCE[reduction], _stream(s2)), "fm_kl_fwd")
@@ -343,7 +366,7 @@ def kl_loss_grad(s2, t2, inv_temperature: float, reduction: str, grad_dtype, inp
     loss = torch.empty((), device=dev, dtype=torch.float32)
     inplace = inplace and grad_dtype == s2.dtype
     g = s2 if inplace else torch.empty((n, v), device=dev, dtype=grad_dtype)
-    with torch.cuda.device(dev):
+    with _guard(dev):
         def call(out):
             return lib().fm_kl_loss_grad(_ptr(s2), _ptr(t2), buf[0].data_ptr(), buf[1].data_ptr(),
                                          buf[2].data_ptr(), _ptr(loss), _ptr(out), n, v,
@@ -370,7 +393,7 @@ def kl_fwd_topk(s2, t2, k: int, inv_temperature: float, reduction: str, index_dt
     probs = torch.empty((n, k), device=dev, dtype=torch.float32) if want_probs else None
     idx = torch.empty((n, k), device=dev, dtype=index_dtype)
     bits = 64 if index_dtype == torch.int64 else 32
-    with torch.cuda.device(dev):
+    with _guard(dev):
         rc = lib().fm_kl_fwd_topk(_ptr(s2), _ptr(t2), buf[0].data_ptr(), buf[1].data_ptr(),
                                   buf[2].data_ptr(), _ptr(loss), _ptr(vals), _ptr(idx), _ptr(probs),
                                   n, v, int(k), dtype_code(s2.dtype), bits, float(inv_temperature),
@@ -386,7 +409,7 @@ def kl_bwd(s2, t2, lse_s, lse_t, grad_out, per_row: bool, grad_dtype, inv_temper
     _dense(s2, t2, lse_s, lse_t, grad_out)
     n, v = s2.shape
     g = torch.empty((n, v), device=s2.device, dtype=grad_dtype)
-    with torch.cuda.device(s2.device):
+    with _guard(s2.device):
         _check(lib().fm_kl_bwd(_ptr(s2), _ptr(t2), _ptr(lse_s), _ptr(lse_t), _ptr(grad_out),
                                1 if per_row else 0, _ptr(g), n, v, dtype_code(s2.dtype),
                                dtype_code(grad_dtype), float(inv_temperature), float(scale),
@@ -401,7 +424,7 @@ def topk(x2, k: int, index_dtype=torch.int64, want_values: bool = True):
     vals = torch.empty((n, k), device=x2.device, dtype=x2.dtype) if want_values else None
     idx = torch.empty((n, k), device=x2.device, dtype=index_dtype)
     bits = 64 if index_dtype == torch.int64 else 32
-    with torch.cuda.device(x2.device):
+    with _guard(x2.device):
         _check(lib().fm_topk(_ptr(x2), _ptr(vals), _ptr(idx), n, v, int(k), dtype_code(x2.dtype),
                              bits, _stream(x2)), "fm_topk")
     return vals, idx
@@ -411,7 +434,7 @@ def softmax_fwd(x2):
     _dense(x2)
     n, v = x2.shape
     y = torch.empty_like(x2)
-    with torch.cuda.device(x2.device):
+    with _guard(x2.device):
         _check(lib().fm_softmax_fwd(_ptr(x2), _ptr(y), n, v, dtype_code(x2.dtype), _stream(x2)),
                "fm_softmax_fwd")
     return y
@@ -429,7 +452,7 @@ def route(logits2, k: int, want_permutation: bool = True, want_stats: bool = Fal
     slot = torch.empty(n * k, device=dev, dtype=torch.int32) if want_permutation else None
     order = torch.empty(n * k, device=dev, dtype=torch.int32) if want_permutation else None
     stats = torch.empty(e + 1, device=dev, dtype=torch.float32) if want_stats else None
-    with torch.cuda.device(dev):
+    with _guard(dev):
         nbytes = int(lib().fm_route_workspace(n, e, k))
         ws = torch.empty(max(nbytes, 16), device=dev, dtype=torch.uint8)
         _check(lib().fm_route(_ptr(logits2), _ptr(idx), _ptr(wts), _ptr(counts), _ptr(slot),
@@ -446,7 +469,7 @@ def moe_gather(x2, order, k: int, scale_flat=None):
     _dense(x2, order, scale_flat)
     n, d = x2.shape
     xs = torch.empty((n * k, d), device=x2.device, dtype=x2.dtype)
-    with torch.cuda.device(x2.device):
+    with _guard(x2.device):
         _check(lib().fm_moe_gather(_ptr(x2), _ptr(order), _ptr(scale_flat), _ptr(xs), n, d, int(k),
                                    dtype_code(x2.dtype), _stream(x2)), "fm_moe_gather")
     return xs
@@ -457,7 +480,7 @@ def moe_combine(ys, weights, slot, n: int, k: int):
     _dense(ys, weights, slot)
     d = ys.shape[1]
     out = torch.empty((n, d), device=ys.device, dtype=ys.dtype)
-    with torch.cuda.device(ys.device):
+    with _guard(ys.device):
         _check(lib().fm_moe_combine(_ptr(ys), _ptr(weights), _ptr(slot), _ptr(out), n, d, int(k),
                                     dtype_code(ys.dtype), _stream(ys)), "fm_moe_combine")
     return out
@@ -468,7 +491,7 @@ def moe_combine_dw(ys, dout, slot, n: int, k: int):
     _dense(ys, dout, slot)
     d = ys.shape[1]
     dw = torch.empty((n, k), device=ys.device, dtype=torch.float32)
-    with torch.cuda.device(ys.device):
+    with _guard(ys.device):
         _check(lib().fm_moe_combine_dw(_ptr(ys), _ptr(dout), _ptr(slot), _ptr(dw), n, d, int(k),
                                        dtype_code(ys.dtype), _stream(ys)), "fm_moe_combine_dw")
     return dw
@@ -478,7 +501,7 @@ def moe_combine_dw(ys, dout, slot, n: int, k: int):
 def swiglu_fwd(gate, up):
     _dense(gate, up)
     y = torch.empty_like(gate)
-    with torch.cuda.device(gate.device):
+    with _guard(gate.device):
         _check(lib().fm_swiglu_fwd(_ptr(gate), _ptr(up), _ptr(y), gate.numel(), dtype_code(gate.dtype),
                                    _stream(gate)), "fm_swiglu_fwd")
     return y
@@ -487,7 +510,7 @@ def swiglu_fwd(gate, up):
 def swiglu_bwd(gate, up, dy):
     _dense(gate, up, dy)
     dg, du = torch.empty_like(gate), torch.empty_like(up)
-    with torch.cuda.device(gate.device):
+    with _guard(gate.device):
         _check(lib().fm_swiglu_bwd(_ptr(gate), _ptr(up), _ptr(dy), _ptr(dg), _ptr(du), gate.numel(),
                                    dtype_code(gate.dtype), _stream(gate)), "fm_swiglu_bwd")
     return dg, du
@@ -498,7 +521,7 @@ def swiglu_split_fwd(x2):
     _dense(x2)
     rows, w = x2.shape
     y = torch.empty((rows, w // 2), device=x2.device, dtype=x2.dtype)
-    with torch.cuda.device(x2.device):
+    with _guard(x2.device):
         _check(lib().fm_swiglu_split_fwd(_ptr(x2), _ptr(y), rows, w // 2, dtype_code(x2.dtype),
                                          _stream(x2)), "fm_swiglu_split_fwd")
     return y
@@ -508,7 +531,7 @@ def swiglu_split_bwd(x2, dy2):
     _dense(x2, dy2)
     rows, w = x2.shape
     dx = torch.empty_like(x2)
-    with torch.cuda.device(x2.device):
+    with _guard(x2.device):
         _check(lib().fm_swiglu_split_bwd(_ptr(x2), _ptr(dy2), _ptr(dx), rows, w // 2,
                                          dtype_code(x2.dtype), _stream(x2)), "fm_swiglu_split_bwd")
     return dx
@@ -521,7 +544,7 @@ def qk_norm_rope_fwd(x4, w, cos, sin, eps: float):
     b, t, h, d = x4.shape
     out = torch.empty_like(x4)
     rstd = torch.empty(b * t * h, device=x4.device, dtype=torch.float32)
-    with torch.cuda.device(x4.device):
+    with _guard(x4.device):
         _check(lib().fm_qk_norm_rope_fwd(_ptr(x4), _ptr(w), _ptr(cos), _ptr(sin), _ptr(out), _ptr(rstd),
                                          b, t, h, d, dtype_code(x4.dtype), dtype_code(w.dtype), float(eps),
                                          _stream(x4)), "fm_qk_norm_rope_fwd")
@@ -533,7 +556,7 @@ def qk_norm_rope_bwd(x4, w, cos, sin, rstd, dout, want_dw: bool = True):
     b, t, h, d = x4.shape
     dx = torch.empty_like(x4)
     dw = torch.empty_like(w) if want_dw else None
-    with torch.cuda.device(x4.device):
+    with _guard(x4.device):
         nbytes = int(lib().fm_qk_norm_rope_bwd_workspace(b, t, h, d)) if want_dw else 0
         ws = torch.empty(max(nbytes, 16), device=x4.device, dtype=torch.uint8) if want_dw else None
         _check(lib().fm_qk_norm_rope_bwd(_ptr(x4), _ptr(w), _ptr(cos), _ptr(sin), _ptr(rstd), _ptr(dout),
