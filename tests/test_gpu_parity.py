@@ -60,7 +60,7 @@ def assert_close_lowp(got, ref, dt, what, ulps=2.0, cancel=0.0, cancel_lowp=0.0)
 
 # ------------------------------------------------------------------ RMSNorm
 NORM_CASES = [
-    # n, d, x dtype, w dtype, eps      (first one: BASELINE config 1 at 1/8 of the rows)
+    # n, d, x dtype, w dtype, eps      (first one: the RMSNorm benchmark shape at 1/8 of the rows)
     (1024, 1024, BF16, F32, 1e-6), (64, 8192, BF16, BF16, 1e-6), (33, 768, F16, F16, 1e-5),
     (17, 100, F32, F32, 1e-6), (5, 7, BF16, F32, 1e-6), (300, 5120, BF16, F32, 1e-6),
     (16, 64, BF16, BF16, 1e-6), (3, 1, F32, F32, 1e-6), (6, 8, F32, F32, 1e-6), (1, 3, F32, F32, 1e-6),
