@@ -44,25 +44,28 @@ __global__ __launch_bounds__(THREADS) void ce_fwd_kernel(const T* __restrict__ l
       const int c = c0 + u * THREADS + tid;
       if (c < sp.nvec) raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
     }
+    // the maximum is taken on the raw logits and scaled once per batch, so each element costs
+    // one max, one fma and one exp2
     float z[UNROLL][EPV];
-    float cm = st.m;
+    float raw_max = -INFINITY;
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const int c = c0 + u * THREADS + tid;
       if (c < sp.nvec) {
         Elem<T>::unpack(raw[u], z[u]);
 #pragma unroll
-        for (int e = 0; e < EPV; ++e) { z[u][e] *= kLog2e; cm = fmaxf(cm, z[u][e]); }
+        for (int e = 0; e < EPV; ++e) raw_max = fmaxf(raw_max, z[u][e]);
       } else {
 #pragma unroll
         for (int e = 0; e < EPV; ++e) z[u][e] = -INFINITY;
       }
     }
+    const float cm = fmaxf(st.m, raw_max * kLog2e);   // st.m is finite, so cm is
     float acc = st.s * fast_exp2(st.m - cm);
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
 #pragma unroll
-      for (int e = 0; e < EPV; ++e) acc += fast_exp2(z[u][e] - cm);
+      for (int e = 0; e < EPV; ++e) acc += fast_exp2(__builtin_fmaf(z[u][e], kLog2e, -cm));
     }
     st.m = cm;
     st.s = acc;

@@ -32,8 +32,10 @@ __device__ __forceinline__ void kl_update(KLState& k, const u32x4 (&rs)[UNROLL],
                                           const u32x4 (&rt)[UNROLL], int c_first, int stride,
                                           int nvec, float c1) {
   constexpr int EPV = Elem<T>::kVec;
+  // maxima are taken on the raw logits and scaled once per batch; the temperature scale rides
+  // in the fma that feeds exp2, and the (t - s) factor of A is scaled once per batch too
   float zs[UNROLL][EPV], zt[UNROLL][EPV];
-  float cms = k.ms, cmt = k.mt;
+  float raw_ms = -INFINITY, raw_mt = -INFINITY;
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
     const int c = c_first + u * stride;
@@ -42,34 +44,30 @@ __device__ __forceinline__ void kl_update(KLState& k, const u32x4 (&rs)[UNROLL],
       Elem<T>::unpack(rt[u], zt[u]);
 #pragma unroll
       for (int e = 0; e < EPV; ++e) {
-        zs[u][e] *= c1;
-        zt[u][e] *= c1;
-        cms = fmaxf(cms, zs[u][e]);
-        cmt = fmaxf(cmt, zt[u][e]);
+        raw_ms = fmaxf(raw_ms, zs[u][e]);
+        raw_mt = fmaxf(raw_mt, zt[u][e]);
       }
-    } else {
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) { zs[u][e] = -INFINITY; zt[u][e] = -INFINITY; }
     }
   }
+  const float cms = fmaxf(k.ms, raw_ms * c1), cmt = fmaxf(k.mt, raw_mt * c1);   // finite: k.ms, k.mt are
   float ds = k.ds * fast_exp2(k.ms - cms);
   const float ft = fast_exp2(k.mt - cmt);
   float dt = k.dt * ft;
-  float a = k.a * ft;
+  float a_raw = 0.f;
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
     const int c = c_first + u * stride;
     if (c < nvec) {   // uniform per vector; keeps (-inf) - (-inf) out of the A term
 #pragma unroll
       for (int e = 0; e < EPV; ++e) {
-        ds += fast_exp2(zs[u][e] - cms);
-        const float et = fast_exp2(zt[u][e] - cmt);
+        ds += fast_exp2(__builtin_fmaf(zs[u][e], c1, -cms));
+        const float et = fast_exp2(__builtin_fmaf(zt[u][e], c1, -cmt));
         dt += et;
-        a += et * (zt[u][e] - zs[u][e]);
+        a_raw += et * (zt[u][e] - zs[u][e]);
       }
     }
   }
-  k.ms = cms; k.ds = ds; k.mt = cmt; k.dt = dt; k.a = a;
+  k.ms = cms; k.ds = ds; k.mt = cmt; k.dt = dt; k.a = k.a * ft + a_raw * c1;
 }
 
 // One scalar column.

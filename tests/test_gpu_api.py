@@ -437,7 +437,7 @@ def test_kl_div_logits_topk_autograd_and_wide_rows():
     sr = s.to("cuda").requires_grad_(True)
     ref = kernels.kl_div_logits(sr, t.to("cuda"), temperature=2.0)
     ref.backward()
-    assert loss.item() == pytest.approx(ref.item(), rel=1e-6)
+    assert loss.item() == pytest.approx(ref.item(), rel=1e-4)     # two kernels, two summation orders
     assert torch.allclose(sd.grad.float(), sr.grad.float(), rtol=1e-2, atol=1e-9)
     assert not probs.requires_grad and idx.dtype == torch.int32
     assert torch.equal(idx.cpu().long(), O.topk(t, 16)[1])

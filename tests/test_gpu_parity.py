@@ -408,7 +408,7 @@ def test_kl_loss_and_gradient_in_one_pass(n, v, dt, T, gdt, reduction):
     # against the two-pass kernels
     loss2, rows2, ls, lt = _hip.kl_fwd(sd, td, 1.0 / T, reduction)
     g2 = _hip.kl_bwd(sd, td, ls, lt, None, False, gdt, 1.0 / T, 1.0 / n if reduction == "mean" else 1.0)
-    assert loss2.item() == pytest.approx(loss.item(), rel=2e-5, abs=1e-7)
+    assert loss2.item() == pytest.approx(loss.item(), rel=1e-4, abs=5e-7)
     assert_close_lowp(grad, g2.float().cpu(), gdt, "vs two-pass", ulps=2.0, cancel=cancel)
     # written over the student when the dtypes agree and the row fits the register file
     loss3, g3, _ = _hip.kl_loss_grad(sd, td, 1.0 / T, reduction, gdt, inplace=True)
