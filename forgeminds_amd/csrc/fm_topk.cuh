@@ -153,12 +153,24 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
     const int active = (sp.nvec > ne ? sp.nvec : ne) < THREADS ? (sp.nvec > ne ? sp.nvec : ne) : THREADS;
     const int nfull = active >> 6;
     const int j = nfull > 0 ? (k + nfull - 1) / nfull : 65;
+    // Only the bits a value of type T can set are searched (the masked key is a lower bound
+    // of the key with nothing representable in between), two bits per step: three ballots
+    // that do not depend on each other instead of two dependent rounds.
     uint32_t tw = 0u;
     if (j <= 64 && wave < nfull) {
-      for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t mk = mykey & KMASK;
+      int bit = 31;
+      for (; bit - 1 >= KeyBits<T>::low; bit -= 2) {
+        const int shift = bit - 1;
+        const int c1 = __builtin_popcountll(__ballot(mk >= (tw | (1u << shift))));
+        const int c2 = __builtin_popcountll(__ballot(mk >= (tw | (2u << shift))));
+        const int c3 = __builtin_popcountll(__ballot(mk >= (tw | (3u << shift))));
+        const uint32_t dgt = c3 >= j ? 3u : (c2 >= j ? 2u : (c1 >= j ? 1u : 0u));
+        tw |= dgt << shift;
+      }
+      if (bit >= KeyBits<T>::low) {   // an odd number of key bits leaves one
         const uint32_t trial = tw | (1u << bit);
-        const int cnt = __builtin_popcountll(__ballot(mykey >= trial));
-        if (cnt >= j) tw = trial;
+        if (__builtin_popcountll(__ballot(mk >= trial)) >= j) tw = trial;
       }
     }
     if (lane == 0) s_tau[wave] = (wave < nfull || j > 64) ? tw : 0xFFFFFFFFu;
@@ -350,8 +362,18 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
       const unsigned long long me = ccomp[jx];
       const int i0 = part * per;
       const int i1 = i0 + per < C ? i0 + per : C;
+      // every lane reads the same candidate (an LDS broadcast); eight reads in flight hide
+      // the LDS latency that a one-at-a-time loop would pay per candidate
       int r = 0;
-      for (int i = i0; i < i1; ++i) r += ccomp[i] > me ? 1 : 0;
+      int i = i0;
+      for (; i + 8 <= i1; i += 8) {
+        unsigned long long o[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) o[u] = ccomp[i + u];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) r += o[u] > me ? 1 : 0;
+      }
+      for (; i < i1; ++i) r += ccomp[i] > me ? 1 : 0;
       if (parts == 1) crank[jx] = r; else atomicAdd(&crank[jx], r);
     }
   }
