@@ -17,7 +17,9 @@ from __future__ import annotations
 import torch
 
 from . import _fallback as fb
-from . import _hip
+import typing
+
+from . import _hip, _ops
 from ._common import _note, fast_ok
 
 
@@ -50,6 +52,47 @@ class _CrossEntropyFn(torch.autograd.Function):
         return dl.view(ctx.shape), None, None, None, None
 
 
+# ------------------------------------------------------------------ traced: custom ops
+# While tracing, the two-pass dataflow is used (forward keeps the per-row log-sum-exp, backward
+# recomputes the softmax): it is purely functional, which is what a traced graph needs.
+def _ce_impl(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int,
+             mean: bool) -> typing.Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    lg2 = logits.contiguous().view(-1, logits.shape[-1])
+    loss, lse, n_valid, _rows = _hip.ce_fwd(lg2, labels.contiguous().view(-1), ignore_index,
+                                            "mean" if mean else "sum")
+    return loss.clone(), lse, n_valid.clone()
+
+
+def _ce_fake(logits, labels, ignore_index, mean):
+    rows = logits.numel() // logits.shape[-1]
+    f32 = dict(device=logits.device, dtype=torch.float32)
+    return torch.empty((), **f32), torch.empty(rows, **f32), torch.empty((), **f32)
+
+
+def _ce_bwd_impl(logits: torch.Tensor, labels: torch.Tensor, lse: torch.Tensor, n_valid: torch.Tensor,
+                 g: torch.Tensor, ignore_index: int, mean: bool) -> torch.Tensor:
+    lg2 = logits.contiguous().view(-1, logits.shape[-1])
+    g32 = g.detach().to(torch.float32).contiguous()
+    dl = _hip.ce_bwd(lg2, labels.contiguous().view(-1), lse, n_valid if mean else None, g32, ignore_index)
+    return dl.view(logits.shape)
+
+
+def _ce_setup(ctx, inputs, output):
+    logits, labels, ignore_index, mean = inputs
+    ctx.save_for_backward(logits, labels, output[1], output[2])
+    ctx.ignore_index, ctx.mean = ignore_index, mean
+
+
+def _ce_autograd(ctx, g, _glse, _gn):
+    logits, labels, lse, n_valid = ctx.saved_tensors
+    return _CE_BWD_OP(logits, labels, lse, n_valid, g, ctx.ignore_index, ctx.mean), None, None, None
+
+
+_CE_BWD_OP = _ops.define_backward("cross_entropy", _ce_bwd_impl,
+                                  lambda logits, labels, lse, n_valid, g, ignore_index, mean: torch.empty_like(logits))
+_CE_OP = _ops.define("cross_entropy", _ce_impl, _ce_fake, _ce_setup, _ce_autograd)
+
+
 def cross_entropy(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int = -100,
                   reduction: str = "mean", inplace: bool = False) -> torch.Tensor:
     """fp32 scalar CE over the last dim of ``logits``.
@@ -74,6 +117,8 @@ def cross_entropy(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int 
         return fb.cross_entropy(logits, labels, ignore_index, reduction)
     if not fast_ok(logits):
         return fb.cross_entropy(logits, labels, ignore_index, reduction)
+    if _CE_OP is not None and _ops.wanted():
+        return _CE_OP(logits, labels, int(ignore_index), reduction == "mean")[0]
     return _CrossEntropyFn.apply(logits, labels, int(ignore_index), reduction, bool(inplace))
 
 

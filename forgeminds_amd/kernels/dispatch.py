@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from . import _hip
-from ._common import _note, fast_ok
+from ._common import _note, fast_ok, tracing
 
 
 def _inverse(perm: torch.Tensor) -> torch.Tensor:
@@ -72,7 +72,7 @@ def moe_gather(x: torch.Tensor, order: torch.Tensor, k: int,
     if k > 8 or x.numel() == 0 or order.device != x.device:
         _note("moe_gather shape")
         return x[(order // k).long()]
-    if not fast_ok(x):
+    if tracing() or not fast_ok(x):      # a traced graph gets the tensor expression
         return x[(order // k).long()]
     order = _i32(order)
     if slot is None:
@@ -96,7 +96,7 @@ def moe_combine(ys: torch.Tensor, weights: torch.Tensor, slot: torch.Tensor,
     if k > 8 or ys.numel() == 0 or slot.device != ys.device or weights.device != ys.device:
         _note("moe_combine shape")
         return torch_path()
-    if not fast_ok(ys, weights):
+    if tracing() or not fast_ok(ys, weights):
         return torch_path()
     slot = _i32(slot)
     if order is None:

@@ -18,8 +18,10 @@ from __future__ import annotations
 import torch
 
 from . import _fallback as fb
-from . import _hip
-from ._common import _note, fast_ok
+import typing
+
+from . import _hip, _ops
+from ._common import _note, fast_ok, tracing
 
 _REDUCTIONS = ("mean", "sum", "none")
 
@@ -105,6 +107,57 @@ class _KLDivTopkFn(torch.autograd.Function):
         return grad.view(shape), None, None, None, None, None, None
 
 
+# ------------------------------------------------------------------ traced: custom ops
+# While tracing, the functional two-pass dataflow: the forward keeps the two per-row
+# log-sum-exps, the backward recomputes both softmaxes.
+_RED = ("none", "sum", "mean")
+
+
+def _kl_impl(student: torch.Tensor, teacher: torch.Tensor, reduction: int,
+             inv_t: float) -> typing.Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    v = student.shape[-1]
+    s2, t2 = student.contiguous().view(-1, v), teacher.contiguous().view(-1, v)
+    loss, rows, lse_s, lse_t = _hip.kl_fwd(s2, t2, inv_t, _RED[reduction])
+    out = rows.clone().view(student.shape[:-1]) if reduction == 0 else loss
+    return out, lse_s.clone(), lse_t.clone()       # the three are rows of one buffer
+
+
+def _kl_fake(student, teacher, reduction, inv_t):
+    rows = student.numel() // student.shape[-1]
+    f32 = dict(device=student.device, dtype=torch.float32)
+    out = torch.empty(student.shape[:-1], **f32) if reduction == 0 else torch.empty((), **f32)
+    return out, torch.empty(rows, **f32), torch.empty(rows, **f32)
+
+
+def _kl_bwd_impl(student: torch.Tensor, teacher: torch.Tensor, lse_s: torch.Tensor, lse_t: torch.Tensor,
+                 g: torch.Tensor, reduction: int, inv_t: float, fp32_grad: bool) -> torch.Tensor:
+    v = student.shape[-1]
+    s2, t2 = student.contiguous().view(-1, v), teacher.contiguous().view(-1, v)
+    g32 = g.detach().to(torch.float32).contiguous().view(-1)
+    scale = 1.0 / s2.shape[0] if reduction == 2 else 1.0
+    gdt = torch.float32 if fp32_grad else student.dtype
+    return _hip.kl_bwd(s2, t2, lse_s, lse_t, g32, reduction == 0, gdt, inv_t, scale).view(student.shape)
+
+
+def _kl_bwd_fake(student, teacher, lse_s, lse_t, g, reduction, inv_t, fp32_grad):
+    return torch.empty_like(student, dtype=torch.float32 if fp32_grad else student.dtype)
+
+
+def _kl_setup(ctx, inputs, output):
+    student, teacher, reduction, inv_t = inputs
+    ctx.save_for_backward(student, teacher, output[1], output[2])
+    ctx.reduction, ctx.inv_t = reduction, inv_t
+
+
+def _kl_autograd(ctx, g, _g1, _g2):
+    student, teacher, lse_s, lse_t = ctx.saved_tensors
+    return _KL_BWD_OP(student, teacher, lse_s, lse_t, g, ctx.reduction, ctx.inv_t, False), None, None, None
+
+
+_KL_BWD_OP = _ops.define_backward("kl_div", _kl_bwd_impl, _kl_bwd_fake)
+_KL_OP = _ops.define("kl_div", _kl_impl, _kl_fake, _kl_setup, _kl_autograd)
+
+
 def _kernel_ok(*tensors) -> bool:
     if any(t.numel() >= 2 ** 31 * 4 for t in tensors):
         _note("kl numel")
@@ -134,6 +187,8 @@ def kl_div_logits(student: torch.Tensor, teacher: torch.Tensor, reduction: str =
         return fb.kl_div_logits(student, teacher, reduction, temperature)
     if not _kernel_ok(student, teacher):
         return fb.kl_div_logits(student, teacher, reduction, temperature)
+    if _KL_OP is not None and _ops.wanted() and grad_dtype in (None, student.dtype):
+        return _KL_OP(student, teacher, _RED.index(reduction), 1.0 / float(temperature))[0]
     return _KLDivFn.apply(student, teacher, reduction, grad_dtype, float(temperature), bool(reuse))
 
 
@@ -159,7 +214,7 @@ def kl_div_logits_topk(student: torch.Tensor, teacher: torch.Tensor, k: int,
     ok = (student.shape == teacher.shape and student.shape[-1] > 0 and student.numel() > 0
           and student.dtype == teacher.dtype and k <= 512
           and grad_dtype in (None, student.dtype, torch.float32))
-    if not ok or not _kernel_ok(student, teacher):
+    if not ok or tracing() or not _kernel_ok(student, teacher):
         if ok is False:
             _note("kl operands")
         loss = fb.kl_div_logits(student, teacher, reduction, temperature)

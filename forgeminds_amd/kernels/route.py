@@ -16,7 +16,7 @@ import torch
 
 from . import _fallback as fb
 from . import _hip
-from ._common import _note, fast_ok
+from ._common import _note, fast_ok, tracing
 
 MAX_EXPERTS = 512
 MAX_TOP_K = 8
@@ -126,6 +126,8 @@ def moe_route(logits: torch.Tensor, k: int, with_aux: bool = False) -> Routing:
         raise RuntimeError(f"selected index k out of range (got {k} vs {e})")
     if e > MAX_EXPERTS or k > MAX_TOP_K or n * k >= 2 ** 31 - 1:
         _note("route shape")
+        return _torch_route(logits, k, with_aux)
+    if tracing():      # no op is registered for the router: a traced graph gets the tensor expression
         return _torch_route(logits, k, with_aux)
     if not fast_ok(logits):
         return _torch_route(logits, k, with_aux)

@@ -492,3 +492,46 @@ def test_layer_norm_autograd_module_and_op_path():
     fn = torch.compile(lambda t: kernels.layer_norm(t, wd.detach(), bd.detach()).float().sum(), fullgraph=True,
                        backend="eager")
     assert torch.isfinite(fn(x.to(DEV)))
+
+
+def test_losses_and_moe_pieces_trace_in_one_graph():
+    g = torch.Generator().manual_seed(61)
+    lg = (2 * torch.randn(40, 700, generator=g)).bfloat16().to(DEV)
+    lab = torch.randint(0, 700, (40,), generator=g).to(DEV)
+    lab[::9] = -100
+    t = (lg.float() + 0.5 * torch.randn(40, 700, generator=g).to(DEV)).bfloat16()
+    for name in ("cross_entropy", "cross_entropy_backward", "kl_div", "kl_div_backward"):
+        assert hasattr(torch.ops.forgemind, name), name
+
+    def both(fn):
+        a = lg.clone().requires_grad_(True)
+        out = fn(a)
+        out.sum().backward()
+        b = lg.clone().requires_grad_(True)
+        cout = torch.compile(fn, fullgraph=True, backend="eager")(b)
+        cout.sum().backward()
+        assert torch.allclose(out, cout, rtol=1e-5, atol=1e-7)
+        assert close(b.grad, a.grad)
+    both(lambda a: kernels.cross_entropy(a, lab))
+    both(lambda a: kernels.cross_entropy(a, lab, reduction="sum"))
+    both(lambda a: kernels.kl_div_logits(a, t, temperature=2.0))
+    both(lambda a: kernels.kl_div_logits(a, t, "none"))
+    both(lambda a: kernels.kl_div_logits_topk(a, t, 8)[0])
+    # the exported graph keeps the loss as one node
+    class M(nn.Module):
+        def forward(self, a):
+            return kernels.cross_entropy(a, lab)
+    ep = torch.export.export(M(), (lg,))
+    targets = [str(n.target) for n in ep.graph.nodes if n.op == "call_function"]
+    assert "forgemind.cross_entropy.default" in targets, targets
+    # router and token moves: the traced graph gets the tensor expression, same results
+    rl = torch.round(torch.randn(200, 16, generator=g) * 64).to(DEV) / 64
+    x = torch.randn(200, 64, generator=g).to(DEV)
+
+    def moe(a):
+        r = kernels.moe_route(rl, 2)
+        xs = kernels.moe_gather(a, r.order, 2, r.slot)
+        return kernels.moe_combine(xs, r.weights, r.slot, r.order)
+    eager = moe(x)
+    traced = torch.compile(moe, fullgraph=True, backend="eager")(x)
+    assert torch.allclose(eager, traced, rtol=1e-5, atol=1e-6)
