@@ -12,6 +12,7 @@ import types
 import torch
 import torch.nn as nn
 
+from .layernorm import layer_norm
 from .swiglu import swiglu, swiglu_split
 from .norm import rms_norm
 
@@ -56,6 +57,19 @@ def _patch_norm(m: nn.Module) -> None:
     _swap_forward(m, forward)
 
 
+def _is_last_dim_layernorm(m: nn.Module) -> bool:
+    return isinstance(m, nn.LayerNorm) and len(m.normalized_shape) == 1
+
+
+def _patch_layernorm(m: nn.Module) -> None:
+    def forward(self, x):
+        if self.weight is None:      # elementwise_affine=False
+            return layer_norm(x, torch.ones(self.normalized_shape, device=x.device, dtype=x.dtype), None, self.eps)
+        return layer_norm(x, self.weight, self.bias, self.eps)
+
+    _swap_forward(m, forward)
+
+
 def _patch_mlp(m: nn.Module) -> None:
     def forward(self, x):
         return self.w2(swiglu(self.w1(x), self.w3(x)))
@@ -88,13 +102,22 @@ def patch(module: nn.Module, split: bool = False, kind: "str | None" = None) -> 
     """Fuse one module in place; ``True`` if it was recognised (or already patched).
 
     ``kind="norm"`` / ``kind="mlp"`` skips detection by class name and validates the structure
-    instead, raising ``TypeError`` when it does not fit. ``split=True`` additionally merges
+    instead, raising ``TypeError`` when it does not fit. ``kind="layernorm"`` is the only way a
+    ``torch.nn.LayerNorm`` is touched (it is not an RMSNorm, and the reference leaves it alone:
+    ``tests/test_nn_blocks.py:170-172``). ``split=True`` additionally merges
     ``w1|w3`` of an MLP into one ``gate_up`` projection (renames parameters).
     """
     if getattr(module, "_fm_norm", False) or getattr(module, "_fm_mlp", False):
         return True
-    if kind not in (None, "norm", "mlp"):
-        raise ValueError(f"kind must be 'norm', 'mlp' or None, got {kind!r}")
+    if kind not in (None, "norm", "mlp", "layernorm"):
+        raise ValueError(f"kind must be 'norm', 'mlp', 'layernorm' or None, got {kind!r}")
+    if kind == "layernorm":
+        if not _is_last_dim_layernorm(module):
+            raise TypeError(f"patch(kind='layernorm') needs a torch.nn.LayerNorm over the last "
+                            f"dimension, got {type(module).__name__}")
+        _patch_layernorm(module)
+        module._fm_norm = True
+        return True
     if kind == "norm" and not _has_vector_weight(module):
         raise TypeError(f"patch(kind='norm') needs a 1-D weight Parameter, "
                         f"{type(module).__name__} has {getattr(module, 'weight', None)!r}")
@@ -113,13 +136,19 @@ def patch(module: nn.Module, split: bool = False, kind: "str | None" = None) -> 
 
 
 def enable(model: nn.Module, norm: bool = True, swiglu_mlp: bool = True,
-           split: bool = False) -> nn.Module:
-    """Patch every recognised module of ``model``; counts land on ``model._fm_fused``."""
+           split: bool = False, layer_norm: bool = False) -> nn.Module:
+    """Patch every recognised module of ``model``; counts land on ``model._fm_fused``.
+
+    ``layer_norm=True`` (off by default) also routes ``torch.nn.LayerNorm`` modules over the last
+    dimension through the LayerNorm kernels; they are counted with the norms."""
     n_norm = n_mlp = 0
     for m in model.modules():
         if getattr(m, "_fm_norm", False) or getattr(m, "_fm_mlp", False):
             continue
-        if norm and _looks_like_rmsnorm(m):
+        if layer_norm and _is_last_dim_layernorm(m):
+            patch(m, kind="layernorm")
+            n_norm += 1
+        elif norm and _looks_like_rmsnorm(m):
             patch(m)
             n_norm += 1
         elif swiglu_mlp and _looks_like_swiglu_mlp(m):

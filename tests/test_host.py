@@ -413,3 +413,21 @@ def test_layer_norm_torch_path_and_module():
     with pytest.raises(ValueError):
         m(torch.randn(2, 23))
     assert fm.nn.LayerNorm(8, bias=False).bias is None and fm.nn.LayerNorm(8, elementwise_affine=False).weight is None
+
+
+def test_layernorm_is_only_patched_on_request():
+    ln = nn.LayerNorm(16)
+    assert kernels.patch(ln) is False                           # reference tests/test_nn_blocks.py:170-172
+    with pytest.raises(TypeError):
+        kernels.patch(nn.Linear(4, 4), kind="layernorm")
+    x = torch.randn(5, 16)
+    before = ln(x).detach().clone()
+    assert kernels.patch(ln, kind="layernorm") is True and kernels.patch(ln) is True
+    assert torch.allclose(ln(x), before, atol=2e-6)
+    kernels.revert(ln)
+    assert "forward" not in ln.__dict__ and torch.equal(ln(x), before)
+    model = nn.Sequential(nn.LayerNorm(16), nn.Linear(16, 16), nn.LayerNorm(16, elementwise_affine=False))
+    assert kernels.enable(model)._fm_fused == {"norm": 0, "mlp": 0}
+    ref = model(x).detach().clone()
+    assert kernels.enable(model, layer_norm=True)._fm_fused == {"norm": 2, "mlp": 0}
+    assert torch.allclose(model(x), ref, atol=2e-6)
