@@ -475,6 +475,7 @@ def measure(torch, w, steps, warmup):
         "rows_per_s": round(w.rows / ms * 1e3, 1),
         "dominant_kernel": w.dominant,
         "dominant_ms_avg": round(avg, 5), "dominant_ms_min": round(best, 5),
+        "dominant_ms_median": round(med, 5),
         "dominant_gbps": round(w.dominant_bytes / avg / 1e6, 1),
     }
     if hasattr(w, "warm_step"):      # same buffers every step: served by the Infinity Cache
