@@ -1,8 +1,10 @@
 #!/usr/bin/env python3
 """Benchmark of the packed-kernel hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload ce|rmsnorm|add_rmsnorm|kl|topk|route]
-                    [--no-extras] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extras] [--no-cpu]
+
+NAME: ce (headline), ce_one_pass, rmsnorm, add_rmsnorm, add_layernorm, kl, kl_topk, topk, route,
+moe_dispatch, swiglu, qk_norm_rope.
 
 A step is one pass of the hot path (forward + backward) over one batch of synthetic,
 seeded input that is already resident in HBM, launched straight through the C ABI of

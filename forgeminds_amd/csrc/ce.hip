@@ -6,7 +6,9 @@
 // Forward: one workgroup per row, one read of the row. Each thread runs an online
 // (max, sum-exp) over its share of the row in the base-2 domain, the workgroup merges
 // the pairs, and lse[row] is saved. Backward: the softmax is recomputed from lse instead of
-// being stored, so the whole fwd+bwd moves 2 + 2 + 2 bytes per bf16 logit.
+// being stored, so the whole fwd+bwd moves 2 + 2 + 2 bytes per bf16 logit. A second form
+// (ce_loss_grad_kernel) produces the loss and the gradient from one read of rows that fit the
+// register file: 2 + 2 bytes per logit.
 #include "fm_vocab.cuh"
 
 using namespace fm;

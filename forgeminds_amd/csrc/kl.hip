@@ -8,6 +8,8 @@
 //   KL = (sum_j e^{t_j - m_t} (t_j - s_j)) / d_t - lse_t + lse_s
 // a thread carries (m_s, d_s, m_t, d_t, A) and rescales d_t and A whenever its teacher
 // maximum moves. The backward recomputes both softmaxes from the saved lse values.
+// Two more forms: kl_loss_grad_kernel writes the gradient in the forward from one read of rows
+// that fit the register file, and kl_fwd_topk_kernel also selects the teacher's top-k.
 // All exponentials run in the base-2 domain; the temperature is folded into the scale.
 #include "fm_topk.cuh"
 
