@@ -203,7 +203,10 @@ __global__ __launch_bounds__(kBwdBlock) void norm_bwd_kernel(
     const bool valid = row < n;
     const int64_t base = row * (int64_t)d;
     // x and dy stay packed in registers between the two sweeps (half the footprint of fp32)
-    u32x4 rx[ITERS], rg[ITERS], rr[ITERS];   // rr: the residual-stream gradient, fetched with the rest
+    // rr: the residual-stream gradient, fetched with the rest where the register budget allows
+    // (the LayerNorm form carries a second set of accumulators and fetches it late instead)
+    constexpr bool EARLY_RES = !LN;
+    u32x4 rx[ITERS], rg[ITERS], rr[EARLY_RES ? ITERS : 1];
     const float r = valid ? rstd[row] : 0.f;
     float mu = 0.f;
     if constexpr (LN) mu = valid ? mean[row] : 0.f;
@@ -214,7 +217,9 @@ __global__ __launch_bounds__(kBwdBlock) void norm_bwd_kernel(
       if (valid && c < nvec) {
         rx[i] = load16_stream(x + base + (int64_t)c * EPV);
         rg[i] = load16_stream(dy + base + (int64_t)c * EPV);
-        if (gxn != nullptr) rr[i] = load16_stream(gxn + base + (int64_t)c * EPV);
+        if constexpr (EARLY_RES) {
+          if (gxn != nullptr) rr[i] = load16_stream(gxn + base + (int64_t)c * EPV);
+        }
       }
     }
 #pragma unroll
@@ -252,7 +257,8 @@ __global__ __launch_bounds__(kBwdBlock) void norm_bwd_kernel(
           o[e] = ((gv[e] * wv[i][e] - gmean) - ((xv[e] - mu) * r) * cmean) * r;
         if (gxn != nullptr) {
           float rv[EPV];
-          Elem<T>::unpack(rr[i], rv);
+          if constexpr (EARLY_RES) Elem<T>::unpack(rr[i], rv);
+          else Elem<T>::unpack(load16_stream(gxn + base + (int64_t)c * EPV), rv);
 #pragma unroll
           for (int e = 0; e < EPV; ++e) o[e] += rv[e];
         }
