@@ -142,6 +142,83 @@ __global__ __launch_bounds__(THREADS) void topk_lds_kernel(const T* __restrict__
                                          nullptr, 0.f, 0.f);
 }
 
+// Rows of up to 1024 elements: one wave per row, four rows per workgroup. Lane l holds the
+// elements l, l + 64, ... as keys in registers; the k-th key comes from a bitwise search whose
+// counts are wave ballots (no memory traffic, no workgroup barrier inside the search), the
+// selected elements take slots in LDS (greater first, then the first ties in index order) and
+// are ranked by counting among themselves.
+constexpr int kWaveRows = 4;
+
+template <typename T, int EPL>
+__global__ __launch_bounds__(64 * kWaveRows) void topk_wave_kernel(const T* __restrict__ x,
+                                                                    T* __restrict__ values,
+                                                                    int32_t* __restrict__ idx32,
+                                                                    int64_t* __restrict__ idx64, int64_t n,
+                                                                    int v, int k) {
+  __shared__ unsigned long long sel[kWaveRows][kMaxK];
+  constexpr uint32_t KMASK = KeyBits<T>::mask;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row = (int64_t)blockIdx.x * kWaveRows + wave;
+  const bool valid = row < n;                  // uniform per wave; nobody leaves before the barrier
+  const T* rp = x + (valid ? row : 0) * (int64_t)v;
+  uint32_t mk[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) {
+    const int col = lane + 64 * e;
+    // 0 is below the key of every value (-inf maps to 0x007FFFFF), so empty slots never win
+    mk[e] = (valid && col < v) ? (key_of(Elem<T>::load1(rp + col)) & KMASK) : 0u;
+  }
+  uint32_t kth = 0u;
+  for (int bit = 31; bit >= KeyBits<T>::low; --bit) {
+    const uint32_t trial = kth | (1u << bit);
+    int cnt = 0;
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) cnt += __builtin_popcountll(__ballot(mk[e] >= trial));
+    if (cnt >= k) kth = trial;
+  }
+  int c_gt = 0;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) c_gt += __builtin_popcountll(__ballot(mk[e] > kth));
+  const int need = k - c_gt;                   // ties admitted, lowest columns first
+  const unsigned long long below = (1ull << lane) - 1ull;
+  int base_gt = 0, base_eq = 0;
+  unsigned long long* my = sel[wave];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) {              // ascending e, ascending lane: ascending column
+    const int col = lane + 64 * e;
+    const unsigned long long m_gt = __ballot(mk[e] > kth);
+    const unsigned long long m_eq = __ballot(mk[e] == kth && mk[e] != 0u);
+    const unsigned long long item = ((unsigned long long)mk[e] << 32) | (uint32_t)(~col);
+    if (mk[e] > kth) my[base_gt + __builtin_popcountll(m_gt & below)] = item;
+    if (mk[e] == kth && mk[e] != 0u) {
+      const int t = base_eq + __builtin_popcountll(m_eq & below);
+      if (t < need) my[c_gt + t] = item;
+    }
+    base_gt += __builtin_popcountll(m_gt);
+    base_eq += __builtin_popcountll(m_eq);
+  }
+  __syncthreads();
+  if (!valid) return;
+  for (int s = lane; s < k; s += 64) {
+    const unsigned long long me = my[s];
+    int r = 0;
+    int i = 0;
+    for (; i + 8 <= k; i += 8) {
+      unsigned long long o[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) o[u] = my[i + u];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) r += o[u] > me ? 1 : 0;
+    }
+    for (; i < k; ++i) r += my[i] > me ? 1 : 0;
+    const int col = (int)(~(uint32_t)(me & 0xFFFFFFFFull));
+    const int64_t o = row * (int64_t)k + r;
+    if (idx32 != nullptr) idx32[o] = col;
+    if (idx64 != nullptr) idx64[o] = col;
+    if (values != nullptr) values[o] = rp[col];
+  }
+}
+
 // widest row (in 16-byte vectors) whose key prefixes fit the LDS budget
 constexpr int kLdsMaxVec = 20480;
 
@@ -162,7 +239,17 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
                      i64, v, k, vec_ok)
   int variant = fm_host::get_param(fm_host::P_TOPK_VARIANT);
   if (variant == 0) variant = nvec <= 3072 ? 1 : (nvec <= 12288 ? 2 : 3);
-  if (v <= kCap) GOL(256, 4);             // every element is a candidate; no prefixes used
+  if (v <= 64 * 16) {                     // short rows: a wave per row
+    const dim3 wgrid((unsigned)((n + kWaveRows - 1) / kWaveRows));
+#define GOW(EPL_)                                                                                 \
+  hipLaunchKernelGGL((topk_wave_kernel<T, EPL_>), wgrid, dim3(64 * kWaveRows), 0, st, xp, vp, i32, i64, n, v, k)
+    if (v <= 64) GOW(1);
+    else if (v <= 128) GOW(2);
+    else if (v <= 256) GOW(4);
+    else if (v <= 512) GOW(8);
+    else GOW(16);
+#undef GOW
+  }
   else if (nvec > kLdsMaxVec) {
     if (nvec <= 1024 * 32) GO(1024, 32);
     else GO(1024, 0);

@@ -495,7 +495,9 @@ def test_kl_fwd_topk_ties_unaligned_and_unsupported():
 TOPK_CASES = [(32, 128256, 64, BF16), (8, 4096, 64, F32), (4, 64, 8, F32), (3, 5000, 512, BF16),
               (4, 20000, 100, F16), (2, 300000, 17, BF16), (3, 9000, 5, F32), (2, 100, 99, F32),
               (1, 512, 512, F32), (5, 1, 1, F32), (2, 600, 4, F32), (4, 5000, 512, F32),
-              (2, 1025, 3, BF16), (3, 70000, 512, F32), (6, 50257, 64, BF16), (2, 140000, 64, F32)]
+              (2, 1025, 3, BF16), (3, 70000, 512, F32), (6, 50257, 64, BF16), (2, 140000, 64, F32),
+              (1000, 64, 8, F32), (333, 128, 2, BF16), (77, 200, 200, F16), (50, 1024, 512, BF16),
+              (41, 1000, 64, F32), (9, 7, 7, BF16), (130, 513, 100, F16), (5, 1024, 1, F32)]
 
 
 @pytest.mark.parametrize("n,v,k,dt", TOPK_CASES)
@@ -541,6 +543,15 @@ def test_topk_ties_nans_zeros_and_degenerate_rows():
     for dt, v, k in ((BF16, 2048, 256), (F32, 1500, 300), (F16, 4096, 512), (BF16, 1100, 512)):
         x = (3 * torch.randn(5, v, generator=g)).to(dt)
         assert torch.equal(run(x, k), O.topk(x, k)[1])
+    # short rows (a wave per row): ties, NaNs, -inf and signed zeros
+    x = torch.randint(0, 4, (300, 700), generator=g).to(BF16)
+    x[::3, ::5] = float("nan")
+    x[1::3, 1::7] = float("-inf")
+    x[2::3, ::2] = -0.0
+    for k in (1, 17, 64, 300, 512):
+        assert torch.equal(run(x, k), O.topk(x, k)[1])
+    z = torch.zeros(5, 64)
+    assert torch.equal(run(z, 64), torch.arange(64).expand(5, 64))
     # negative NaN payloads and a row of -inf
     x = torch.full((2, 3000), float("-inf"))
     x[0, 17] = -torch.tensor(float("nan"))
