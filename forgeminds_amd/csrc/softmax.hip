@@ -137,6 +137,43 @@ __global__ __launch_bounds__(RowBlock<TPR>::value) void softmax_rows_kernel(cons
   }
 }
 
+// Narrow rows whose width is not a whole number of 16-byte vectors (or whose buffers are not
+// 16-byte aligned): the same scheme with one element per load. Lane t of a row's TPR lanes holds
+// elements t, t + TPR, ...
+template <typename T, int TPR, int ITERS>
+__global__ __launch_bounds__(256) void softmax_rows_scalar_kernel(const T* __restrict__ x,
+                                                                  T* __restrict__ y, int64_t n, int v) {
+  constexpr int RPB = 256 / TPR;
+  const int tid = threadIdx.x;
+  const int rib = tid / TPR;
+  const int t = tid % TPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + rib;
+  const bool valid = row < n;
+  const int64_t base = row * (int64_t)v;
+  float z[ITERS];
+  float m = kNegBig;
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * TPR + t;
+    z[i] = (valid && c < v) ? Elem<T>::load1(x + base + c) * kLog2e : -INFINITY;
+    m = fmaxf(m, z[i]);
+  }
+  m = group_reduce<TPR, OpMax>(m);
+  float ssum = 0.f;
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    z[i] = fast_exp2(z[i] - m);
+    ssum += z[i];
+  }
+  ssum = group_reduce<TPR, OpSum>(ssum);
+  const float inv = 1.f / ssum;
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * TPR + t;
+    if (valid && c < v) Elem<T>::store1(y + base + c, z[i] * inv);
+  }
+}
+
 #define FM_SOFTMAX_SHAPES(X) \
   X(4, 1) X(8, 1) X(16, 1) X(32, 1) X(64, 1) X(64, 2) X(128, 2) X(256, 2) X(256, 4) X(512, 4) X(512, 8) X(1024, 8)
 
@@ -167,6 +204,19 @@ void launch(const void* x, void* y, int64_t n, int v, bool vec_ok, hipStream_t s
   }
     FM_SOFTMAX_SHAPES(X)
 #undef X
+  }
+  if (v <= 64 * 16) {   // narrow, not vectorisable: lane groups with one element per load
+    const int tpr = v <= 16 * 16 ? 16 : 64;
+    int iters = 1;
+    while (tpr * iters < v) iters *= 2;
+    const dim3 sgrid((unsigned)((n + 256 / tpr - 1) / (256 / tpr)));
+#define GOS(TPR_, IT_)                                                                             \
+  if (tpr == TPR_ && iters == IT_) {                                                               \
+    hipLaunchKernelGGL((softmax_rows_scalar_kernel<T, TPR_, IT_>), sgrid, dim3(256), 0, st, xp, yp, n, v); \
+    return;                                                                                        \
+  }
+    GOS(16, 1) GOS(16, 2) GOS(16, 4) GOS(16, 8) GOS(16, 16) GOS(64, 8) GOS(64, 16)
+#undef GOS
   }
   const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 4);
   const dim3 grid((unsigned)n);

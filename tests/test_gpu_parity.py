@@ -575,7 +575,8 @@ def test_topk_unaligned_rows():
                                      (8, 50257, BF16), (6, 300, F16), (2, 128256, BF16),
                                      (1000, 64, F32), (77, 16, BF16), (3, 4, F32), (33, 512, BF16),
                                      (130, 8, F16), (9, 8192, BF16), (5, 32768, F16), (3, 65536, BF16),
-                                     (257, 2048, F32), (4, 32000, BF16)])
+                                     (257, 2048, F32), (4, 32000, BF16), (1000, 33, BF16), (77, 7, F32),
+                                     (300, 257, F16), (65, 1023, BF16), (40, 100, F32), (9, 513, F32)])
 def test_softmax(n, v, dt):
     x = torch.randn(n, v, generator=gen(21)).to(dt)
     y = _hip.softmax_fwd(x.to(DEV))
