@@ -147,11 +147,20 @@ def _stream(t: torch.Tensor):
 _SAME_DEVICE = contextlib.nullcontext()
 
 
+_current_device = getattr(torch._C, "_cuda_getDevice", None) or torch.cuda.current_device
+
+
 def _guard(dev: torch.device):
     """Make ``dev`` current for the launch; free when it already is (the usual case)."""
-    if dev.index is None or dev.index == torch.cuda.current_device():
+    if dev.index is None or dev.index == _current_device():
         return _SAME_DEVICE
     return torch.cuda.device(dev)
+
+
+def _rows(x: torch.Tensor):
+    """(rows, width) of a dense tensor whose last dimension is the row."""
+    d = x.shape[-1]
+    return x.numel() // d, d
 
 
 def _check(rc: int, what: str) -> None:
@@ -172,9 +181,9 @@ def set_param(name: str, value: int) -> None:
 
 # ------------------------------------------------------------------ norm
 def rmsnorm_fwd(x2: torch.Tensor, w: torch.Tensor, eps: float):
-    """x2 [n, d] contiguous, w [d] -> (y [n, d], rstd [n] fp32)."""
+    """x2 [..., d] contiguous, w [d] -> (y like x2, rstd [rows] fp32)."""
     _dense(x2, w)
-    n, d = x2.shape
+    n, d = _rows(x2)
     y = torch.empty_like(x2)
     rstd = torch.empty(n, device=x2.device, dtype=torch.float32)
     with _guard(x2.device):
@@ -200,7 +209,7 @@ def _norm_ws(n: int, d: int, x: torch.Tensor, want_dw: bool):
 def rmsnorm_bwd(x2, w, rstd, dy2, want_dw: bool = True):
     """-> (dx [n, d], dw [d] in w.dtype or None)."""
     _dense(x2, w, rstd, dy2)
-    n, d = x2.shape
+    n, d = _rows(x2)
     dx = torch.empty_like(x2)
     dw = torch.empty_like(w) if want_dw else None
     with _guard(x2.device):
@@ -214,7 +223,7 @@ def rmsnorm_bwd(x2, w, rstd, dy2, want_dw: bool = True):
 def add_rmsnorm_fwd(x2, delta2, w, eps: float):
     """-> (xn [n, d], y [n, d], rstd [n] fp32)."""
     _dense(x2, delta2, w)
-    n, d = x2.shape
+    n, d = _rows(x2)
     xn = torch.empty_like(x2)
     y = torch.empty_like(x2)
     rstd = torch.empty(n, device=x2.device, dtype=torch.float32)
@@ -229,7 +238,7 @@ def add_rmsnorm_fwd(x2, delta2, w, eps: float):
 def add_rmsnorm_bwd(xn2, w, rstd, gy2, gxn2, want_dw: bool = True):
     """-> (dx [n, d] (== ddelta), dw or None). gxn2 may be None (no gradient on the sum)."""
     _dense(xn2, w, rstd, gy2, gxn2)
-    n, d = xn2.shape
+    n, d = _rows(xn2)
     dx = torch.empty_like(xn2)
     dw = torch.empty_like(w) if want_dw else None
     with _guard(xn2.device):
@@ -244,7 +253,7 @@ def add_rmsnorm_bwd(xn2, w, rstd, gy2, gxn2, want_dw: bool = True):
 def layernorm_fwd(x2, w, b, eps: float, delta2=None):
     """-> (xn or None, y [n, d], mean [n], rstd [n]); with ``delta2`` the residual-add form."""
     _dense(x2, w, b, delta2)
-    n, d = x2.shape
+    n, d = _rows(x2)
     y = torch.empty_like(x2)
     stats = torch.empty(2, n, device=x2.device, dtype=torch.float32)
     xn = torch.empty_like(x2) if delta2 is not None else None
@@ -264,7 +273,7 @@ def layernorm_fwd(x2, w, b, eps: float, delta2=None):
 def layernorm_bwd(x2, w, mean, rstd, dy2, gxn2=None, want_dw: bool = True, want_db: bool = True):
     """-> (dx [n, d], dw or None, db or None); ``x2`` is the normalised input (xn of the add form)."""
     _dense(x2, w, mean, rstd, dy2, gxn2)
-    n, d = x2.shape
+    n, d = _rows(x2)
     dx = torch.empty_like(x2)
     dw = torch.empty_like(w) if want_dw else None
     db = torch.empty_like(w) if want_db else None

@@ -20,20 +20,16 @@ from . import _hip, _ops
 from ._common import _note, fast_ok
 
 
-def _flat(t: torch.Tensor) -> torch.Tensor:
-    return t.contiguous().view(-1, t.shape[-1])
+def _c(t):
+    return t if t is None or t.is_contiguous() else t.contiguous()
 
 
 def _launch_fwd(x, w, b, eps, delta=None):
-    xn2, y2, mean, rstd = _hip.layernorm_fwd(_flat(x), w.contiguous(), None if b is None else b.contiguous(),
-                                             eps, None if delta is None else _flat(delta))
-    return (None if xn2 is None else xn2.view(x.shape)), y2.view(x.shape), mean, rstd
+    return _hip.layernorm_fwd(_c(x), _c(w), _c(b), eps, _c(delta))
 
 
 def _launch_bwd(x, w, mean, rstd, dy, gxn=None, want_dw=True, want_db=True):
-    dx2, dw, db = _hip.layernorm_bwd(_flat(x), w.contiguous(), mean, rstd, _flat(dy),
-                                     None if gxn is None else _flat(gxn), want_dw, want_db)
-    return dx2.view(x.shape), dw, db
+    return _hip.layernorm_bwd(_c(x), _c(w), mean, rstd, _c(dy), _c(gxn), want_dw, want_db)
 
 
 # ------------------------------------------------------------------ eager: autograd.Function

@@ -24,29 +24,25 @@ from . import _hip, _ops
 from ._common import _note, fast_ok
 
 
-def _flat(t: torch.Tensor) -> torch.Tensor:
-    return t.contiguous().view(-1, t.shape[-1])
+def _c(t: torch.Tensor) -> torch.Tensor:
+    # is_contiguous() is a tenth of the cost of a contiguous() that has nothing to do
+    return t if t.is_contiguous() else t.contiguous()
 
 
 def _launch_rms_fwd(x, w, eps):
-    y2, rstd = _hip.rmsnorm_fwd(_flat(x), w.contiguous(), eps)
-    return y2.view(x.shape), rstd
+    return _hip.rmsnorm_fwd(_c(x), _c(w), eps)
 
 
 def _launch_rms_bwd(x, w, rstd, dy, want_dw=True):
-    dx2, dw = _hip.rmsnorm_bwd(_flat(x), w.contiguous(), rstd, _flat(dy), want_dw)
-    return dx2.view(x.shape), dw
+    return _hip.rmsnorm_bwd(_c(x), _c(w), rstd, _c(dy), want_dw)
 
 
 def _launch_addrms_fwd(x, delta, w, eps):
-    xn2, y2, rstd = _hip.add_rmsnorm_fwd(_flat(x), _flat(delta), w.contiguous(), eps)
-    return xn2.view(x.shape), y2.view(x.shape), rstd
+    return _hip.add_rmsnorm_fwd(_c(x), _c(delta), _c(w), eps)
 
 
 def _launch_addrms_bwd(xn, w, rstd, gxn, gy, want_dw=True):
-    g_res = None if gxn is None else _flat(gxn)
-    dx2, dw = _hip.add_rmsnorm_bwd(_flat(xn), w.contiguous(), rstd, _flat(gy), g_res, want_dw)
-    return dx2.view(xn.shape), dw
+    return _hip.add_rmsnorm_bwd(_c(xn), _c(w), rstd, _c(gy), None if gxn is None else _c(gxn), want_dw)
 
 
 # ------------------------------------------------------------------ eager: autograd.Function
