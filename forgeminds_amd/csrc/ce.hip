@@ -475,9 +475,12 @@ int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float
     else LAUNCH(T, 1024, 8);                   \
   } while (0)
   // the fewest threads that hold the row in at most 8 vectors each: small workgroups keep
-  // several rows per compute unit in different phases (loading, reducing, storing)
+  // several rows per compute unit in different phases (loading, reducing, storing). fp16 and
+  // fp32 rows stop at 4 vectors below 1024 threads: with 8 the compiler keeps the converted
+  // values of all of them alive (over 220 registers, one workgroup per unit).
+  const int per_thread = dtype == FM_BF16 ? 8 : 4;
   int threads = pref == 256 || pref == 512 || pref == 1024 ? pref : 256;
-  while (threads < 1024 && nvec > (int64_t)threads * 8) threads *= 2;
+  while (threads < 1024 && nvec > (int64_t)threads * per_thread) threads *= 2;
   int iters = 2;
   while ((int64_t)threads * iters < nvec) iters *= 2;
   if (dtype == FM_F32) BY_SHAPE(float);
