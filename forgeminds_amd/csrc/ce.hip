@@ -331,6 +331,98 @@ __global__ __launch_bounds__(1024) void scale_inplace_kernel(T* x, const float* 
     Elem<T>::store1(x + i, Elem<T>::load1(x + i) * f);
 }
 
+// Narrow rows (up to 1024 logits, e.g. classification heads): a row is owned by TPR lanes of a
+// wave, each holding ITERS elements (t, t + TPR, ...), several rows per workgroup. LOSS writes
+// lse / row_loss, GRAD writes (softmax - onehot) * scale with scale = grad_out / n_valid (each
+// NULL pointer counts as 1). Any alignment, one element per load.
+template <typename T, int TPR, int ITERS, bool LOSS, bool GRAD>
+__global__ __launch_bounds__(256) void ce_rows_kernel(const T* logits, const int64_t* __restrict__ labels,
+                                                      const float* __restrict__ n_valid,
+                                                      const float* __restrict__ grad_out,
+                                                      float* __restrict__ lse, float* __restrict__ row_loss,
+                                                      T* dlogits, int64_t n, int v, int64_t ignore_index) {
+  constexpr int RPB = 256 / TPR;
+  const int tid = threadIdx.x;
+  const int rib = tid / TPR;
+  const int t = tid % TPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + rib;
+  const bool valid = row < n;
+  const int64_t base = row * (int64_t)v;
+  const int64_t y64 = valid ? labels[row] : ignore_index;
+  const bool ignored = y64 == ignore_index;
+  const int y = (y64 >= 0 && y64 < v) ? (int)y64 : -1;
+  float z[ITERS];
+  float m = kNegBig;
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * TPR + t;
+    // an ignored row of the gradient-only form is not read at all
+    z[i] = (valid && c < v && (LOSS || !ignored)) ? Elem<T>::load1(logits + base + c) * kLog2e : -INFINITY;
+    m = fmaxf(m, z[i]);
+  }
+  m = group_reduce<TPR, OpMax>(m);
+  float ssum = 0.f;
+  float ylogit2 = 0.f;          // the label's logit (times log2 e), found among the lane's elements
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    if (i * TPR + t == y) ylogit2 = z[i];
+    z[i] = fast_exp2(z[i] - m);
+    ssum += z[i];
+  }
+  ssum = group_reduce<TPR, OpSum>(ssum);
+  const float l2 = m + fast_log2(ssum);
+  if constexpr (LOSS) {
+    ylogit2 = group_reduce<TPR, OpSum>(ylogit2);     // one lane holds it, the others add 0
+    if (valid && t == 0) {
+      const float l = l2 * kLn2;
+      if (lse != nullptr) lse[row] = l;
+      row_loss[row] = ignored ? 0.f : (y >= 0 ? l - ylogit2 * kLn2 : __builtin_nanf(""));
+    }
+  }
+  if constexpr (GRAD) {
+    const float scale = (grad_out != nullptr ? *grad_out : 1.f) / (n_valid != nullptr ? *n_valid : 1.f);
+    const float inv = 1.f / ssum;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = i * TPR + t;
+      if (valid && c < v) {
+        float p = ignored ? 0.f : z[i] * inv;
+        if (c == y && !ignored) p -= 1.f;
+        Elem<T>::store1(dlogits + base + c, ignored ? 0.f : p * scale);
+      }
+    }
+  }
+}
+
+// rows of up to 1024 logits go to ce_rows_kernel; returns false for wider rows
+template <typename T, bool LOSS, bool GRAD>
+bool launch_rows(const void* logits, const int64_t* labels, const float* n_valid, const float* grad_out,
+                 float* lse, float* row_loss, void* dlogits, int64_t n, int v, int64_t ignore_index,
+                 hipStream_t st) {
+  if (v > 64 * 16) return false;
+  const int tpr = v <= 16 * 16 ? 16 : 64;
+  int iters = 1;
+  while (tpr * iters < v) iters *= 2;
+  const dim3 grid((unsigned)((n + 256 / tpr - 1) / (256 / tpr)));
+#define GOR(TPR_, IT_)                                                                              \
+  if (tpr == TPR_ && iters == IT_) {                                                                \
+    hipLaunchKernelGGL((ce_rows_kernel<T, TPR_, IT_, LOSS, GRAD>), grid, dim3(256), 0, st,          \
+                       static_cast<const T*>(logits), labels, n_valid, grad_out, lse, row_loss,     \
+                       static_cast<T*>(dlogits), n, v, ignore_index);                               \
+    return true;                                                                                    \
+  }
+  GOR(16, 1) GOR(16, 2) GOR(16, 4) GOR(16, 8) GOR(16, 16) GOR(64, 8) GOR(64, 16)
+#undef GOR
+  return false;
+}
+
+#define FM_CE_BY_DTYPE(dtype, CALL)              \
+  do {                                           \
+    if ((dtype) == FM_F32) { CALL(float); }      \
+    else if ((dtype) == FM_BF16) { CALL(bf16_t); } \
+    else { CALL(f16_t); }                        \
+  } while (0)
+
 template <typename T>
 int launch_fwd(const void* logits, const int64_t* labels, float* lse, float* row_loss, int64_t n,
                int v, int64_t ignore_index, bool vec_ok, hipStream_t st) {
@@ -386,13 +478,19 @@ int fm_ce_fwd(const void* logits, const int64_t* labels, float* lse, float* row_
   FM_CHECK_ARG(loss && n_valid, "fm_ce_fwd: NULL scalar output");
   FM_CHECK_ARG(n == 0 || (logits && labels && lse && row_loss), "fm_ce_fwd: NULL pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  bool narrow = false;
   if (n > 0) {
+#define CALL(T) narrow = launch_rows<T, true, false>(logits, labels, nullptr, nullptr, lse, row_loss, nullptr, n, (int)v, ignore_index, st)
+    FM_CE_BY_DTYPE(dtype, CALL);
+#undef CALL
+  }
+  if (n > 0 && !narrow) {
     const bool vec_ok = fm_host::aligned16(logits);
     if (dtype == FM_F32) launch_fwd<float>(logits, labels, lse, row_loss, n, (int)v, ignore_index, vec_ok, st);
     else if (dtype == FM_BF16) launch_fwd<bf16_t>(logits, labels, lse, row_loss, n, (int)v, ignore_index, vec_ok, st);
     else launch_fwd<f16_t>(logits, labels, lse, row_loss, n, (int)v, ignore_index, vec_ok, st);
-    FM_CHECK_LAUNCH("fm_ce_fwd");
   }
+  if (n > 0) FM_CHECK_LAUNCH("fm_ce_fwd");
   hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, st, row_loss, labels, n,
                      ignore_index, reduction == FM_REDUCE_MEAN ? 1 : 0, loss, n_valid);
   FM_CHECK_LAUNCH("fm_ce_fwd(finalize)");
@@ -407,6 +505,14 @@ int fm_ce_bwd(const void* logits, const int64_t* labels, const float* lse, const
   if (n == 0) return FM_OK;
   FM_CHECK_ARG(logits && labels && lse && dlogits, "fm_ce_bwd: NULL pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  bool narrow = false;
+#define CALL(T) narrow = launch_rows<T, false, true>(logits, labels, n_valid, grad_out, nullptr, nullptr, dlogits, n, (int)v, ignore_index, st)
+  FM_CE_BY_DTYPE(dtype, CALL);
+#undef CALL
+  if (narrow) {
+    FM_CHECK_LAUNCH("fm_ce_bwd");
+    return FM_OK;
+  }
   const bool vec_ok = fm_host::aligned16(logits) && fm_host::aligned16(dlogits);
   if (dtype == FM_F32) launch_bwd<float>(logits, labels, lse, n_valid, grad_out, dlogits, n, (int)v, ignore_index, vec_ok, st);
   else if (dtype == FM_BF16) launch_bwd<bf16_t>(logits, labels, lse, n_valid, grad_out, dlogits, n, (int)v, ignore_index, vec_ok, st);
@@ -427,6 +533,24 @@ int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int esize = dtype == FM_F32 ? 4 : 2;
   const int64_t nvec = v / (16 / esize);
+  if (n > 0 && v <= 64 * 16) {   // narrow rows: lane groups, any alignment, in place allowed
+    const bool mean_ = reduction == FM_REDUCE_MEAN;
+    if (mean_) {
+      hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(1024), 0, st, labels, n, ignore_index, n_valid);
+      FM_CHECK_LAUNCH("fm_ce_loss_grad(count)");
+    }
+    bool done = false;
+#define CALL(T) done = launch_rows<T, true, true>(logits, labels, mean_ ? n_valid : nullptr, nullptr, lse, row_loss, dlogits, n, (int)v, ignore_index, st)
+    FM_CE_BY_DTYPE(dtype, CALL);
+#undef CALL
+    if (done) {
+      FM_CHECK_LAUNCH("fm_ce_loss_grad");
+      hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, st, row_loss, labels, n, ignore_index,
+                         mean_ ? 1 : 0, loss, n_valid);
+      FM_CHECK_LAUNCH("fm_ce_loss_grad(finalize)");
+      return FM_OK;
+    }
+  }
   const bool one_pass = n > 0 && fm_host::aligned16(logits) && fm_host::aligned16(dlogits) &&
                         nvec <= 8 * 1024;
   if (!one_pass) {

@@ -400,8 +400,11 @@ def test_moe_layer_matches_the_reference_expression():
     ref = torch.zeros_like(xr).index_add_(0, tok, ys.to(xr.dtype))
     ref.square().sum().backward()
     assert torch.allclose(out, ref, rtol=1e-4, atol=1e-5)
-    assert torch.allclose(gx, xr.grad, rtol=1e-3, atol=1e-5)
-    assert torch.allclose(gate_g, layer.router.gate.weight.grad, rtol=1e-3, atol=1e-5)
+    # the reference side sums with atomics (index_add_), so its own last bits move from run to run:
+    # tolerances are relative to each tensor's scale
+    assert torch.allclose(gx, xr.grad, rtol=1e-3, atol=1e-4 * float(xr.grad.abs().max()))
+    gw = layer.router.gate.weight.grad
+    assert torch.allclose(gate_g, gw, rtol=1e-3, atol=1e-4 * float(gw.abs().max()))
 
 
 def test_qk_norm_rope_surface_and_op_path():

@@ -236,7 +236,8 @@ def test_layernorm_determinism_unaligned_and_empty():
 
 # ------------------------------------------------------------------ cross entropy
 CE_CASES = [(512, 32000, BF16), (7, 50257, BF16), (5, 1000, F32), (4, 7, F16), (9, 16, F32),
-            (3, 128256, BF16), (6, 32001, F32), (33, 4096, F16), (2, 1, F32), (64, 50257, F32)]
+            (3, 128256, BF16), (6, 32001, F32), (33, 4096, F16), (2, 1, F32), (64, 50257, F32),
+            (1000, 100, BF16), (300, 257, F16), (50, 1024, F32), (70, 33, BF16), (129, 600, BF16)]
 
 
 @pytest.mark.parametrize("n,v,dt", CE_CASES)
@@ -278,10 +279,10 @@ def test_ce_loss_and_gradient_in_one_pass(n, v, dt, reduction):
     y = torch.randint(0, v, (n,), generator=g)
     y[torch.rand(n, generator=g) < 0.2] = -100
     o64, _ = O.cross_entropy(lg, y, acc=torch.float64)
-    _, ograd = O.cross_entropy(lg, y)
+    _, ograd = O.cross_entropy(lg.float(), y)        # unrounded: the sum form rescales it
     n_valid = max(1, int((y != -100).sum()))
     if reduction == "sum":
-        o64, ograd = o64 * n_valid, ograd.float() * n_valid
+        o64, ograd = o64 * n_valid, ograd * n_valid
     lgd, yd = lg.to(DEV), y.to(DEV)
     keep = lgd.clone()
     loss, dl, nv, rows = _hip.ce_loss_grad(lgd, yd, -100, reduction)
