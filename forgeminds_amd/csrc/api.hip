@@ -18,6 +18,7 @@ const char* const kParamNames[fm_host::P_COUNT] = {
     "topk_variant",
     "vocab_unroll",
     "norm_fwd_blocks_per_cu",
+    "ce_rows_max_v",
 };
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cus[kMaxDevices];

@@ -100,7 +100,17 @@ __global__ __launch_bounds__(1024) void ce_finalize_kernel(const float* __restri
   __shared__ int si[16];
   float a = 0.f;
   int cnt = 0;
-  for (int64_t i = threadIdx.x; i < n; i += 1024) {
+  // eight rows' loads in flight per thread; the additions keep the order stated above
+  int64_t i = threadIdx.x;
+  for (; i + 7 * 1024 < n; i += 8 * 1024) {
+    float r[8];
+    int64_t l[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) { r[u] = row_loss[i + u * 1024]; l[u] = labels[i + u * 1024]; }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) { a += r[u]; cnt += l[u] != ignore_index ? 1 : 0; }
+  }
+  for (; i < n; i += 1024) {
     a += row_loss[i];
     cnt += labels[i] != ignore_index ? 1 : 0;
   }
@@ -187,7 +197,15 @@ __global__ __launch_bounds__(1024) void ce_count_kernel(const int64_t* __restric
                                                         float* __restrict__ n_valid) {
   __shared__ int si[16];
   int cnt = 0;
-  for (int64_t i = threadIdx.x; i < n; i += 1024) cnt += labels[i] != ignore_index ? 1 : 0;
+  int64_t i = threadIdx.x;
+  for (; i + 7 * 1024 < n; i += 8 * 1024) {
+    int64_t l[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) l[u] = labels[i + u * 1024];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) cnt += l[u] != ignore_index ? 1 : 0;
+  }
+  for (; i < n; i += 1024) cnt += labels[i] != ignore_index ? 1 : 0;
   cnt = wave_sum_i(cnt);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   if (lane == 0) si[wave] = cnt;
@@ -395,11 +413,19 @@ __global__ __launch_bounds__(256) void ce_rows_kernel(const T* logits, const int
 }
 
 // rows of up to 1024 logits go to ce_rows_kernel; returns false for wider rows
+// Widest row the lane-group kernel takes (tunable downwards with "ce_rows_max_v").
+inline int rows_max_v() {
+  const int p = fm_host::get_param(fm_host::P_CE_ROWS_MAX_V);
+  return p > 0 && p < 64 * 16 ? p : 64 * 16;
+}
+
 template <typename T, bool LOSS, bool GRAD>
 bool launch_rows(const void* logits, const int64_t* labels, const float* n_valid, const float* grad_out,
                  float* lse, float* row_loss, void* dlogits, int64_t n, int v, int64_t ignore_index,
                  hipStream_t st) {
-  if (v > 64 * 16) return false;
+  if (v > rows_max_v()) return false;
+  // fp32 gradients of rows past 512 classes go faster through the workgroup-per-row kernels
+  if (GRAD && sizeof(T) == 4 && v > 512) return false;
   const int tpr = v <= 16 * 16 ? 16 : 64;
   int iters = 1;
   while (tpr * iters < v) iters *= 2;
@@ -533,7 +559,7 @@ int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int esize = dtype == FM_F32 ? 4 : 2;
   const int64_t nvec = v / (16 / esize);
-  if (n > 0 && v <= 64 * 16) {   // narrow rows: lane groups, any alignment, in place allowed
+  if (n > 0 && v <= rows_max_v() && !(esize == 4 && v > 512)) {   // narrow rows: lane groups, any alignment, in place allowed
     const bool mean_ = reduction == FM_REDUCE_MEAN;
     if (mean_) {
       hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(1024), 0, st, labels, n, ignore_index, n_valid);

@@ -241,7 +241,15 @@ __global__ __launch_bounds__(1024) void kl_finalize_kernel(const float* __restri
                                                            float* __restrict__ loss) {
   __shared__ float sf[16];
   float a = 0.f;
-  for (int64_t i = threadIdx.x; i < n; i += 1024) a += row_kl[i];
+  int64_t i = threadIdx.x;
+  for (; i + 7 * 1024 < n; i += 8 * 1024) {   // eight loads in flight; additions in the same order
+    float r[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) r[u] = row_kl[i + u * 1024];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) a += r[u];
+  }
+  for (; i < n; i += 1024) a += row_kl[i];
   a = wave_sum(a);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   if (lane == 0) sf[wave] = a;

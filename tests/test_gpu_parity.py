@@ -237,7 +237,8 @@ def test_layernorm_determinism_unaligned_and_empty():
 # ------------------------------------------------------------------ cross entropy
 CE_CASES = [(512, 32000, BF16), (7, 50257, BF16), (5, 1000, F32), (4, 7, F16), (9, 16, F32),
             (3, 128256, BF16), (6, 32001, F32), (33, 4096, F16), (2, 1, F32), (64, 50257, F32),
-            (1000, 100, BF16), (300, 257, F16), (50, 1024, F32), (70, 33, BF16), (129, 600, BF16)]
+            (1000, 100, BF16), (300, 257, F16), (50, 1024, F32), (70, 33, BF16), (129, 600, BF16),
+            (300, 512, F32), (40, 513, F32)]
 
 
 @pytest.mark.parametrize("n,v,dt", CE_CASES)
