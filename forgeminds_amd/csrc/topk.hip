@@ -238,8 +238,20 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
   hipLaunchKernelGGL((topk_lds_kernel<T, TH, UN>), grid, dim3(TH), (size_t)(nvec + 8) * 2, st, xp, vp, i32, \
                      i64, v, k, vec_ok)
   int variant = fm_host::get_param(fm_host::P_TOPK_VARIANT);
+  const bool forced = variant != 0;       // a forced variant also bypasses the wave-per-row kernel
   if (variant == 0) variant = nvec <= 3072 ? 1 : (nvec <= 12288 ? 2 : 3);
-  if (v <= 64 * 16) {                     // short rows: a wave per row
+  if (!forced) {
+    // the threshold search needs k <= 63 x (full waves of the row); more threads give more of
+    // them while the row has a vector for each. Past half of that bound the candidates mostly
+    // overflow anyway; the exact path that then runs costs a pass per key bit, which for the 16
+    // bits of a half type is cheaper at the smaller workgroup (measured), for fp32's 32 is not.
+    const int64_t whole = v / EPV;
+    auto cap = [&](int threads) { return (int)(std::min<int64_t>(threads, whole) / 64) * 63; };
+    auto pays = [&](int threads) { return sizeof(T) == 4 || 2 * k <= cap(threads) + 8; };
+    if (variant == 1 && k > cap(256) && cap(512) > cap(256) && pays(512)) variant = 2;
+    if (variant == 2 && k > cap(512) && cap(1024) > cap(512) && pays(1024)) variant = 3;
+  }
+  if (v <= 64 * 16 && !forced) {          // short rows: a wave per row
     const dim3 wgrid((unsigned)((n + kWaveRows - 1) / kWaveRows));
 #define GOW(EPL_)                                                                                 \
   hipLaunchKernelGGL((topk_wave_kernel<T, EPL_>), wgrid, dim3(64 * kWaveRows), 0, st, xp, vp, i32, i64, n, v, k)

@@ -499,7 +499,8 @@ TOPK_CASES = [(32, 128256, 64, BF16), (8, 4096, 64, F32), (4, 64, 8, F32), (3, 5
               (1, 512, 512, F32), (5, 1, 1, F32), (2, 600, 4, F32), (4, 5000, 512, F32),
               (2, 1025, 3, BF16), (3, 70000, 512, F32), (6, 50257, 64, BF16), (2, 140000, 64, F32),
               (1000, 64, 8, F32), (333, 128, 2, BF16), (77, 200, 200, F16), (50, 1024, 512, BF16),
-              (41, 1000, 64, F32), (9, 7, 7, BF16), (130, 513, 100, F16), (5, 1024, 1, F32)]
+              (41, 1000, 64, F32), (9, 7, 7, BF16), (130, 513, 100, F16), (5, 1024, 1, F32),
+              (6, 4096, 256, BF16), (5, 8192, 512, F32), (4, 8192, 256, F16), (3, 16384, 512, F32)]
 
 
 @pytest.mark.parametrize("n,v,k,dt", TOPK_CASES)
