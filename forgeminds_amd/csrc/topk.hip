@@ -142,80 +142,199 @@ __global__ __launch_bounds__(THREADS) void topk_lds_kernel(const T* __restrict__
                                          nullptr, 0.f, 0.f);
 }
 
-// Rows of up to 1024 elements: one wave per row, four rows per workgroup. Lane l holds the
-// elements l, l + 64, ... as keys in registers; the k-th key comes from a bitwise search whose
-// counts are wave ballots (no memory traffic, no workgroup barrier inside the search), the
-// selected elements take slots in LDS (greater first, then the first ties in index order) and
-// are ranked by counting among themselves.
-constexpr int kWaveRows = 4;
+// Rows of up to 2048 elements: one wave per row (a 64-thread workgroup each), the whole row as
+// keys in registers (EPL per lane; 16-byte loads when the rows are aligned, else lane-strided
+// scalars). No step depends on the order of the registers:
+//   1. tau = the k-th largest of the lanes' group maxima (ballot search, one to four compares a
+//      bit) -- at least k elements reach it;
+//   2. elements >= tau become candidates (key, kWaveMaxV - column) in LDS; when at most
+//      64 exist each lane takes one and they are ranked by counting, which ends the row; up to
+//      kWaveCand are reloaded, four a lane, and searched instead of the row (otherwise the
+//      row's own registers are searched: heavy ties, or k too large for step 1);
+//   3. wave_select: bitwise search for the k-th key, then, when more ties exist than places,
+//      a bitwise search over the reversed column for the last tie admitted (lowest columns
+//      win); winners take LDS slots and are ranked by counting among themselves.
+constexpr int kWaveMaxV = 2048;
+constexpr int kWaveCand = 256;
 
-template <typename T, int EPL>
-__global__ __launch_bounds__(64 * kWaveRows) void topk_wave_kernel(const T* __restrict__ x,
-                                                                    T* __restrict__ values,
-                                                                    int32_t* __restrict__ idx32,
-                                                                    int64_t* __restrict__ idx64, int64_t n,
-                                                                    int v, int k) {
-  __shared__ unsigned long long sel[kWaveRows][kMaxK];
-  constexpr uint32_t KMASK = KeyBits<T>::mask;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t row = (int64_t)blockIdx.x * kWaveRows + wave;
-  const bool valid = row < n;                  // uniform per wave; nobody leaves before the barrier
-  const T* rp = x + (valid ? row : 0) * (int64_t)v;
-  uint32_t mk[EPL];
-#pragma unroll
-  for (int e = 0; e < EPL; ++e) {
-    const int col = lane + 64 * e;
-    // 0 is below the key of every value (-inf maps to 0x007FFFFF), so empty slots never win
-    mk[e] = (valid && col < v) ? (key_of(Elem<T>::load1(rp + col)) & KMASK) : 0u;
-  }
+template <typename T, int NR>
+__device__ __forceinline__ void wave_select(const uint32_t (&key)[NR], const uint32_t (&rc)[NR], int nreg,
+                                            int k, unsigned long long* buf, const T* rp, int64_t row,
+                                            T* __restrict__ values, int32_t* __restrict__ idx32,
+                                            int64_t* __restrict__ idx64) {
+  const int lane = threadIdx.x;
+  const unsigned long long below = (1ull << lane) - 1ull;
   uint32_t kth = 0u;
   for (int bit = 31; bit >= KeyBits<T>::low; --bit) {
     const uint32_t trial = kth | (1u << bit);
     int cnt = 0;
 #pragma unroll
-    for (int e = 0; e < EPL; ++e) cnt += __builtin_popcountll(__ballot(mk[e] >= trial));
+    for (int e = 0; e < NR; ++e)
+      if (e < nreg) cnt += __builtin_popcountll(__ballot(key[e] >= trial));
     if (cnt >= k) kth = trial;
   }
-  int c_gt = 0;
+  int c_gt = 0, c_eq = 0;
 #pragma unroll
-  for (int e = 0; e < EPL; ++e) c_gt += __builtin_popcountll(__ballot(mk[e] > kth));
-  const int need = k - c_gt;                   // ties admitted, lowest columns first
-  const unsigned long long below = (1ull << lane) - 1ull;
-  int base_gt = 0, base_eq = 0;
-  unsigned long long* my = sel[wave];
-#pragma unroll
-  for (int e = 0; e < EPL; ++e) {              // ascending e, ascending lane: ascending column
-    const int col = lane + 64 * e;
-    const unsigned long long m_gt = __ballot(mk[e] > kth);
-    const unsigned long long m_eq = __ballot(mk[e] == kth && mk[e] != 0u);
-    const unsigned long long item = ((unsigned long long)mk[e] << 32) | (uint32_t)(~col);
-    if (mk[e] > kth) my[base_gt + __builtin_popcountll(m_gt & below)] = item;
-    if (mk[e] == kth && mk[e] != 0u) {
-      const int t = base_eq + __builtin_popcountll(m_eq & below);
-      if (t < need) my[c_gt + t] = item;
+  for (int e = 0; e < NR; ++e)
+    if (e < nreg) {
+      c_gt += __builtin_popcountll(__ballot(key[e] > kth));
+      c_eq += __builtin_popcountll(__ballot(key[e] == kth));
     }
-    base_gt += __builtin_popcountll(m_gt);
-    base_eq += __builtin_popcountll(m_eq);
+  const int need = k - c_gt;          // places left for the c_eq ties (kth > 0: empty slots never tie)
+  uint32_t cth = 0u;                  // ties whose reversed column reaches cth are admitted
+  if (need < c_eq) {
+    for (int bit = 11; bit >= 0; --bit) {   // reversed columns are 1..kWaveMaxV = 1 << 11
+      const uint32_t trial = cth | (1u << bit);
+      int cnt = 0;
+#pragma unroll
+      for (int e = 0; e < NR; ++e)
+        if (e < nreg) cnt += __builtin_popcountll(__ballot(key[e] == kth && rc[e] >= trial));
+      if (cnt >= need) cth = trial;
+    }
   }
+  __syncthreads();                    // the candidates in buf have been read
+  int base = 0;
+#pragma unroll
+  for (int e = 0; e < NR; ++e)
+    if (e < nreg) {
+      const bool win = key[e] > kth || (key[e] == kth && rc[e] >= cth);
+      const unsigned long long m = __ballot(win);
+      if (win) buf[base + __builtin_popcountll(m & below)] = ((unsigned long long)key[e] << 32) | rc[e];
+      base += __builtin_popcountll(m);
+    }
   __syncthreads();
-  if (!valid) return;
   for (int s = lane; s < k; s += 64) {
-    const unsigned long long me = my[s];
+    const unsigned long long me = buf[s];
     int r = 0;
     int i = 0;
     for (; i + 8 <= k; i += 8) {
       unsigned long long o[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) o[u] = my[i + u];
+      for (int u = 0; u < 8; ++u) o[u] = buf[i + u];
 #pragma unroll
       for (int u = 0; u < 8; ++u) r += o[u] > me ? 1 : 0;
     }
-    for (; i < k; ++i) r += my[i] > me ? 1 : 0;
-    const int col = (int)(~(uint32_t)(me & 0xFFFFFFFFull));
+    for (; i < k; ++i) r += buf[i] > me ? 1 : 0;
+    const int col = kWaveMaxV - (int)(uint32_t)(me & 0xFFFFFFFFull);
     const int64_t o = row * (int64_t)k + r;
     if (idx32 != nullptr) idx32[o] = col;
     if (idx64 != nullptr) idx64[o] = col;
     if (values != nullptr) values[o] = rp[col];
+  }
+}
+
+template <typename T, int EPL, bool VEC>
+__global__ __launch_bounds__(64) void topk_wave_kernel(const T* __restrict__ x, T* __restrict__ values,
+                                                        int32_t* __restrict__ idx32,
+                                                        int64_t* __restrict__ idx64, int v, int k) {
+  __shared__ unsigned long long buf[kMaxK];
+  constexpr uint32_t KMASK = KeyBits<T>::mask;
+  constexpr int EPV = Elem<T>::kVec;
+  static_assert(!VEC || EPL % EPV == 0, "whole vectors per lane");
+  const int lane = threadIdx.x;
+  const int64_t row = blockIdx.x;
+  const T* rp = x + row * (int64_t)v;
+  auto col_of = [&](int e) { return VEC ? ((e / EPV) * 64 + lane) * EPV + (e % EPV) : lane + 64 * e; };
+  // 0 is below the key of every value (-inf maps to 0x007FFFFF), so empty slots never win
+  uint32_t mk[EPL];
+  if constexpr (VEC) {
+#pragma unroll
+    for (int g = 0; g < EPL / EPV; ++g) {
+      const int c0 = (g * 64 + lane) * EPV;
+      if (c0 < v) {
+        float f[EPV];
+        Elem<T>::unpack(load16_stream(rp + c0), f);
+#pragma unroll
+        for (int i = 0; i < EPV; ++i) mk[g * EPV + i] = key_of(f[i]) & KMASK;
+      } else {
+#pragma unroll
+        for (int i = 0; i < EPV; ++i) mk[g * EPV + i] = 0u;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) {
+      const int col = lane + 64 * e;
+      mk[e] = col < v ? (key_of(Elem<T>::load1(rp + col)) & KMASK) : 0u;
+    }
+  }
+  // step 1: group maxima (one group per lane for small k, up to four otherwise)
+  constexpr int GM = EPL < 4 ? EPL : 4;
+  uint32_t gm[GM];
+#pragma unroll
+  for (int g = 0; g < GM; ++g) gm[g] = 0u;
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) gm[e % GM] = gm[e % GM] > mk[e] ? gm[e % GM] : mk[e];
+  int groups = GM;
+  if (k <= 16) {
+#pragma unroll
+    for (int g = 1; g < GM; ++g) {
+      gm[0] = gm[0] > gm[g] ? gm[0] : gm[g];
+      gm[g] = 0u;
+    }
+    groups = 1;
+  }
+  uint32_t tau = 0u;
+  if (k <= 64 * groups) {
+    for (int bit = 31; bit >= KeyBits<T>::low; --bit) {
+      const uint32_t trial = tau | (1u << bit);
+      int cnt = 0;
+#pragma unroll
+      for (int g = 0; g < GM; ++g)
+        if (g < groups) cnt += __builtin_popcountll(__ballot(gm[g] >= trial));
+      if (cnt >= k) tau = trial;
+    }
+  }
+  // step 2: candidates
+  const unsigned long long below = (1ull << lane) - 1ull;
+  int ncand = 0;
+  uint32_t rc[EPL];
+#pragma unroll
+  for (int e = 0; e < EPL; ++e) {
+    rc[e] = (uint32_t)(kWaveMaxV - col_of(e));
+    const bool c = mk[e] >= tau && mk[e] != 0u;
+    const unsigned long long m = __ballot(c);
+    if (m == 0ull) continue;          // most registers hold no candidate
+    if (c) {
+      const int s = ncand + __builtin_popcountll(m & below);
+      if (s < kWaveCand) buf[s] = ((unsigned long long)mk[e] << 32) | rc[e];
+    }
+    ncand += __builtin_popcountll(m);
+  }
+  __syncthreads();
+  if (ncand <= 64) {
+    // at most one candidate a lane: rank them all by counting; ranks below k are the output
+    const unsigned long long me = lane < ncand ? buf[lane] : 0ull;
+    int r = 0;
+    int i = 0;
+    for (; i + 8 <= ncand; i += 8) {
+      unsigned long long o[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) o[u] = buf[i + u];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) r += o[u] > me ? 1 : 0;
+    }
+    for (; i < ncand; ++i) r += buf[i] > me ? 1 : 0;
+    if (lane < ncand && r < k) {
+      const int col = kWaveMaxV - (int)(uint32_t)(me & 0xFFFFFFFFull);
+      const int64_t o = row * (int64_t)k + r;
+      if (idx32 != nullptr) idx32[o] = col;
+      if (idx64 != nullptr) idx64[o] = col;
+      if (values != nullptr) values[o] = rp[col];
+    }
+  } else if (ncand <= kWaveCand) {
+    constexpr int CR = kWaveCand / 64;
+    uint32_t ck[CR], cc[CR];
+#pragma unroll
+    for (int j = 0; j < CR; ++j) {
+      const int s = lane + 64 * j;
+      const unsigned long long item = s < ncand ? buf[s] : 0ull;
+      ck[j] = (uint32_t)(item >> 32);
+      cc[j] = (uint32_t)(item & 0xFFFFFFFFull);
+    }
+    wave_select<T, CR>(ck, cc, (ncand + 63) / 64, k, buf, rp, row, values, idx32, idx64);
+  } else {
+    wave_select<T, EPL>(mk, rc, EPL, k, buf, rp, row, values, idx32, idx64);
   }
 }
 
@@ -251,15 +370,26 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
     if (variant == 1 && k > cap(256) && cap(512) > cap(256) && pays(512)) variant = 2;
     if (variant == 2 && k > cap(512) && cap(1024) > cap(512) && pays(1024)) variant = 3;
   }
-  if (v <= 64 * 16 && !forced) {          // short rows: a wave per row
-    const dim3 wgrid((unsigned)((n + kWaveRows - 1) / kWaveRows));
-#define GOW(EPL_)                                                                                 \
-  hipLaunchKernelGGL((topk_wave_kernel<T, EPL_>), wgrid, dim3(64 * kWaveRows), 0, st, xp, vp, i32, i64, n, v, k)
-    if (v <= 64) GOW(1);
-    else if (v <= 128) GOW(2);
-    else if (v <= 256) GOW(4);
-    else if (v <= 512) GOW(8);
-    else GOW(16);
+  if (v <= kWaveMaxV && !forced) {       // short rows: a wave per row
+    int epl = 1;
+    while (64 * epl < v) epl *= 2;
+    const bool wvec = vec_ok && v % EPV == 0 && epl >= EPV;
+#define GOW(EPL_, VEC_)                                                                            \
+  hipLaunchKernelGGL((topk_wave_kernel<T, EPL_, VEC_>), grid, dim3(64), 0, st, xp, vp, i32, i64, v, k)
+#define GOWV(EPL_)                                                                                 \
+  if constexpr (EPL_ % EPV == 0) {                                                                 \
+    if (wvec) GOW(EPL_, true);                                                                     \
+    else GOW(EPL_, false);                                                                         \
+  } else {                                                                                         \
+    GOW(EPL_, false);                                                                              \
+  }
+    if (epl == 1) { GOWV(1) }
+    else if (epl == 2) { GOWV(2) }
+    else if (epl == 4) { GOWV(4) }
+    else if (epl == 8) { GOWV(8) }
+    else if (epl == 16) { GOWV(16) }
+    else { GOWV(32) }
+#undef GOWV
 #undef GOW
   }
   else if (nvec > kLdsMaxVec) {
