@@ -555,6 +555,25 @@ def test_topk_ties_nans_zeros_and_degenerate_rows():
         assert torch.equal(run(x, k), O.topk(x, k)[1])
     z = torch.zeros(5, 64)
     assert torch.equal(run(z, 64), torch.arange(64).expand(5, 64))
+    # the same kernel with 16-byte loads (aligned rows): all-equal rows, few distinct values,
+    # k up to the row width, and fp16 values one ulp apart
+    for dt in (BF16, F16, F32):
+        for v, ks in ((8, (1, 8)), (100, (1, 5, 100)), (1024, (1, 64, 100, 512)), (2048, (7, 64, 257, 512))):
+            z = torch.full((3, v), -1.5, dtype=dt)
+            x = torch.randint(0, 5, (6, v), generator=g).to(dt)
+            x[::2, ::9] = float("nan")
+            x[1::2, 3::4] = float("-inf")
+            for k in ks:
+                assert torch.equal(run(z, k), torch.arange(k).expand(3, k)), (dt, v, k)
+                assert torch.equal(run(x, k), O.topk(x, k)[1]), (dt, v, k)
+    steps = torch.randint(0, 8, (40, 2048), generator=g).float()
+    x = (1.0 + steps * 2.0 ** -10).to(F16) * torch.where(torch.rand(40, 2048, generator=g) < 0.5, 1.0, -1.0).to(F16)
+    for k in (3, 64, 200):
+        assert torch.equal(run(x, k), O.topk(x, k)[1])
+    x = (3 * torch.randn(50, 2048, generator=g)).to(BF16)
+    assert torch.equal(run(x, 2048 // 4), O.topk(x, 512)[1])
+    x = (3 * torch.randn(9, 300, generator=g))
+    assert torch.equal(run(x, 300), O.topk(x, 300)[1])
     # negative NaN payloads and a row of -inf
     x = torch.full((2, 3000), float("-inf"))
     x[0, 17] = -torch.tensor(float("nan"))
@@ -569,6 +588,9 @@ def test_topk_unaligned_rows():
         assert torch.equal(idx.cpu().long(), O.topk(x, 33)[1])
     base = (3 * torch.randn(3 * 9000 + 1, generator=g)).bfloat16().to(DEV)
     x = base[1:].view(3, 9000)                                        # base pointer off by 2 bytes
+    _, idx = _hip.topk(x, 20, torch.int32)
+    assert torch.equal(idx.cpu().long(), O.topk(x.cpu(), 20)[1])
+    x = base[1:1 + 12 * 2048].view(12, 2048)                          # the same for wave-per-row rows
     _, idx = _hip.topk(x, 20, torch.int32)
     assert torch.equal(idx.cpu().long(), O.topk(x.cpu(), 20)[1])
 
