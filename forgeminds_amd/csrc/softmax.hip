@@ -7,6 +7,9 @@
 // rows per workgroup when they are narrow), read once, reduced (maximum, then sum) and written.
 // Other rows take one workgroup each: an online (max, sum-exp) pass, then a second pass over
 // the row (served by L2 for rows that fit) that writes exp2(z - m) / s.
+//
+// Backward (forgemind/kernels/softmax.py:108-115: dx = (dy - sum(dy * y)) * y): the same three
+// shapes over two inputs, fp32 math on the stored y and dy, one rounding at the store.
 #include "fm_vocab.cuh"
 
 using namespace fm;
@@ -174,6 +177,145 @@ __global__ __launch_bounds__(256) void softmax_rows_scalar_kernel(const T* __res
   }
 }
 
+
+// ---------------------------------------------------------------- backward
+template <typename T, int THREADS, int UNROLL>
+__global__ __launch_bounds__(THREADS) void softmax_bwd_kernel(const T* __restrict__ y,
+                                                               const T* __restrict__ dy,
+                                                               T* __restrict__ dx, int v, bool vec_ok) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int NW = THREADS / 64;
+  __shared__ float smem[NW];
+  const int64_t row = blockIdx.x;
+  const T* yp = y + row * (int64_t)v;
+  const T* gp = dy + row * (int64_t)v;
+  T* op = dx + row * (int64_t)v;
+  const RowSplit sp = split_row<EPV>(row, v, vec_ok);
+  const int tid = threadIdx.x;
+  const int ne = edge_count(sp, v);
+  float dot = 0.f;
+  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+    u32x4 ry[UNROLL], rg[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) {
+        ry[u] = load16(yp + sp.head + (int64_t)c * EPV);
+        rg[u] = load16(gp + sp.head + (int64_t)c * EPV);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) {
+        float a[EPV], b[EPV];
+        Elem<T>::unpack(ry[u], a);
+        Elem<T>::unpack(rg[u], b);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) dot += a[e] * b[e];
+      }
+    }
+  }
+  for (int e = tid; e < ne; e += THREADS) {
+    const int col = edge_col(sp, e);
+    dot += Elem<T>::load1(yp + col) * Elem<T>::load1(gp + col);
+  }
+  dot = block_sum<NW>(dot, smem);
+  for (int c = tid; c < sp.nvec; c += THREADS) {
+    float a[EPV], b[EPV], o[EPV];
+    Elem<T>::unpack(load16(yp + sp.head + (int64_t)c * EPV), a);
+    Elem<T>::unpack(load16(gp + sp.head + (int64_t)c * EPV), b);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) o[e] = (b[e] - dot) * a[e];
+    store16_stream(op + sp.head + (int64_t)c * EPV, Elem<T>::pack(o));
+  }
+  for (int e = tid; e < ne; e += THREADS) {
+    const int col = edge_col(sp, e);
+    Elem<T>::store1(op + col, (Elem<T>::load1(gp + col) - dot) * Elem<T>::load1(yp + col));
+  }
+}
+
+template <typename T, int TPR, int ITERS>
+__global__ __launch_bounds__(RowBlock<TPR>::value) void softmax_bwd_rows_kernel(const T* __restrict__ y,
+                                                                                 const T* __restrict__ dy,
+                                                                                 T* __restrict__ dx,
+                                                                                 int64_t n, int v) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int BLOCK = RowBlock<TPR>::value;
+  constexpr int RPB = BLOCK / TPR;
+  __shared__ float smem[RPB * (TPR > 64 ? TPR / 64 : 1)];
+  const int tid = threadIdx.x;
+  const int rib = tid / TPR;
+  const int t = tid % TPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + rib;
+  const bool valid = row < n;
+  const int nvec = v / EPV;
+  const int64_t base = row * (int64_t)v;
+  u32x4 ry[ITERS], rg[ITERS];      // both rows stay packed between the dot product and the store
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * TPR + t;
+    if (valid && c < nvec) {
+      ry[i] = load16_stream(y + base + (int64_t)c * EPV);
+      rg[i] = load16_stream(dy + base + (int64_t)c * EPV);
+    } else {
+      ry[i] = u32x4{0u, 0u, 0u, 0u};
+      rg[i] = u32x4{0u, 0u, 0u, 0u};
+    }
+  }
+  float dot = 0.f;
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    float a[EPV], b[EPV];
+    Elem<T>::unpack(ry[i], a);
+    Elem<T>::unpack(rg[i], b);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) dot += a[e] * b[e];
+  }
+  dot = row_reduce<TPR, OpSum>(dot, smem, rib, t);
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * TPR + t;
+    if (valid && c < nvec) {
+      float a[EPV], b[EPV], o[EPV];
+      Elem<T>::unpack(ry[i], a);
+      Elem<T>::unpack(rg[i], b);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) o[e] = (b[e] - dot) * a[e];
+      store16_stream(dx + base + (int64_t)c * EPV, Elem<T>::pack(o));
+    }
+  }
+}
+
+template <typename T, int TPR, int ITERS>
+__global__ __launch_bounds__(256) void softmax_bwd_rows_scalar_kernel(const T* __restrict__ y,
+                                                                      const T* __restrict__ dy,
+                                                                      T* __restrict__ dx, int64_t n, int v) {
+  constexpr int RPB = 256 / TPR;
+  const int tid = threadIdx.x;
+  const int rib = tid / TPR;
+  const int t = tid % TPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + rib;
+  const bool valid = row < n;
+  const int64_t base = row * (int64_t)v;
+  float a[ITERS], b[ITERS];
+  float dot = 0.f;
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * TPR + t;
+    const bool in = valid && c < v;
+    a[i] = in ? Elem<T>::load1(y + base + c) : 0.f;
+    b[i] = in ? Elem<T>::load1(dy + base + c) : 0.f;
+    dot += a[i] * b[i];
+  }
+  dot = group_reduce<TPR, OpSum>(dot);
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * TPR + t;
+    if (valid && c < v) Elem<T>::store1(dx + base + c, (b[i] - dot) * a[i]);
+  }
+}
+
 #define FM_SOFTMAX_SHAPES(X) \
   X(4, 1) X(8, 1) X(16, 1) X(32, 1) X(64, 1) X(64, 2) X(128, 2) X(256, 2) X(256, 4) X(512, 4) X(512, 8) X(1024, 8)
 
@@ -226,6 +368,48 @@ void launch(const void* x, void* y, int64_t n, int v, bool vec_ok, hipStream_t s
 #undef LAUNCH
 }
 
+template <typename T>
+void launch_bwd(const void* y, const void* dy, void* dx, int64_t n, int v, bool vec_ok, hipStream_t st) {
+  const T* yp = static_cast<const T*>(y);
+  const T* gp = static_cast<const T*>(dy);
+  T* op = static_cast<T*>(dx);
+  constexpr int EPV = Elem<T>::kVec;
+  int tpr = 0, iters = 0;
+  // two packed rows in registers, on the plans of the forward; half types stop at 64 KiB rows
+  // (their unpacked copies would not fit the 128 registers of a 1024-thread workgroup)
+  if (vec_ok && v % EPV == 0 && v / EPV <= (sizeof(T) == 4 ? 8192 : 4096) &&
+      rows_plan(v / EPV, &tpr, &iters)) {
+#define X(TPR_, IT_)                                                                               \
+  if (tpr == TPR_ && iters == IT_) {                                                               \
+    constexpr int RPB = RowBlock<TPR_>::value / TPR_;                                              \
+    hipLaunchKernelGGL((softmax_bwd_rows_kernel<T, TPR_, IT_>), dim3((unsigned)((n + RPB - 1) / RPB)), \
+                       dim3(RowBlock<TPR_>::value), 0, st, yp, gp, op, n, v);                      \
+    return;                                                                                        \
+  }
+    FM_SOFTMAX_SHAPES(X)
+#undef X
+  }
+  if (v <= 64 * 16) {
+    const int tpr = v <= 16 * 16 ? 16 : 64;
+    int iters = 1;
+    while (tpr * iters < v) iters *= 2;
+    const dim3 sgrid((unsigned)((n + 256 / tpr - 1) / (256 / tpr)));
+#define GOS(TPR_, IT_)                                                                             \
+  if (tpr == TPR_ && iters == IT_) {                                                               \
+    hipLaunchKernelGGL((softmax_bwd_rows_scalar_kernel<T, TPR_, IT_>), sgrid, dim3(256), 0, st, yp, gp, op, n, v); \
+    return;                                                                                        \
+  }
+    GOS(16, 1) GOS(16, 2) GOS(16, 4) GOS(16, 8) GOS(16, 16) GOS(64, 8) GOS(64, 16)
+#undef GOS
+  }
+  const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 4);
+  const dim3 grid((unsigned)n);
+#define LAUNCH(TH, UN) \
+  hipLaunchKernelGGL((softmax_bwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, yp, gp, op, v, vec_ok)
+  FM_VOCAB_DISPATCH(sh, LAUNCH);
+#undef LAUNCH
+}
+
 }  // namespace
 
 extern "C" int fm_softmax_fwd(const void* x, void* y, int64_t n, int64_t v, int dtype,
@@ -245,5 +429,25 @@ extern "C" int fm_softmax_fwd(const void* x, void* y, int64_t n, int64_t v, int 
   else if (dtype == FM_BF16) launch<bf16_t>(x, y, n, (int)v, vec_ok, st);
   else launch<f16_t>(x, y, n, (int)v, vec_ok, st);
   FM_CHECK_LAUNCH("fm_softmax_fwd");
+  return FM_OK;
+}
+
+extern "C" int fm_softmax_bwd(const void* y, const void* dy, void* dx, int64_t n, int64_t v, int dtype,
+                              fm_stream_t stream) {
+  FM_CHECK_ARG(n >= 0 && v > 0, "fm_softmax_bwd: bad shape n=%lld v=%lld", (long long)n, (long long)v);
+  FM_CHECK_ARG(dtype == FM_F32 || dtype == FM_F16 || dtype == FM_BF16, "fm_softmax_bwd: bad dtype %d",
+               dtype);
+  if (n > 0x7fffffffLL || v > 0x7fffffffLL) {
+    fm_host::set_error("fm_softmax_bwd: n and v must be below 2^31");
+    return FM_ERR_UNSUPPORTED;
+  }
+  if (n == 0) return FM_OK;
+  FM_CHECK_ARG(y && dy && dx, "fm_softmax_bwd: NULL pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool vec_ok = fm_host::aligned16(y) && fm_host::aligned16(dy) && fm_host::aligned16(dx);
+  if (dtype == FM_F32) launch_bwd<float>(y, dy, dx, n, (int)v, vec_ok, st);
+  else if (dtype == FM_BF16) launch_bwd<bf16_t>(y, dy, dx, n, (int)v, vec_ok, st);
+  else launch_bwd<f16_t>(y, dy, dx, n, (int)v, vec_ok, st);
+  FM_CHECK_LAUNCH("fm_softmax_bwd");
   return FM_OK;
 }

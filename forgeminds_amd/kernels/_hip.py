@@ -56,6 +56,7 @@ SIGNATURES = {
     "fm_kl_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _i64, _i64, _int, _int, _f32, _f32, _vp]),
     "fm_topk": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _int, _vp]),
     "fm_softmax_fwd": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
+    "fm_softmax_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _vp]),
     "fm_route_workspace": (_sz, [_i64, _int, _int]),
     "fm_moe_gather": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "fm_moe_combine": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
@@ -447,6 +448,17 @@ def softmax_fwd(x2):
         _check(lib().fm_softmax_fwd(_ptr(x2), _ptr(y), n, v, dtype_code(x2.dtype), _stream(x2)),
                "fm_softmax_fwd")
     return y
+
+
+def softmax_bwd(y2, dy2):
+    """dx = (dy - sum(dy * y, -1)) * y for y2 = softmax(x2)."""
+    _dense(y2, dy2)
+    n, v = y2.shape
+    dx = torch.empty_like(y2)
+    with _guard(y2.device):
+        _check(lib().fm_softmax_bwd(_ptr(y2), _ptr(dy2), _ptr(dx), n, v, dtype_code(y2.dtype),
+                                    _stream(y2)), "fm_softmax_bwd")
+    return dx
 
 
 def route(logits2, k: int, want_permutation: bool = True, want_stats: bool = False):

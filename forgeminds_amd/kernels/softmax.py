@@ -1,7 +1,8 @@
 """``softmax`` over the last dimension on the HIP kernel.
 
 Call surface of the reference's ``forgemind/kernels/softmax.py:118-139``; the backward is
-the closed form ``(g - sum(g * y)) * y`` in tensor ops (reference ``softmax.py:107-115``).
+the closed form ``(g - sum(g * y)) * y`` (reference ``softmax.py:107-115``), in one kernel with
+fp32 math on the saved ``y`` (tensor ops when the incoming gradient has another dtype).
 """
 
 from __future__ import annotations
@@ -24,8 +25,11 @@ class _Softmax(torch.autograd.Function):
         (y,) = ctx.saved_tensors
         if g is None:
             return None
-        inner = (g * y).sum(dim=-1, keepdim=True)
-        return (g - inner) * y
+        if g.dtype != y.dtype or not g.is_cuda:
+            inner = (g * y).sum(dim=-1, keepdim=True)
+            return (g - inner) * y
+        v = y.shape[-1]
+        return _hip.softmax_bwd(y.contiguous().view(-1, v), g.contiguous().view(-1, v)).view(y.shape)
 
 
 def softmax(x: torch.Tensor, dim: int = -1, dtype: "torch.dtype | None" = None) -> torch.Tensor:

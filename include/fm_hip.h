@@ -231,6 +231,12 @@ int fm_topk(const void* x, void* values, void* indices, int64_t n, int64_t v, in
  * Replaces _softmax_kernel (forgemind/kernels/softmax.py:27-80): y = exp(x - max) / sum. */
 int fm_softmax_fwd(const void* x, void* y, int64_t n, int64_t v, int dtype, fm_stream_t stream);
 
+/* Replaces the tensor expression of _Softmax.backward (forgemind/kernels/softmax.py:108-115):
+ * dx = (dy - sum(dy * y)) * y per row, fp32 math on the stored y and dy, one rounding.
+ * y, dy, dx: [n, v] of dtype, three distinct buffers. */
+int fm_softmax_bwd(const void* y, const void* dy, void* dx, int64_t n, int64_t v, int dtype,
+                   fm_stream_t stream);
+
 /* ------------------------------------------------------------------ MoE router + dispatch permutation
  * Replaces the aten sequence of Router.forward and MoE.forward
  * (forgemind/moe.py:86-91, 52-60, 232-236): probs = softmax(logits) in fp32; top-k of probs

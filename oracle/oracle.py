@@ -187,6 +187,13 @@ def softmax(x, acc=torch.float32):
     return (e / e.sum(dim=-1, keepdim=True)).to(x.dtype)
 
 
+def softmax_bwd(y, dy, acc=torch.float32):
+    """Reference forgemind/kernels/softmax.py:108-115: (dy - sum(dy * y)) * y from the saved
+    output, here in ``acc`` on the stored values with one rounding to y.dtype."""
+    yf, gf = _up(y, acc), _up(dy, acc)
+    return ((gf - (gf * yf).sum(dim=-1, keepdim=True)) * yf).to(y.dtype)
+
+
 # ------------------------------------------------------------------ top-k (canonical order)
 def topk(x, k):
     """values (x.dtype), indices (int64). Canonical order of forgemind/kernels/topk.py:13-19,

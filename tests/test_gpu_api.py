@@ -270,6 +270,16 @@ def test_topk_softmax_surface_on_gpu():
     torch.softmax(xr, -1).backward(gr)
     assert torch.allclose(y, torch.softmax(xr, -1), rtol=1e-5, atol=1e-6)
     assert torch.allclose(xs.grad, xr.grad, rtol=1e-4, atol=1e-6)
+    # bf16 attention-shaped input; an fp32 gradient arriving on a bf16 output takes tensor ops
+    xb = torch.randn(2, 4, 128, 128, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    gb = torch.randn(2, 4, 128, 128, device=DEV, dtype=torch.bfloat16)
+    kernels.softmax(xb).backward(gb)
+    x32 = xb.detach().float().requires_grad_(True)
+    torch.softmax(x32, -1).backward(gb.float())
+    assert ((xb.grad.float() - x32.grad).abs().max() / x32.grad.abs().max()).item() < 1e-2
+    xb.grad = None
+    (kernels.softmax(xb).float() * gb.float()).sum().backward()
+    assert ((xb.grad.float() - x32.grad).abs().max() / x32.grad.abs().max()).item() < 1e-2
     fn = torch.compile(lambda t: kernels.topk(kernels.softmax(t), 8)[0].sum(), fullgraph=True, backend="eager")
     fn(xs)                                                   # traces to aten, no graph break
 

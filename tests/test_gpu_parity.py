@@ -610,6 +610,36 @@ def test_softmax(n, v, dt):
     assert torch.allclose(y.float().sum(-1).cpu(), torch.ones(n), atol=1e-2)
 
 
+@pytest.mark.parametrize("n,v,dt", [(4, 64, F32), (5, 1000, F32), (7, 1, F32), (8, 50257, BF16), (6, 300, F16),
+                                     (2, 128256, BF16), (1000, 64, F32), (77, 16, BF16), (33, 512, BF16),
+                                     (9, 8192, BF16), (5, 32768, F16), (3, 65536, BF16), (257, 2048, F32),
+                                     (4, 32000, BF16), (1000, 33, BF16), (65, 1023, BF16), (9, 513, F32),
+                                     (3, 40000, F32), (6, 16384, F32)])
+def test_softmax_bwd(n, v, dt):
+    g = gen(22)
+    y = torch.softmax(2 * torch.randn(n, v, generator=g), -1).to(dt)
+    dy = torch.randn(n, v, generator=g).to(dt)
+    dx = _hip.softmax_bwd(y.to(DEV), dy.to(DEV))
+    ref = O.softmax_bwd(y, dy)
+    # (dy - dot) * y: the subtraction cancels up to |dy| + |dot| before it is scaled by y
+    cancel = float((dy.float().abs().max() + 1) * y.float().max())
+    assert_close_lowp(dx, ref, dt, "softmax_bwd", ulps=2.0, cancel=cancel)
+    ref64 = O.softmax_bwd(y.double(), dy.double(), acc=torch.float64)
+    assert rel_max(dx, ref64) <= (1e-2 if dt != F32 else 1e-5)
+
+
+def test_softmax_bwd_unaligned_base_and_determinism():
+    g = gen(23)
+    for v in (9000, 700):
+        base = torch.softmax(torch.randn(3, v, generator=g), -1).bfloat16().reshape(-1)
+        pad = torch.zeros(1, dtype=BF16)
+        y = torch.cat((pad, base)).to(DEV)[1:].view(3, v)                 # base pointer off by 2 bytes
+        dy = torch.randn(3, v, generator=g).bfloat16().to(DEV)
+        dx = _hip.softmax_bwd(y, dy)
+        assert_close_lowp(dx, O.softmax_bwd(y.cpu(), dy.cpu()), BF16, "softmax_bwd", ulps=2.0, cancel=4.0)
+        assert torch.equal(dx, _hip.softmax_bwd(y, dy))
+
+
 def test_softmax_nan_and_neg_inf_rows():
     y = _hip.softmax_fwd(torch.tensor([[float("nan"), 1.0, 2.0]], device=DEV))
     assert math.isnan(y[0, 0].item())

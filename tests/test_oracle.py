@@ -278,6 +278,29 @@ def test_softmax_matches_torch():
     assert all(math.isnan(v) for v in y[0].tolist())
 
 
+def test_softmax_bwd_matches_autograd():
+    # pinned by torch's own derivative of softmax and by what the mathematics fixes: gradient
+    # rows sum to zero, a constant upstream gradient gives zero, a one-hot y gives zero
+    for shape in [(4, 64), (5, 1000), (2, 3, 97), (7, 1)]:
+        x = torch.randn(*shape, dtype=torch.float64, requires_grad=True)
+        g = torch.randn(*shape, dtype=torch.float64)
+        y = torch.softmax(x, -1)
+        y.backward(g)
+        got = O.softmax_bwd(y.detach(), g, acc=torch.float64)
+        assert torch.allclose(got, x.grad, rtol=1e-12, atol=1e-14)
+        assert got.sum(-1).abs().max() < 1e-12
+    y = torch.softmax(torch.randn(3, 50), -1)
+    assert O.softmax_bwd(y, torch.full((3, 50), 2.5)).abs().max() < 1e-6
+    onehot = torch.zeros(2, 9)
+    onehot[:, 4] = 1.0
+    assert O.softmax_bwd(onehot, torch.randn(2, 9)).abs().max() == 0
+    yb = torch.softmax(torch.randn(4, 300), -1).bfloat16()
+    gb = torch.randn(4, 300).bfloat16()
+    assert O.softmax_bwd(yb, gb).dtype == torch.bfloat16
+    ref = O.softmax_bwd(yb.double(), gb.double(), acc=torch.float64)
+    assert torch.allclose(O.softmax_bwd(yb, gb).double(), ref, rtol=2 ** -7, atol=1e-6)
+
+
 # ------------------------------------------------------------------ top-k
 def _canonical(v, idx):
     k = v.shape[-1]
