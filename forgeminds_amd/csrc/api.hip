@@ -19,6 +19,7 @@ const char* const kParamNames[fm_host::P_COUNT] = {
     "vocab_unroll",
     "norm_fwd_blocks_per_cu",
     "ce_rows_max_v",
+    "norm_wide_min_vec",
 };
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cus[kMaxDevices];

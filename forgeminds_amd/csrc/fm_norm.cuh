@@ -494,6 +494,202 @@ __global__ __launch_bounds__(256) void dw_generic(const T* __restrict__ x,
   }
 }
 
+// ---------------------------------------------------------------- wide rows (16-byte vectors, streamed)
+// Rows too wide for the register path (more than 4096 vectors) whose width is a whole number
+// of vectors and whose buffers are aligned: one 1024-thread workgroup per row, the row read
+// with 16-byte loads, reduced, and read again from cache for the output (LayerNorm: once more
+// in between, for the centred second moment). Thread t owns the same vectors in every pass, so
+// the sum x + delta it stored in the first pass is its own to re-read.
+constexpr int kWideThreads = 1024;
+
+template <typename T, typename WT, bool ADD, bool LN>
+__global__ __launch_bounds__(kWideThreads) void norm_fwd_wide(
+    const T* __restrict__ x, const T* __restrict__ delta, const WT* __restrict__ w,
+    const WT* __restrict__ bias, T* __restrict__ xn, T* __restrict__ y, float* __restrict__ mean,
+    float* __restrict__ rstd, int d, float eps) {
+  constexpr int EPV = Elem<T>::kVec;
+  __shared__ float smem[kWideThreads / 64];
+  const int tid = threadIdx.x;
+  const int nvec = d / EPV;
+  const int64_t base = (int64_t)blockIdx.x * d;
+  const T* src = ADD ? xn + base : x + base;   // what the later passes read
+  float ss = 0.f;
+  for (int c0 = tid; c0 < nvec; c0 += 2 * kWideThreads) {
+    const int c1 = c0 + kWideThreads;
+    u32x4 ra[2], rb[2];
+    ra[0] = load16_stream(x + base + (int64_t)c0 * EPV);
+    if (c1 < nvec) ra[1] = load16_stream(x + base + (int64_t)c1 * EPV);
+    if constexpr (ADD) {
+      rb[0] = load16_stream(delta + base + (int64_t)c0 * EPV);
+      if (c1 < nvec) rb[1] = load16_stream(delta + base + (int64_t)c1 * EPV);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = u == 0 ? c0 : c1;
+      if (c < nvec) {
+        float v[EPV];
+        Elem<T>::unpack(ra[u], v);
+        if constexpr (ADD) {
+          float dv[EPV];
+          Elem<T>::unpack(rb[u], dv);
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) v[e] += dv[e];
+          const u32x4 packed = Elem<T>::pack(v);
+          store16(xn + base + (int64_t)c * EPV, packed);
+          Elem<T>::unpack(packed, v);          // normalise the rounded sum, as the reference does
+        }
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) ss += LN ? v[e] : v[e] * v[e];
+      }
+    }
+  }
+  ss = row_reduce<kWideThreads, OpSum>(ss, smem, 0, tid);
+  float mu = 0.f;
+  if constexpr (LN) {
+    mu = ss / (float)d;
+    ss = 0.f;
+    for (int c = tid; c < nvec; c += kWideThreads) {
+      float v[EPV];
+      Elem<T>::unpack(load16(src + (int64_t)c * EPV), v);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) ss += (v[e] - mu) * (v[e] - mu);
+    }
+    ss = row_reduce<kWideThreads, OpSum>(ss, smem, 0, tid);
+  }
+  const float r = rsqrtf(ss / (float)d + eps);
+  if (tid == 0) {
+    rstd[blockIdx.x] = r;
+    if constexpr (LN) mean[blockIdx.x] = mu;
+  }
+  for (int c = tid; c < nvec; c += kWideThreads) {
+    float v[EPV], wv[EPV], o[EPV];
+    Elem<T>::unpack(load16(src + (int64_t)c * EPV), v);
+    load_w<T, WT>(w, c * EPV, wv);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) o[e] = ((v[e] - mu) * r) * wv[e];
+    if constexpr (LN) {
+      if (bias != nullptr) {
+        float bv[EPV];
+        load_w<T, WT>(bias, c * EPV, bv);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] += bv[e];
+      }
+    }
+    store16_stream(y + base + (int64_t)c * EPV, Elem<T>::pack(o));
+  }
+}
+
+template <typename T, typename WT, bool LN>
+__global__ __launch_bounds__(kWideThreads) void norm_bwd_wide(
+    const T* __restrict__ x, const WT* __restrict__ w, const float* __restrict__ mean,
+    const float* __restrict__ rstd, const T* __restrict__ dy, const T* __restrict__ gxn,
+    T* __restrict__ dx, T* __restrict__ dd, int d) {
+  constexpr int EPV = Elem<T>::kVec;
+  __shared__ float smem[kWideThreads / 64];
+  const int tid = threadIdx.x;
+  const int nvec = d / EPV;
+  const int64_t base = (int64_t)blockIdx.x * d;
+  const float r = rstd[blockIdx.x];
+  float mu = 0.f;
+  if constexpr (LN) mu = mean[blockIdx.x];
+  float dot = 0.f, gsum = 0.f;
+  for (int c0 = tid; c0 < nvec; c0 += 2 * kWideThreads) {
+    const int c1 = c0 + kWideThreads;
+    u32x4 rx[2], rg[2];
+    rx[0] = load16(x + base + (int64_t)c0 * EPV);
+    rg[0] = load16(dy + base + (int64_t)c0 * EPV);
+    if (c1 < nvec) {
+      rx[1] = load16(x + base + (int64_t)c1 * EPV);
+      rg[1] = load16(dy + base + (int64_t)c1 * EPV);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = u == 0 ? c0 : c1;
+      if (c < nvec) {
+        float xv[EPV], gv[EPV], wv[EPV];
+        Elem<T>::unpack(rx[u], xv);
+        Elem<T>::unpack(rg[u], gv);
+        load_w<T, WT>(w, c * EPV, wv);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+          const float g = gv[e] * wv[e];
+          dot += g * ((xv[e] - mu) * r);
+          gsum += g;
+        }
+      }
+    }
+  }
+  dot = row_reduce<kWideThreads, OpSum>(dot, smem, 0, tid);
+  const float cmean = dot / (float)d;
+  float gmean = 0.f;
+  if constexpr (LN) gmean = row_reduce<kWideThreads, OpSum>(gsum, smem, 0, tid) / (float)d;
+  for (int c = tid; c < nvec; c += kWideThreads) {
+    float xv[EPV], gv[EPV], wv[EPV], o[EPV];
+    Elem<T>::unpack(load16(x + base + (int64_t)c * EPV), xv);
+    Elem<T>::unpack(load16(dy + base + (int64_t)c * EPV), gv);
+    load_w<T, WT>(w, c * EPV, wv);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) o[e] = ((gv[e] * wv[e] - gmean) - ((xv[e] - mu) * r) * cmean) * r;
+    if (gxn != nullptr) {
+      float rv[EPV];
+      Elem<T>::unpack(load16_stream(gxn + base + (int64_t)c * EPV), rv);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) o[e] += rv[e];
+    }
+    const u32x4 packed = Elem<T>::pack(o);
+    store16_stream(dx + base + (int64_t)c * EPV, packed);
+    if (dd != nullptr) store16_stream(dd + base + (int64_t)c * EPV, packed);
+  }
+}
+
+// dW (and, for LN, db) partials of the wide path: grid (ceil(nvec / 64), chunks); a workgroup
+// owns 64 vector columns and the rows of its chunk, four row lanes of 64 threads each; the
+// four are folded in a fixed order. Partial rows as in dw_generic.
+template <typename T, bool LN>
+__global__ __launch_bounds__(256) void dw_wide(const T* __restrict__ x, const float* __restrict__ mean,
+                                                const float* __restrict__ rstd,
+                                                const T* __restrict__ dy, float* __restrict__ partial,
+                                                int64_t n, int d, int64_t rows_per_chunk) {
+  constexpr int EPV = Elem<T>::kVec;
+  __shared__ float s[4][64][EPV + 1];
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int nvec = d / EPV;
+  const int c = blockIdx.x * 64 + lane;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_chunk;
+  const int64_t r1 = (r0 + rows_per_chunk < n) ? r0 + rows_per_chunk : n;
+  const int64_t pcols = LN ? 2 * (int64_t)d : d;
+  float acc[EPV], accb[EPV];
+#pragma unroll
+  for (int e = 0; e < EPV; ++e) { acc[e] = 0.f; accb[e] = 0.f; }
+  if (c < nvec) {
+    for (int64_t r = r0 + g; r < r1; r += 4) {
+      float xv[EPV], gv[EPV];
+      Elem<T>::unpack(load16(x + r * d + (int64_t)c * EPV), xv);
+      Elem<T>::unpack(load16(dy + r * d + (int64_t)c * EPV), gv);
+      const float rs = rstd[r];
+      float mu = 0.f;
+      if constexpr (LN) mu = mean[r];
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        acc[e] += gv[e] * ((xv[e] - mu) * rs);
+        if constexpr (LN) accb[e] += gv[e];
+      }
+    }
+  }
+#pragma unroll
+  for (int which = 0; which < (LN ? 2 : 1); ++which) {
+    if (which == 1) __syncthreads();
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) s[g][lane][e] = which == 0 ? acc[e] : accb[e];
+    __syncthreads();
+    if (g == 0 && c < nvec) {
+      float* out = partial + (int64_t)blockIdx.y * pcols + (int64_t)which * d + (int64_t)c * EPV;
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) out[e] = (s[0][lane][e] + s[1][lane][e]) + (s[2][lane][e] + s[3][lane][e]);
+    }
+  }
+}
+
 __global__ void zero_u16_kernel(uint16_t* p, int64_t n) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0;
@@ -502,6 +698,8 @@ __global__ void zero_u16_kernel(uint16_t* p, int64_t n) {
 // ---------------------------------------------------------------- host: plan + dispatch
 struct Plan {
   bool vec;        // register-resident vector path
+  bool wide;       // streamed vector path (rows past the register path)
+  bool bwd_vec, bwd_wide;  // the same two for the backward, whose register path ends earlier
   int tpr, iters;  // threads per row, 16-byte vectors per thread
   int rpb;         // rows per workgroup
   int64_t tiles;   // row tiles of the forward (vector path)
@@ -516,7 +714,16 @@ Plan make_plan(int64_t n, int64_t d, int x_dtype, bool aligned) {
   Plan p{};
   const int epv = 16 / elem_size(x_dtype);
   const int64_t nvec = d / epv;
-  p.vec = aligned && (d % epv == 0) && nvec <= 4096;
+  // rows of more than `reg_max` vectors are streamed (tunable downwards with "norm_wide_min_vec")
+  int64_t reg_max = fm_host::get_param(fm_host::P_NORM_WIDE_MIN_VEC);
+  if (reg_max <= 0 || reg_max > 4096) reg_max = 4096;
+  p.vec = aligned && (d % epv == 0) && nvec <= reg_max;
+  p.wide = aligned && (d % epv == 0) && nvec > reg_max;
+  // the backward of half types keeps x, dy and two fp32 column sets per thread: past 2048
+  // vectors that no longer fits 128 registers, and streaming the row is faster than spilling
+  const int64_t bwd_max = (elem_size(x_dtype) == 2 && reg_max > 2048) ? 2048 : reg_max;
+  p.bwd_vec = p.vec && nvec <= bwd_max;
+  p.bwd_wide = aligned && (d % epv == 0) && nvec > bwd_max;
   if (p.vec) {
     if (nvec <= 64) {
       int t = 4;
@@ -537,6 +744,8 @@ Plan make_plan(int64_t n, int64_t d, int x_dtype, bool aligned) {
     const int block = p.tpr > kMinBlock ? p.tpr : kMinBlock;
     p.rpb = block / p.tpr;
     p.tiles = (n + p.rpb - 1) / p.rpb;
+  }
+  if (p.bwd_vec) {
     p.bwd_tiles = (n + (kBwdBlock / p.tpr) - 1) / (kBwdBlock / p.tpr);
     int per_cu = fm_host::get_param(fm_host::P_NORM_BWD_BLOCKS_PER_CU);
     if (per_cu <= 0) per_cu = 1;
@@ -578,6 +787,11 @@ int launch_fwd(const Plan& p, const void* x, const void* delta, const void* w, c
   const WT* bp = static_cast<const WT*>(bias);
   T* xnp = static_cast<T*>(xn);
   T* yp = static_cast<T*>(y);
+  if (p.wide) {
+    hipLaunchKernelGGL((norm_fwd_wide<T, WT, ADD, LN>), dim3((unsigned)n), dim3(kWideThreads), 0, st, xp,
+                       dp, wp, bp, xnp, yp, mean, rstd, (int)d, eps);
+    return FM_OK;
+  }
   if (!p.vec) {
     hipLaunchKernelGGL((norm_fwd_generic<T, WT, ADD, LN>), dim3((unsigned)n), dim3(256), 0, st, xp, dp,
                        wp, bp, xnp, yp, mean, rstd, d, eps);
@@ -617,7 +831,16 @@ int launch_bwd(const Plan& p, const void* x, const void* w, const float* mean, c
   T* ddp = static_cast<T*>(dd);
   if (dw == nullptr && db == nullptr) partial = nullptr;
   const int pcols = (int)(LN ? 2 * d : d);
-  if (!p.vec) {
+  if (p.bwd_wide) {
+    hipLaunchKernelGGL((norm_bwd_wide<T, WT, LN>), dim3((unsigned)n), dim3(kWideThreads), 0, st, xp, wp,
+                       mean, rstd, dyp, gp, dxp, ddp, (int)d);
+    if (partial != nullptr) {
+      const int nvec = (int)(d / Elem<T>::kVec);
+      dim3 grid((unsigned)((nvec + 63) / 64), (unsigned)p.bwd_blocks);
+      hipLaunchKernelGGL((dw_wide<T, LN>), grid, dim3(256), 0, st, xp, mean, rstd, dyp, partial, n, (int)d,
+                         p.rows_per_chunk);
+    }
+  } else if (!p.bwd_vec) {
     hipLaunchKernelGGL((norm_bwd_generic<T, WT, LN>), dim3((unsigned)n), dim3(256), 0, st, xp, wp, mean,
                        rstd, dyp, gp, dxp, ddp, d);
     if (partial != nullptr) {

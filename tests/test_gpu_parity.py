@@ -66,6 +66,9 @@ NORM_CASES = [
     (16, 64, BF16, BF16, 1e-6), (3, 1, F32, F32, 1e-6), (6, 8, F32, F32, 1e-6), (1, 3, F32, F32, 1e-6),
     (9, 16384, BF16, F32, 1e-6), (4, 40000, F16, F32, 1e-6), (130, 3072, F32, F32, 1e-6),
     (7, 12288, BF16, BF16, 1e-5), (2, 24576, BF16, F32, 1e-5),
+    # rows past the register path: streamed 16-byte vectors (and, one row wider, scalars)
+    (5, 40960, BF16, F32, 1e-6), (3, 65536, F16, F16, 1e-5), (6, 20480, F32, F32, 1e-6),
+    (300, 32768, BF16, BF16, 1e-6), (2, 131080, BF16, F32, 1e-6), (3, 40961, BF16, F32, 1e-6),
 ]
 
 
@@ -121,7 +124,8 @@ def test_rmsnorm_unaligned_views_take_the_any_width_path():
 
 ADD_CASES = [(256, 8192, BF16, F32, 1e-5), (9, 24, F32, F32, 1e-6), (10, 33, BF16, BF16, 1e-6),
              (6, 8, F32, F32, 1e-6), (5, 7, F32, F32, 1e-6), (40, 4096, F16, F16, 1e-5),
-             (12, 2048, BF16, F32, 1e-5)]
+             (12, 2048, BF16, F32, 1e-5), (7, 40960, BF16, F32, 1e-5), (5, 20480, F32, F32, 1e-6),
+             (260, 24576, F16, F16, 1e-5)]
 
 
 @pytest.mark.parametrize("n,d,dt,wdt,eps", ADD_CASES)
@@ -155,6 +159,8 @@ LN_CASES = [
     (16, 64, BF16, BF16, 1e-5, True), (3, 1, F32, F32, 1e-5, True), (6, 8, F32, F32, 1e-5, True),
     (9, 16384, BF16, F32, 1e-5, True), (4, 40000, F16, F32, 1e-5, True), (130, 3072, F32, F32, 1e-5, True),
     (7, 12288, BF16, BF16, 1e-5, True), (2, 24576, BF16, F32, 1e-5, False), (40, 4096, BF16, F32, 1e-5, True),
+    (5, 40960, BF16, F32, 1e-5, True), (3, 65536, F16, F16, 1e-5, False), (6, 20480, F32, F32, 1e-5, True),
+    (270, 32768, BF16, BF16, 1e-5, True),
 ]
 
 
@@ -193,7 +199,8 @@ def test_layernorm_fwd_bwd(n, d, dt, wdt, eps, bias):
 
 
 @pytest.mark.parametrize("n,d,dt,wdt", [(128, 8192, BF16, F32), (9, 24, F32, F32), (10, 33, BF16, BF16),
-                                        (40, 4096, F16, F16), (12, 2048, BF16, F32)])
+                                        (40, 4096, F16, F16), (12, 2048, BF16, F32), (6, 40960, BF16, F32),
+                                        (4, 24576, F32, F32)])
 def test_add_layernorm_fwd_bwd(n, d, dt, wdt):
     g = gen(1034)
     x = torch.randn(n, d, generator=g).to(dt)
