@@ -466,6 +466,110 @@ void launch_bwd(const void* s, const void* t, const float* lse_s, const float* l
 #undef LAUNCH
 }
 
+// Narrow rows (at most 1024 classes: classifier distillation, not vocabularies): TPR lanes per
+// row, several rows per 256-thread workgroup, both rows in registers (ITERS scalar loads each
+// per lane), any alignment. LOSS writes the log-sum-exps and the row's KL; GRAD writes the
+// gradient, from the sums just computed (LOSS) or from saved log-sum-exps. dstudent may be
+// the student buffer when the dtypes agree: each element is read by the lane that writes it.
+template <typename T, typename GT, int TPR, int ITERS, bool LOSS, bool GRAD>
+__global__ __launch_bounds__(256) void kl_rows_kernel(const T* student, const T* __restrict__ teacher,
+                                                      float* lse_s, float* lse_t,
+                                                      float* __restrict__ row_kl,
+                                                      const float* __restrict__ grad_out,
+                                                      int grad_per_row, GT* dstudent, int64_t n, int v,
+                                                      float inv_temp, float mul) {
+  constexpr int RPB = 256 / TPR;
+  const int tid = threadIdx.x;
+  const int rib = tid / TPR;
+  const int t = tid % TPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + rib;
+  const bool valid = row < n;
+  const int64_t base = row * (int64_t)v;
+  const float c1 = kLog2e * inv_temp;
+  float zs[ITERS], zt[ITERS];
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * TPR + t;
+    const bool in = valid && c < v;
+    zs[i] = in ? Elem<T>::load1(student + base + c) * c1 : -INFINITY;
+    zt[i] = in ? Elem<T>::load1(teacher + base + c) * c1 : -INFINITY;
+  }
+  float l2s, l2t;
+  if constexpr (LOSS) {
+    float ms = kNegBig, mt = kNegBig;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) { ms = fmaxf(ms, zs[i]); mt = fmaxf(mt, zt[i]); }
+    ms = group_reduce<TPR, OpMax>(ms);
+    mt = group_reduce<TPR, OpMax>(mt);
+    float ds = 0.f, dt = 0.f, a = 0.f;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = i * TPR + t;
+      if (valid && c < v) {            // keeps (-inf) - (-inf) of the padding out of the A term
+        ds += fast_exp2(zs[i] - ms);
+        const float et = fast_exp2(zt[i] - mt);
+        dt += et;
+        a += et * (zt[i] - zs[i]);
+      }
+    }
+    ds = group_reduce<TPR, OpSum>(ds);
+    dt = group_reduce<TPR, OpSum>(dt);
+    a = group_reduce<TPR, OpSum>(a);
+    l2s = ms + fast_log2(ds);
+    l2t = mt + fast_log2(dt);
+    if (valid && t == 0) {
+      if (lse_s != nullptr) lse_s[row] = l2s * kLn2;
+      if (lse_t != nullptr) lse_t[row] = l2t * kLn2;
+      row_kl[row] = (a / dt - l2t + l2s) * kLn2;
+    }
+  } else {
+    l2s = valid ? lse_s[row] * kLog2e : 0.f;
+    l2t = valid ? lse_t[row] * kLog2e : 0.f;
+  }
+  if constexpr (GRAD) {
+    float g = mul;
+    if (grad_out != nullptr && valid) g *= grad_per_row ? grad_out[row] : grad_out[0];
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = i * TPR + t;
+      if (valid && c < v)
+        Elem<GT>::store1(dstudent + base + c, (fast_exp2(zs[i] - l2s) - fast_exp2(zt[i] - l2t)) * g);
+    }
+  }
+}
+
+constexpr int kRowsMaxV = 1024;
+
+template <typename T, typename GT, bool LOSS, bool GRAD>
+bool launch_rows(const void* student, const void* teacher, float* lse_s, float* lse_t, float* row_kl,
+                 const float* grad_out, int grad_per_row, void* dstudent, int64_t n, int v, float inv_temp,
+                 float mul, hipStream_t st) {
+  if (v > kRowsMaxV) return false;
+  const int tpr = v <= 16 * 16 ? 16 : 64;
+  int iters = 1;
+  while (tpr * iters < v) iters *= 2;
+  const dim3 grid((unsigned)((n + 256 / tpr - 1) / (256 / tpr)));
+#define GOR(TPR_, IT_)                                                                             \
+  if (tpr == TPR_ && iters == IT_) {                                                               \
+    hipLaunchKernelGGL((kl_rows_kernel<T, GT, TPR_, IT_, LOSS, GRAD>), grid, dim3(256), 0, st,     \
+                       static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t, \
+                       row_kl, grad_out, grad_per_row, static_cast<GT*>(dstudent), n, v, inv_temp, mul); \
+    return true;                                                                                   \
+  }
+  GOR(16, 1) GOR(16, 2) GOR(16, 4) GOR(16, 8) GOR(16, 16) GOR(64, 8) GOR(64, 16)
+#undef GOR
+  return false;
+}
+
+#define FM_KL_BY_DTYPES(dtype, grad_dtype, CALL)                        \
+  do {                                                                  \
+    if ((dtype) == FM_F32) { CALL(float, float); }                      \
+    else if ((dtype) == FM_BF16 && (grad_dtype) == FM_BF16) { CALL(bf16_t, bf16_t); } \
+    else if ((dtype) == FM_BF16) { CALL(bf16_t, float); }               \
+    else if ((grad_dtype) == FM_F16) { CALL(f16_t, f16_t); }            \
+    else { CALL(f16_t, float); }                                        \
+  } while (0)
+
 int check_shape(const char* what, int64_t n, int64_t v, int dtype) {
   FM_CHECK_ARG(n >= 0 && v > 0, "%s: bad shape n=%lld v=%lld", what, (long long)n, (long long)v);
   FM_CHECK_ARG(dtype == FM_F32 || dtype == FM_F16 || dtype == FM_BF16, "%s: bad dtype %d", what,
@@ -490,7 +594,16 @@ int fm_kl_fwd(const void* student, const void* teacher, float* lse_s, float* lse
                "fm_kl_fwd: bad reduction %d", reduction);
   FM_CHECK_ARG(n == 0 || (student && teacher && lse_s && lse_t && row_kl), "fm_kl_fwd: NULL pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (n > 0) {
+  bool narrow = false;
+  if (n > 0 && v <= kRowsMaxV) {
+#define CALL(T, GT) \
+  narrow = launch_rows<T, GT, true, false>(student, teacher, lse_s, lse_t, row_kl, nullptr, 0, nullptr, n, \
+                                           (int)v, inv_temperature, 0.f, st)
+    FM_KL_BY_DTYPES(dtype, dtype, CALL);
+#undef CALL
+    if (narrow) FM_CHECK_LAUNCH("fm_kl_fwd");
+  }
+  if (n > 0 && !narrow) {
     const bool vec_ok = fm_host::aligned16(student) && fm_host::aligned16(teacher);
     if (dtype == FM_F32) launch_fwd<float>(student, teacher, lse_s, lse_t, row_kl, n, (int)v, inv_temperature, vec_ok, st);
     else if (dtype == FM_BF16) launch_fwd<bf16_t>(student, teacher, lse_s, lse_t, row_kl, n, (int)v, inv_temperature, vec_ok, st);
@@ -572,6 +685,19 @@ int fm_kl_bwd(const void* student, const void* teacher, const float* lse_s, cons
   if (n == 0) return FM_OK;
   FM_CHECK_ARG(student && teacher && lse_s && lse_t && dstudent, "fm_kl_bwd: NULL pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (v <= kRowsMaxV) {
+    bool narrow = false;
+#define CALL(T, GT)                                                                                 \
+  narrow = launch_rows<T, GT, false, true>(student, teacher, const_cast<float*>(lse_s),             \
+                                           const_cast<float*>(lse_t), nullptr, grad_out, grad_per_row, \
+                                           dstudent, n, (int)v, inv_temperature, inv_temperature * scale, st)
+    FM_KL_BY_DTYPES(dtype, grad_dtype, CALL);
+#undef CALL
+    if (narrow) {
+      FM_CHECK_LAUNCH("fm_kl_bwd");
+      return FM_OK;
+    }
+  }
   const bool vec_ok = fm_host::aligned16(student) && fm_host::aligned16(teacher) &&
                       fm_host::aligned16(dstudent);
 #define CALL(T, GT) \
@@ -604,6 +730,22 @@ int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, floa
   const float scale = (reduction == FM_REDUCE_MEAN && n > 0) ? 1.f / (float)n : 1.f;
   const int esize = dtype == FM_F32 ? 4 : 2;
   const int64_t nvec = v / (16 / esize);
+  if (n > 0 && v <= kRowsMaxV) {   // narrow rows: lane groups, any alignment, in place allowed
+    bool narrow = false;
+#define CALL(T, GT)                                                                                  \
+  narrow = launch_rows<T, GT, true, true>(student, teacher, lse_s, lse_t, row_kl, nullptr, 0, dstudent, n, \
+                                          (int)v, inv_temperature, inv_temperature * scale, st)
+    FM_KL_BY_DTYPES(dtype, grad_dtype, CALL);
+#undef CALL
+    if (narrow) {
+      FM_CHECK_LAUNCH("fm_kl_loss_grad");
+      if (loss != nullptr) {
+        hipLaunchKernelGGL(kl_finalize_kernel, dim3(1), dim3(1024), 0, st, row_kl, n, scale, loss);
+        FM_CHECK_LAUNCH("fm_kl_loss_grad(finalize)");
+      }
+      return FM_OK;
+    }
+  }
   const bool one_pass = n > 0 && fm_host::aligned16(student) && fm_host::aligned16(teacher) &&
                         fm_host::aligned16(dstudent) && nvec <= kOnePassMaxVec;
   if (!one_pass) {
