@@ -317,17 +317,31 @@ __global__ __launch_bounds__(256) void softmax_bwd_rows_scalar_kernel(const T* _
 }
 
 #define FM_SOFTMAX_SHAPES(X) \
-  X(4, 1) X(8, 1) X(16, 1) X(32, 1) X(64, 1) X(64, 2) X(128, 2) X(256, 2) X(256, 4) X(512, 4) X(512, 8) X(1024, 8)
+  X(1, 1) X(2, 1) X(4, 1) X(8, 1) X(16, 1) X(32, 1) X(64, 1) X(64, 2) X(128, 2) X(256, 2) X(256, 4) X(512, 4) X(512, 8) X(1024, 8)
 
 // threads per row and vectors per thread for a row of nvec 16-byte vectors; false: too wide
 bool rows_plan(int64_t nvec, int* tpr, int* iters) {
-  static const int kPlans[][3] = {{4, 4, 1},     {8, 8, 1},      {16, 16, 1},    {32, 32, 1},
+  static const int kPlans[][3] = {{1, 1, 1},     {2, 2, 1},      {4, 4, 1},     {8, 8, 1},      {16, 16, 1},    {32, 32, 1},
                                   {64, 64, 1},   {128, 64, 2},   {256, 128, 2},  {512, 256, 2},
                                   {1024, 256, 4}, {2048, 512, 4}, {4096, 512, 8}, {8192, 1024, 8}};
   for (auto& pl : kPlans) {
     if (nvec <= pl[0]) { *tpr = pl[1]; *iters = pl[2]; return true; }
   }
   return false;
+}
+
+// lanes per row and elements per lane of the scalar lane-group kernels (v <= 1024): about
+// four elements a lane for the narrowest rows, so that rows of a few elements do not idle
+// most of a 16-lane group
+void scalar_plan(int v, int* tpr, int* iters) {
+  int t = 1;
+  while (t < 16 && 4 * t < v) t *= 2;
+  if (v > 16 * 16) t = 64;
+  int it = 1;
+  while (t * it < v) it *= 2;
+  if (t >= 16 && it < 4) it = 4;      // the instantiated shapes
+  *tpr = t;
+  *iters = it;
 }
 
 template <typename T>
@@ -348,16 +362,16 @@ void launch(const void* x, void* y, int64_t n, int v, bool vec_ok, hipStream_t s
 #undef X
   }
   if (v <= 64 * 16) {   // narrow, not vectorisable: lane groups with one element per load
-    const int tpr = v <= 16 * 16 ? 16 : 64;
-    int iters = 1;
-    while (tpr * iters < v) iters *= 2;
+    int tpr, iters;
+    scalar_plan(v, &tpr, &iters);
     const dim3 sgrid((unsigned)((n + 256 / tpr - 1) / (256 / tpr)));
 #define GOS(TPR_, IT_)                                                                             \
   if (tpr == TPR_ && iters == IT_) {                                                               \
     hipLaunchKernelGGL((softmax_rows_scalar_kernel<T, TPR_, IT_>), sgrid, dim3(256), 0, st, xp, yp, n, v); \
     return;                                                                                        \
   }
-    GOS(16, 1) GOS(16, 2) GOS(16, 4) GOS(16, 8) GOS(16, 16) GOS(64, 8) GOS(64, 16)
+    GOS(1, 1) GOS(1, 2) GOS(1, 4) GOS(2, 4) GOS(4, 4) GOS(8, 4)
+    GOS(16, 4) GOS(16, 8) GOS(16, 16) GOS(64, 8) GOS(64, 16)
 #undef GOS
   }
   const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 4);
@@ -390,16 +404,16 @@ void launch_bwd(const void* y, const void* dy, void* dx, int64_t n, int v, bool 
 #undef X
   }
   if (v <= 64 * 16) {
-    const int tpr = v <= 16 * 16 ? 16 : 64;
-    int iters = 1;
-    while (tpr * iters < v) iters *= 2;
+    int tpr, iters;
+    scalar_plan(v, &tpr, &iters);
     const dim3 sgrid((unsigned)((n + 256 / tpr - 1) / (256 / tpr)));
 #define GOS(TPR_, IT_)                                                                             \
   if (tpr == TPR_ && iters == IT_) {                                                               \
     hipLaunchKernelGGL((softmax_bwd_rows_scalar_kernel<T, TPR_, IT_>), sgrid, dim3(256), 0, st, yp, gp, op, n, v); \
     return;                                                                                        \
   }
-    GOS(16, 1) GOS(16, 2) GOS(16, 4) GOS(16, 8) GOS(16, 16) GOS(64, 8) GOS(64, 16)
+    GOS(1, 1) GOS(1, 2) GOS(1, 4) GOS(2, 4) GOS(4, 4) GOS(8, 4)
+    GOS(16, 4) GOS(16, 8) GOS(16, 16) GOS(64, 8) GOS(64, 16)
 #undef GOS
   }
   const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 4);
