@@ -73,6 +73,7 @@ __device__ __forceinline__ int block_excl_scan(int v, int* smem, int nw, int* to
 }
 
 constexpr int kWorkCap = 2048;  // vectors that may be revisited in phase B
+constexpr int kSortFrom = 128;  // candidate counts above this are sorted instead of counted
 
 // Where the vector maxima of the streaming pass live.
 enum VecMax { kVecMaxNone = 0, kVecMaxRegs = 1, kVecMaxLds = 2 };
@@ -153,106 +154,143 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
     const int active = (sp.nvec > ne ? sp.nvec : ne) < THREADS ? (sp.nvec > ne ? sp.nvec : ne) : THREADS;
     const int nfull = active >> 6;
     const int j = nfull > 0 ? (k + nfull - 1) / nfull : 65;
-    // Only the bits a value of type T can set are searched (the masked key is a lower bound
-    // of the key with nothing representable in between), two bits per step: three ballots
-    // that do not depend on each other instead of two dependent rounds.
-    uint32_t tw = 0u;
-    if (j <= 64 && wave < nfull) {
-      const uint32_t mk = mykey & KMASK;
-      int bit = 31;
-      for (; bit - 1 >= KeyBits<T>::low; bit -= 2) {
-        const int shift = bit - 1;
-        const int c1 = __builtin_popcountll(__ballot(mk >= (tw | (1u << shift))));
-        const int c2 = __builtin_popcountll(__ballot(mk >= (tw | (2u << shift))));
-        const int c3 = __builtin_popcountll(__ballot(mk >= (tw | (3u << shift))));
-        const uint32_t dgt = c3 >= j ? 3u : (c2 >= j ? 2u : (c1 >= j ? 1u : 0u));
-        tw |= dgt << shift;
-      }
-      if (bit >= KeyBits<T>::low) {   // an odd number of key bits leaves one
-        const uint32_t trial = tw | (1u << bit);
-        if (__builtin_popcountll(__ballot(mk >= trial)) >= j) tw = trial;
-      }
-    }
-    if (lane == 0) s_tau[wave] = (wave < nfull || j > 64) ? tw : 0xFFFFFFFFu;
-    if (tid == 0) { s_count = 0; s_nwork = 0; }
-    __syncthreads();
-    uint32_t tau = s_tau[0];
-#pragma unroll
-    for (int i = 1; i < NW; ++i) tau = tau < s_tau[i] ? tau : s_tau[i];
-    // float image of tau; keys at or below key(-inf) admit everything, the NaN key only NaNs
-    const float tau_f = tau <= 0x007FFFFFu ? -INFINITY
-                                           : (tau == 0xFFFFFFFFu ? __builtin_nanf("") : float_of_key(tau));
-    const bool only_nan = tau == 0xFFFFFFFFu;
-    auto take_of = [&](float f) { return only_nan ? (f != f) : !(f < tau_f); };
-
-    // ---- phase B: candidates
-    auto consider = [&](float f, int col) {
-      if (take_of(f)) {
-        const int slot = atomicAdd(&s_count, 1);
-        if (slot < kCap) ccomp[slot] = ((unsigned long long)key_of(f) << 32) | (uint32_t)(~col);
-      }
-    };
-    auto scan_vec = [&](const u32x4& raw, int c) {
-      float f[EPV];
-      Elem<T>::unpack(raw, f);
-      bool any = false;
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) any |= take_of(f[e]);
-      if (any) {
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) consider(f[e], sp.head + c * EPV + e);
-      }
-    };
-    if constexpr (VMAX != kVecMaxNone) {
-      // B1: vectors that can hold a candidate go to the work list
-      auto list = [&](int c) {
-        const int slot = atomicAdd(&s_nwork, 1);
-        if (slot < kWorkCap) work[slot] = c;
-      };
-      if constexpr (VMAX == kVecMaxRegs) {
-#pragma unroll
-        for (int i = 0; i < ITERS; ++i) {
-          const int c = i * THREADS + tid;
-          if (c < sp.nvec && take_of(vmax[i])) list(c);
+    if (j > 64) {
+      // no full wave can bound the k-th value from below (k beyond 63 per full wave): every
+      // element would become a candidate, so the exact path is taken at once
+      C = kCap + 1;
+    } else {
+      // Only the bits a value of type T can set are searched (the masked key is a lower bound
+      // of the key with nothing representable in between), two bits per step: three ballots
+      // that do not depend on each other instead of two dependent rounds.
+      uint32_t tw = 0u;
+      if (j <= 64 && wave < nfull) {
+        const uint32_t mk = mykey & KMASK;
+        int bit = 31;
+        for (; bit - 1 >= KeyBits<T>::low; bit -= 2) {
+          const int shift = bit - 1;
+          const int c1 = __builtin_popcountll(__ballot(mk >= (tw | (1u << shift))));
+          const int c2 = __builtin_popcountll(__ballot(mk >= (tw | (2u << shift))));
+          const int c3 = __builtin_popcountll(__ballot(mk >= (tw | (3u << shift))));
+          const uint32_t dgt = c3 >= j ? 3u : (c2 >= j ? 2u : (c1 >= j ? 1u : 0u));
+          tw |= dgt << shift;
         }
-      } else {
-        const uint32_t tau_hi = tau >> 16;
-        const uint64_t* quad = reinterpret_cast<const uint64_t*>(vhi);
-        for (int q = tid; q * 4 < sp.nvec; q += THREADS) {
-          const uint64_t four = quad[q];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int c = q * 4 + e;
-            if (c < sp.nvec && (uint32_t)((four >> (16 * e)) & 0xFFFFu) >= tau_hi) list(c);
+        if (bit >= KeyBits<T>::low) {   // an odd number of key bits leaves one
+          const uint32_t trial = tw | (1u << bit);
+          if (__builtin_popcountll(__ballot(mk >= trial)) >= j) tw = trial;
+        }
+      }
+      if (lane == 0) s_tau[wave] = (wave < nfull || j > 64) ? tw : 0xFFFFFFFFu;
+      if (tid == 0) { s_count = 0; s_nwork = 0; }
+      __syncthreads();
+      uint32_t tau = s_tau[0];
+  #pragma unroll
+      for (int i = 1; i < NW; ++i) tau = tau < s_tau[i] ? tau : s_tau[i];
+      // float image of tau; keys at or below key(-inf) admit everything, the NaN key only NaNs
+      const float tau_f = tau <= 0x007FFFFFu ? -INFINITY
+                                             : (tau == 0xFFFFFFFFu ? __builtin_nanf("") : float_of_key(tau));
+      const bool only_nan = tau == 0xFFFFFFFFu;
+      auto take_of = [&](float f) { return only_nan ? (f != f) : !(f < tau_f); };
+
+      // ---- phase B: candidates
+      auto consider = [&](float f, int col) {
+        if (take_of(f)) {
+          const int slot = atomicAdd(&s_count, 1);
+          if (slot < kCap) ccomp[slot] = ((unsigned long long)key_of(f) << 32) | (uint32_t)(~col);
+        }
+      };
+      auto scan_vec = [&](const u32x4& raw, int c) {
+        float f[EPV];
+        Elem<T>::unpack(raw, f);
+        bool any = false;
+  #pragma unroll
+        for (int e = 0; e < EPV; ++e) any |= take_of(f[e]);
+        if (any) {
+  #pragma unroll
+          for (int e = 0; e < EPV; ++e) consider(f[e], sp.head + c * EPV + e);
+        }
+      };
+      if constexpr (VMAX != kVecMaxNone) {
+        // B1: vectors that can hold a candidate go to the work list
+        auto list = [&](int c) {
+          const int slot = atomicAdd(&s_nwork, 1);
+          if (slot < kWorkCap) work[slot] = c;
+        };
+        if constexpr (VMAX == kVecMaxRegs) {
+  #pragma unroll
+          for (int i = 0; i < ITERS; ++i) {
+            const int c = i * THREADS + tid;
+            if (c < sp.nvec && take_of(vmax[i])) list(c);
+          }
+        } else {
+          const uint32_t tau_hi = tau >> 16;
+          const uint64_t* quad = reinterpret_cast<const uint64_t*>(vhi);
+          for (int q = tid; q * 4 < sp.nvec; q += THREADS) {
+            const uint64_t four = quad[q];
+  #pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int c = q * 4 + e;
+              if (c < sp.nvec && (uint32_t)((four >> (16 * e)) & 0xFFFFu) >= tau_hi) list(c);
+            }
           }
         }
+        __syncthreads();
+        const int nwork = s_nwork;
+        overflow = nwork > kWorkCap;
+        // B2: revisit only those vectors, spread over the whole workgroup
+        if (!overflow) {
+          for (int w = tid; w < nwork; w += THREADS) {
+            const int c = work[w];
+            scan_vec(load16(rp + sp.head + (int64_t)c * EPV), c);
+          }
+        }
+      } else {
+        for (int c = tid; c < sp.nvec; c += THREADS) scan_vec(load16(rp + sp.head + (int64_t)c * EPV), c);
+      }
+      for (int e = tid; e < ne; e += THREADS) {
+        const int col = edge_col(sp, e);
+        consider(Elem<T>::load1(rp + col), col);
       }
       __syncthreads();
-      const int nwork = s_nwork;
-      overflow = nwork > kWorkCap;
-      // B2: revisit only those vectors, spread over the whole workgroup
-      if (!overflow) {
-        for (int w = tid; w < nwork; w += THREADS) {
-          const int c = work[w];
-          scan_vec(load16(rp + sp.head + (int64_t)c * EPV), c);
-        }
-      }
-    } else {
-      for (int c = tid; c < sp.nvec; c += THREADS) scan_vec(load16(rp + sp.head + (int64_t)c * EPV), c);
-    }
-    for (int e = tid; e < ne; e += THREADS) {
-      const int col = edge_col(sp, e);
-      consider(Elem<T>::load1(rp + col), col);
-    }
-    __syncthreads();
-    C = s_count;
-    __syncthreads();
-    if (overflow) C = kCap + 1;
+      C = s_count;
+      __syncthreads();
+      if (overflow) C = kCap + 1;
 
+    }
     if (C > kCap) {
-      // ---- exact path: k-th key by bitwise search over the whole row
+      // ---- exact path: k-th key by bitwise search over the whole row. Rows of up to RK vectors
+      // per thread keep their (masked) keys in registers for the search; wider rows are
+      // re-read once per key bit. Empty slots hold 0, which no predicate below accepts.
+      constexpr int RK = 4;
+      const bool cached = sp.nvec <= THREADS * RK && ne <= THREADS;
+      uint32_t ck[RK][EPV];
+      uint32_t ek = 0u;
+      if (cached) {
+#pragma unroll
+        for (int i = 0; i < RK; ++i) {
+          const int c = i * THREADS + tid;
+          if (c < sp.nvec) {
+            float f[EPV];
+            Elem<T>::unpack(load16(rp + sp.head + (int64_t)c * EPV), f);
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) ck[i][e] = key_of(f[e]) & KMASK;
+          } else {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) ck[i][e] = 0u;
+          }
+        }
+        if (tid < ne) ek = key_of(Elem<T>::load1(rp + edge_col(sp, tid))) & KMASK;
+      }
       auto count_if = [&](auto pred) {
         int cnt = 0;
+        if (cached) {
+#pragma unroll
+          for (int i = 0; i < RK; ++i) {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) cnt += pred(ck[i][e]) ? 1 : 0;
+          }
+          cnt += pred(ek) ? 1 : 0;
+          return block_sum_int(cnt, s_int, NW);
+        }
         for (int c = tid; c < sp.nvec; c += THREADS) {
           float f[EPV];
           Elem<T>::unpack(load16(rp + sp.head + (int64_t)c * EPV), f);
@@ -347,6 +385,37 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
       __syncthreads();
       C = k;
     }
+  }
+
+  // ---- many candidates for the size of the workgroup: a bitonic sort of the slots (key
+  // descending, then column ascending; zero padding sorts last) puts output slot r at position
+  // r for log^2 steps of work, where counting costs one read of every candidate per candidate
+  if (C > kSortFrom && C * C > 256 * THREADS) {
+    int cp = 2 * kSortFrom;
+    while (cp < C) cp <<= 1;
+    for (int s = C + tid; s < cp; s += THREADS) ccomp[s] = 0ull;
+    __syncthreads();
+    for (int size = 2; size <= cp; size <<= 1) {
+      for (int stride = size >> 1; stride > 0; stride >>= 1) {
+        for (int t = tid; t < cp / 2; t += THREADS) {
+          const int lo = 2 * t - (t & (stride - 1));
+          const int hi = lo + stride;
+          const bool desc = (lo & size) == 0;
+          const unsigned long long a = ccomp[lo], b = ccomp[hi];
+          if ((a < b) == desc) { ccomp[lo] = b; ccomp[hi] = a; }
+        }
+        __syncthreads();
+      }
+    }
+    for (int r = tid; r < k; r += THREADS) {
+      const int col = (int)(~(uint32_t)(ccomp[r] & 0xFFFFFFFFull));
+      const int64_t o = row * (int64_t)k + r;
+      if (idx32 != nullptr) idx32[o] = col;
+      if (idx64 != nullptr) idx64[o] = col;
+      if (values != nullptr) values[o] = rp[col];
+      if (probs != nullptr) probs[o] = fast_exp2(Elem<T>::load1(rp + col) * c1 - lse2);
+    }
+    return;
   }
 
   // ---- rank the C candidates by counting; rank r < k goes to output slot r

@@ -203,18 +203,39 @@ __device__ __forceinline__ void wave_select(const uint32_t (&key)[NR], const uin
       base += __builtin_popcountll(m);
     }
   __syncthreads();
+  if (k > 64) {
+    // many winners: a bitonic sort of the slots (padded with zeros, which sort last) costs
+    // log^2 steps where counting costs k reads per winner
+    int kp = 128;
+    while (kp < k) kp <<= 1;
+    for (int s = k + lane; s < kp; s += 64) buf[s] = 0ull;
+    __syncthreads();
+    for (int size = 2; size <= kp; size <<= 1) {
+      for (int stride = size >> 1; stride > 0; stride >>= 1) {
+        for (int t = lane; t < kp / 2; t += 64) {
+          const int lo = 2 * t - (t & (stride - 1));
+          const int hi = lo + stride;
+          const bool desc = (lo & size) == 0;
+          const unsigned long long a = buf[lo], b = buf[hi];
+          if ((a < b) == desc) { buf[lo] = b; buf[hi] = a; }
+        }
+        __syncthreads();
+      }
+    }
+    for (int s = lane; s < k; s += 64) {
+      const unsigned long long me = buf[s];
+      const int col = kWaveMaxV - (int)(uint32_t)(me & 0xFFFFFFFFull);
+      const int64_t o = row * (int64_t)k + s;
+      if (idx32 != nullptr) idx32[o] = col;
+      if (idx64 != nullptr) idx64[o] = col;
+      if (values != nullptr) values[o] = rp[col];
+    }
+    return;
+  }
   for (int s = lane; s < k; s += 64) {
     const unsigned long long me = buf[s];
     int r = 0;
-    int i = 0;
-    for (; i + 8 <= k; i += 8) {
-      unsigned long long o[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) o[u] = buf[i + u];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) r += o[u] > me ? 1 : 0;
-    }
-    for (; i < k; ++i) r += buf[i] > me ? 1 : 0;
+    for (int i = 0; i < k; ++i) r += buf[i] > me ? 1 : 0;
     const int col = kWaveMaxV - (int)(uint32_t)(me & 0xFFFFFFFFull);
     const int64_t o = row * (int64_t)k + r;
     if (idx32 != nullptr) idx32[o] = col;
@@ -360,15 +381,26 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
   const bool forced = variant != 0;       // a forced variant also bypasses the wave-per-row kernel
   if (variant == 0) variant = nvec <= 3072 ? 1 : (nvec <= 12288 ? 2 : 3);
   if (!forced) {
-    // the threshold search needs k <= 63 x (full waves of the row); more threads give more of
-    // them while the row has a vector for each. Past half of that bound the candidates mostly
-    // overflow anyway; the exact path that then runs costs a pass per key bit, which for the 16
-    // bits of a half type is cheaper at the smaller workgroup (measured), for fp32's 32 is not.
+    // The threshold search needs k <= 63 x (full waves of the row); more threads give more of
+    // them while the row has a vector for each, and it pays while k stays within half of that
+    // bound (past it the candidates mostly overflow anyway). Otherwise the exact path runs for
+    // certain: the smallest workgroup whose threads can keep the row's keys in registers
+    // (four vectors each), else the largest.
     const int64_t whole = v / EPV;
     auto cap = [&](int threads) { return (int)(std::min<int64_t>(threads, whole) / 64) * 63; };
-    auto pays = [&](int threads) { return sizeof(T) == 4 || 2 * k <= cap(threads) + 8; };
-    if (variant == 1 && k > cap(256) && cap(512) > cap(256) && pays(512)) variant = 2;
-    if (variant == 2 && k > cap(512) && cap(1024) > cap(512) && pays(1024)) variant = 3;
+    auto pays = [&](int threads) { return 2 * k <= cap(threads) + 8; };
+    const int threads_of[4] = {0, 256, 512, 1024};
+    if (k > cap(threads_of[variant])) {
+      int pick = 0;
+      for (int cand = variant + 1; cand <= 3 && pick == 0; ++cand)
+        if (cap(threads_of[cand]) > cap(threads_of[cand - 1]) && pays(threads_of[cand])) pick = cand;
+      if (pick == 0) {
+        pick = 3;
+        for (int cand = 3; cand >= 1; --cand)
+          if (whole <= (int64_t)threads_of[cand] * 4) pick = cand;
+      }
+      variant = pick;
+    }
   }
   if (v <= kWaveMaxV && !forced) {       // short rows: a wave per row
     int epl = 1;
