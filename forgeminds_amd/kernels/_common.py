@@ -110,6 +110,17 @@ def fast_ok(*tensors) -> bool:
     return True
 
 
+def wants_grad(*tensors) -> bool:
+    """Will autograd record this call? An inference call goes straight to the launcher and skips
+    the ``autograd.Function`` object (a few microseconds of host time per call)."""
+    if not torch.is_grad_enabled():
+        return False
+    for t in tensors:
+        if t is not None and t.requires_grad:
+            return True
+    return False
+
+
 def next_pow2(n: int) -> int:
     n = max(int(n), 1)
     return 1 << (n - 1).bit_length()

@@ -17,7 +17,7 @@ import torch
 
 from . import _fallback as fb
 from . import _hip, _ops
-from ._common import _note, fast_ok
+from ._common import _note, fast_ok, wants_grad
 
 
 def _c(t):
@@ -176,6 +176,8 @@ def layer_norm(x: torch.Tensor, w: torch.Tensor, b: "torch.Tensor | None" = None
             _note("layer_norm op without bias")
             return fb.layer_norm(x, w, b, eps)
         return _LN_OP(x, w, b, float(eps))[0]
+    if not wants_grad(x, w, b):
+        return _launch_fwd(x, w, b, float(eps))[1]
     return _LayerNormFn.apply(x, w, b, float(eps))
 
 
@@ -193,6 +195,8 @@ def add_layer_norm(x: torch.Tensor, delta: torch.Tensor, w: torch.Tensor,
             return fb.add_layer_norm(x, delta, w, b, eps)
         xn, y, _mean, _rstd = _ADDLN_OP(x, delta, w, b, float(eps))
         return xn, y
+    if not wants_grad(x, delta, w, b):
+        return _launch_fwd(x, w, b, float(eps), delta)[:2]
     return _AddLayerNormFn.apply(x, delta, w, b, float(eps))
 
 

@@ -21,7 +21,7 @@ import torch
 
 from . import _fallback as fb
 from . import _hip, _ops
-from ._common import _note, fast_ok
+from ._common import _note, fast_ok, wants_grad
 
 
 def _c(t: torch.Tensor) -> torch.Tensor:
@@ -172,6 +172,8 @@ def rms_norm(x: torch.Tensor, w: torch.Tensor, eps: float = 1e-6) -> torch.Tenso
         return fb.rms_norm(x, w, eps)
     if _RMS_OP is not None and _ops.wanted():
         return _RMS_OP(x, w, float(eps))[0]
+    if not wants_grad(x, w):
+        return _launch_rms_fwd(x, w, float(eps))[0]
     return _RMSNormFn.apply(x, w, float(eps))
 
 
@@ -185,4 +187,6 @@ def add_rms_norm(x: torch.Tensor, delta: torch.Tensor, w: torch.Tensor, eps: flo
     if _ADDRMS_OP is not None and _ops.wanted():
         xn, y, _rstd = _ADDRMS_OP(x, delta, w, float(eps))
         return xn, y
+    if not wants_grad(x, delta, w):
+        return _launch_addrms_fwd(x, delta, w, float(eps))[:2]
     return _AddRMSNormFn.apply(x, delta, w, float(eps))

@@ -12,7 +12,7 @@ import torch
 
 from . import _fallback as fb
 from . import _hip, _ops
-from ._common import _note, fast_ok
+from ._common import _note, fast_ok, wants_grad
 
 MAX_HEAD_DIM = 512
 
@@ -99,6 +99,8 @@ def qk_norm_rope(x: torch.Tensor, w: torch.Tensor, cos: torch.Tensor, sin: torch
         return _torch_path(x, w, cos, sin, eps)
     if _OP is not None and _ops.wanted():
         return _OP(x, w, cos, sin, float(eps))[0]
+    if not wants_grad(x, w):
+        return _launch_fwd(x, w, cos, sin, float(eps))[0]
     return _QKNormRoPE.apply(x, w, cos, sin, float(eps))
 
 

@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from . import _common, _hip
-from ._common import fast_ok
+from ._common import fast_ok, wants_grad
 
 
 class _Softmax(torch.autograd.Function):
@@ -47,6 +47,8 @@ def softmax(x: torch.Tensor, dim: int = -1, dtype: "torch.dtype | None" = None) 
         return torch.softmax(x, dim=-1)
     if not fast_ok(x):
         return torch.softmax(x, dim=-1)
+    if not wants_grad(x):
+        return _hip.softmax_fwd(x.contiguous().view(-1, x.shape[-1])).view(x.shape)
     return _Softmax.apply(x)
 
 

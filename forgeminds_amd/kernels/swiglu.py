@@ -13,7 +13,7 @@ import torch
 
 from . import _fallback as fb
 from . import _hip, _ops
-from ._common import _note, fast_ok
+from ._common import _note, fast_ok, wants_grad
 
 
 def _launch_fwd(gate, up):
@@ -113,6 +113,8 @@ def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
         return fb.swiglu(gate, up)
     if _SW_OP is not None and _ops.wanted():
         return _SW_OP(gate, up)
+    if not wants_grad(gate, up):
+        return _launch_fwd(gate, up)
     return _SwiGLUFn.apply(gate, up)
 
 
@@ -127,6 +129,8 @@ def swiglu_split(gate_up: torch.Tensor) -> torch.Tensor:
         return fb.swiglu_split(gate_up)
     if _SWS_OP is not None and _ops.wanted():
         return _SWS_OP(gate_up)
+    if not wants_grad(gate_up):
+        return _launch_split_fwd(gate_up)
     return _SwiGLUSplitFn.apply(gate_up)
 
 

@@ -12,7 +12,7 @@ import torch
 
 from . import _common, _fallback as fb
 from . import _hip
-from ._common import fast_ok
+from ._common import fast_ok, wants_grad
 
 #: the kernel ranks at most this many outputs per row; larger k takes the torch path
 MAX_K = 512
@@ -68,6 +68,9 @@ def topk(x: torch.Tensor, k: int, dim: int = -1, sorted: bool = True):
         if x.is_floating_point():
             return fb.topk_canonical(x, k)
         return torch.topk(x, k, dim=-1, sorted=True)
+    if not wants_grad(x):
+        vals, idx = _hip.topk(x.contiguous().view(-1, n), k, torch.int64)
+        return vals.view(x.shape[:-1] + (k,)), idx.view(x.shape[:-1] + (k,))
     return _TopK.apply(x, k)
 
 
