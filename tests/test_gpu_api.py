@@ -53,6 +53,35 @@ def test_gpu_calls_take_the_hip_path():
     assert "dtype torch.float64" in kernels.stats()["reasons"]
 
 
+def test_inference_calls_record_no_graph_and_give_the_same_bits():
+    x = torch.randn(64, 256, device=DEV, dtype=torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(256, device=DEV)).bfloat16()
+    b = torch.zeros_like(w)
+    xg, wg = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    cos, sin = torch.randn(8, 32, device=DEV), torch.randn(8, 32, device=DEV)
+    calls = [
+        (lambda a, ww: kernels.rms_norm(a, ww), (x, w), (xg, wg)),
+        (lambda a, ww: kernels.add_rms_norm(a, a, ww)[1], (x, w), (xg, wg)),
+        (lambda a, ww: kernels.layer_norm(a, ww, b), (x, w), (xg, wg)),
+        (lambda a, ww: kernels.add_layer_norm(a, a, ww, b)[1], (x, w), (xg, wg)),
+        (lambda a, ww: kernels.softmax(a), (x, w), (xg, wg)),
+        (lambda a, ww: kernels.swiglu(a, a), (x, w), (xg, wg)),
+        (lambda a, ww: kernels.swiglu_split(a), (x, w), (xg, wg)),
+        (lambda a, ww: kernels.topk(a, 5)[0], (x, w), (xg, wg)),
+        (lambda a, ww: kernels.qk_norm_rope(a.view(1, 8, 8, 256)[..., :64].contiguous(), ww[:64].contiguous(), cos, sin),
+         (x, w), (xg, wg)),
+    ]
+    for fn, plain, tracked in calls:
+        y0 = fn(*plain)
+        assert y0.grad_fn is None and not y0.requires_grad
+        y1 = fn(*tracked)
+        assert y1.grad_fn is not None
+        assert torch.equal(y0, y1.detach())
+        with torch.no_grad():
+            y2 = fn(*tracked)
+        assert y2.grad_fn is None and torch.equal(y2, y0)
+
+
 @pytest.mark.parametrize("dt,wdt", [(torch.bfloat16, torch.float32), (torch.bfloat16, torch.bfloat16),
                                     (torch.float32, torch.float32), (torch.float16, torch.float16)])
 def test_rms_norm_autograd_matches_oracle(dt, wdt):
