@@ -409,6 +409,61 @@ def test_launches_are_graph_capturable():
         assert all(torch.equal(a, b) for a, b in zip((y, dx, dw), ref))
 
 
+def test_loss_selection_and_routing_launches_replay_in_a_graph():
+    """The rest of the library under capture (outputs come from the graph's own pool): every
+    replay gives the bits of the eager call, with eager work and synchronisations in between."""
+    g = torch.Generator().manual_seed(77)
+    lg = (2 * torch.randn(300, 4096, generator=g)).bfloat16().to(DEV)
+    narrow = torch.randn(700, 100, generator=g).to(DEV)
+    y = torch.randint(0, 4096, (300,), generator=g).to(DEV)
+    y[::7] = -100
+    yn = torch.randint(0, 100, (700,), generator=g).to(DEV)
+    s_, t_ = lg, (lg.float() + 0.5 * torch.randn(300, 4096, generator=g).to(DEV)).bfloat16()
+    wide = (3 * torch.randn(8, 128256, generator=g)).bfloat16().to(DEV)
+    short = torch.randn(500, 1000, generator=g).to(DEV)
+    logits = torch.randn(2048, 64, generator=g).to(DEV)
+    xs = torch.randn(2048, 512, generator=g).bfloat16().to(DEV)
+
+    def step():
+        out = []
+        loss, dl, nv, rows = _hip.ce_loss_grad(lg, y, -100, "mean")
+        out += [loss, dl, nv, rows]
+        loss2, lse, nv2, rows2 = _hip.ce_fwd(narrow, yn, -100, "mean")
+        out += [loss2, lse, _hip.ce_bwd(narrow, yn, lse, nv2, None, -100)]
+        kl, rkl, ls, lt = _hip.kl_fwd(s_, t_, 0.5, "mean")
+        out += [kl, rkl, _hip.kl_bwd(s_, t_, ls, lt, None, False, torch.bfloat16, 0.5, 1.0 / 300)]
+        out += [t for t in _hip.kl_fwd_topk(wide, wide, 64, 1.0, "mean", torch.int32) if t is not None]
+        out += list(_hip.topk(wide, 64, torch.int32)) + list(_hip.topk(short, 8, torch.int64))
+        out += list(_hip.topk(short, 300, torch.int32))
+        sm = _hip.softmax_fwd(short)
+        out += [sm, _hip.softmax_bwd(sm, short)]
+        idx, wts, counts, slot, order = _hip.route(logits, 2)
+        gathered = _hip.moe_gather(xs, order, 2)
+        out += [idx, wts, counts, slot, order, gathered, _hip.moe_combine(gathered, wts, slot, 2048, 2)]
+        out += [_hip.swiglu_split_fwd(xs), _hip.swiglu_split_bwd(xs, xs[:, :256].contiguous())]
+        return out
+
+    eager = [t.clone() for t in step()]
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                           # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            outs = step()
+    for _ in range(3):
+        for t in outs:
+            t.zero_()
+        _hip.softmax_fwd(short)                          # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(outs, eager):
+            assert torch.equal(a, b)
+
+
 def test_moe_layer_matches_the_reference_expression():
     """MoE.forward of forgemind/moe.py:227-251 written with aten ops vs the fused pipeline."""
     g = torch.Generator().manual_seed(7)
