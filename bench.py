@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extras] [--no-cpu]
 
-NAME: ce (headline), ce_one_pass, rmsnorm, add_rmsnorm, add_layernorm, kl, kl_topk, topk, route,
+NAME: ce (headline), ce_one_pass, rmsnorm, add_rmsnorm, add_layernorm, kl, kl_one_launch, kl_topk, topk, route,
 moe_dispatch, swiglu, qk_norm_rope.
 
 A step is one pass of the hot path (forward + backward) over one batch of synthetic,
@@ -51,7 +51,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="ce",
-                    choices=["ce", "ce_one_pass", "rmsnorm", "add_rmsnorm", "add_layernorm", "kl", "kl_topk", "topk", "route", "moe_dispatch", "swiglu", "qk_norm_rope"])
+                    choices=["ce", "ce_one_pass", "rmsnorm", "add_rmsnorm", "add_layernorm", "kl", "kl_one_launch", "kl_topk", "topk", "route", "moe_dispatch", "swiglu", "qk_norm_rope"])
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
@@ -262,7 +262,7 @@ def make_workload(name, torch, L, dev):
         w.tensors = (lg, y)
         return w
 
-    if name in ("kl", "kl_topk", "topk"):
+    if name in ("kl", "kl_one_launch", "kl_topk", "topk"):
         n, v = 4096, 128256
         g.manual_seed(1005)
         s = (3 * torch.randn(n, v, device=dev, generator=g)).bfloat16()
@@ -292,6 +292,28 @@ def make_workload(name, torch, L, dev):
         def bwd():
             _check(L.fm_kl_bwd(s.data_ptr(), t.data_ptr(), b3[0].data_ptr(), b3[1].data_ptr(), None, 0,
                                gs.data_ptr(), n, v, BF, BF, 0.5, 1.0 / n, st), "fm_kl_bwd")
+
+        if name == "kl_one_launch":
+            one = torch.ones((), device=dev)
+
+            def both():
+                _check(L.fm_kl_loss_grad(s.data_ptr(), t.data_ptr(), b3[0].data_ptr(), b3[1].data_ptr(),
+                                         b3[2].data_ptr(), ls.data_ptr(), gs.data_ptr(), n, v, BF, BF, 0.5, 2,
+                                         st), "fm_kl_loss_grad")
+
+            def step():
+                both()      # forward: loss, and the gradient from a second sweep served by cache
+                _check(L.fm_scale_inplace(gs.data_ptr(), one.data_ptr(), n * v, BF, st),
+                       "fm_scale_inplace")   # backward: upstream gradient 1, nothing to move
+
+            w.step = step
+            w.dominant_launch = both
+            w.dominant = "kl_loss_grad_wide_kernel<bf16,bf16,1024,2>"
+            w.dominant_bytes = w.bytes = n * v * 6
+            w.desc = (f"KL loss + gradient in one launch bf16 [{n},{v}], T=2, mean; HBM dataflow read s,t + "
+                      "write g = 6 B/logit pair (the second sweep of s,t is served by the memory-side cache)")
+            w.rows = n
+            return w
 
         if name == "kl_topk":
             idx = torch.empty(n, 64, device=dev, dtype=torch.int32)
@@ -623,7 +645,7 @@ def main():
     torch.cuda.empty_cache()
     if not a.no_extras:
         extras = {a.workload: res}
-        for name in ["rmsnorm", "add_rmsnorm", "add_layernorm", "ce", "ce_one_pass", "kl", "kl_topk", "topk", "route", "moe_dispatch", "swiglu", "qk_norm_rope"]:
+        for name in ["rmsnorm", "add_rmsnorm", "add_layernorm", "ce", "ce_one_pass", "kl", "kl_one_launch", "kl_topk", "topk", "route", "moe_dispatch", "swiglu", "qk_norm_rope"]:
             if name == a.workload:
                 continue
             wl = make_workload(name, torch, L, dev)

@@ -190,6 +190,124 @@ __global__ __launch_bounds__(THREADS) void ce_bwd_kernel(const T* __restrict__ l
   }
 }
 
+// Rows too wide for registers (or unaligned buffers), loss and gradient in ONE launch: the
+// streaming log-sum-exp, the workgroup merge, then a second sweep over the same row that writes
+// the gradient. The first sweep reads with ordinary (cached) loads so that the second finds
+// the row in the memory-side cache instead of HBM. dlogits may be the logits buffer itself:
+// every element is re-read by the thread that writes it.
+template <typename T, int THREADS, int UNROLL>
+__global__ __launch_bounds__(THREADS) void ce_loss_grad_wide_kernel(const T* logits,
+                                                                     const int64_t* __restrict__ labels,
+                                                                     const float* __restrict__ n_valid,
+                                                                     float* __restrict__ lse,
+                                                                     float* __restrict__ row_loss,
+                                                                     T* dlogits, int v,
+                                                                     int64_t ignore_index, bool vec_ok) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int NW = THREADS / 64;
+  __shared__ float smem[2 * NW];
+  const int64_t row = blockIdx.x;
+  const T* rp = logits + row * (int64_t)v;
+  T* gp = dlogits + row * (int64_t)v;
+  const RowSplit sp = split_row<EPV>(row, v, vec_ok);
+  const int tid = threadIdx.x;
+  const int ne = edge_count(sp, v);
+  const int64_t y64 = labels[row];
+
+  if (y64 == ignore_index) {  // ignored row: zeros, and the logits are never read
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    for (int c = tid; c < sp.nvec; c += THREADS) store16_stream(gp + sp.head + (int64_t)c * EPV, zero);
+    for (int e = tid; e < ne; e += THREADS) Elem<T>::store1(gp + edge_col(sp, e), 0.f);
+    if (tid == 0) {
+      row_loss[row] = 0.f;
+      if (lse != nullptr) lse[row] = 0.f;
+    }
+    return;
+  }
+  const int y = (y64 >= 0 && y64 < v) ? (int)y64 : -1;
+  float ylogit = 0.f;
+  if (tid == 0 && y >= 0) ylogit = Elem<T>::load1(rp + y);
+
+  MaxSum st{kNegBig, 0.f};
+  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+    u32x4 raw[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) raw[u] = load16(rp + sp.head + (int64_t)c * EPV);
+    }
+    float z[UNROLL][EPV];
+    float raw_max = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) {
+        Elem<T>::unpack(raw[u], z[u]);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) raw_max = fmaxf(raw_max, z[u][e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) z[u][e] = -INFINITY;
+      }
+    }
+    const float cm = fmaxf(st.m, raw_max * kLog2e);
+    float acc = st.s * fast_exp2(st.m - cm);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) acc += fast_exp2(__builtin_fmaf(z[u][e], kLog2e, -cm));
+    }
+    st.m = cm;
+    st.s = acc;
+  }
+  for (int e = tid; e < ne; e += THREADS) {
+    const float z = Elem<T>::load1(rp + edge_col(sp, e)) * kLog2e;
+    const float cm = fmaxf(st.m, z);
+    st.s = st.s * fast_exp2(st.m - cm) + fast_exp2(z - cm);
+    st.m = cm;
+  }
+  const MaxSum tot = block_merge<NW>(st, smem);
+  const float l2 = tot.m + fast_log2(tot.s);
+  const float scale = 1.f / (n_valid != nullptr ? *n_valid : 1.f);
+  if (tid == 0) {
+    const float l = l2 * kLn2;
+    if (lse != nullptr) lse[row] = l;
+    row_loss[row] = y >= 0 ? l - ylogit : __builtin_nanf("");
+  }
+  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+    u32x4 raw[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) {
+        float z[EPV], o[EPV];
+        Elem<T>::unpack(raw[u], z);
+        const int col0 = sp.head + c * EPV;
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] = fast_exp2(z[e] * kLog2e - l2);
+        if (y >= col0 && y < col0 + EPV) {
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) o[e] -= (col0 + e == y) ? 1.f : 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] *= scale;
+        store16_stream(gp + col0, Elem<T>::pack(o));
+      }
+    }
+  }
+  for (int e = tid; e < ne; e += THREADS) {
+    const int col = edge_col(sp, e);
+    float p = fast_exp2(Elem<T>::load1(rp + col) * kLog2e - l2);
+    if (col == y) p -= 1.f;
+    Elem<T>::store1(gp + col, p * scale);
+  }
+}
+
 // Number of rows whose label is not ignore_index, as the float the gradient is divided by
 // (at least 1). One workgroup; runs ahead of ce_loss_grad_kernel, which needs the count.
 __global__ __launch_bounds__(1024) void ce_count_kernel(const int64_t* __restrict__ labels, int64_t n,
@@ -580,22 +698,27 @@ int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float
   const bool one_pass = n > 0 && fm_host::aligned16(logits) && fm_host::aligned16(dlogits) &&
                         nvec <= 8 * 1024;
   if (!one_pass) {
-    // rows too wide for the register file (or unaligned buffers): the two-pass kernels,
-    // which give the same outputs; lse is then needed as scratch
-    if (n > 0 && lse == nullptr) {
-      fm_host::set_error("fm_ce_loss_grad: lse is required for rows of more than %d bytes or unaligned buffers",
-                         8 * 1024 * 16);
-      return FM_ERR_INVALID;
+    // rows too wide for the register file (or unaligned buffers): two sweeps in one launch
+    if (n > 0) {
+      const bool mean_ = reduction == FM_REDUCE_MEAN;
+      if (mean_) {
+        hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(1024), 0, st, labels, n, ignore_index, n_valid);
+        FM_CHECK_LAUNCH("fm_ce_loss_grad(count)");
+      }
+      const bool vec_ok = fm_host::aligned16(logits) && fm_host::aligned16(dlogits);
+      const dim3 wgrid((unsigned)n);
+#define WIDE(T)                                                                                   \
+  hipLaunchKernelGGL((ce_loss_grad_wide_kernel<T, 1024, 2>), wgrid, dim3(1024), 0, st,            \
+                     static_cast<const T*>(logits), labels, mean_ ? n_valid : nullptr, lse, row_loss, \
+                     static_cast<T*>(dlogits), (int)v, ignore_index, vec_ok)
+      FM_CE_BY_DTYPE(dtype, WIDE);
+#undef WIDE
+      FM_CHECK_LAUNCH("fm_ce_loss_grad");
     }
-    if (n > 0 && dlogits == logits) {
-      fm_host::set_error("fm_ce_loss_grad: the gradient can overwrite the logits only for aligned rows of "
-                         "at most %d bytes", 8 * 1024 * 16);
-      return FM_ERR_UNSUPPORTED;
-    }
-    rc = fm_ce_fwd(logits, labels, lse, row_loss, loss, n_valid, n, v, dtype, ignore_index, reduction, stream);
-    if (rc != FM_OK) return rc;
-    return fm_ce_bwd(logits, labels, lse, reduction == FM_REDUCE_MEAN ? n_valid : nullptr, nullptr, dlogits,
-                     n, v, dtype, ignore_index, stream);
+    hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, st, row_loss, labels, n, ignore_index,
+                       reduction == FM_REDUCE_MEAN ? 1 : 0, loss, n_valid);
+    FM_CHECK_LAUNCH("fm_ce_loss_grad(finalize)");
+    return FM_OK;
   }
   const bool mean = reduction == FM_REDUCE_MEAN;
   const int pref = fm_host::get_param(fm_host::P_VOCAB_THREADS);

@@ -466,6 +466,96 @@ void launch_bwd(const void* s, const void* t, const float* lse_s, const float* l
 #undef LAUNCH
 }
 
+// Rows too wide for registers, loss and gradient in ONE launch: the streaming forward, the
+// workgroup merge, then a second sweep over the same row that writes the gradient. The first
+// sweep reads with ordinary (cached) loads so that the second finds the row in the memory-side
+// cache instead of HBM (the rows in flight, one or two per compute unit, fit it). The gradient
+// is for an upstream gradient of 1 and may overwrite the student (each element is re-read by
+// the thread that writes it).
+template <typename T, typename GT, int THREADS, int UNROLL>
+__global__ __launch_bounds__(THREADS) void kl_loss_grad_wide_kernel(const T* student,
+                                                                     const T* __restrict__ teacher,
+                                                                     float* __restrict__ lse_s,
+                                                                     float* __restrict__ lse_t,
+                                                                     float* __restrict__ row_kl,
+                                                                     GT* dstudent, int v, float inv_temp,
+                                                                     float mul, bool vec_ok) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int NW = THREADS / 64;
+  __shared__ float smem[5 * NW];
+  const int64_t row = blockIdx.x;
+  const T* sp_ = student + row * (int64_t)v;
+  const T* tp_ = teacher + row * (int64_t)v;
+  GT* gp = dstudent + row * (int64_t)v;
+  const RowSplit sp = split_row<EPV>(row, v, vec_ok);
+  const int tid = threadIdx.x;
+  const int ne = edge_count(sp, v);
+  const float c1 = kLog2e * inv_temp;
+
+  KLState k{kNegBig, 0.f, kNegBig, 0.f, 0.f};
+  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+    u32x4 rs[UNROLL], rt[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) {
+        rs[u] = load16(sp_ + sp.head + (int64_t)c * EPV);
+        rt[u] = load16(tp_ + sp.head + (int64_t)c * EPV);
+      }
+    }
+    kl_update<T, UNROLL>(k, rs, rt, c0 + tid, THREADS, sp.nvec, c1);
+  }
+  for (int e = tid; e < ne; e += THREADS) {
+    const int col = edge_col(sp, e);
+    kl_update1(k, Elem<T>::load1(sp_ + col) * c1, Elem<T>::load1(tp_ + col) * c1);
+  }
+  float l2s, l2t, kl2;
+  kl_merge<NW>(k, smem, &l2s, &l2t, &kl2);
+  if (tid == 0) {
+    if (lse_s != nullptr) lse_s[row] = l2s * kLn2;
+    if (lse_t != nullptr) lse_t[row] = l2t * kLn2;
+    row_kl[row] = kl2 * kLn2;
+  }
+  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+    u32x4 rs[UNROLL], rt[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) {
+        rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
+        rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) {
+        float zs[EPV], zt[EPV], o[EPV];
+        Elem<T>::unpack(rs[u], zs);
+        Elem<T>::unpack(rt[u], zt);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e)
+          o[e] = (fast_exp2(zs[e] * c1 - l2s) - fast_exp2(zt[e] * c1 - l2t)) * mul;
+        GT* dst = gp + sp.head + (int64_t)c * EPV;
+        if constexpr (sizeof(GT) == sizeof(T)) {
+          store16_stream(dst, Elem<GT>::pack(o));
+        } else {
+          static_assert(sizeof(GT) == 4 && EPV == 8, "gradient is the logits' dtype or fp32");
+          float lo[4] = {o[0], o[1], o[2], o[3]}, hi[4] = {o[4], o[5], o[6], o[7]};
+          store16_stream(dst, Elem<float>::pack(lo));
+          store16_stream(dst + 4, Elem<float>::pack(hi));
+        }
+      }
+    }
+  }
+  for (int e = tid; e < ne; e += THREADS) {
+    const int col = edge_col(sp, e);
+    const float ps = fast_exp2(Elem<T>::load1(sp_ + col) * c1 - l2s);
+    const float pt = fast_exp2(Elem<T>::load1(tp_ + col) * c1 - l2t);
+    Elem<GT>::store1(gp + col, (ps - pt) * mul);
+  }
+}
+
 // Narrow rows (at most 1024 classes: classifier distillation, not vocabularies): TPR lanes per
 // row, several rows per 256-thread workgroup, both rows in registers (ITERS scalar loads each
 // per lane), any alignment. LOSS writes the log-sum-exps and the row's KL; GRAD writes the
@@ -749,21 +839,29 @@ int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, floa
   const bool one_pass = n > 0 && fm_host::aligned16(student) && fm_host::aligned16(teacher) &&
                         fm_host::aligned16(dstudent) && nvec <= kOnePassMaxVec;
   if (!one_pass) {
-    if (n > 0 && dstudent == student) {
-      fm_host::set_error("fm_kl_loss_grad: the gradient can overwrite the student only for aligned rows "
-                         "of at most %d bytes", kOnePassMaxVec * 16);
-      return FM_ERR_UNSUPPORTED;
+    if (n == 0) {
+      return fm_kl_fwd(student, teacher, lse_s, lse_t, row_kl, loss, n, v, dtype, inv_temperature, reduction,
+                       stream);
     }
-    if (n > 0 && (lse_s == nullptr || lse_t == nullptr)) {
-      fm_host::set_error("fm_kl_loss_grad: lse_s and lse_t are required for rows of more than %d bytes or "
-                         "unaligned buffers", kOnePassMaxVec * 16);
-      return FM_ERR_INVALID;
+    // wide (or unaligned) rows: two sweeps in one launch, the second served by cache. With a
+    // gradient in another dtype than the student the buffers must differ, which the argument
+    // check above already ensures.
+    const bool vec_ok = fm_host::aligned16(student) && fm_host::aligned16(teacher) &&
+                        fm_host::aligned16(dstudent);
+    const float mul_w = inv_temperature * scale;
+    const dim3 wgrid((unsigned)n);
+#define WIDE(T, GT)                                                                                \
+  hipLaunchKernelGGL((kl_loss_grad_wide_kernel<T, GT, 1024, 2>), wgrid, dim3(1024), 0, st,         \
+                     static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t,  \
+                     row_kl, static_cast<GT*>(dstudent), (int)v, inv_temperature, mul_w, vec_ok)
+    FM_KL_BY_DTYPES(dtype, grad_dtype, WIDE);
+#undef WIDE
+    FM_CHECK_LAUNCH("fm_kl_loss_grad");
+    if (loss != nullptr) {
+      hipLaunchKernelGGL(kl_finalize_kernel, dim3(1), dim3(1024), 0, st, row_kl, n, scale, loss);
+      FM_CHECK_LAUNCH("fm_kl_loss_grad(finalize)");
     }
-    rc = fm_kl_fwd(student, teacher, lse_s, lse_t, row_kl, loss, n, v, dtype, inv_temperature, reduction,
-                   stream);
-    if (rc != FM_OK) return rc;
-    return fm_kl_bwd(student, teacher, lse_s, lse_t, nullptr, 0, dstudent, n, v, dtype, grad_dtype,
-                     inv_temperature, scale, stream);
+    return FM_OK;
   }
   // the fewest threads that hold both rows in at most 4 vectors each per thread
   int threads = 256;

@@ -156,10 +156,9 @@ int fm_ce_bwd(const void* logits, const int64_t* labels, const float* lse, const
  * Rows stay in registers between the log-sum-exp and the store, so the step moves 2 + 2
  * bytes per 16-bit logit instead of 2 + 2 + 2. dlogits may be the logits buffer itself
  * (the way the reference's KL writes its gradient into an owned student tensor,
- * kernels/kl.py:146-150, 157-160). lse may be NULL when rows are at most 128 KiB and both
- * buffers are 16-byte aligned; wider rows run fm_ce_fwd + fm_ce_bwd internally, need lse, and
- * cannot be rewritten in place (FM_ERR_UNSUPPORTED when dlogits == logits).
- * lse of ignored rows is written as 0 by the one-pass form (those rows are not read). */
+ * kernels/kl.py:146-150, 157-160); lse may be NULL. Rows wider than 128 KiB (or unaligned
+ * buffers) are swept twice inside the same launch, the second sweep served by the
+ * memory-side cache. lse of ignored rows is written as 0 (those rows are not read). */
 int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float* row_loss,
                     float* loss, float* n_valid, void* dlogits, int64_t n, int64_t v, int dtype,
                     int64_t ignore_index, int reduction, fm_stream_t stream);
@@ -186,10 +185,10 @@ int fm_kl_fwd(const void* student, const void* teacher, float* lse_s, float* lse
  * fm_kl_fwd's outputs plus dstudent = fm_kl_bwd's result for grad_out = 1 and
  * scale = 1/n (FM_REDUCE_MEAN) or 1 (FM_REDUCE_SUM). Rows of at most 64 KiB stay in
  * registers between the log-sum-exps and the store (4 + 2 bytes per pair of 16-bit logits
- * instead of 4 + 4 + 2) and dstudent may then be the student buffer itself when
- * grad_dtype == dtype (kl.py:146-150, reuse=True). Wider rows run fm_kl_fwd + fm_kl_bwd
- * internally, need lse_s / lse_t (otherwise optional) and cannot be rewritten in place
- * (FM_ERR_UNSUPPORTED). fm_scale_inplace applies an upstream gradient other than 1. */
+ * instead of 4 + 4 + 2); wider rows are swept twice inside the same launch, the second
+ * sweep served by the memory-side cache. dstudent may be the student buffer itself when
+ * grad_dtype == dtype (kl.py:146-150, reuse=True); lse_s / lse_t may be NULL.
+ * fm_scale_inplace applies an upstream gradient other than 1. */
 int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, float* lse_t,
                     float* row_kl, float* loss, void* dstudent, int64_t n, int64_t v, int dtype,
                     int grad_dtype, float inv_temperature, int reduction, fm_stream_t stream);
