@@ -3,7 +3,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extras] [--no-cpu]
 
-NAME: ce (headline), ce_one_pass, rmsnorm, add_rmsnorm, add_layernorm, kl, kl_one_launch, kl_topk, topk, route,
+NAME: ce (headline), ce_one_pass, rmsnorm, add_rmsnorm, add_layernorm, kl, kl_one_launch, kl_topk, kl_topk_one_launch, topk,
+route,
 moe_dispatch, swiglu, qk_norm_rope.
 
 A step is one pass of the hot path (forward + backward) over one batch of synthetic,
@@ -51,7 +52,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="ce",
-                    choices=["ce", "ce_one_pass", "rmsnorm", "add_rmsnorm", "add_layernorm", "kl", "kl_one_launch", "kl_topk", "topk", "route", "moe_dispatch", "swiglu", "qk_norm_rope"])
+                    choices=["ce", "ce_one_pass", "rmsnorm", "add_rmsnorm", "add_layernorm", "kl", "kl_one_launch", "kl_topk", "kl_topk_one_launch", "topk", "route", "moe_dispatch", "swiglu", "qk_norm_rope"])
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
@@ -262,7 +263,7 @@ def make_workload(name, torch, L, dev):
         w.tensors = (lg, y)
         return w
 
-    if name in ("kl", "kl_one_launch", "kl_topk", "topk"):
+    if name in ("kl", "kl_one_launch", "kl_topk", "kl_topk_one_launch", "topk"):
         n, v = 4096, 128256
         g.manual_seed(1005)
         s = (3 * torch.randn(n, v, device=dev, generator=g)).bfloat16()
@@ -312,6 +313,29 @@ def make_workload(name, torch, L, dev):
             w.dominant_bytes = w.bytes = n * v * 6
             w.desc = (f"KL loss + gradient in one launch bf16 [{n},{v}], T=2, mean; HBM dataflow read s,t + "
                       "write g = 6 B/logit pair (the second sweep of s,t is served by the memory-side cache)")
+            w.rows = n
+            return w
+
+        if name == "kl_topk_one_launch":
+            one = torch.ones((), device=dev)
+            idx = torch.empty(n, 64, device=dev, dtype=torch.int32)
+            pr = torch.empty(n, 64, device=dev)
+
+            def both():
+                _check(L.fm_kl_loss_grad_topk(s.data_ptr(), t.data_ptr(), b3[0].data_ptr(), b3[1].data_ptr(),
+                                              b3[2].data_ptr(), ls.data_ptr(), gs.data_ptr(), None, idx.data_ptr(),
+                                              pr.data_ptr(), n, v, 64, BF, 32, 0.5, 2, st), "fm_kl_loss_grad_topk")
+
+            def step():
+                both()
+                _check(L.fm_scale_inplace(gs.data_ptr(), one.data_ptr(), n * v, BF, st), "fm_scale_inplace")
+
+            w.step = step
+            w.dominant_launch = both
+            w.dominant = "kl_fwd_topk_kernel<bf16,512,2>"
+            w.dominant_bytes = w.bytes = n * v * 6
+            w.desc = (f"KL loss + gradient + teacher top-64 in one launch bf16 [{n},{v}], T=2, mean; HBM "
+                      "dataflow 6 B/logit pair")
             w.rows = n
             return w
 
@@ -645,7 +669,7 @@ def main():
     torch.cuda.empty_cache()
     if not a.no_extras:
         extras = {a.workload: res}
-        for name in ["rmsnorm", "add_rmsnorm", "add_layernorm", "ce", "ce_one_pass", "kl", "kl_one_launch", "kl_topk", "topk", "route", "moe_dispatch", "swiglu", "qk_norm_rope"]:
+        for name in ["rmsnorm", "add_rmsnorm", "add_layernorm", "ce", "ce_one_pass", "kl", "kl_one_launch", "kl_topk", "kl_topk_one_launch", "topk", "route", "moe_dispatch", "swiglu", "qk_norm_rope"]:
             if name == a.workload:
                 continue
             wl = make_workload(name, torch, L, dev)

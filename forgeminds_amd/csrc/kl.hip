@@ -117,6 +117,54 @@ __device__ __forceinline__ void kl_merge(const KLState& k, float* smem, float* l
   *kl2 = A / Dt - *l2t + *l2s;
 }
 
+// One sweep over a row that writes (softmax(s) - softmax(t)) * mul from the row's base-2
+// log-sum-exps: the body of the backward, shared by the kernels that append it to a forward.
+template <typename T, typename GT, int THREADS, int UNROLL>
+__device__ __forceinline__ void kl_grad_sweep(const T* sp_, const T* tp_, GT* gp, const RowSplit& sp,
+                                              int v, float c1, float l2s, float l2t, float mul) {
+  constexpr int EPV = Elem<T>::kVec;
+  const int tid = threadIdx.x;
+  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+    u32x4 rs[UNROLL], rt[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) {
+        rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
+        rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      if (c < sp.nvec) {
+        float zs[EPV], zt[EPV], o[EPV];
+        Elem<T>::unpack(rs[u], zs);
+        Elem<T>::unpack(rt[u], zt);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e)
+          o[e] = (fast_exp2(zs[e] * c1 - l2s) - fast_exp2(zt[e] * c1 - l2t)) * mul;
+        GT* dst = gp + sp.head + (int64_t)c * EPV;
+        if constexpr (sizeof(GT) == sizeof(T)) {
+          store16_stream(dst, Elem<GT>::pack(o));
+        } else {  // fp32 gradient next to 16-bit logits: two 16-byte stores
+          static_assert(sizeof(GT) == 4 && EPV == 8, "gradient is the logits' dtype or fp32");
+          float lo[4] = {o[0], o[1], o[2], o[3]}, hi[4] = {o[4], o[5], o[6], o[7]};
+          store16_stream(dst, Elem<float>::pack(lo));
+          store16_stream(dst + 4, Elem<float>::pack(hi));
+        }
+      }
+    }
+  }
+  const int ne = edge_count(sp, v);
+  for (int e = tid; e < ne; e += THREADS) {
+    const int col = edge_col(sp, e);
+    const float ps = fast_exp2(Elem<T>::load1(sp_ + col) * c1 - l2s);
+    const float pt = fast_exp2(Elem<T>::load1(tp_ + col) * c1 - l2t);
+    Elem<GT>::store1(gp + col, (ps - pt) * mul);
+  }
+}
+
 template <typename T, int THREADS, int UNROLL>
 __global__ __launch_bounds__(THREADS) void kl_fwd_kernel(const T* __restrict__ student,
                                                           const T* __restrict__ teacher,
@@ -171,7 +219,7 @@ __global__ __launch_bounds__(THREADS) void kl_fwd_topk_kernel(
     const T* __restrict__ student, const T* __restrict__ teacher, float* __restrict__ lse_s,
     float* __restrict__ lse_t, float* __restrict__ row_kl, T* __restrict__ tk_values,
     int32_t* __restrict__ tk_idx32, int64_t* __restrict__ tk_idx64, float* __restrict__ tk_probs,
-    int v, int k, float inv_temp, bool vec_ok) {
+    T* __restrict__ dstudent, float mul, int v, int k, float inv_temp, bool vec_ok) {
   constexpr int EPV = Elem<T>::kVec;
   constexpr int NW = THREADS / 64;
   __shared__ float smem[5 * NW];
@@ -198,8 +246,13 @@ __global__ __launch_bounds__(THREADS) void kl_fwd_topk_kernel(
     for (int u = 0; u < UNROLL; ++u) {
       const int c = c0 + u * THREADS + tid;
       if (c < sp.nvec) {
-        rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
-        rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
+        if (dstudent != nullptr) {   // a gradient sweep follows: leave the row to the caches
+          rs[u] = load16(sp_ + sp.head + (int64_t)c * EPV);
+          rt[u] = load16(tp_ + sp.head + (int64_t)c * EPV);
+        } else {
+          rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
+          rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
+        }
       }
     }
     kl_update<T, UNROLL>(st, rs, rt, c0 + tid, THREADS, sp.nvec, c1);
@@ -233,6 +286,8 @@ __global__ __launch_bounds__(THREADS) void kl_fwd_topk_kernel(
   const float none[1] = {0.f};
   topk_finish<T, THREADS, 1, kVecMaxLds>(tp_, sp, v, k, none, vhi, fm, has_nan, sh, row, tk_values,
                                          tk_idx32, tk_idx64, tk_probs, c1, l2t);
+  if (dstudent != nullptr)
+    kl_grad_sweep<T, T, THREADS, UNROLL>(sp_, tp_, dstudent + row * (int64_t)v, sp, v, c1, l2s, l2t, mul);
 }
 
 // loss = sum(row_kl) * scale in a fixed order (thread i adds rows i, i+1024, ...).
@@ -516,44 +571,7 @@ __global__ __launch_bounds__(THREADS) void kl_loss_grad_wide_kernel(const T* stu
     if (lse_t != nullptr) lse_t[row] = l2t * kLn2;
     row_kl[row] = kl2 * kLn2;
   }
-  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
-    u32x4 rs[UNROLL], rt[UNROLL];
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) {
-        rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
-        rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) {
-        float zs[EPV], zt[EPV], o[EPV];
-        Elem<T>::unpack(rs[u], zs);
-        Elem<T>::unpack(rt[u], zt);
-#pragma unroll
-        for (int e = 0; e < EPV; ++e)
-          o[e] = (fast_exp2(zs[e] * c1 - l2s) - fast_exp2(zt[e] * c1 - l2t)) * mul;
-        GT* dst = gp + sp.head + (int64_t)c * EPV;
-        if constexpr (sizeof(GT) == sizeof(T)) {
-          store16_stream(dst, Elem<GT>::pack(o));
-        } else {
-          static_assert(sizeof(GT) == 4 && EPV == 8, "gradient is the logits' dtype or fp32");
-          float lo[4] = {o[0], o[1], o[2], o[3]}, hi[4] = {o[4], o[5], o[6], o[7]};
-          store16_stream(dst, Elem<float>::pack(lo));
-          store16_stream(dst + 4, Elem<float>::pack(hi));
-        }
-      }
-    }
-  }
-  for (int e = tid; e < ne; e += THREADS) {
-    const int col = edge_col(sp, e);
-    const float ps = fast_exp2(Elem<T>::load1(sp_ + col) * c1 - l2s);
-    const float pt = fast_exp2(Elem<T>::load1(tp_ + col) * c1 - l2t);
-    Elem<GT>::store1(gp + col, (ps - pt) * mul);
-  }
+  kl_grad_sweep<T, GT, THREADS, UNROLL>(sp_, tp_, gp, sp, v, c1, l2s, l2t, mul);
 }
 
 // Narrow rows (at most 1024 classes: classifier distillation, not vocabularies): TPR lanes per
@@ -708,27 +726,27 @@ int fm_kl_fwd(const void* student, const void* teacher, float* lse_s, float* lse
   return FM_OK;
 }
 
-int fm_kl_fwd_topk(const void* student, const void* teacher, float* lse_s, float* lse_t,
-                   float* row_kl, float* loss, void* topk_values, void* topk_indices,
-                   float* topk_probs, int64_t n, int64_t v, int k, int dtype, int index_bits,
-                   float inv_temperature, int reduction, fm_stream_t stream) {
-  int rc = check_shape("fm_kl_fwd_topk", n, v, dtype);
+static int kl_topk_entry(const char* what, const void* student, const void* teacher, float* lse_s,
+                         float* lse_t, float* row_kl, float* loss, void* dstudent, void* topk_values,
+                         void* topk_indices, float* topk_probs, int64_t n, int64_t v, int k, int dtype,
+                         int index_bits, float inv_temperature, int reduction, fm_stream_t stream) {
+  int rc = check_shape(what, n, v, dtype);
   if (rc != FM_OK) return rc;
   FM_CHECK_ARG(reduction == FM_REDUCE_NONE || reduction == FM_REDUCE_SUM || reduction == FM_REDUCE_MEAN,
-               "fm_kl_fwd_topk: bad reduction %d", reduction);
-  FM_CHECK_ARG(index_bits == 32 || index_bits == 64, "fm_kl_fwd_topk: index_bits must be 32 or 64");
-  FM_CHECK_ARG(k >= 1 && k <= v, "fm_kl_fwd_topk: selected index k out of range (k=%d, v=%lld)", k,
+               "%s: bad reduction %d", what, reduction);
+  FM_CHECK_ARG(index_bits == 32 || index_bits == 64, "%s: index_bits must be 32 or 64", what);
+  FM_CHECK_ARG(k >= 1 && k <= v, "%s: selected index k out of range (k=%d, v=%lld)", what, k,
                (long long)v);
-  FM_CHECK_ARG(inv_temperature > 0.f, "fm_kl_fwd_topk: the temperature must be positive");
+  FM_CHECK_ARG(inv_temperature > 0.f, "%s: the temperature must be positive", what);
   const int esize = dtype == FM_F32 ? 4 : 2;
   const int64_t nvec_max = v / (16 / esize);
   if (k > kMaxK || nvec_max > kFusedMaxVec) {
-    fm_host::set_error("fm_kl_fwd_topk: k <= %d and rows of at most %d bytes are fused (k=%d, v=%lld); "
-                       "call fm_kl_fwd and fm_topk instead", kMaxK, kFusedMaxVec * 16, k, (long long)v);
+    fm_host::set_error("%s: k <= %d and rows of at most %d bytes are fused (k=%d, v=%lld); "
+                       "call fm_kl_fwd and fm_topk instead", what, kMaxK, kFusedMaxVec * 16, k, (long long)v);
     return FM_ERR_UNSUPPORTED;
   }
   FM_CHECK_ARG(n == 0 || (student && teacher && lse_s && lse_t && row_kl && topk_indices),
-               "fm_kl_fwd_topk: NULL pointer");
+               "%s: NULL pointer", what);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (n > 0) {
     const bool vec_ok = fm_host::aligned16(student) && fm_host::aligned16(teacher);
@@ -738,11 +756,13 @@ int fm_kl_fwd_topk(const void* student, const void* teacher, float* lse_s, float
     if (threads != 256 && threads != 1024) threads = 512;
     const size_t lds = (size_t)((nvec_max + 3) / 4 * 4 + 4) * sizeof(uint16_t);
     const dim3 grid((unsigned)n);
+    // gradient (when asked for) is for an upstream gradient of 1
+    const float mul = inv_temperature * ((reduction == FM_REDUCE_MEAN) ? 1.f / (float)n : 1.f);
 #define LAUNCH(T, TH)                                                                              \
   hipLaunchKernelGGL((kl_fwd_topk_kernel<T, TH, 2>), grid, dim3(TH), lds, st,                      \
                      static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t, \
-                     row_kl, static_cast<T*>(topk_values), i32, i64, topk_probs, (int)v, k,        \
-                     inv_temperature, vec_ok)
+                     row_kl, static_cast<T*>(topk_values), i32, i64, topk_probs,                   \
+                     static_cast<T*>(dstudent), mul, (int)v, k, inv_temperature, vec_ok)
 #define BY_THREADS(T)                      \
   do {                                     \
     if (threads == 256) LAUNCH(T, 256);    \
@@ -754,14 +774,36 @@ int fm_kl_fwd_topk(const void* student, const void* teacher, float* lse_s, float
     else BY_THREADS(f16_t);
 #undef BY_THREADS
 #undef LAUNCH
-    FM_CHECK_LAUNCH("fm_kl_fwd_topk");
+    FM_CHECK_LAUNCH(what);
   }
   if (reduction != FM_REDUCE_NONE && loss != nullptr) {
     const float scale = (reduction == FM_REDUCE_MEAN && n > 0) ? 1.f / (float)n : 1.f;
     hipLaunchKernelGGL(kl_finalize_kernel, dim3(1), dim3(1024), 0, st, row_kl, n, scale, loss);
-    FM_CHECK_LAUNCH("fm_kl_fwd_topk(finalize)");
+    FM_CHECK_LAUNCH(what);
   }
   return FM_OK;
+}
+
+int fm_kl_fwd_topk(const void* student, const void* teacher, float* lse_s, float* lse_t,
+                   float* row_kl, float* loss, void* topk_values, void* topk_indices,
+                   float* topk_probs, int64_t n, int64_t v, int k, int dtype, int index_bits,
+                   float inv_temperature, int reduction, fm_stream_t stream) {
+  return kl_topk_entry("fm_kl_fwd_topk", student, teacher, lse_s, lse_t, row_kl, loss, nullptr, topk_values,
+                       topk_indices, topk_probs, n, v, k, dtype, index_bits, inv_temperature, reduction,
+                       stream);
+}
+
+int fm_kl_loss_grad_topk(const void* student, const void* teacher, float* lse_s, float* lse_t,
+                         float* row_kl, float* loss, void* dstudent, void* topk_values,
+                         void* topk_indices, float* topk_probs, int64_t n, int64_t v, int k, int dtype,
+                         int index_bits, float inv_temperature, int reduction, fm_stream_t stream) {
+  FM_CHECK_ARG(reduction == FM_REDUCE_SUM || reduction == FM_REDUCE_MEAN,
+               "fm_kl_loss_grad_topk: reduction must be sum or mean (got %d)", reduction);
+  FM_CHECK_ARG(n == 0 || (dstudent != nullptr && dstudent != student),
+               "fm_kl_loss_grad_topk: dstudent must be a buffer of its own");
+  return kl_topk_entry("fm_kl_loss_grad_topk", student, teacher, lse_s, lse_t, row_kl, loss, dstudent,
+                       topk_values, topk_indices, topk_probs, n, v, k, dtype, index_bits, inv_temperature,
+                       reduction, stream);
 }
 
 int fm_kl_bwd(const void* student, const void* teacher, const float* lse_s, const float* lse_t,

@@ -53,6 +53,8 @@ SIGNATURES = {
     "fm_kl_loss_grad": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _f32, _int, _vp]),
     "fm_kl_fwd_topk": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _int,
                               _f32, _int, _vp]),
+    "fm_kl_loss_grad_topk": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int,
+                                    _int, _f32, _int, _vp]),
     "fm_kl_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _i64, _i64, _int, _int, _f32, _f32, _vp]),
     "fm_topk": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _int, _int, _vp]),
     "fm_softmax_fwd": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
@@ -391,12 +393,15 @@ def kl_loss_grad(s2, t2, inv_temperature: float, reduction: str, grad_dtype, inp
 
 
 def kl_fwd_topk(s2, t2, k: int, inv_temperature: float, reduction: str, index_dtype=torch.int64,
-                want_values: bool = False, want_probs: bool = True):
+                want_values: bool = False, want_probs: bool = True, want_grad: bool = False):
     """-> (loss or None, row_kl, lse_s, lse_t, values or None, idx, probs or None); None when the
-    shape is outside what the fused kernel takes (the caller then runs the two kernels)."""
+    shape is outside what the fused kernel takes (the caller then runs the two kernels).
+    ``want_grad`` (reduction sum or mean) appends the student's gradient for an upstream
+    gradient of 1, written by the same launch."""
     _dense(s2, t2)
     n, v = s2.shape
     dev = s2.device
+    grad = torch.empty_like(s2) if want_grad else None
     buf = torch.empty(3, n, device=dev, dtype=torch.float32)
     loss = torch.empty((), device=dev, dtype=torch.float32) if reduction != "none" else None
     vals = torch.empty((n, k), device=dev, dtype=t2.dtype) if want_values else None
@@ -404,13 +409,21 @@ def kl_fwd_topk(s2, t2, k: int, inv_temperature: float, reduction: str, index_dt
     idx = torch.empty((n, k), device=dev, dtype=index_dtype)
     bits = 64 if index_dtype == torch.int64 else 32
     with _guard(dev):
-        rc = lib().fm_kl_fwd_topk(_ptr(s2), _ptr(t2), buf[0].data_ptr(), buf[1].data_ptr(),
-                                  buf[2].data_ptr(), _ptr(loss), _ptr(vals), _ptr(idx), _ptr(probs),
-                                  n, v, int(k), dtype_code(s2.dtype), bits, float(inv_temperature),
-                                  REDUCE[reduction], _stream(s2))
+        if want_grad:
+            rc = lib().fm_kl_loss_grad_topk(_ptr(s2), _ptr(t2), buf[0].data_ptr(), buf[1].data_ptr(),
+                                            buf[2].data_ptr(), _ptr(loss), _ptr(grad), _ptr(vals), _ptr(idx),
+                                            _ptr(probs), n, v, int(k), dtype_code(s2.dtype), bits,
+                                            float(inv_temperature), REDUCE[reduction], _stream(s2))
+        else:
+            rc = lib().fm_kl_fwd_topk(_ptr(s2), _ptr(t2), buf[0].data_ptr(), buf[1].data_ptr(),
+                                      buf[2].data_ptr(), _ptr(loss), _ptr(vals), _ptr(idx), _ptr(probs),
+                                      n, v, int(k), dtype_code(s2.dtype), bits, float(inv_temperature),
+                                      REDUCE[reduction], _stream(s2))
     if rc == 2:   # FM_ERR_UNSUPPORTED
         return None
-    _check(rc, "fm_kl_fwd_topk")
+    _check(rc, "fm_kl_loss_grad_topk" if want_grad else "fm_kl_fwd_topk")
+    if want_grad:
+        return loss, buf[2], buf[0], buf[1], vals, idx, probs, grad
     return loss, buf[2], buf[0], buf[1], vals, idx, probs
 
 

@@ -79,15 +79,26 @@ class _KLDivTopkFn(torch.autograd.Function):
         s2 = student.contiguous().view(-1, v)
         t2 = teacher.contiguous().view(-1, v)
         inv_t = 1.0 / float(temperature)
-        out = _hip.kl_fwd_topk(s2, t2, k, inv_t, reduction, index_dtype)
+        gdt = grad_dtype or student.dtype
+        ctx.in_forward = False
+        ctx.spent = False
+        # KL, the teacher's top-k and (when the student needs it, in its own dtype) the gradient
+        # for an upstream gradient of 1, all from one launch
+        with_grad = reduction != "none" and ctx.needs_input_grad[0] and gdt == student.dtype
+        out = _hip.kl_fwd_topk(s2.detach(), t2, k, inv_t, reduction, index_dtype, want_grad=with_grad)
         if out is None:   # row too wide for the fused kernel: two launches, same results
+            with_grad = False
             loss, rows, lse_s, lse_t = _hip.kl_fwd(s2, t2, inv_t, reduction)
             vals, idx = _hip.topk(t2, k, index_dtype)
             probs = torch.exp(vals.float() * inv_t - lse_t[:, None])
         else:
-            loss, rows, lse_s, lse_t, _, idx, probs = out
-        ctx.save_for_backward(s2, t2, lse_s, lse_t)
-        ctx.meta = (student.shape, reduction, grad_dtype or student.dtype, inv_t)
+            loss, rows, lse_s, lse_t, _, idx, probs = out[:7]
+        if with_grad:
+            ctx.in_forward = True
+            ctx.save_for_backward(out[7])
+        else:
+            ctx.save_for_backward(s2, t2, lse_s, lse_t)
+        ctx.meta = (student.shape, reduction, gdt, inv_t)
         lead = student.shape[:-1]
         probs = probs.view(*lead, k)
         idx = idx.view(*lead, k)
@@ -98,8 +109,16 @@ class _KLDivTopkFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g, _gp, _gi):
-        s2, t2, lse_s, lse_t = ctx.saved_tensors
         shape, reduction, gdt, inv_t = ctx.meta
+        if ctx.in_forward:
+            (grad,) = ctx.saved_tensors
+            if ctx.spent:
+                raise RuntimeError("kl_div_logits_topk: the gradient buffer written in the forward was "
+                                   "already consumed by a backward pass; run the forward again")
+            ctx.spent = True
+            _hip.scale_inplace(grad, g.detach().to(torch.float32).contiguous())
+            return grad.view(shape), None, None, None, None, None, None
+        s2, t2, lse_s, lse_t = ctx.saved_tensors
         n = s2.shape[0]
         g32 = g.detach().to(torch.float32).contiguous().view(-1)
         scale = 1.0 / n if reduction == "mean" else 1.0

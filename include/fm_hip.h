@@ -206,6 +206,16 @@ int fm_kl_fwd_topk(const void* student, const void* teacher, float* lse_s, float
                    float* topk_probs, int64_t n, int64_t v, int k, int dtype, int index_bits,
                    float inv_temperature, int reduction, fm_stream_t stream);
 
+/* fm_kl_fwd_topk that also writes the gradient of the student in the same launch (a second
+ * sweep of the row, served by the memory-side cache, after the selection): dstudent [n, v] of
+ * dtype = fm_kl_bwd's result for grad_out = 1 and scale = 1/n (FM_REDUCE_MEAN) or 1
+ * (FM_REDUCE_SUM), a buffer of its own. One launch for a whole distillation step (KL, its
+ * gradient, the teacher's top-k). No counterpart in the reference (see fm_kl_fwd_topk). */
+int fm_kl_loss_grad_topk(const void* student, const void* teacher, float* lse_s, float* lse_t,
+                         float* row_kl, float* loss, void* dstudent, void* topk_values,
+                         void* topk_indices, float* topk_probs, int64_t n, int64_t v, int k, int dtype,
+                         int index_bits, float inv_temperature, int reduction, fm_stream_t stream);
+
 /* Gradient wrt the (unscaled) student logits, recomputed from the saved lse values
  * (the reference stores it from the forward, kl.py:112-134, and rescales it in
  * _KLDivFn.backward, kl.py:181-191):

@@ -478,6 +478,20 @@ def test_kl_fwd_topk_matches_the_two_kernels(n, v, k, dt, T):
         assert torch.allclose(ls, ls2, rtol=1e-6, atol=2e-6) and torch.allclose(lt, lt2, rtol=1e-6, atol=2e-6)
         want = torch.gather(torch.softmax(t.double() / T, -1), -1, oi)
         assert torch.allclose(probs.cpu().double(), want, rtol=1e-4, atol=1e-9)
+    # the same launch also writing the student's gradient: every other output keeps its bits
+    keep = sd.clone()
+    full = _hip.kl_fwd_topk(sd, td, k, 1.0 / T, "mean", torch.int64, want_values=True, want_probs=True,
+                            want_grad=True)
+    torch.cuda.synchronize()
+    assert torch.equal(sd, keep)
+    for a, b in zip(full[:7], out):
+        assert torch.equal(a, b)
+    _, ograd = O.kl_div(s, t, "mean", T)
+    lse_mag = 1.0 + float(torch.logsumexp(s.double() / T, -1).abs().max())
+    assert_close_lowp(full[7], ograd, dt, "dstudent", ulps=3.0, cancel=lse_mag / (T * n))
+    summed = _hip.kl_fwd_topk(sd, td, k, 1.0 / T, "sum", torch.int32, want_grad=True)
+    _, ograd_sum = O.kl_div(s, t, "sum", T)
+    assert_close_lowp(summed[7], ograd_sum, dt, "dstudent (sum)", ulps=3.0, cancel=lse_mag / T)
 
 
 def test_kl_fwd_topk_ties_unaligned_and_unsupported():
