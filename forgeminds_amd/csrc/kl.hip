@@ -214,7 +214,7 @@ __global__ __launch_bounds__(THREADS) void kl_fwd_kernel(const T* __restrict__ s
 // the temperature are monotone, so the order is that of the probabilities). The streaming pass
 // leaves a 16-bit key prefix of every teacher vector's maximum in LDS (2 bytes per 16 bytes of
 // row), so the selection revisits only the few vectors that can hold a winner.
-template <typename T, int THREADS, int UNROLL>
+template <typename T, int THREADS, int UNROLL, bool GRAD>
 __global__ __launch_bounds__(THREADS) void kl_fwd_topk_kernel(
     const T* __restrict__ student, const T* __restrict__ teacher, float* __restrict__ lse_s,
     float* __restrict__ lse_t, float* __restrict__ row_kl, T* __restrict__ tk_values,
@@ -246,7 +246,7 @@ __global__ __launch_bounds__(THREADS) void kl_fwd_topk_kernel(
     for (int u = 0; u < UNROLL; ++u) {
       const int c = c0 + u * THREADS + tid;
       if (c < sp.nvec) {
-        if (dstudent != nullptr) {   // a gradient sweep follows: leave the row to the caches
+        if constexpr (GRAD) {   // a gradient sweep follows: leave the row to the caches
           rs[u] = load16(sp_ + sp.head + (int64_t)c * EPV);
           rt[u] = load16(tp_ + sp.head + (int64_t)c * EPV);
         } else {
@@ -286,7 +286,7 @@ __global__ __launch_bounds__(THREADS) void kl_fwd_topk_kernel(
   const float none[1] = {0.f};
   topk_finish<T, THREADS, 1, kVecMaxLds>(tp_, sp, v, k, none, vhi, fm, has_nan, sh, row, tk_values,
                                          tk_idx32, tk_idx64, tk_probs, c1, l2t);
-  if (dstudent != nullptr)
+  if constexpr (GRAD)
     kl_grad_sweep<T, T, THREADS, UNROLL>(sp_, tp_, dstudent + row * (int64_t)v, sp, v, c1, l2s, l2t, mul);
 }
 
@@ -758,11 +758,16 @@ static int kl_topk_entry(const char* what, const void* student, const void* teac
     const dim3 grid((unsigned)n);
     // gradient (when asked for) is for an upstream gradient of 1
     const float mul = inv_temperature * ((reduction == FM_REDUCE_MEAN) ? 1.f / (float)n : 1.f);
-#define LAUNCH(T, TH)                                                                              \
-  hipLaunchKernelGGL((kl_fwd_topk_kernel<T, TH, 2>), grid, dim3(TH), lds, st,                      \
+#define LAUNCH_AS(T, TH, GRAD_)                                                                     \
+  hipLaunchKernelGGL((kl_fwd_topk_kernel<T, TH, 2, GRAD_>), grid, dim3(TH), lds, st,               \
                      static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t, \
                      row_kl, static_cast<T*>(topk_values), i32, i64, topk_probs,                   \
                      static_cast<T*>(dstudent), mul, (int)v, k, inv_temperature, vec_ok)
+#define LAUNCH(T, TH)                         \
+  do {                                        \
+    if (dstudent != nullptr) LAUNCH_AS(T, TH, true); \
+    else LAUNCH_AS(T, TH, false);             \
+  } while (0)
 #define BY_THREADS(T)                      \
   do {                                     \
     if (threads == 256) LAUNCH(T, 256);    \
@@ -774,6 +779,7 @@ static int kl_topk_entry(const char* what, const void* student, const void* teac
     else BY_THREADS(f16_t);
 #undef BY_THREADS
 #undef LAUNCH
+#undef LAUNCH_AS
     FM_CHECK_LAUNCH(what);
   }
   if (reduction != FM_REDUCE_NONE && loss != nullptr) {
