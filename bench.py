@@ -303,7 +303,7 @@ def make_workload(name, torch, L, dev):
                                          st), "fm_kl_loss_grad")
 
             def step():
-                both()      # forward: loss, and the gradient from a second sweep served by cache
+                both()      # forward: loss, and the gradient from a second sweep of each row
                 _check(L.fm_scale_inplace(gs.data_ptr(), one.data_ptr(), n * v, BF, st),
                        "fm_scale_inplace")   # backward: upstream gradient 1, nothing to move
 
@@ -312,7 +312,7 @@ def make_workload(name, torch, L, dev):
             w.dominant = "kl_loss_grad_wide_kernel<bf16,bf16,1024,2>"
             w.dominant_bytes = w.bytes = n * v * 6
             w.desc = (f"KL loss + gradient in one launch bf16 [{n},{v}], T=2, mean; HBM dataflow read s,t + "
-                      "write g = 6 B/logit pair (the second sweep of s,t is served by the memory-side cache)")
+                      "write g = 6 B/logit pair (each row is swept a second time right after the first, inside the launch)")
             w.rows = n
             return w
 

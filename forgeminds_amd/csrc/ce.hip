@@ -192,8 +192,8 @@ __global__ __launch_bounds__(THREADS) void ce_bwd_kernel(const T* __restrict__ l
 
 // Rows too wide for registers (or unaligned buffers), loss and gradient in ONE launch: the
 // streaming log-sum-exp, the workgroup merge, then a second sweep over the same row that writes
-// the gradient. The first sweep reads with ordinary (cached) loads so that the second finds
-// the row in the memory-side cache instead of HBM. dlogits may be the logits buffer itself:
+// the gradient. The second sweep follows the first at once, so a cache that still holds the
+// row serves it (the first sweep uses ordinary loads for that reason). dlogits may be the logits buffer itself:
 // every element is re-read by the thread that writes it.
 template <typename T, int THREADS, int UNROLL>
 __global__ __launch_bounds__(THREADS) void ce_loss_grad_wide_kernel(const T* logits,

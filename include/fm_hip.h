@@ -157,8 +157,8 @@ int fm_ce_bwd(const void* logits, const int64_t* labels, const float* lse, const
  * bytes per 16-bit logit instead of 2 + 2 + 2. dlogits may be the logits buffer itself
  * (the way the reference's KL writes its gradient into an owned student tensor,
  * kernels/kl.py:146-150, 157-160); lse may be NULL. Rows wider than 128 KiB (or unaligned
- * buffers) are swept twice inside the same launch, the second sweep served by the
- * memory-side cache. lse of ignored rows is written as 0 (those rows are not read). */
+ * buffers) are swept twice inside the same launch (the second sweep follows the first at
+ * once, while the rows in flight still fit the memory-side cache). lse of ignored rows is written as 0 (those rows are not read). */
 int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float* row_loss,
                     float* loss, float* n_valid, void* dlogits, int64_t n, int64_t v, int dtype,
                     int64_t ignore_index, int reduction, fm_stream_t stream);
@@ -185,8 +185,8 @@ int fm_kl_fwd(const void* student, const void* teacher, float* lse_s, float* lse
  * fm_kl_fwd's outputs plus dstudent = fm_kl_bwd's result for grad_out = 1 and
  * scale = 1/n (FM_REDUCE_MEAN) or 1 (FM_REDUCE_SUM). Rows of at most 64 KiB stay in
  * registers between the log-sum-exps and the store (4 + 2 bytes per pair of 16-bit logits
- * instead of 4 + 4 + 2); wider rows are swept twice inside the same launch, the second
- * sweep served by the memory-side cache. dstudent may be the student buffer itself when
+ * instead of 4 + 4 + 2); wider rows are swept twice inside the same launch (the second
+ * sweep follows the first at once, while the rows in flight fit the memory-side cache). dstudent may be the student buffer itself when
  * grad_dtype == dtype (kl.py:146-150, reuse=True); lse_s / lse_t may be NULL.
  * fm_scale_inplace applies an upstream gradient other than 1. */
 int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, float* lse_t,
@@ -207,7 +207,7 @@ int fm_kl_fwd_topk(const void* student, const void* teacher, float* lse_s, float
                    float inv_temperature, int reduction, fm_stream_t stream);
 
 /* fm_kl_fwd_topk that also writes the gradient of the student in the same launch (a second
- * sweep of the row, served by the memory-side cache, after the selection): dstudent [n, v] of
+ * sweep of the row after the selection): dstudent [n, v] of
  * dtype = fm_kl_bwd's result for grad_out = 1 and scale = 1/n (FM_REDUCE_MEAN) or 1
  * (FM_REDUCE_SUM), a buffer of its own. One launch for a whole distillation step (KL, its
  * gradient, the teacher's top-k). No counterpart in the reference (see fm_kl_fwd_topk). */
