@@ -18,13 +18,18 @@ namespace {
 constexpr int kMaxK = 8;
 
 // dst[s, :] = scale * src[order[s] / k, :],  scale = w[order[s]] if w else 1
+// A destination row is owned by `g` threads (a power of two up to 256: as many as the row has
+// 16-byte vectors), 256 / g rows per workgroup.
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void gather_kernel(const T* __restrict__ src,
                                                       const int32_t* __restrict__ order,
                                                       const float* __restrict__ w,
-                                                      T* __restrict__ dst, int d, int k) {
+                                                      T* __restrict__ dst, int64_t total, int d, int k,
+                                                      int g) {
   constexpr int EPV = Elem<T>::kVec;
-  const int64_t s = blockIdx.x;
+  const int rib = threadIdx.x / g, l = threadIdx.x % g;
+  const int64_t s = (int64_t)blockIdx.x * (256 / g) + rib;
+  if (s >= total) return;
   const int p = order[s];
   const int64_t t = p / k;
   const float scale = w != nullptr ? w[p] : 1.f;
@@ -32,19 +37,32 @@ __global__ __launch_bounds__(256) void gather_kernel(const T* __restrict__ src,
   T* dp = dst + s * (int64_t)d;
   if constexpr (VEC) {
     const int nvec = d / EPV;
-    for (int c = threadIdx.x; c < nvec; c += 256) {
-      u32x4 raw = load16(sp + c * EPV);
-      if (w != nullptr) {
-        float f[EPV];
-        Elem<T>::unpack(raw, f);
+    // four loads in flight per thread: a row is a few vectors per thread, and one load at a
+    // time leaves the memory system idle between a load and its store
+    for (int c0 = l; c0 < nvec; c0 += 4 * g) {
+      u32x4 raw[4];
 #pragma unroll
-        for (int e = 0; e < EPV; ++e) f[e] *= scale;
-        raw = Elem<T>::pack(f);
+      for (int u = 0; u < 4; ++u) {
+        const int c = c0 + u * g;
+        if (c < nvec) raw[u] = load16(sp + c * EPV);
       }
-      store16_stream(dp + c * EPV, raw);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = c0 + u * g;
+        if (c < nvec) {
+          if (w != nullptr) {
+            float f[EPV];
+            Elem<T>::unpack(raw[u], f);
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) f[e] *= scale;
+            raw[u] = Elem<T>::pack(f);
+          }
+          store16_stream(dp + c * EPV, raw[u]);
+        }
+      }
     }
   } else {
-    for (int j = threadIdx.x; j < d; j += 256) Elem<T>::store1(dp + j, Elem<T>::load1(sp + j) * scale);
+    for (int j = l; j < d; j += g) Elem<T>::store1(dp + j, Elem<T>::load1(sp + j) * scale);
   }
 }
 
@@ -168,14 +186,21 @@ int fm_moe_gather(const void* x, const int32_t* order, const float* scale, void*
   if (n == 0) return FM_OK;
   FM_CHECK_ARG(x && order && xs, "fm_moe_gather: NULL pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const dim3 grid((unsigned)(n * k));
+  const int64_t total = n * k;
 #define CALL(T)                                                                                  \
-  if (vec_ok<T>(d, x, xs))                                                                       \
-    hipLaunchKernelGGL((gather_kernel<T, true>), grid, dim3(256), 0, st, static_cast<const T*>(x), \
-                       order, scale, static_cast<T*>(xs), (int)d, k);                            \
-  else                                                                                           \
-    hipLaunchKernelGGL((gather_kernel<T, false>), grid, dim3(256), 0, st, static_cast<const T*>(x), \
-                       order, scale, static_cast<T*>(xs), (int)d, k)
+  {                                                                                              \
+    const bool vec = vec_ok<T>(d, x, xs);                                                        \
+    const int64_t units = vec ? d / Elem<T>::kVec : d;   /* loads a row takes */                  \
+    int g = 8;                                                                                   \
+    while (g < 256 && g < units) g *= 2;                                                         \
+    const dim3 grid((unsigned)((total + 256 / g - 1) / (256 / g)));                              \
+    if (vec)                                                                                     \
+      hipLaunchKernelGGL((gather_kernel<T, true>), grid, dim3(256), 0, st, static_cast<const T*>(x), \
+                         order, scale, static_cast<T*>(xs), total, (int)d, k, g);                \
+    else                                                                                         \
+      hipLaunchKernelGGL((gather_kernel<T, false>), grid, dim3(256), 0, st, static_cast<const T*>(x), \
+                         order, scale, static_cast<T*>(xs), total, (int)d, k, g);                \
+  }
   FM_BY_DTYPE(dtype, CALL);
 #undef CALL
   FM_CHECK_LAUNCH("fm_moe_gather");
