@@ -19,7 +19,7 @@
 
 namespace fm {
 
-constexpr int kCap = 1024;  // candidate slots in LDS
+constexpr int kCap = 1024;  // candidate slots in LDS (twice that for 1024-thread workgroups)
 constexpr int kMaxK = 512;
 
 __device__ __forceinline__ uint32_t key_of(float f) {
@@ -73,7 +73,8 @@ __device__ __forceinline__ int block_excl_scan(int v, int* smem, int nw, int* to
 }
 
 constexpr int kWorkCap = 2048;  // vectors that may be revisited in phase B
-constexpr int kSortFrom = 128;  // candidate counts above this are sorted instead of counted
+constexpr int kSortFrom = 128;  // candidate counts above this are sorted instead of counted ...
+constexpr int kRankSlots = 512; // ... when C * C > 256 * threads, so counting never sees more than this
 
 // Where the vector maxima of the streaming pass live.
 enum VecMax { kVecMaxNone = 0, kVecMaxRegs = 1, kVecMaxLds = 2 };
@@ -84,10 +85,14 @@ __device__ __forceinline__ uint32_t key_prefix(uint32_t key) {
   return p > 0xFFFFu ? 0xFFFFu : p;
 }
 
-template <int THREADS, int VMAX>
+// BIG doubles the candidate slots: for k above 256 the threshold of a 1024-thread workgroup
+// admits one to two thousand elements, which then still avoid the exact path. It is a separate
+// instantiation because it costs the ordinary case (k = 64: 280 against 190 us per launch).
+template <int THREADS, int VMAX, bool BIG = false>
 struct TopkShared {
-  unsigned long long ccomp[kCap];  // (key << 32) | ~index : larger is better
-  int crank[kCap];
+  static constexpr int kSlots = BIG ? 2 * kCap : kCap;
+  unsigned long long ccomp[kSlots];  // (key << 32) | ~index : larger is better
+  int crank[kRankSlots];   // counting ranks at most this many candidates (more are sorted)
   int work[VMAX ? kWorkCap : 1];
   int s_int[THREADS / 64];
   uint32_t s_tau[THREADS / 64];
@@ -112,11 +117,11 @@ __device__ __forceinline__ float fold_vector_max(const u32x4& raw) {
 // vector c's maximum for the whole row, padded with zeros to a multiple of four entries and
 // 8-byte aligned; with kVecMaxNone the row is walked a second time. Outputs go to row `orow` of the [rows, k] arrays;
 // `probs` (optional) receives exp2(x * c1 - lse2) of the selected elements.
-template <typename T, int THREADS, int NV, int VMAX>
+template <typename T, int THREADS, int NV, int VMAX, bool BIG = false>
 __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowSplit& sp, int v, int k,
                                             const float (&vmax)[NV], const uint16_t* vhi, float fm,
                                             bool has_nan,
-                                            TopkShared<THREADS, VMAX>& sh, int64_t orow,
+                                            TopkShared<THREADS, VMAX, BIG>& sh, int64_t orow,
                                             T* __restrict__ values, int32_t* __restrict__ idx32,
                                             int64_t* __restrict__ idx64, float* __restrict__ probs,
                                             float c1, float lse2) {
@@ -124,6 +129,7 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
   constexpr int NW = THREADS / 64;
   constexpr int ITERS = NV;
   constexpr uint32_t KMASK = KeyBits<T>::mask;
+  constexpr int CAP = TopkShared<THREADS, VMAX, BIG>::kSlots;
   unsigned long long* ccomp = sh.ccomp;
   int* crank = sh.crank;
   int* work = sh.work;
@@ -138,7 +144,7 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
 
   int C = 0;
   bool overflow = false;
-  if (v <= kCap) {
+  if (v <= CAP) {
     // short row: every element is a candidate
     for (int j = tid; j < v; j += THREADS)
       ccomp[j] = ((unsigned long long)key_of(Elem<T>::load1(rp + j)) << 32) | (uint32_t)(~j);
@@ -157,7 +163,7 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
     if (j > 64) {
       // no full wave can bound the k-th value from below (k beyond 63 per full wave): every
       // element would become a candidate, so the exact path is taken at once
-      C = kCap + 1;
+      C = CAP + 1;
     } else {
       // Only the bits a value of type T can set are searched (the masked key is a lower bound
       // of the key with nothing representable in between), two bits per step: three ballots
@@ -195,7 +201,7 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
       auto consider = [&](float f, int col) {
         if (take_of(f)) {
           const int slot = atomicAdd(&s_count, 1);
-          if (slot < kCap) ccomp[slot] = ((unsigned long long)key_of(f) << 32) | (uint32_t)(~col);
+          if (slot < CAP) ccomp[slot] = ((unsigned long long)key_of(f) << 32) | (uint32_t)(~col);
         }
       };
       auto scan_vec = [&](const u32x4& raw, int c) {
@@ -253,10 +259,10 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
       __syncthreads();
       C = s_count;
       __syncthreads();
-      if (overflow) C = kCap + 1;
+      if (overflow) C = CAP + 1;
 
     }
-    if (C > kCap) {
+    if (C > CAP) {
       // ---- exact path: k-th key by bitwise search over the whole row. Rows of up to RK vectors
       // per thread keep their (masked) keys in registers for the search; wider rows are
       // re-read once per key bit. Empty slots hold 0, which no predicate below accepts.

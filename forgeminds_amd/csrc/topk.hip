@@ -30,14 +30,14 @@ using namespace fm;
 
 namespace {
 
-template <typename T, int THREADS, int ITERS>
+template <typename T, int THREADS, int ITERS, bool BIG>
 __global__ __launch_bounds__(THREADS, (ITERS > 0 && ITERS <= 16 && THREADS == 1024) ? 8 : 1)
 void topk_kernel(const T* __restrict__ x, T* __restrict__ values, int32_t* __restrict__ idx32,
                  int64_t* __restrict__ idx64, int v, int k, bool vec_ok) {
   constexpr int EPV = Elem<T>::kVec;
   constexpr bool VMAX = ITERS > 0;   // vector maxima live in registers
   constexpr int NV = VMAX ? ITERS : 1;
-  __shared__ TopkShared<THREADS, VMAX ? kVecMaxRegs : kVecMaxNone> sh;
+  __shared__ TopkShared<THREADS, VMAX ? kVecMaxRegs : kVecMaxNone, BIG> sh;
 
   const int64_t row = blockIdx.x;
   const T* rp = x + row * (int64_t)v;
@@ -47,7 +47,7 @@ void topk_kernel(const T* __restrict__ x, T* __restrict__ values, int32_t* __res
   float vmax[NV];
   float fm = -INFINITY;
   bool has_nan = false;
-  if (v > kCap) {
+  if (v > TopkShared<THREADS, VMAX ? kVecMaxRegs : kVecMaxNone, BIG>::kSlots) {
     // ---- phase A: vector maxima and the thread's group maximum
     if constexpr (VMAX) {
 #pragma unroll
@@ -85,20 +85,20 @@ void topk_kernel(const T* __restrict__ x, T* __restrict__ values, int32_t* __res
 #pragma unroll
     for (int i = 0; i < NV; ++i) vmax[i] = 0.f;
   }
-  topk_finish<T, THREADS, NV, VMAX ? kVecMaxRegs : kVecMaxNone>(rp, sp, v, k, vmax, nullptr, fm, has_nan, sh,
+  topk_finish<T, THREADS, NV, VMAX ? kVecMaxRegs : kVecMaxNone, BIG>(rp, sp, v, k, vmax, nullptr, fm, has_nan, sh,
                                                                 row, values, idx32, idx64, nullptr, 0.f, 0.f);
 }
 
 // Variant that leaves a 16-bit key prefix of every vector's maximum in LDS instead of the
 // maxima in registers: few registers, so several workgroups share a compute unit and one
 // row's selection overlaps the next row's streaming read.
-template <typename T, int THREADS, int UNROLL>
+template <typename T, int THREADS, int UNROLL, bool BIG>
 __global__ __launch_bounds__(THREADS) void topk_lds_kernel(const T* __restrict__ x, T* __restrict__ values,
                                                            int32_t* __restrict__ idx32,
                                                            int64_t* __restrict__ idx64, int v, int k,
                                                            bool vec_ok) {
   constexpr int EPV = Elem<T>::kVec;
-  __shared__ TopkShared<THREADS, kVecMaxLds> sh;
+  __shared__ TopkShared<THREADS, kVecMaxLds, BIG> sh;
   extern __shared__ __align__(16) uint16_t vhi[];
   const int64_t row = blockIdx.x;
   const T* rp = x + row * (int64_t)v;
@@ -106,7 +106,7 @@ __global__ __launch_bounds__(THREADS) void topk_lds_kernel(const T* __restrict__
   const RowSplit sp = split_row<EPV>(row, v, vec_ok);
   float fm = -INFINITY;
   bool has_nan = false;
-  if (v > kCap) {
+  if (v > TopkShared<THREADS, kVecMaxLds, BIG>::kSlots) {
     {  // zero the padding of the last quad of prefixes
       const int p = ((sp.nvec + 3) & ~3) - 1 - tid;
       if (tid < 3 && p >= sp.nvec) vhi[p] = 0;
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(THREADS) void topk_lds_kernel(const T* __restrict__
     }
   }
   const float none[1] = {0.f};
-  topk_finish<T, THREADS, 1, kVecMaxLds>(rp, sp, v, k, none, vhi, fm, has_nan, sh, row, values, idx32, idx64,
+  topk_finish<T, THREADS, 1, kVecMaxLds, BIG>(rp, sp, v, k, none, vhi, fm, has_nan, sh, row, values, idx32, idx64,
                                          nullptr, 0.f, 0.f);
 }
 
@@ -372,11 +372,12 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
   constexpr int EPV = Elem<T>::kVec;
   const int64_t nvec = (v + EPV - 1) / EPV + 1;  // upper bound on whole vectors of any row
   const dim3 grid((unsigned)n);
-#define GO(TH, IT)                                                                               \
-  hipLaunchKernelGGL((topk_kernel<T, TH, IT>), grid, dim3(TH), 0, st, xp, vp, i32, i64, v, k, vec_ok)
-#define GOL(TH, UN)                                                                              \
-  hipLaunchKernelGGL((topk_lds_kernel<T, TH, UN>), grid, dim3(TH), (size_t)(nvec + 8) * 2, st, xp, vp, i32, \
-                     i64, v, k, vec_ok)
+#define GO(TH, IT, BIG_)                                                                         \
+  hipLaunchKernelGGL((topk_kernel<T, TH, IT, BIG_>), grid, dim3(TH), 0, st, xp, vp, i32, i64, v, k, vec_ok)
+#define GOL(TH, UN, BIG_)                                                                        \
+  hipLaunchKernelGGL((topk_lds_kernel<T, TH, UN, BIG_>), grid, dim3(TH), (size_t)(nvec + 8) * 2, st, xp, vp, \
+                     i32, i64, v, k, vec_ok)
+  const bool big = k > 256;               // twice the candidate slots (1024-thread forms only)
   int variant = fm_host::get_param(fm_host::P_TOPK_VARIANT);
   const bool forced = variant != 0;       // a forced variant also bypasses the wave-per-row kernel
   if (variant == 0) variant = nvec <= 3072 ? 1 : (nvec <= 12288 ? 2 : 3);
@@ -425,11 +426,17 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
 #undef GOW
   }
   else if (nvec > kLdsMaxVec) {
-    if (nvec <= 1024 * 32) GO(1024, 32);
-    else GO(1024, 0);
-  } else if (variant == 1) GOL(256, 4);
-  else if (variant == 2) GOL(512, 4);
-  else GOL(1024, 4);
+    if (nvec <= 1024 * 32) {
+      if (big) GO(1024, 32, true);
+      else GO(1024, 32, false);
+    } else {
+      if (big) GO(1024, 0, true);
+      else GO(1024, 0, false);
+    }
+  } else if (variant == 1) GOL(256, 4, false);
+  else if (variant == 2) GOL(512, 4, false);
+  else if (big) GOL(1024, 4, true);
+  else GOL(1024, 4, false);
 #undef GO
 #undef GOL
   return FM_OK;
