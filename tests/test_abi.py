@@ -67,4 +67,12 @@ def test_argument_validation_happens_before_any_launch(lib):
     # empty problems are a no-op that succeeds
     assert lib.fm_rmsnorm_fwd(None, None, None, None, 0, 8, 2, 2, 1e-6, None) == 0
     assert lib.fm_softmax_fwd(None, None, 0, 8, 2, None) == 0
+    assert lib.fm_softmax_bwd(None, None, None, 0, 8, 2, None) == 0
+    assert lib.fm_softmax_bwd(None, None, None, 4, 0, 2, None) == 1
+    # the one-launch distillation step validates like its parts
+    args = (None,) * 10
+    assert lib.fm_kl_loss_grad_topk(*args, 4, 8, 9, 2, 32, 1.0, 2, None) == 1          # k > v
+    assert lib.fm_kl_loss_grad_topk(*args, 4, 8, 2, 2, 32, 1.0, 0, None) == 1          # reduction none
+    assert b"sum or mean" in lib.fm_last_error()
+    assert lib.fm_kl_loss_grad_topk(*args, 4, 8, 2, 2, 32, 1.0, 2, None) == 1          # no gradient buffer
     assert lib.fm_rmsnorm_bwd_workspace(0, 8, 2) == 0
