@@ -319,16 +319,10 @@ def ce_loss_grad(logits2, labels, ignore_index: int, reduction: str, inplace: bo
     scalars = torch.empty(2, device=dev, dtype=torch.float32)
     dl = logits2 if inplace else torch.empty_like(logits2)
     with _guard(dev):
-        def call(out):
-            return lib().fm_ce_loss_grad(_ptr(logits2), _ptr(labels), buf[0].data_ptr(), buf[1].data_ptr(),
-                                         scalars[0:].data_ptr(), scalars[1:].data_ptr(), _ptr(out), n, v,
-                                         dtype_code(logits2.dtype), int(ignore_index), REDUCE[reduction],
-                                         _stream(logits2))
-        rc = call(dl)
-        if rc == 2 and inplace:     # rows too wide to be rewritten in place: a buffer of its own
-            dl = torch.empty_like(logits2)
-            rc = call(dl)
-        _check(rc, "fm_ce_loss_grad")
+        _check(lib().fm_ce_loss_grad(_ptr(logits2), _ptr(labels), buf[0].data_ptr(), buf[1].data_ptr(),
+                                     scalars[0:].data_ptr(), scalars[1:].data_ptr(), _ptr(dl), n, v,
+                                     dtype_code(logits2.dtype), int(ignore_index), REDUCE[reduction],
+                                     _stream(logits2)), "fm_ce_loss_grad")
     return scalars[0], dl, scalars[1], buf[1][:n]
 
 
@@ -370,7 +364,7 @@ def kl_fwd(s2, t2, inv_temperature: float, reduction: str):
 
 def kl_loss_grad(s2, t2, inv_temperature: float, reduction: str, grad_dtype, inplace: bool = False):
     """-> (loss fp32 scalar, dstudent [n, v], row_kl); the gradient is for an upstream gradient of 1
-    and lands in ``s2`` itself when ``inplace`` (same dtype, rows narrow enough)."""
+    and lands in ``s2`` itself when ``inplace`` and the gradient has the student's dtype."""
     _dense(s2, t2)
     n, v = s2.shape
     dev = s2.device
@@ -379,16 +373,10 @@ def kl_loss_grad(s2, t2, inv_temperature: float, reduction: str, grad_dtype, inp
     inplace = inplace and grad_dtype == s2.dtype
     g = s2 if inplace else torch.empty((n, v), device=dev, dtype=grad_dtype)
     with _guard(dev):
-        def call(out):
-            return lib().fm_kl_loss_grad(_ptr(s2), _ptr(t2), buf[0].data_ptr(), buf[1].data_ptr(),
-                                         buf[2].data_ptr(), _ptr(loss), _ptr(out), n, v,
-                                         dtype_code(s2.dtype), dtype_code(grad_dtype),
-                                         float(inv_temperature), REDUCE[reduction], _stream(s2))
-        rc = call(g)
-        if rc == 2 and inplace:     # rows too wide to be rewritten in place: a buffer of its own
-            g = torch.empty((n, v), device=dev, dtype=grad_dtype)
-            rc = call(g)
-        _check(rc, "fm_kl_loss_grad")
+        _check(lib().fm_kl_loss_grad(_ptr(s2), _ptr(t2), buf[0].data_ptr(), buf[1].data_ptr(),
+                                     buf[2].data_ptr(), _ptr(loss), _ptr(g), n, v, dtype_code(s2.dtype),
+                                     dtype_code(grad_dtype), float(inv_temperature), REDUCE[reduction],
+                                     _stream(s2)), "fm_kl_loss_grad")
     return loss, g, buf[2]
 
 

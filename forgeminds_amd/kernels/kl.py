@@ -252,7 +252,7 @@ def kl_distill_loss(hs: torch.Tensor, ht: torch.Tensor, w: torch.Tensor, teacher
 
     Same structure as the reference's ``kl.py:209-233``: the teacher head runs under
     ``no_grad``; one chunk of student logits exists at a time in the forward, and its gradient
-    is written over it (``reuse=True``, as in the reference) when the rows are narrow enough.
+    is written over it (``reuse=True``, as in the reference).
     """
     hs2 = hs.reshape(-1, hs.shape[-1])
     ht2 = ht.reshape(-1, ht.shape[-1])
