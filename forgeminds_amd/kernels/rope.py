@@ -89,8 +89,15 @@ def qk_norm_rope(x: torch.Tensor, w: torch.Tensor, cos: torch.Tensor, sin: torch
     if x.dim() != 4:
         raise ValueError(f"qk_norm_rope expects [B, T, H, D], got {tuple(x.shape)}")
     b, t, h, d = x.shape
-    if d % 2 != 0 or w.numel() != d or cos.shape != sin.shape or cos.shape[-2:] != (t, d // 2):
-        raise ValueError(f"qk_norm_rope: x {tuple(x.shape)}, w {tuple(w.shape)}, cos {tuple(cos.shape)} disagree")
+    if d % 2 != 0:
+        raise ValueError(f"qk_norm_rope rotates pairs of features, so the head dim must be even; got {d}")
+    need = t * (d // 2)
+    if w.numel() != d or cos.numel() < need or sin.numel() < need:
+        raise ValueError(f"qk_norm_rope: x {tuple(x.shape)}, w {tuple(w.shape)}, cos {tuple(cos.shape)}, "
+                         f"sin {tuple(sin.shape)} disagree")
+    # [T, D/2] or any shape whose first T * D/2 elements are that table (reference rope.py:231-238)
+    cos = cos.reshape(-1)[:need].reshape(t, d // 2)
+    sin = sin.reshape(-1)[:need].reshape(t, d // 2)
     ok_w = w.dtype == x.dtype or (w.dtype == torch.float32 and x.dtype in (torch.float16, torch.bfloat16))
     if d > MAX_HEAD_DIM or x.numel() == 0 or not ok_w or cos.dim() != 2 or cos.device != x.device:
         _note("qk_norm_rope shape")

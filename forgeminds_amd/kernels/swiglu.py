@@ -121,7 +121,7 @@ def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
 def swiglu_split(gate_up: torch.Tensor) -> torch.Tensor:
     """``silu(x[..., :h]) * x[..., h:]`` for a fused gate|up projection of width ``2h``."""
     if gate_up.dim() < 1 or gate_up.shape[-1] % 2 != 0:
-        raise ValueError(f"swiglu_split needs an even last dim, got {tuple(gate_up.shape)}")
+        raise ValueError(f"swiglu_split needs an even last dimension (gate|up), got {gate_up.shape[-1] if gate_up.dim() else 0}")
     if gate_up.numel() == 0:
         _note("swiglu_split empty")
         return fb.swiglu_split(gate_up)

@@ -522,6 +522,11 @@ def test_qk_norm_rope_surface_and_op_path():
     assert all(torch.allclose(a, b, rtol=1e-4, atol=1e-4) for a, b in zip(eager, ref))
     with pytest.raises(ValueError):
         kernels.qk_norm_rope(x[0], w, cos, sin)
+    # a broadcast-shaped table and a longer one give the bits of the [T, D/2] call
+    base = kernels.qk_norm_rope(x, w, cos, sin)
+    assert torch.equal(kernels.qk_norm_rope(x, w, cos.view(1, 9, 1, 32), sin.view(1, 9, 1, 32)), base)
+    pad = torch.randn(7, 32, device=DEV)
+    assert torch.equal(kernels.qk_norm_rope(x, w, torch.cat((cos, pad)), torch.cat((sin, pad))), base)
 
 
 def test_kl_div_logits_topk_autograd_and_wide_rows():

@@ -364,10 +364,26 @@ def test_out_of_path_names_keep_their_torch_expression():
     assert torch.allclose(kernels.swiglu(g, u), F.silu(g) * u, atol=2e-6)
     x = torch.randn(7, 16)
     assert torch.allclose(kernels.swiglu_split(x), F.silu(x[..., :8]) * x[..., 8:], atol=2e-6)
-    with pytest.raises(ValueError):
+    # messages the reference's tests match on (tests/test_kernels.py:209-220, test_edge_cases.py:129-139)
+    with pytest.raises(ValueError, match="even last dimension"):
         kernels.swiglu_split(torch.randn(3, 7))
-    q = kernels.qk_norm_rope(torch.randn(2, 5, 3, 8), torch.randn(8), torch.randn(5, 4), torch.randn(5, 4))
+    with pytest.raises(ValueError, match="must be even"):
+        kernels.qk_norm_rope(torch.randn(1, 8, 4, 63), torch.randn(63), torch.randn(8, 32), torch.randn(8, 32))
+    with pytest.raises((RuntimeError, ValueError)):
+        kernels.swiglu(torch.randn(4), torch.randn(5))
+    one = torch.randn(5, 2)
+    assert torch.allclose(kernels.swiglu_split(one), F.silu(one[..., :1]) * one[..., 1:], atol=1e-6)
+    xq, wq = torch.randn(2, 5, 3, 8), torch.randn(8)
+    cos, sin = torch.randn(5, 4), torch.randn(5, 4)
+    q = kernels.qk_norm_rope(xq, wq, cos, sin)
     assert q.shape == (2, 5, 3, 8)
+    # cos / sin: [T, D/2], a broadcast shape, or a longer table whose first T rows are used
+    # (reference kernels/rope.py:231-238)
+    assert torch.equal(kernels.qk_norm_rope(xq, wq, cos.view(1, 5, 1, 4), sin.view(1, 5, 1, 4)), q)
+    longer = torch.cat((cos, torch.randn(3, 4))), torch.cat((sin, torch.randn(3, 4)))
+    assert torch.equal(kernels.qk_norm_rope(xq, wq, *longer), q)
+    with pytest.raises(ValueError):
+        kernels.qk_norm_rope(xq, wq, cos[:4], sin[:4])
     o = kernels.newton_schulz(torch.randn(8, 16))
     assert o.shape == (8, 16)
 
