@@ -104,9 +104,9 @@ _SWS_OP = _ops.define("swiglu_split", _sws_impl,
 
 def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """``F.silu(gate) * up`` with fp32 math and one rounding."""
-    if gate.shape != up.shape:
-        raise ValueError(f"swiglu: gate {tuple(gate.shape)} and up {tuple(up.shape)} differ")
-    if gate.dtype != up.dtype or gate.numel() == 0 or gate.device != up.device:
+    # differing shapes go to the torch expression, which broadcasts or raises as torch does
+    # (reference kernels/swiglu.py:140-142, 291-297)
+    if gate.shape != up.shape or gate.dtype != up.dtype or gate.numel() == 0 or gate.device != up.device:
         _note("swiglu operands")
         return fb.swiglu(gate, up)
     if not fast_ok(gate, up):

@@ -371,6 +371,8 @@ def test_out_of_path_names_keep_their_torch_expression():
         kernels.qk_norm_rope(torch.randn(1, 8, 4, 63), torch.randn(63), torch.randn(8, 32), torch.randn(8, 32))
     with pytest.raises((RuntimeError, ValueError)):
         kernels.swiglu(torch.randn(4), torch.randn(5))
+    gb, ub = torch.randn(4, 8), torch.randn(8)            # broadcastable: the torch expression, as in the reference
+    assert torch.allclose(kernels.swiglu(gb, ub), F.silu(gb) * ub, atol=2e-6)
     one = torch.randn(5, 2)
     assert torch.allclose(kernels.swiglu_split(one), F.silu(one[..., :1]) * one[..., 1:], atol=1e-6)
     xq, wq = torch.randn(2, 5, 3, 8), torch.randn(8)
