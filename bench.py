@@ -590,9 +590,10 @@ def kbench_style(torch):
 
 # ---------------------------------------------------------------------------- CPU baseline
 def cpu_baseline(torch):
-    """The CPU oracle's CE forward + backward on a bounded sample of the headline workload."""
+    """The CPU oracle's CE forward + backward on the headline workload's own shape (all 8192 rows:
+    a few seconds of CPU work, bounded at 25 s)."""
     from oracle import oracle as O
-    rows, v = 1024, 32000
+    rows, v = 8192, 32000
     g = torch.Generator(device="cpu").manual_seed(1002)
     lg = (2 * torch.randn(rows, v, generator=g)).bfloat16()
     y = torch.randint(0, v, (rows,), generator=g)
@@ -609,8 +610,8 @@ def cpu_baseline(torch):
             break
     return {
         "value": round(rows * v * 6 / best / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-        "sample": f"oracle.cross_entropy fwd+bwd on {rows} of 8192 rows x {v} bf16 logits, "
-                  f"min of 3, {best * 1e3:.1f} ms, same 6 B/logit accounting",
+        "sample": f"oracle.cross_entropy fwd+bwd on all {rows} rows x {v} bf16 logits, "
+                  f"min of up to 3 passes, {best * 1e3:.1f} ms, same 6 B/logit accounting",
     }
 
 
