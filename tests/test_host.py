@@ -433,6 +433,44 @@ def test_layer_norm_torch_path_and_module():
     assert fm.nn.LayerNorm(8, bias=False).bias is None and fm.nn.LayerNorm(8, elementwise_affine=False).weight is None
 
 
+def test_swiglu_module_layouts_agree():
+    """fm.nn.SwiGLU (reference nn.py:150-217, tests/test_nn_blocks.py:118-157): the eager
+    expression, and the same answer from the stacked gate_up layout."""
+    torch.manual_seed(0)
+    mlp = fm.nn.SwiGLU(16, hidden=24)
+    x = torch.randn(5, 16)
+    ref = mlp.w2(F.silu(mlp.w1(x)) * mlp.w3(x))
+    assert torch.allclose(mlp(x), ref, atol=1e-6)
+    assert fm.nn.SwiGLU(8).hidden == 32 and "16 -> 24 -> 16" in repr(mlp)
+    stacked = mlp.to_split(inplace=False)
+    assert torch.allclose(stacked(x), ref, atol=1e-6)
+    assert sorted(stacked.state_dict()) == ["gate_up.weight", "w2.weight"]
+    assert hasattr(mlp, "w1") and not hasattr(mlp, "gate_up") and mlp.split is False    # original untouched
+    assert stacked.to_split() is stacked
+    assert mlp.to_split() is mlp and mlp.split is True and not hasattr(mlp, "w3")
+    assert torch.allclose(mlp(x), ref, atol=1e-6)
+    direct = fm.nn.SwiGLU(16, hidden=24, split=True)
+    direct.load_state_dict(stacked.state_dict())
+    assert torch.allclose(direct(x), ref, atol=1e-6)
+    with pytest.raises(ValueError):
+        fm.nn.SwiGLU(0)
+    with pytest.raises(ValueError):
+        fm.nn.SwiGLU(8, hidden=0)
+    lop = fm.nn.SwiGLU(8, 12, bias=True)
+    lop.w3.bias = None
+    with pytest.raises(ValueError, match="bias"):
+        lop.to_split()
+    assert kernels.patch(fm.nn.SwiGLU(8, 16)) is True
+
+
+def test_swiglu_module_gradcheck():
+    torch.manual_seed(0)
+    mlp = fm.nn.SwiGLU(8, hidden=12, bias=True).double()
+    x = torch.randn(2, 8, dtype=torch.float64, requires_grad=True)
+    assert torch.autograd.gradcheck(mlp, (x,))
+    assert torch.autograd.gradcheck(mlp.to_split(inplace=False), (x,))
+
+
 def test_layernorm_is_only_patched_on_request():
     ln = nn.LayerNorm(16)
     assert kernels.patch(ln) is False                           # reference tests/test_nn_blocks.py:170-172
