@@ -88,12 +88,16 @@ __device__ __forceinline__ uint32_t key_prefix(uint32_t key) {
 // BIG doubles the candidate slots: for k above 256 the threshold of a 1024-thread workgroup
 // admits one to two thousand elements, which then still avoid the exact path. It is a separate
 // instantiation because it costs the ordinary case (k = 64: 280 against 190 us per launch).
-template <int THREADS, int VMAX, bool BIG = false>
+// SMALL halves slots and work list instead: 11 KB of LDS per workgroup, so that fourteen
+// 128-thread workgroups share a compute unit (rows of a few thousand elements, k <= 64).
+enum TopkSize { kTopkNormal = 0, kTopkBig = 1, kTopkSmall = 2 };
+template <int THREADS, int VMAX, int SZ = kTopkNormal>
 struct TopkShared {
-  static constexpr int kSlots = BIG ? 2 * kCap : kCap;
+  static constexpr int kSlots = SZ == kTopkBig ? 2 * kCap : (SZ == kTopkSmall ? kCap / 2 : kCap);
+  static constexpr int kWork = SZ == kTopkSmall ? kWorkCap / 2 : kWorkCap;
   unsigned long long ccomp[kSlots];  // (key << 32) | ~index : larger is better
   int crank[kRankSlots];   // counting ranks at most this many candidates (more are sorted)
-  int work[VMAX ? kWorkCap : 1];
+  int work[VMAX ? kWork : 1];
   int s_int[THREADS / 64];
   uint32_t s_tau[THREADS / 64];
   int s_count, s_nwork;
@@ -117,7 +121,7 @@ __device__ __forceinline__ float fold_vector_max(const u32x4& raw) {
 // vector c's maximum for the whole row, padded with zeros to a multiple of four entries and
 // 8-byte aligned; with kVecMaxNone the row is walked a second time. Outputs go to row `orow` of the [rows, k] arrays;
 // `probs` (optional) receives exp2(x * c1 - lse2) of the selected elements.
-template <typename T, int THREADS, int NV, int VMAX, bool BIG = false>
+template <typename T, int THREADS, int NV, int VMAX, int BIG = kTopkNormal>
 __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowSplit& sp, int v, int k,
                                             const float (&vmax)[NV], const uint16_t* vhi, float fm,
                                             bool has_nan,
@@ -130,6 +134,7 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
   constexpr int ITERS = NV;
   constexpr uint32_t KMASK = KeyBits<T>::mask;
   constexpr int CAP = TopkShared<THREADS, VMAX, BIG>::kSlots;
+  constexpr int WORK = TopkShared<THREADS, VMAX, BIG>::kWork;
   unsigned long long* ccomp = sh.ccomp;
   int* crank = sh.crank;
   int* work = sh.work;
@@ -219,7 +224,7 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
         // B1: vectors that can hold a candidate go to the work list
         auto list = [&](int c) {
           const int slot = atomicAdd(&s_nwork, 1);
-          if (slot < kWorkCap) work[slot] = c;
+          if (slot < WORK) work[slot] = c;
         };
         if constexpr (VMAX == kVecMaxRegs) {
   #pragma unroll
@@ -241,7 +246,7 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
         }
         __syncthreads();
         const int nwork = s_nwork;
-        overflow = nwork > kWorkCap;
+        overflow = nwork > WORK;
         // B2: revisit only those vectors, spread over the whole workgroup
         if (!overflow) {
           for (int w = tid; w < nwork; w += THREADS) {

@@ -30,7 +30,7 @@ using namespace fm;
 
 namespace {
 
-template <typename T, int THREADS, int ITERS, bool BIG>
+template <typename T, int THREADS, int ITERS, int BIG>
 __global__ __launch_bounds__(THREADS, (ITERS > 0 && ITERS <= 16 && THREADS == 1024) ? 8 : 1)
 void topk_kernel(const T* __restrict__ x, T* __restrict__ values, int32_t* __restrict__ idx32,
                  int64_t* __restrict__ idx64, int v, int k, bool vec_ok) {
@@ -92,7 +92,7 @@ void topk_kernel(const T* __restrict__ x, T* __restrict__ values, int32_t* __res
 // Variant that leaves a 16-bit key prefix of every vector's maximum in LDS instead of the
 // maxima in registers: few registers, so several workgroups share a compute unit and one
 // row's selection overlaps the next row's streaming read.
-template <typename T, int THREADS, int UNROLL, bool BIG>
+template <typename T, int THREADS, int UNROLL, int BIG>
 __global__ __launch_bounds__(THREADS) void topk_lds_kernel(const T* __restrict__ x, T* __restrict__ values,
                                                            int32_t* __restrict__ idx32,
                                                            int64_t* __restrict__ idx64, int v, int k,
@@ -361,6 +361,9 @@ __global__ __launch_bounds__(64) void topk_wave_kernel(const T* __restrict__ x, 
 
 // widest row (in 16-byte vectors) whose key prefixes fit the LDS budget
 constexpr int kLdsMaxVec = 20480;
+// largest k the 128-thread form takes: the threshold of two full waves then still leaves the
+// candidates within its 512 slots
+constexpr int kSmallMaxK = 72;
 
 template <typename T>
 int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, int index_bits,
@@ -402,6 +405,10 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
       }
       variant = pick;
     }
+    // Rows of up to 48 KiB with a small k are bound by the latency of the phases after the
+    // read, not by the read: two waves per row and half the LDS put fourteen rows on a compute
+    // unit instead of eight (1.2-1.8x on rows of 2-24 K elements; even by 64 KiB rows).
+    if (whole <= 3072 && k <= kSmallMaxK) variant = 4;
   }
   if (v <= kWaveMaxV && !forced) {       // short rows: a wave per row
     int epl = 1;
@@ -433,7 +440,8 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
       if (big) GO(1024, 0, true);
       else GO(1024, 0, false);
     }
-  } else if (variant == 1) GOL(256, 4, false);
+  } else if (variant == 4) GOL(128, 4, kTopkSmall);
+  else if (variant == 1) GOL(256, 4, false);
   else if (variant == 2) GOL(512, 4, false);
   else if (big) GOL(1024, 4, true);
   else GOL(1024, 4, false);

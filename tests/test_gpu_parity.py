@@ -610,6 +610,48 @@ def test_topk_ties_nans_zeros_and_degenerate_rows():
     assert torch.equal(run(x, 4), O.topk(x, 4)[1])
 
 
+def test_topk_two_wave_rows():
+    """Rows of 2-24 K elements with k <= 72 take the 128-thread form (512 candidate slots, half
+    the work list): random rows around its bounds, then inputs that overflow its slots or its
+    work list and fall to the exact path, NaN / -inf rows, and unaligned rows."""
+    g = gen(1012)
+
+    def run(t, k):
+        _, i = _hip.topk(t.to(DEV), k, torch.int64)
+        return i.cpu()
+    for dt, n, v, ks in ((BF16, 40, 2049, (1, 64, 72, 73)), (F16, 9, 8191, (8, 72)), (BF16, 7, 24576, (1, 33, 72)),
+                         (F32, 12, 2304, (2, 72)), (F32, 6, 12288, (64, 72, 73)), (BF16, 5, 24584, (72,)),
+                         (F32, 4, 12290, (64,)), (BF16, 300, 4096, (64,))):
+        x = (3 * torch.randn(n, v, generator=g)).to(dt)
+        for k in ks:
+            vals, idx = _hip.topk(x.to(DEV), k, torch.int32)
+            ov, oi = O.topk(x, k)
+            assert torch.equal(idx.cpu().long(), oi) and torch.equal(vals.cpu(), ov), (dt, v, k)
+    # every element equal, few distinct values, one vector in each group of eight holding the
+    # maximum (the work list sees every vector), a row of NaNs, -inf with a few finite values
+    for dt in (BF16, F32):
+        for v in (4096, 9000, 20000):
+            z = torch.full((3, v), 0.25, dtype=dt)
+            assert torch.equal(run(z, 72), torch.arange(72).expand(3, 72))
+            x = torch.randint(0, 4, (5, v), generator=g).to(dt)
+            assert torch.equal(run(x, 64), O.topk(x, 64)[1]), (dt, v)
+            x = torch.randn(4, v, generator=g).to(dt)
+            x[:, ::8] = 9.0
+            assert torch.equal(run(x, 50), O.topk(x, 50)[1]), (dt, v)
+            x = torch.randn(4, v, generator=g).to(dt)
+            x[0] = float("nan")
+            x[1] = float("-inf")
+            x[1, 5::1000] = 1.0
+            x[2, 3::5] = float("nan")
+            x[3, ::2] = -0.0
+            x[3, 1::2] = 0.0
+            for k in (1, 20, 72):
+                assert torch.equal(run(x, k), O.topk(x, k)[1]), (dt, v, k)
+    base = (3 * torch.randn(1 + 6 * 5003, generator=g)).to(BF16).to(DEV)
+    x = base[1:].view(6, 5003)                                        # rows start 2 bytes off 16-byte alignment
+    assert torch.equal(run(x, 40), O.topk(x.cpu(), 40)[1])
+
+
 def test_topk_unaligned_rows():
     g = gen(12)
     for dt, v in ((BF16, 50257), (F32, 32001), (F16, 4099)):
