@@ -20,6 +20,7 @@ const char* const kParamNames[fm_host::P_COUNT] = {
     "norm_fwd_blocks_per_cu",
     "ce_rows_max_v",
     "norm_wide_min_vec",
+    "rows_vec_max",
 };
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cus[kMaxDevices];

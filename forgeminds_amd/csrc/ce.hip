@@ -530,6 +530,135 @@ __global__ __launch_bounds__(256) void ce_rows_kernel(const T* logits, const int
   }
 }
 
+// The same lane groups with 16-byte accesses, for rows that are a whole number of aligned
+// vectors: lane t of a row's TPR lanes holds vectors t, t + TPR, ... packed, and unpacks them
+// once per pass (maximum, sum, gradient). The gradient may overwrite the logits: the label's
+// logit is taken from the registers, and a lane stores only what it loaded.
+template <typename T, int TPR, int ITERS, bool LOSS, bool GRAD>
+__global__ __launch_bounds__(256) void ce_vrows_kernel(const T* logits, const int64_t* __restrict__ labels,
+                                                       const float* __restrict__ n_valid,
+                                                       const float* __restrict__ grad_out,
+                                                       float* __restrict__ lse, float* __restrict__ row_loss,
+                                                       T* dlogits, int64_t n, int v, int64_t ignore_index) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int RPB = 256 / TPR;
+  const int tid = threadIdx.x;
+  const int rib = tid / TPR;
+  const int t = tid % TPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + rib;
+  const bool valid = row < n;
+  const int64_t base = row * (int64_t)v;
+  const int nvec = v / EPV;
+  const int64_t y64 = valid ? labels[row] : ignore_index;
+  const bool ignored = y64 == ignore_index;
+  const int y = (y64 >= 0 && y64 < v) ? (int)y64 : -1;
+  // an ignored row of the gradient-only form is not read at all
+  const bool read = valid && (LOSS || !ignored);
+  u32x4 r[ITERS];
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * TPR + t;
+    if (read && c < nvec) r[i] = load16_stream(logits + base + (int64_t)c * EPV);
+  }
+  float m = kNegBig;
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    if (read && i * TPR + t < nvec) {
+      float f[EPV];
+      Elem<T>::unpack(r[i], f);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) m = fmaxf(m, f[e] * kLog2e);
+    }
+  }
+  m = group_reduce<TPR, OpMax>(m);
+  // a NaN anywhere must reach the whole row: fmaxf drops it, so it is carried in the sum
+  float ssum = 0.f;
+  float ylogit2 = 0.f;          // the label's logit (times log2 e), found among the lane's elements
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * TPR + t;
+    if (read && c < nvec) {
+      float f[EPV];
+      Elem<T>::unpack(r[i], f);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        const float z = f[e] * kLog2e;
+        if (LOSS && c * EPV + e == y) ylogit2 = z;
+        ssum += fast_exp2(z - m);
+      }
+    }
+  }
+  ssum = group_reduce<TPR, OpSum>(ssum);
+  const float l2 = m + fast_log2(ssum);
+  if constexpr (LOSS) {
+    ylogit2 = group_reduce<TPR, OpSum>(ylogit2);     // one lane holds it, the others add 0
+    if (valid && t == 0) {
+      const float l = l2 * kLn2;
+      if (lse != nullptr) lse[row] = l;
+      row_loss[row] = ignored ? 0.f : (y >= 0 ? l - ylogit2 * kLn2 : __builtin_nanf(""));
+    }
+  }
+  if constexpr (GRAD) {
+    const float scale = (grad_out != nullptr ? *grad_out : 1.f) / (n_valid != nullptr ? *n_valid : 1.f);
+    const float inv = 1.f / ssum;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = i * TPR + t;
+      if (valid && c < nvec) {
+        float f[EPV], o[EPV];
+        if (!ignored) Elem<T>::unpack(r[i], f);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+          float p = ignored ? 0.f : fast_exp2(f[e] * kLog2e - m) * inv;
+          if (c * EPV + e == y && !ignored) p -= 1.f;
+          o[e] = ignored ? 0.f : p * scale;
+        }
+        store16_stream(dlogits + base + (int64_t)c * EPV, Elem<T>::pack(o));
+      }
+    }
+  }
+}
+
+// Widest row, in 16-byte vectors, of the vector lane-group kernel (tunable downwards with
+// "rows_vec_max"; the forward alone takes twice the width of the forms that write a gradient).
+constexpr int kVRowsMaxVec = 512;
+
+bool vrows_fits(int v, int esize, bool bf16, const void* logits, const void* dlogits, bool loss, bool grad) {
+  const int epv = 16 / esize;
+  int lim = fm_host::get_param(fm_host::P_ROWS_VEC_MAX);
+  // eight vectors per lane only pay for bf16 (the other types then run at a quarter of the occupancy)
+  const int top = loss && !grad && esize == 2 && bf16 ? kVRowsMaxVec : kVRowsMaxVec / 2;
+  if (lim <= 0 || lim > top) lim = top;
+  return v % epv == 0 && v / epv <= lim && fm_host::aligned16(logits) && (!grad || fm_host::aligned16(dlogits));
+}
+
+template <typename T, bool LOSS, bool GRAD>
+bool launch_vrows(const void* logits, const int64_t* labels, const float* n_valid, const float* grad_out,
+                  float* lse, float* row_loss, void* dlogits, int64_t n, int v, int64_t ignore_index,
+                  hipStream_t st) {
+  constexpr int EPV = Elem<T>::kVec;
+  if (!vrows_fits(v, (int)sizeof(T), std::is_same<T, bf16_t>::value, logits, dlogits, LOSS, GRAD)) return false;
+  // four vectors a lane where the row has them: a wave then keeps 4 KiB in flight, and narrow
+  // rows share it (a 512-element bf16 row takes 16 lanes, not 64)
+  const int nvec = v / EPV;
+  int tpr = 4;
+  while (tpr < 64 && tpr * 4 < nvec) tpr *= 2;
+  int iters = 1;
+  while (tpr * iters < nvec) iters *= 2;
+  const dim3 grid((unsigned)((n + 256 / tpr - 1) / (256 / tpr)));
+#define GOV(TPR_, IT_)                                                                              \
+  if (tpr == TPR_ && iters == IT_) {                                                                \
+    hipLaunchKernelGGL((ce_vrows_kernel<T, TPR_, IT_, LOSS, GRAD>), grid, dim3(256), 0, st,         \
+                       static_cast<const T*>(logits), labels, n_valid, grad_out, lse, row_loss,     \
+                       static_cast<T*>(dlogits), n, v, ignore_index);                               \
+    return true;                                                                                    \
+  }
+  GOV(4, 1) GOV(4, 2) GOV(4, 4) GOV(8, 4) GOV(16, 4) GOV(32, 4) GOV(64, 4)
+  if constexpr (std::is_same<T, bf16_t>::value && LOSS && !GRAD) { GOV(64, 8) }
+#undef GOV
+  return false;
+}
+
 // rows of up to 1024 logits go to ce_rows_kernel; returns false for wider rows
 // Widest row the lane-group kernel takes (tunable downwards with "ce_rows_max_v").
 inline int rows_max_v() {
@@ -541,6 +670,8 @@ template <typename T, bool LOSS, bool GRAD>
 bool launch_rows(const void* logits, const int64_t* labels, const float* n_valid, const float* grad_out,
                  float* lse, float* row_loss, void* dlogits, int64_t n, int v, int64_t ignore_index,
                  hipStream_t st) {
+  if (launch_vrows<T, LOSS, GRAD>(logits, labels, n_valid, grad_out, lse, row_loss, dlogits, n, v, ignore_index, st))
+    return true;
   if (v > rows_max_v()) return false;
   // fp32 gradients of rows past 512 classes go faster through the workgroup-per-row kernels
   if (GRAD && sizeof(T) == 4 && v > 512) return false;
@@ -571,7 +702,8 @@ template <typename T>
 int launch_fwd(const void* logits, const int64_t* labels, float* lse, float* row_loss, int64_t n,
                int v, int64_t ignore_index, bool vec_ok, hipStream_t st) {
   const T* lp = static_cast<const T*>(logits);
-  const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 512, 4);
+  // the forward alone keeps 256 threads up to 24 KiB rows (16 KiB rows: 50 against 65 us per 256 MiB)
+  const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 512, 4, 24 * 1024);
   const dim3 grid((unsigned)n);
 #define LAUNCH(TH, UN)                                                                          \
   hipLaunchKernelGGL((ce_fwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, lp, labels, lse, row_loss, \
@@ -677,7 +809,8 @@ int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float
   hipStream_t st = static_cast<hipStream_t>(stream);
   const int esize = dtype == FM_F32 ? 4 : 2;
   const int64_t nvec = v / (16 / esize);
-  if (n > 0 && v <= rows_max_v() && !(esize == 4 && v > 512)) {   // narrow rows: lane groups, any alignment, in place allowed
+  if (n > 0 && (vrows_fits((int)v, esize, dtype == FM_BF16, logits, dlogits, true, true) ||
+                (v <= rows_max_v() && !(esize == 4 && v > 512)))) {   // narrow rows: lane groups, in place allowed
     const bool mean_ = reduction == FM_REDUCE_MEAN;
     if (mean_) {
       hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(1024), 0, st, labels, n, ignore_index, n_valid);

@@ -106,10 +106,11 @@ namespace fm_host {
 // in flight. `pref_threads` is the per-kernel default (read-only kernels do best with 512
 // threads on 64 KB rows, kernels that also write with 1024); both can be overridden for sweeps.
 struct VocabShape { int threads, unroll; };
-inline VocabShape vocab_shape(int64_t v, int esize, int pref_threads, int pref_unroll) {
+inline VocabShape vocab_shape(int64_t v, int esize, int pref_threads, int pref_unroll,
+                              int64_t small_below = 16 * 1024) {
   VocabShape s{pref_threads, pref_unroll};
   const int64_t bytes = v * esize;
-  if (bytes < 16 * 1024) s.threads = 256;
+  if (bytes < small_below) s.threads = 256;
   else if (bytes < 48 * 1024 && s.threads > 512) s.threads = 512;
   const int t = get_param(P_VOCAB_THREADS);
   if (t == 256 || t == 512 || t == 1024) s.threads = t;

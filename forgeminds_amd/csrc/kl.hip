@@ -647,12 +647,153 @@ __global__ __launch_bounds__(256) void kl_rows_kernel(const T* student, const T*
   }
 }
 
+// The same lane groups with 16-byte accesses, for rows that are a whole number of aligned
+// vectors: lane t of a row's TPR lanes keeps vectors t, t + TPR, ... of both rows packed and
+// unpacks them once per pass. The gradient may overwrite the student (a lane stores only what it
+// loaded).
+template <typename T, typename GT, int TPR, int ITERS, bool LOSS, bool GRAD>
+__global__ __launch_bounds__(256) void kl_vrows_kernel(const T* student, const T* __restrict__ teacher,
+                                                       float* lse_s, float* lse_t,
+                                                       float* __restrict__ row_kl,
+                                                       const float* __restrict__ grad_out,
+                                                       int grad_per_row, GT* dstudent, int64_t n, int v,
+                                                       float inv_temp, float mul) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int RPB = 256 / TPR;
+  const int tid = threadIdx.x;
+  const int rib = tid / TPR;
+  const int t = tid % TPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + rib;
+  const bool valid = row < n;
+  const int64_t base = row * (int64_t)v;
+  const int nvec = v / EPV;
+  const float c1 = kLog2e * inv_temp;
+  u32x4 rs[ITERS], rt[ITERS];
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * TPR + t;
+    if (valid && c < nvec) {
+      rs[i] = load16_stream(student + base + (int64_t)c * EPV);
+      rt[i] = load16_stream(teacher + base + (int64_t)c * EPV);
+    }
+  }
+  float l2s, l2t;
+  if constexpr (LOSS) {
+    float ms = kNegBig, mt = kNegBig;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      if (valid && i * TPR + t < nvec) {
+        float zs[EPV], zt[EPV];
+        Elem<T>::unpack(rs[i], zs);
+        Elem<T>::unpack(rt[i], zt);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) { ms = fmaxf(ms, zs[e] * c1); mt = fmaxf(mt, zt[e] * c1); }
+      }
+    }
+    ms = group_reduce<TPR, OpMax>(ms);
+    mt = group_reduce<TPR, OpMax>(mt);
+    float ds = 0.f, dt = 0.f, a = 0.f;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      if (valid && i * TPR + t < nvec) {
+        float zs[EPV], zt[EPV];
+        Elem<T>::unpack(rs[i], zs);
+        Elem<T>::unpack(rt[i], zt);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+          const float x = zs[e] * c1, y = zt[e] * c1;
+          ds += fast_exp2(x - ms);
+          const float et = fast_exp2(y - mt);
+          dt += et;
+          a += et * (y - x);
+        }
+      }
+    }
+    ds = group_reduce<TPR, OpSum>(ds);
+    dt = group_reduce<TPR, OpSum>(dt);
+    a = group_reduce<TPR, OpSum>(a);
+    l2s = ms + fast_log2(ds);
+    l2t = mt + fast_log2(dt);
+    if (valid && t == 0) {
+      if (lse_s != nullptr) lse_s[row] = l2s * kLn2;
+      if (lse_t != nullptr) lse_t[row] = l2t * kLn2;
+      row_kl[row] = (a / dt - l2t + l2s) * kLn2;
+    }
+  } else {
+    l2s = valid ? lse_s[row] * kLog2e : 0.f;
+    l2t = valid ? lse_t[row] * kLog2e : 0.f;
+  }
+  if constexpr (GRAD) {
+    float g = mul;
+    if (grad_out != nullptr && valid) g *= grad_per_row ? grad_out[row] : grad_out[0];
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = i * TPR + t;
+      if (valid && c < nvec) {
+        float zs[EPV], zt[EPV], o[EPV];
+        Elem<T>::unpack(rs[i], zs);
+        Elem<T>::unpack(rt[i], zt);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] = (fast_exp2(zs[e] * c1 - l2s) - fast_exp2(zt[e] * c1 - l2t)) * g;
+        GT* dst = dstudent + base + (int64_t)c * EPV;
+        if constexpr (sizeof(GT) == sizeof(T)) {
+          store16_stream(dst, Elem<GT>::pack(o));
+        } else {  // fp32 gradient next to 16-bit logits: two 16-byte stores
+          static_assert(sizeof(GT) == 4 && EPV == 8, "gradient is the logits' dtype or fp32");
+          float lo[4] = {o[0], o[1], o[2], o[3]}, hi[4] = {o[4], o[5], o[6], o[7]};
+          store16_stream(dst, Elem<float>::pack(lo));
+          store16_stream(dst + 4, Elem<float>::pack(hi));
+        }
+      }
+    }
+  }
+}
+
+// Widest row, in 16-byte vectors, of the vector lane-group kernel (tunable downwards with
+// "rows_vec_max").
+constexpr int kVRowsMaxVec = 256;
+
+template <typename T, typename GT, bool LOSS, bool GRAD>
+bool launch_vrows(const void* student, const void* teacher, float* lse_s, float* lse_t, float* row_kl,
+                  const float* grad_out, int grad_per_row, void* dstudent, int64_t n, int v, float inv_temp,
+                  float mul, hipStream_t st) {
+  constexpr int EPV = Elem<T>::kVec;
+  int lim = fm_host::get_param(fm_host::P_ROWS_VEC_MAX);
+  if (lim <= 0 || lim > kVRowsMaxVec) lim = kVRowsMaxVec;
+  if (v % EPV != 0 || v / EPV > lim || !fm_host::aligned16(student) || !fm_host::aligned16(teacher) ||
+      (GRAD && !fm_host::aligned16(dstudent)))
+    return false;
+  // two vectors of each row a lane where the rows have them: a wave then keeps 4 KiB in
+  // flight, and narrow rows share it
+  const int nvec = v / EPV;
+  int tpr = 4;
+  while (tpr < 64 && tpr * 2 < nvec) tpr *= 2;
+  int iters = 1;
+  while (tpr * iters < nvec) iters *= 2;
+  const dim3 grid((unsigned)((n + 256 / tpr - 1) / (256 / tpr)));
+#define GOV(TPR_, IT_)                                                                             \
+  if (tpr == TPR_ && iters == IT_) {                                                               \
+    hipLaunchKernelGGL((kl_vrows_kernel<T, GT, TPR_, IT_, LOSS, GRAD>), grid, dim3(256), 0, st,    \
+                       static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t, \
+                       row_kl, grad_out, grad_per_row, static_cast<GT*>(dstudent), n, v, inv_temp, mul); \
+    return true;                                                                                   \
+  }
+  GOV(4, 1) GOV(4, 2) GOV(8, 2) GOV(16, 2) GOV(32, 2) GOV(64, 2) GOV(64, 4)
+#undef GOV
+  return false;
+}
+
 constexpr int kRowsMaxV = 1024;
+// widest row either lane-group kernel can take (the vector form, fp16 / bf16)
+constexpr int kRowsReach = kVRowsMaxVec * 8 > kRowsMaxV ? kVRowsMaxVec * 8 : kRowsMaxV;
 
 template <typename T, typename GT, bool LOSS, bool GRAD>
 bool launch_rows(const void* student, const void* teacher, float* lse_s, float* lse_t, float* row_kl,
                  const float* grad_out, int grad_per_row, void* dstudent, int64_t n, int v, float inv_temp,
                  float mul, hipStream_t st) {
+  if (launch_vrows<T, GT, LOSS, GRAD>(student, teacher, lse_s, lse_t, row_kl, grad_out, grad_per_row, dstudent,
+                                      n, v, inv_temp, mul, st))
+    return true;
   if (v > kRowsMaxV) return false;
   const int tpr = v <= 16 * 16 ? 16 : 64;
   int iters = 1;
@@ -704,7 +845,7 @@ int fm_kl_fwd(const void* student, const void* teacher, float* lse_s, float* lse
   FM_CHECK_ARG(n == 0 || (student && teacher && lse_s && lse_t && row_kl), "fm_kl_fwd: NULL pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
   bool narrow = false;
-  if (n > 0 && v <= kRowsMaxV) {
+  if (n > 0 && v <= kRowsReach) {
 #define CALL(T, GT) \
   narrow = launch_rows<T, GT, true, false>(student, teacher, lse_s, lse_t, row_kl, nullptr, 0, nullptr, n, \
                                            (int)v, inv_temperature, 0.f, st)
@@ -824,7 +965,7 @@ int fm_kl_bwd(const void* student, const void* teacher, const float* lse_s, cons
   if (n == 0) return FM_OK;
   FM_CHECK_ARG(student && teacher && lse_s && lse_t && dstudent, "fm_kl_bwd: NULL pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (v <= kRowsMaxV) {
+  if (v <= kRowsReach) {
     bool narrow = false;
 #define CALL(T, GT)                                                                                 \
   narrow = launch_rows<T, GT, false, true>(student, teacher, const_cast<float*>(lse_s),             \
@@ -869,7 +1010,7 @@ int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, floa
   const float scale = (reduction == FM_REDUCE_MEAN && n > 0) ? 1.f / (float)n : 1.f;
   const int esize = dtype == FM_F32 ? 4 : 2;
   const int64_t nvec = v / (16 / esize);
-  if (n > 0 && v <= kRowsMaxV) {   // narrow rows: lane groups, any alignment, in place allowed
+  if (n > 0 && v <= kRowsReach) {   // narrow rows: lane groups, in place allowed
     bool narrow = false;
 #define CALL(T, GT)                                                                                  \
   narrow = launch_rows<T, GT, true, true>(student, teacher, lse_s, lse_t, row_kl, nullptr, 0, dstudent, n, \

@@ -245,7 +245,11 @@ def test_layernorm_determinism_unaligned_and_empty():
 CE_CASES = [(512, 32000, BF16), (7, 50257, BF16), (5, 1000, F32), (4, 7, F16), (9, 16, F32),
             (3, 128256, BF16), (6, 32001, F32), (33, 4096, F16), (2, 1, F32), (64, 50257, F32),
             (1000, 100, BF16), (300, 257, F16), (50, 1024, F32), (70, 33, BF16), (129, 600, BF16),
-            (300, 512, F32), (40, 513, F32)]
+            (300, 512, F32), (40, 513, F32),
+            # rows that are whole aligned 16-byte vectors: every lane-group shape of the vector form
+            (257, 24, BF16), (130, 64, BF16), (99, 128, F16), (65, 256, BF16), (300, 512, BF16),
+            (50, 1024, BF16), (18, 1000, BF16), (37, 2048, BF16), (21, 4096, BF16), (37, 2048, F16),
+            (21, 1536, F16), (33, 96, F32), (19, 2048, F32), (1025, 8, F32), (23, 2040, BF16)]
 
 
 @pytest.mark.parametrize("n,v,dt", CE_CASES)
@@ -314,6 +318,52 @@ def test_ce_loss_and_gradient_in_one_pass(n, v, dt, reduction):
     assert_close_lowp(dl, dl3.float().cpu(), dt, "vs two-pass", ulps=2.0, cancel=cancel)
 
 
+def test_ce_kl_vector_rows_agree_with_the_scalar_form():
+    """Narrow rows of whole aligned vectors take 16-byte loads; the same rows one element per
+    load (the form for other widths and alignments, forced here through the tuning knob) must
+    give the same answers, special values included."""
+    g = gen(1040)
+    for dt, v in ((BF16, 512), (F16, 1024), (F32, 256), (BF16, 2048)):
+        n = 37
+        lg = (2 * torch.randn(n, v, generator=g)).to(dt)
+        lg[0, 5] = float("nan")
+        lg[1] = float("-inf")
+        lg[1, 7] = 1.0
+        lg[2, 3] = float("inf")
+        y = torch.randint(0, v, (n,), generator=g)
+        y[3] = -100
+        y[4] = v + 5                       # out of range: the loss of that row is NaN, as in torch
+        y[1] = 7
+        t = (lg.float() + 0.5 * torch.randn(n, v, generator=g)).to(dt)
+        lgd, yd, td = lg.to(DEV), y.to(DEV), t.to(DEV)
+        res = []
+        for limit in (0, 1):
+            _hip.set_param("rows_vec_max", limit)
+            loss, lse, nv, rows = _hip.ce_fwd(lgd, yd, -100, "sum")
+            dl = _hip.ce_bwd(lgd, yd, lse, nv, None, -100)
+            l1, d1, _, r1 = _hip.ce_loss_grad(lgd, yd, -100, "mean")
+            kl, krows, ls, lt = _hip.kl_fwd(lgd, td, 0.5, "none")
+            kg = _hip.kl_bwd(lgd, td, ls, lt, None, False, dt, 0.5, 1.0)
+            torch.cuda.synchronize()
+            res.append([x.float().cpu() for x in (lse, rows, dl, d1, r1, krows, ls, lt, kg)])
+        _hip.set_param("rows_vec_max", 0)
+        names = ("lse", "rows", "dl", "d1", "r1", "krows", "ls", "lt", "kg")
+        for name, a, b in zip(names, *res):
+            assert torch.equal(a.isnan(), b.isnan()), (dt, v, name)
+            assert torch.allclose(a.nan_to_num(0.0, 1e30, -1e30), b.nan_to_num(0.0, 1e30, -1e30),
+                                  rtol=2e-2 if dt != F32 else 1e-5, atol=1e-6), (dt, v, name)
+        assert res[0][1][4].isnan() and res[0][1][3] == 0 and not res[0][2][3].any()
+    # 16 bytes further into a buffer the rows are still aligned; 2 bytes further they are not
+    base = (2 * torch.randn(9 * 512 + 9, generator=g)).to(BF16).to(DEV)
+    yb = torch.randint(0, 512, (9,), generator=g)
+    for off in (8, 1):
+        view = base[off:off + 9 * 512].view(9, 512)
+        loss, dl, _, _ = _hip.ce_loss_grad(view, yb.to(DEV), -100, "mean")
+        ref, rgrad = O.cross_entropy(view.cpu(), yb)
+        assert loss.item() == pytest.approx(ref.item(), rel=1e-4)
+        assert_close_lowp(dl, rgrad, BF16, f"offset {off}", ulps=3.0, cancel=1.0 / 9)
+
+
 def test_ce_loss_grad_unaligned_and_scale_inplace():
     g = gen(1013)
     base = (2 * torch.randn(5 * 3001 + 1, generator=g)).bfloat16().to(DEV)
@@ -361,7 +411,11 @@ KL_CASES = [(64, 128256, BF16, 2.0), (6, 5000, F32, 1.0), (3, 1, F32, 1.0), (5, 
             (2, 5000, F32, 4.0),
             # narrow rows: lane groups, several rows per workgroup
             (1000, 100, BF16, 2.0), (300, 257, F16, 1.0), (50, 1024, F32, 2.0), (70, 33, BF16, 1.0),
-            (129, 600, BF16, 1.5), (1030, 8, F32, 1.0), (77, 16, BF16, 3.0)]
+            (129, 600, BF16, 1.5), (1030, 8, F32, 1.0), (77, 16, BF16, 3.0),
+            # whole aligned vectors: every lane-group shape of the vector form
+            (257, 24, BF16, 1.0), (130, 64, BF16, 2.0), (99, 128, F16, 1.0), (65, 256, BF16, 1.0),
+            (300, 512, BF16, 2.0), (50, 1024, BF16, 1.0), (37, 2048, BF16, 1.5), (21, 2040, F16, 1.0),
+            (33, 96, F32, 1.0), (19, 1024, F32, 2.0), (40, 520, F32, 1.0)]
 
 
 @pytest.mark.parametrize("n,v,dt,T", KL_CASES)
@@ -401,6 +455,9 @@ KL1_CASES = [(64, 32000, BF16, 2.0, BF16), (6, 5000, F32, 1.0, F32), (3, 1, F32,
              (5, 600, F16, 1.0, F32), (6, 2048, BF16, 2.0, BF16),
              (1000, 100, BF16, 2.0, BF16), (300, 257, F16, 1.0, F32), (50, 1024, F32, 2.0, F32),
              (70, 33, BF16, 1.0, F32), (1030, 8, BF16, 1.0, BF16),
+             (257, 24, BF16, 1.0, F32), (130, 64, BF16, 2.0, BF16), (99, 128, F16, 1.0, F16),
+             (65, 256, BF16, 1.0, BF16), (300, 512, BF16, 2.0, F32), (50, 1024, F16, 1.0, F32),
+             (37, 2048, BF16, 1.5, F32), (33, 96, F32, 1.0, F32), (19, 1024, F32, 2.0, F32),
              # rows past the register path: two sweeps in one launch
              (4, 70000, BF16, 2.0, BF16), (3, 40000, F32, 1.0, F32), (3, 128256, BF16, 2.0, F32),
              (5, 65537, F16, 1.0, F16)]
