@@ -445,7 +445,7 @@ def make_workload(name, torch, L, dev):
 
         w.step = step
         w.dominant_launch = step
-        w.dominant = "route_kernel + permute_kernel"
+        w.dominant = "route_group_kernel + permute_kernel"
         w.dominant_bytes = w.bytes = n * (e * 4 + k * 4 * 4)
         w.desc = f"router softmax + top-{k} + counts + stable permutation, logits fp32 [{n},{e}]"
         w.unit = "rows/s"

@@ -6,16 +6,20 @@
 // Ties are resolved in the canonical order of forgemind/kernels/topk.py:13-16: equal
 // probabilities go to the lowest expert index.
 //
-// Two launches, integer-only bookkeeping:
-//   route_kernel    one wave per row, experts spread over the lanes (lane l owns experts
-//                   l, l+64, ...). Wave max / sum give the softmax; each of the k picks is a
-//                   wave max over order-preserving integer keys followed by a wave min over
-//                   the tied expert indices. A wave keeps four rows in flight so that their
-//                   dependent reduction chains overlap. Each 16-wave workgroup owns a
-//                   contiguous tile of rows and leaves its expert histogram in `hist[tile][e]`.
-//   permute_kernel  every workgroup sums the histograms of the tiles before it (and of all
-//                   tiles, for the expert bases), then walks its own tile in ascending flat
-//                   position and gives each assignment the slot
+// Launches, integer-only bookkeeping:
+//   route_group_kernel  L lanes per row (8, 16, 32 or 64 for up to 64, 128, 256, 512 experts),
+//                   eight neighbouring experts per lane, so a wave works on 64 / L rows at once
+//                   and reads whole rows with 16-byte loads. Group max / sum give the softmax;
+//                   each of the k picks is a group max over order-preserving integer keys
+//                   followed by a group min over the tied expert indices. Each 4-wave workgroup
+//                   owns a contiguous tile of rows and leaves its expert histogram in
+//                   `hist[tile][e]` (and, when asked, a partial row of the statistics).
+//   route_stats_kernel  folds the statistics partials in a fixed order (only when asked for).
+//   hist_scan_kernel    only for many tiles x many experts: exclusive scan of the histograms
+//                   over the tiles, in place, and the expert totals.
+//   permute_kernel  every workgroup takes (or, without the scan, sums) the histograms of the
+//                   tiles before it and the expert totals, then walks its own tile in ascending
+//                   flat position and gives each assignment the slot
 //                     base[e] + (#assignments to e in earlier tiles) + (rank inside the tile),
 //                   which is exactly the position a stable sort by expert would assign.
 #include "fm_common.cuh"
@@ -35,138 +39,160 @@ __device__ __forceinline__ uint32_t key_of(float f) {
   return b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);
 }
 
-constexpr int kRouteThreads = 1024;   // 16 waves per tile
-constexpr int kRowsAtOnce = 4;        // rows a wave works on together (independent chains)
+// Reductions over aligned groups of L consecutive lanes (L = 8, 16 or 32) for the keys and the
+// expert indices; every lane of a group ends with the group's result.
+template <int L>
+__device__ __forceinline__ uint32_t group_max_u(uint32_t v) {
+  if constexpr (L == 64) return wave_max_u(v);
+  auto mx = [](uint32_t a, uint32_t b) { return a > b ? a : b; };
+  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppXor1));
+  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppXor2));
+  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppHalfMirror));
+  if constexpr (L >= 16) v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppMirror));
+  if constexpr (L >= 32) v = mx(v, (uint32_t)__shfl_xor((int)v, 16, 64));
+  return v;
+}
 
-template <typename T, int EPL>
-__global__ __launch_bounds__(kRouteThreads) void route_kernel(const T* __restrict__ logits,
-                                                               int32_t* __restrict__ idx,
-                                                               float* __restrict__ weights,
-                                                               int32_t* __restrict__ hist,
-                                                               float* __restrict__ fstat, int64_t n,
-                                                               int e, int k, int tile_rows) {
-  constexpr int R = kRowsAtOnce;
-  constexpr int NW = kRouteThreads / 64;
-  __shared__ int lh[kMaxE];
-  __shared__ float wstat[NW][EPL * 64];   // per-wave column sums of the probabilities
-  __shared__ float wz[NW];                // per-wave sums of logsumexp^2
-  float psum[EPL];
+template <int L>
+__device__ __forceinline__ int group_min_i(int v) {
+  if constexpr (L == 64) return wave_min_i(v);
+  auto mn = [](int a, int b) { return a < b ? a : b; };
+  v = mn(v, FM_DPP_I(v, kDppXor1));
+  v = mn(v, FM_DPP_I(v, kDppXor2));
+  v = mn(v, FM_DPP_I(v, kDppHalfMirror));
+  if constexpr (L >= 16) v = mn(v, FM_DPP_I(v, kDppMirror));
+  if constexpr (L >= 32) v = mn(v, __shfl_xor(v, 16, 64));
+  return v;
+}
+
+constexpr int kGroupThreads = 256;    // 4 waves per tile
+constexpr int kGE = 8;                // experts a lane holds
+
+// L lanes per row, eight neighbouring experts per lane: a wave works on 64 / L rows at once, reads
+// whole rows with 16-byte loads (VEC: e a multiple of eight, aligned buffer) and reduces over L
+// lanes only. Ties go to the lowest expert index: the lane keeps its first maximum, the group
+// takes the smallest index among the lanes that hold the group's maximum.
+template <typename T, int L, bool VEC>
+__global__ __launch_bounds__(kGroupThreads) void route_group_kernel(const T* __restrict__ logits,
+                                                                     int32_t* __restrict__ idx,
+                                                                     float* __restrict__ weights,
+                                                                     int32_t* __restrict__ hist,
+                                                                     float* __restrict__ fstat, int64_t n,
+                                                                     int e, int k, int tile_rows) {
+  constexpr int NW = kGroupThreads / 64;
+  constexpr int GPW = 64 / L;           // rows per wave and pass
+  __shared__ int lh[L * kGE];
+  __shared__ float wstat[NW][L * kGE];  // per-wave column sums of the probabilities
+  __shared__ float wz[NW];              // per-wave sums of logsumexp^2
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane / L, l = lane % L;
+  const int ex0 = l * kGE;              // this lane's first expert
+  float psum[kGE];
   float zsum = 0.f;
 #pragma unroll
-  for (int q = 0; q < EPL; ++q) psum[q] = 0.f;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  for (int i = tid; i < e; i += kRouteThreads) lh[i] = 0;
+  for (int q = 0; q < kGE; ++q) psum[q] = 0.f;
+  for (int i = tid; i < L * kGE; i += kGroupThreads) lh[i] = 0;
   __syncthreads();
   const int64_t row0 = (int64_t)blockIdx.x * tile_rows;
   const int64_t row1 = row0 + tile_rows < n ? row0 + tile_rows : n;
-  // wave w owns rows row0 + w, + NW, ...; R of them are in flight at once so that the
-  // dependent DPP / readlane chains of different rows overlap
-  for (int64_t rb = row0 + wave; rb < row1; rb += (int64_t)NW * R) {
-    float p[R][EPL];
-    uint32_t key[R][EPL];
-    bool live[R];
+  for (int64_t rb = row0 + wave * GPW; rb < row1; rb += (int64_t)NW * GPW) {
+    const int64_t row = rb + g;
+    const bool live = row < row1;
+    float p[kGE];
+    if constexpr (VEC) {
+      constexpr int EPV = Elem<T>::kVec;
+      if (live && ex0 < e) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int64_t row = rb + (int64_t)r * NW;
-      live[r] = row < row1;
+        for (int h = 0; h < kGE / EPV; ++h) {
+          float part[EPV];
+          Elem<T>::unpack(load16(logits + row * (int64_t)e + ex0 + h * EPV), part);
 #pragma unroll
-      for (int q = 0; q < EPL; ++q) {
-        const int ex = lane + 64 * q;
-        p[r][q] = (live[r] && ex < e) ? Elem<T>::load1(logits + row * (int64_t)e + ex) : -INFINITY;
+          for (int q = 0; q < EPV; ++q) p[h * EPV + q] = part[q];
+        }
+      } else {
+#pragma unroll
+        for (int q = 0; q < kGE; ++q) p[q] = -INFINITY;
       }
+    } else {
+#pragma unroll
+      for (int q = 0; q < kGE; ++q)
+        p[q] = (live && ex0 + q < e) ? Elem<T>::load1(logits + row * (int64_t)e + ex0 + q) : -INFINITY;
     }
-    float m[R], s[R];
+    float m = p[0];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      m[r] = p[r][0];
+    for (int q = 1; q < kGE; ++q) m = fmaxf(m, p[q]);
+    m = group_reduce<L, OpMax>(m);
+    float s = 0.f;
 #pragma unroll
-      for (int q = 1; q < EPL; ++q) m[r] = fmaxf(m[r], p[r][q]);
+    for (int q = 0; q < kGE; ++q) {
+      p[q] = fast_exp2((p[q] - m) * kLog2e);
+      s += p[q];
     }
+    s = group_reduce<L, OpSum>(s);
+    uint32_t key[kGE];
 #pragma unroll
-    for (int r = 0; r < R; ++r) m[r] = wave_max(m[r]);
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      s[r] = 0.f;
-#pragma unroll
-      for (int q = 0; q < EPL; ++q) {
-        p[r][q] = fast_exp2((p[r][q] - m[r]) * kLog2e);
-        s[r] += p[r][q];
-      }
+    for (int q = 0; q < kGE; ++q) {
+      p[q] = p[q] / s;
+      key[q] = (ex0 + q) < e ? key_of(p[q]) : 0u;   // 0 is below every real key
+      if (live && (ex0 + q) < e) psum[q] += p[q];    // rows in ascending order
     }
-#pragma unroll
-    for (int r = 0; r < R; ++r) s[r] = wave_sum(s[r]);
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-#pragma unroll
-      for (int q = 0; q < EPL; ++q) {
-        p[r][q] = p[r][q] / s[r];
-        key[r][q] = (lane + 64 * q) < e ? key_of(p[r][q]) : 0u;   // 0 is below every real key
-        if (live[r] && (lane + 64 * q) < e) psum[q] += p[r][q];    // rows in ascending order
-      }
-      if (live[r]) {
-        const float lse = m[r] + fast_log2(s[r]) * kLn2;
-        zsum += lse * lse;
-      }
+    if (live && l == 0) {
+      const float lse = m + fast_log2(s) * kLn2;
+      zsum += lse * lse;
     }
-    int my_i[R];
-    float my_p[R], wsum[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) { my_i[r] = 0; my_p[r] = 0.f; wsum[r] = 0.f; }
+    int my_i = 0;
+    float my_p = 0.f, wsum = 0.f;
 #pragma unroll
     for (int j = 0; j < kMaxK; ++j) {
       if (j < k) {
-        uint32_t bk[R];
-        int bq[R], wi[R];
+        uint32_t bk = key[0];
+        int bq = 0;
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-          bk[r] = key[r][0];
-          bq[r] = 0;
-#pragma unroll
-          for (int q = 1; q < EPL; ++q) {
-            if (key[r][q] > bk[r]) { bk[r] = key[r][q]; bq[r] = q; }
-          }
+        for (int q = 1; q < kGE; ++q) {
+          if (key[q] > bk) { bk = key[q]; bq = q; }
         }
-        uint32_t wk[R];
+        const uint32_t gk = group_max_u<L>(bk);
+        const int gi = group_min_i<L>((bk == gk) ? ex0 + bq : 0x7fffffff);
+        const int wl = gi >> 3, wq = gi & 7;
+        float pv = p[0];
 #pragma unroll
-        for (int r = 0; r < R; ++r) wk[r] = wave_max_u(bk[r]);
+        for (int q = 1; q < kGE; ++q) pv = (q == wq) ? p[q] : pv;
+        pv = __shfl(pv, (lane & ~(L - 1)) + wl, 64);
 #pragma unroll
-        for (int r = 0; r < R; ++r) wi[r] = wave_min_i((bk[r] == wk[r]) ? lane + 64 * bq[r] : 0x7fffffff);
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          const int wq = wi[r] >> 6, wl = wi[r] & 63;
-          float pv = p[r][0];
-#pragma unroll
-          for (int q = 1; q < EPL; ++q) pv = (q == wq) ? p[r][q] : pv;
-          pv = __shfl(pv, wl, 64);
-#pragma unroll
-          for (int q = 0; q < EPL; ++q) {
-            if (lane == wl && q == wq) key[r][q] = 0u;
-          }
-          wsum[r] += pv;
-          if (lane == j) { my_i[r] = wi[r]; my_p[r] = pv; }
+        for (int q = 0; q < kGE; ++q) {
+          if (l == wl && q == wq) key[q] = 0u;
         }
+        wsum += pv;
+        if (l == j) { my_i = gi; my_p = pv; }
       }
     }
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int64_t row = rb + (int64_t)r * NW;
-      if (live[r] && lane < k) {
-        idx[row * (int64_t)k + lane] = my_i[r];
-        weights[row * (int64_t)k + lane] = my_p[r] / wsum[r];
-        atomicAdd(&lh[my_i[r]], 1);
-      }
+    if (live && l < k) {
+      idx[row * (int64_t)k + l] = my_i;
+      weights[row * (int64_t)k + l] = my_p / wsum;
+      atomicAdd(&lh[my_i], 1);
     }
   }
   if (fstat != nullptr) {
+    // fold the wave's row groups (lanes l, l + L, ...) in group order, then the waves
 #pragma unroll
-    for (int q = 0; q < EPL; ++q) wstat[wave][lane + 64 * q] = psum[q];
+    for (int q = 0; q < kGE; ++q) {
+      float a = psum[q];
+#pragma unroll
+      for (int o = L; o < 64; o <<= 1) a += __shfl_xor(a, o, 64);
+      psum[q] = a;
+    }
+    zsum = wave_sum(zsum);
+    if (g == 0) {
+#pragma unroll
+      for (int q = 0; q < kGE; ++q) wstat[wave][ex0 + q] = psum[q];
+    }
     if (lane == 0) wz[wave] = zsum;
   }
   __syncthreads();
-  for (int i = tid; i < e; i += kRouteThreads) hist[(int64_t)blockIdx.x * e + i] = lh[i];
+  for (int i = tid; i < e; i += kGroupThreads) hist[(int64_t)blockIdx.x * e + i] = lh[i];
   if (fstat != nullptr) {   // fold the waves in wave order: one fp32 partial row per tile
     float* out = fstat + (int64_t)blockIdx.x * (e + 1);
-    for (int i = tid; i < e; i += kRouteThreads) {
+    for (int i = tid; i < e; i += kGroupThreads) {
       float a = wstat[0][i];
 #pragma unroll
       for (int w = 1; w < NW; ++w) a += wstat[w][i];
@@ -181,34 +207,91 @@ __global__ __launch_bounds__(kRouteThreads) void route_kernel(const T* __restric
   }
 }
 
-// Sums the per-tile partial rows [ntiles, e+1] in tile order: stats[0..e) = column sums of the
-// probabilities, stats[e] = sum of logsumexp^2. One workgroup; thread c owns column c.
+// Sums the per-tile partial rows [ntiles, e+1]: stats[0..e) = column sums of the probabilities,
+// stats[e] = sum of logsumexp^2. A workgroup owns 64 columns; wave w adds tiles w, w + 16, ...
+// of a column in that order, then the sixteen partial sums are added in wave order. The order
+// depends on ntiles only, so equal inputs give equal bits.
 __global__ __launch_bounds__(1024) void route_stats_kernel(const float* __restrict__ fstat,
                                                             float* __restrict__ stats, int e,
                                                             int ntiles) {
-  const int c = threadIdx.x;
-  if (c > e) return;
+  __shared__ float part[16][64];
+  const int cols = e + 1;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + lane;
   float a = 0.f;
-  int t = 0;
-  for (; t + 7 < ntiles; t += 8) {
-    float v[8];
+  if (c < cols) {
+    // sixteen loads in flight; the additions stay in tile order
+    int t = wave;
+    for (; t + 15 * 16 < ntiles; t += 16 * 16) {
+      float v[16];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = fstat[(int64_t)(t + u) * (e + 1) + c];
+      for (int u = 0; u < 16; ++u) v[u] = fstat[(int64_t)(t + u * 16) * cols + c];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) a += v[u];
+      for (int u = 0; u < 16; ++u) a += v[u];
+    }
+    for (; t < ntiles; t += 16) a += fstat[(int64_t)t * cols + c];
   }
-  for (; t < ntiles; ++t) a += fstat[(int64_t)t * (e + 1) + c];
-  stats[c] = a;
+  part[wave][lane] = a;
+  __syncthreads();
+  if (wave == 0 && c < cols) {
+    float r = part[0][lane];
+#pragma unroll
+    for (int w = 1; w < 16; ++w) r += part[w][lane];
+    stats[c] = r;
+  }
+}
+
+// Exclusive scan of the tile histograms over the tiles, in place: hist[t][c] becomes the number
+// of assignments to expert c in tiles before t, counts[c] their total. A workgroup owns 16
+// experts; thread (s, c) walks tiles s * per, ..., (s + 1) * per - 1 of expert c.
+__global__ __launch_bounds__(1024) void hist_scan_kernel(int32_t* __restrict__ hist,
+                                                          int32_t* __restrict__ counts, int e,
+                                                          int ntiles) {
+  __shared__ int seg[64][17];
+  const int c = threadIdx.x & 15, sgm = threadIdx.x >> 4;
+  const int col = blockIdx.x * 16 + c;
+  constexpr int kPer = kMaxTiles / 64;   // tiles per segment at most
+  const int per = (ntiles + 63) / 64;
+  const int t0 = sgm * per;
+  int v[kPer];
+  int sum = 0;
+#pragma unroll
+  for (int u = 0; u < kPer; ++u) {
+    const int t = t0 + u;
+    v[u] = (col < e && u < per && t < ntiles) ? hist[(int64_t)t * e + col] : 0;
+  }
+#pragma unroll
+  for (int u = 0; u < kPer; ++u) sum += v[u];
+  seg[sgm][c] = sum;
+  __syncthreads();
+  if (threadIdx.x < 16) {       // one thread per expert: exclusive scan of its 64 segment sums
+    int run = 0;
+    for (int q = 0; q < 64; ++q) {
+      const int w = seg[q][threadIdx.x];
+      seg[q][threadIdx.x] = run;
+      run += w;
+    }
+    if (blockIdx.x * 16 + (int)threadIdx.x < e) counts[blockIdx.x * 16 + threadIdx.x] = run;
+  }
+  __syncthreads();
+  int run = seg[sgm][c];
+#pragma unroll
+  for (int u = 0; u < kPer; ++u) {
+    const int t = t0 + u;
+    if (col < e && u < per && t < ntiles) hist[(int64_t)t * e + col] = run;
+    run += v[u];
+  }
 }
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(256) void permute_kernel(const int32_t* __restrict__ idx,
                                                        const int32_t* __restrict__ hist,
-                                                       int32_t* __restrict__ counts,
+                                                       int32_t* counts,
                                                        int32_t* __restrict__ slot,
                                                        int32_t* __restrict__ order, int64_t n, int e,
-                                                       int k, int tile_rows, int ntiles, int emit) {
+                                                       int k, int tile_rows, int ntiles, int emit,
+                                                       int scanned) {
   // partial sums of the tile histograms: [group][expert], "before my tile" and "all tiles"
   __shared__ int part_b[4 * kMaxE];   // flat [group][e]; groups * e <= 4 * kMaxE on every path
   __shared__ int part_t[4 * kMaxE];
@@ -227,7 +310,14 @@ __global__ __launch_bounds__(256) void permute_kernel(const int32_t* __restrict_
 
   const int e4 = e >> 2;
   int groups;
-  if ((e & 3) == 0 && e4 <= 256 && (e4 & (e4 - 1)) == 0) {
+  if (scanned) {
+    // hist already holds "before my tile" and counts the totals (hist_scan_kernel)
+    groups = 1;
+    for (int col = tid; col < e; col += 256) {
+      part_b[col] = hist[(int64_t)me * e + col];
+      part_t[col] = counts[col];
+    }
+  } else if ((e & 3) == 0 && e4 <= 256 && (e4 & (e4 - 1)) == 0) {
     // 16-byte loads: a thread keeps four neighbouring experts and walks tiles g, g+groups, ...
     groups = 256 / e4;
     if (groups > 16) groups = 16;
@@ -296,7 +386,7 @@ __global__ __launch_bounds__(256) void permute_kernel(const int32_t* __restrict_
       }
       if (wave == 0 && col < e) {
         offs[col] += carry + inc - v;
-        if (me == 0) counts[col] = v;
+        if (me == 0 && !scanned) counts[col] = v;
       }
       carry += __builtin_amdgcn_readlane(inc, 63);
     }
@@ -359,14 +449,20 @@ template <typename T>
 int launch_route(const void* logits, int32_t* idx, float* weights, int32_t* hist, float* fstat,
                  int64_t n, int e, int k, const Tiling& tl, hipStream_t st) {
   const T* lp = static_cast<const T*>(logits);
-  const dim3 grid((unsigned)tl.ntiles), block(kRouteThreads);
-#define GO(EPL) \
-  hipLaunchKernelGGL((route_kernel<T, EPL>), grid, block, 0, st, lp, idx, weights, hist, fstat, n, e, k, tl.tile_rows)
-  if (e <= 64) GO(1);
-  else if (e <= 128) GO(2);
-  else if (e <= 256) GO(4);
-  else GO(8);
-#undef GO
+  const dim3 grid((unsigned)tl.ntiles);
+#define GOG(L_)                                                                                       \
+  do {                                                                                                \
+    if (vec) hipLaunchKernelGGL((route_group_kernel<T, L_, true>), grid, dim3(kGroupThreads), 0, st,  \
+                                lp, idx, weights, hist, fstat, n, e, k, tl.tile_rows);                \
+    else hipLaunchKernelGGL((route_group_kernel<T, L_, false>), grid, dim3(kGroupThreads), 0, st,     \
+                            lp, idx, weights, hist, fstat, n, e, k, tl.tile_rows);                    \
+  } while (0)
+  const bool vec = e % kGE == 0 && fm_host::aligned16(logits);
+  if (e <= 64) GOG(8);
+  else if (e <= 128) GOG(16);
+  else if (e <= 256) GOG(32);
+  else GOG(64);
+#undef GOG
   return FM_OK;
 }
 
@@ -413,12 +509,23 @@ int fm_route(const void* logits, int32_t* idx, float* weights, int32_t* counts, 
   else launch_route<f16_t>(logits, idx, weights, hist, fstat, n, e, k, tl, st);
   FM_CHECK_LAUNCH("fm_route");
   if (stats != nullptr) {
-    hipLaunchKernelGGL(route_stats_kernel, dim3(1), dim3(1024), 0, st, fstat, stats, e, tl.ntiles);
+    hipLaunchKernelGGL(route_stats_kernel, dim3((unsigned)((e + 1 + 63) / 64)), dim3(1024), 0, st, fstat, stats,
+                       e, tl.ntiles);
     FM_CHECK_LAUNCH("fm_route(stats)");
   }
   const int emit = (slot != nullptr || order != nullptr) && n > 0 ? 1 : 0;
-  hipLaunchKernelGGL(permute_kernel, dim3(emit ? (unsigned)tl.ntiles : 1u), dim3(256), 0, st, idx, hist,
-                     counts, slot, order, n, e, k, tl.tile_rows, tl.ntiles, emit);
+  // Many tiles times many experts: every permutation workgroup summing all histograms before
+  // its own would read ntiles^2 * e integers in total; scan them once instead.
+  const int scanned = (int64_t)tl.ntiles * e > 32768 ? 1 : 0;
+  if (scanned) {
+    hipLaunchKernelGGL(hist_scan_kernel, dim3((unsigned)((e + 15) / 16)), dim3(1024), 0, st, hist, counts, e,
+                       tl.ntiles);
+    FM_CHECK_LAUNCH("fm_route(scan)");
+  }
+  if (emit || !scanned) {
+    hipLaunchKernelGGL(permute_kernel, dim3(emit ? (unsigned)tl.ntiles : 1u), dim3(256), 0, st, idx, hist,
+                       counts, slot, order, n, e, k, tl.tile_rows, tl.ntiles, emit, scanned);
+  }
   FM_CHECK_LAUNCH("fm_route(permute)");
   return FM_OK;
 }

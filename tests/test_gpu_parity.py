@@ -791,7 +791,11 @@ def router_inputs(n, e, seed, dtype=F32):
 
 
 ROUTE_CASES = [(16384, 64, 2), (1000, 8, 2), (513, 128, 4), (100, 300, 8), (1, 64, 2), (70000, 16, 1),
-               (257, 512, 8), (4099, 64, 6), (3, 2, 2)]
+               (257, 512, 8), (4099, 64, 6), (3, 2, 2),
+               # many tiles x many experts: the histograms are scanned by a kernel of their own
+               (40000, 64, 2), (9000, 256, 8), (5000, 500, 3), (300000, 8, 1),
+               # expert counts around the lane-group sizes, not multiples of eight
+               (700, 65, 2), (700, 129, 3), (700, 257, 8), (900, 60, 4), (64, 7, 7)]
 
 
 @pytest.mark.parametrize("n,e,k", ROUTE_CASES)
@@ -824,6 +828,19 @@ def test_route_half_precision_logits_and_all_equal_rows():
     oi, ow, oc, oslot, oorder = O.router(lg, 2)
     idx, w, counts, slot, order = _hip.route(lg.to(DEV), 2)
     assert torch.equal(idx.cpu().long(), oi) and torch.equal(order.cpu().long(), oorder)
+    for dt, e, k in ((F16, 128, 4), (BF16, 320, 8), (F16, 24, 3)):
+        lg = router_inputs(777, e, 6, dt)
+        oi, ow, oc, oslot, oorder = O.router(lg, k)
+        idx, w, counts, slot, order = _hip.route(lg.to(DEV), k)
+        assert torch.equal(idx.cpu().long(), oi) and torch.equal(order.cpu().long(), oorder), (dt, e, k)
+        assert torch.equal(counts.cpu().long(), oc) and torch.allclose(w.cpu(), ow, rtol=1e-5, atol=0)
+    # a buffer that starts 4 bytes off a 16-byte line takes the element-wise loads
+    base = torch.zeros(500 * 64 + 1, device=DEV)
+    lg = router_inputs(500, 64, 7)
+    base[1:] = lg.reshape(-1).to(DEV)
+    idx, w, counts, slot, order = _hip.route(base[1:].view(500, 64), 2)
+    oi, ow, oc, oslot, oorder = O.router(lg, 2)
+    assert torch.equal(idx.cpu().long(), oi) and torch.equal(slot.cpu().long(), oslot)
     z = torch.zeros(130, 64, device=DEV)
     idx, w, counts, slot, order = _hip.route(z, 2)
     assert torch.equal(idx.cpu(), torch.tensor([[0, 1]], dtype=torch.int32).expand(130, 2))
