@@ -95,81 +95,117 @@ __global__ __launch_bounds__(kGroupThreads) void route_group_kernel(const T* __r
   __syncthreads();
   const int64_t row0 = (int64_t)blockIdx.x * tile_rows;
   const int64_t row1 = row0 + tile_rows < n ? row0 + tile_rows : n;
-  for (int64_t rb = row0 + wave * GPW; rb < row1; rb += (int64_t)NW * GPW) {
-    const int64_t row = rb + g;
-    const bool live = row < row1;
-    float p[kGE];
-    if constexpr (VEC) {
-      constexpr int EPV = Elem<T>::kVec;
-      if (live && ex0 < e) {
+  // R rows per lane group are in flight at once so that their dependent reduction chains overlap
+  constexpr int R = 2;
+  for (int64_t rb = row0 + wave * GPW; rb < row1; rb += (int64_t)NW * GPW * R) {
+    int64_t row[R];
+    bool live[R];
+    float p[R][kGE];
 #pragma unroll
-        for (int h = 0; h < kGE / EPV; ++h) {
-          float part[EPV];
-          Elem<T>::unpack(load16(logits + row * (int64_t)e + ex0 + h * EPV), part);
+    for (int r = 0; r < R; ++r) {
+      row[r] = rb + (int64_t)r * NW * GPW + g;
+      live[r] = row[r] < row1;
+      if constexpr (VEC) {
+        constexpr int EPV = Elem<T>::kVec;
+        if (live[r] && ex0 < e) {
 #pragma unroll
-          for (int q = 0; q < EPV; ++q) p[h * EPV + q] = part[q];
+          for (int h = 0; h < kGE / EPV; ++h) {
+            float part[EPV];
+            Elem<T>::unpack(load16(logits + row[r] * (int64_t)e + ex0 + h * EPV), part);
+#pragma unroll
+            for (int q = 0; q < EPV; ++q) p[r][h * EPV + q] = part[q];
+          }
+        } else {
+#pragma unroll
+          for (int q = 0; q < kGE; ++q) p[r][q] = -INFINITY;
         }
       } else {
 #pragma unroll
-        for (int q = 0; q < kGE; ++q) p[q] = -INFINITY;
+        for (int q = 0; q < kGE; ++q)
+          p[r][q] = (live[r] && ex0 + q < e) ? Elem<T>::load1(logits + row[r] * (int64_t)e + ex0 + q) : -INFINITY;
       }
-    } else {
-#pragma unroll
-      for (int q = 0; q < kGE; ++q)
-        p[q] = (live && ex0 + q < e) ? Elem<T>::load1(logits + row * (int64_t)e + ex0 + q) : -INFINITY;
     }
-    float m = p[0];
+    float m[R], s[R];
 #pragma unroll
-    for (int q = 1; q < kGE; ++q) m = fmaxf(m, p[q]);
-    m = group_reduce<L, OpMax>(m);
-    float s = 0.f;
+    for (int r = 0; r < R; ++r) {
+      m[r] = p[r][0];
 #pragma unroll
-    for (int q = 0; q < kGE; ++q) {
-      p[q] = fast_exp2((p[q] - m) * kLog2e);
-      s += p[q];
+      for (int q = 1; q < kGE; ++q) m[r] = fmaxf(m[r], p[r][q]);
     }
-    s = group_reduce<L, OpSum>(s);
-    uint32_t key[kGE];
 #pragma unroll
-    for (int q = 0; q < kGE; ++q) {
-      p[q] = p[q] / s;
-      key[q] = (ex0 + q) < e ? key_of(p[q]) : 0u;   // 0 is below every real key
-      if (live && (ex0 + q) < e) psum[q] += p[q];    // rows in ascending order
+    for (int r = 0; r < R; ++r) m[r] = group_reduce<L, OpMax>(m[r]);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      s[r] = 0.f;
+#pragma unroll
+      for (int q = 0; q < kGE; ++q) {
+        p[r][q] = fast_exp2((p[r][q] - m[r]) * kLog2e);
+        s[r] += p[r][q];
+      }
     }
-    if (live && l == 0) {
-      const float lse = m + fast_log2(s) * kLn2;
-      zsum += lse * lse;
+#pragma unroll
+    for (int r = 0; r < R; ++r) s[r] = group_reduce<L, OpSum>(s[r]);
+    uint32_t key[R][kGE];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      // one division per row: eight IEEE divisions a lane were a quarter of the kernel
+      const float inv = 1.f / s[r];
+#pragma unroll
+      for (int q = 0; q < kGE; ++q) {
+        p[r][q] = p[r][q] * inv;
+        key[r][q] = (ex0 + q) < e ? key_of(p[r][q]) : 0u;   // 0 is below every real key
+        if (live[r] && (ex0 + q) < e) psum[q] += p[r][q];    // rows in ascending order
+      }
+      if (live[r] && l == 0) {
+        const float lse = m[r] + fast_log2(s[r]) * kLn2;
+        zsum += lse * lse;
+      }
     }
-    int my_i = 0;
-    float my_p = 0.f, wsum = 0.f;
+    int my_i[R];
+    float my_p[R], wsum[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) { my_i[r] = 0; my_p[r] = 0.f; wsum[r] = 0.f; }
 #pragma unroll
     for (int j = 0; j < kMaxK; ++j) {
       if (j < k) {
-        uint32_t bk = key[0];
-        int bq = 0;
+        uint32_t bk[R], gk[R];
+        int bq[R], gi[R];
 #pragma unroll
-        for (int q = 1; q < kGE; ++q) {
-          if (key[q] > bk) { bk = key[q]; bq = q; }
+        for (int r = 0; r < R; ++r) {
+          bk[r] = key[r][0];
+          bq[r] = 0;
+#pragma unroll
+          for (int q = 1; q < kGE; ++q) {
+            if (key[r][q] > bk[r]) { bk[r] = key[r][q]; bq[r] = q; }
+          }
         }
-        const uint32_t gk = group_max_u<L>(bk);
-        const int gi = group_min_i<L>((bk == gk) ? ex0 + bq : 0x7fffffff);
-        const int wl = gi >> 3, wq = gi & 7;
-        float pv = p[0];
 #pragma unroll
-        for (int q = 1; q < kGE; ++q) pv = (q == wq) ? p[q] : pv;
-        pv = __shfl(pv, (lane & ~(L - 1)) + wl, 64);
+        for (int r = 0; r < R; ++r) gk[r] = group_max_u<L>(bk[r]);
 #pragma unroll
-        for (int q = 0; q < kGE; ++q) {
-          if (l == wl && q == wq) key[q] = 0u;
+        for (int r = 0; r < R; ++r) gi[r] = group_min_i<L>((bk[r] == gk[r]) ? ex0 + bq[r] : 0x7fffffff);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const int wl = gi[r] >> 3, wq = gi[r] & 7;
+          float pv = p[r][0];
+#pragma unroll
+          for (int q = 1; q < kGE; ++q) pv = (q == wq) ? p[r][q] : pv;
+          pv = __shfl(pv, (lane & ~(L - 1)) + wl, 64);
+#pragma unroll
+          for (int q = 0; q < kGE; ++q) {
+            if (l == wl && q == wq) key[r][q] = 0u;
+          }
+          wsum[r] += pv;
+          if (l == j) { my_i[r] = gi[r]; my_p[r] = pv; }
         }
-        wsum += pv;
-        if (l == j) { my_i = gi; my_p = pv; }
       }
     }
-    if (live && l < k) {
-      idx[row * (int64_t)k + l] = my_i;
-      weights[row * (int64_t)k + l] = my_p / wsum;
-      atomicAdd(&lh[my_i], 1);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (live[r] && l < k) {
+        idx[row[r] * (int64_t)k + l] = my_i[r];
+        weights[row[r] * (int64_t)k + l] = my_p[r] / wsum[r];
+        atomicAdd(&lh[my_i[r]], 1);
+      }
     }
   }
   if (fstat != nullptr) {
@@ -297,7 +333,7 @@ __global__ __launch_bounds__(256) void permute_kernel(const int32_t* __restrict_
   __shared__ int part_t[4 * kMaxE];
   __shared__ int total[kMaxE];
   __shared__ int offs[kMaxE];      // next free slot of each expert for this tile
-  __shared__ int wcnt[4][kMaxE];   // per-wave assignment counts of the current chunk
+  __shared__ unsigned long long wmask[4][kMaxE];   // per wave and expert: the lanes assigned to it (current chunk)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int me = blockIdx.x;
 
@@ -363,7 +399,7 @@ __global__ __launch_bounds__(256) void permute_kernel(const int32_t* __restrict_
       }
     }
   }
-  for (int i = tid; i < 4 * kMaxE; i += 256) (&wcnt[0][0])[i] = 0;
+  for (int i = tid; i < 4 * kMaxE; i += 256) (&wmask[0][0])[i] = 0ull;
   __syncthreads();
   for (int col = tid; col < e; col += 256) {
     int tb = 0, tt = 0;
@@ -399,31 +435,23 @@ __global__ __launch_bounds__(256) void permute_kernel(const int32_t* __restrict_
     const bool act = p < p1;
     const int ex = ex_next;
     ex_next = (p + 256 < p1) ? idx[p + 256] : -1;
-    // rank among equal experts inside the wave, in lane (= flat position) order
-    int rank = 0;
-    unsigned long long todo = __ballot(act);
-    while (todo != 0ull) {
-      const int leader = __builtin_ctzll(todo);
-      const int e0 = __builtin_amdgcn_readlane(ex, leader);
-      const unsigned long long same = __ballot(act && ex == e0);
-      if (act && ex == e0) {
-        rank = __builtin_popcountll(same & ((1ull << lane) - 1ull));
-        if (lane == leader) wcnt[wave][e0] = __builtin_popcountll(same);
-      }
-      todo &= ~same;
-    }
+    // rank among equal experts inside the wave, in lane (= flat position) order: the lanes of
+    // an expert as a bit mask (the mask does not depend on the order the atomics land in)
+    if (act) atomicOr(&wmask[wave][ex], 1ull << lane);
     __syncthreads();
     if (act) {
+      const int rank = __builtin_popcountll(wmask[wave][ex] & ((1ull << lane) - 1ull));
       int prior = offs[ex];
-      for (int w = 0; w < wave; ++w) prior += wcnt[w][ex];
+      for (int w = 0; w < wave; ++w) prior += __builtin_popcountll(wmask[w][ex]);
       const int s = prior + rank;
       if (slot != nullptr) slot[p] = s;
       if (order != nullptr) order[s] = (int32_t)p;
     }
     __syncthreads();
     for (int col = tid; col < e; col += 256) {
-      offs[col] += (wcnt[0][col] + wcnt[1][col]) + (wcnt[2][col] + wcnt[3][col]);
-      wcnt[0][col] = 0; wcnt[1][col] = 0; wcnt[2][col] = 0; wcnt[3][col] = 0;
+      offs[col] += (__builtin_popcountll(wmask[0][col]) + __builtin_popcountll(wmask[1][col])) +
+                   (__builtin_popcountll(wmask[2][col]) + __builtin_popcountll(wmask[3][col]));
+      wmask[0][col] = 0ull; wmask[1][col] = 0ull; wmask[2][col] = 0ull; wmask[3][col] = 0ull;
     }
     __syncthreads();
   }
