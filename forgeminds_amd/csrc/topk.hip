@@ -359,6 +359,123 @@ __global__ __launch_bounds__(64) void topk_wave_kernel(const T* __restrict__ x, 
   }
 }
 
+// Rows of at most 512 elements with k <= 8: L lanes per row (8, 16, 32 or 64), eight
+// neighbouring elements per lane, so a wave works on 64 / L rows at once and reads whole rows
+// with 16-byte loads (VEC: v a multiple of eight, aligned buffer). Each of the k picks is a
+// lane-local first maximum, a group maximum over the keys and a group minimum over the indices
+// that hold it -- the canonical order (value descending, index ascending) by construction.
+template <int L>
+__device__ __forceinline__ uint32_t lanes_max_u(uint32_t v) {
+  if constexpr (L == 64) return wave_max_u(v);
+  auto mx = [](uint32_t a, uint32_t b) { return a > b ? a : b; };
+  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppXor1));
+  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppXor2));
+  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppHalfMirror));
+  if constexpr (L >= 16) v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppMirror));
+  if constexpr (L >= 32) v = mx(v, (uint32_t)__shfl_xor((int)v, 16, 64));
+  return v;
+}
+
+template <int L>
+__device__ __forceinline__ int lanes_min_i(int v) {
+  if constexpr (L == 64) return wave_min_i(v);
+  auto mn = [](int a, int b) { return a < b ? a : b; };
+  v = mn(v, FM_DPP_I(v, kDppXor1));
+  v = mn(v, FM_DPP_I(v, kDppXor2));
+  v = mn(v, FM_DPP_I(v, kDppHalfMirror));
+  if constexpr (L >= 16) v = mn(v, FM_DPP_I(v, kDppMirror));
+  if constexpr (L >= 32) v = mn(v, __shfl_xor(v, 16, 64));
+  return v;
+}
+
+constexpr int kGroupMaxV = 512;
+constexpr int kGroupMaxK = 8;
+constexpr int kGroupRows = 2;   // rows a lane group works on together (independent chains)
+
+template <typename T, int L, bool VEC>
+__global__ __launch_bounds__(256) void topk_group_kernel(const T* __restrict__ x, T* __restrict__ values,
+                                                         int32_t* __restrict__ idx32,
+                                                         int64_t* __restrict__ idx64, int64_t n, int v,
+                                                         int k) {
+  constexpr int GE = 8;
+  constexpr int GPW = 64 / L;
+  constexpr int R = kGroupRows;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane / L, l = lane % L;
+  const int c0 = l * GE;
+  const int64_t first = ((int64_t)blockIdx.x * 4 + wave) * (GPW * R);
+  int64_t row[R];
+  bool live[R];
+  uint32_t key[R][GE];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    row[r] = first + r * GPW + g;
+    live[r] = row[r] < n;
+    float f[GE];
+    if constexpr (VEC) {
+      constexpr int EPV = Elem<T>::kVec;
+      if (live[r] && c0 < v) {
+#pragma unroll
+        for (int h = 0; h < GE / EPV; ++h) {
+          float part[EPV];
+          Elem<T>::unpack(load16_stream(x + row[r] * (int64_t)v + c0 + h * EPV), part);
+#pragma unroll
+          for (int q = 0; q < EPV; ++q) f[h * EPV + q] = part[q];
+        }
+      } else {
+#pragma unroll
+        for (int q = 0; q < GE; ++q) f[q] = 0.f;
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < GE; ++q) f[q] = (live[r] && c0 + q < v) ? Elem<T>::load1(x + row[r] * (int64_t)v + c0 + q) : 0.f;
+    }
+#pragma unroll
+    for (int q = 0; q < GE; ++q) key[r][q] = (live[r] && c0 + q < v) ? key_of(f[q]) : 0u;   // 0: below every real key
+  }
+  int mine[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) mine[r] = 0;
+#pragma unroll
+  for (int j = 0; j < kGroupMaxK; ++j) {
+    if (j < k) {
+      uint32_t bk[R], gk[R];
+      int bq[R], gi[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        bk[r] = key[r][0];
+        bq[r] = 0;
+#pragma unroll
+        for (int q = 1; q < GE; ++q) {
+          if (key[r][q] > bk[r]) { bk[r] = key[r][q]; bq[r] = q; }
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) gk[r] = lanes_max_u<L>(bk[r]);
+#pragma unroll
+      for (int r = 0; r < R; ++r) gi[r] = lanes_min_i<L>((bk[r] == gk[r]) ? c0 + bq[r] : 0x7fffffff);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int wl = gi[r] >> 3, wq = gi[r] & 7;
+#pragma unroll
+        for (int q = 0; q < GE; ++q) {
+          if (l == wl && q == wq) key[r][q] = 0u;
+        }
+        if (l == j) mine[r] = gi[r];
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (live[r] && l < k) {
+      const int64_t o = row[r] * (int64_t)k + l;
+      if (idx32 != nullptr) idx32[o] = mine[r];
+      if (idx64 != nullptr) idx64[o] = mine[r];
+      if (values != nullptr) values[o] = x[row[r] * (int64_t)v + mine[r]];
+    }
+  }
+}
+
 // widest row (in 16-byte vectors) whose key prefixes fit the LDS budget
 constexpr int kLdsMaxVec = 20480;
 // largest k the 128-thread form takes: the threshold of two full waves then still leaves the
@@ -410,7 +527,25 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
     // unit instead of eight (1.2-1.8x on rows of 2-24 K elements; even by 64 KiB rows).
     if (whole <= 3072 && k <= kSmallMaxK) variant = 4;
   }
-  if (v <= kWaveMaxV && !forced) {       // short rows: a wave per row
+  // narrow rows, few picks: lane groups. A pick costs a lane group as much as it costs the
+  // wave-per-row kernel, which pays it once per candidate set instead: past 256 columns that is
+  // cheaper from the third pick on.
+  if (v <= kGroupMaxV && k <= (v <= 256 ? kGroupMaxK : 2) && !forced) {
+    const bool gvec = vec_ok && v % 8 == 0;
+#define GOG(L_)                                                                                    \
+  do {                                                                                             \
+    constexpr int rows_per_block = 4 * (64 / L_) * kGroupRows;                                     \
+    const dim3 ggrid((unsigned)((n + rows_per_block - 1) / rows_per_block));                       \
+    if (gvec) hipLaunchKernelGGL((topk_group_kernel<T, L_, true>), ggrid, dim3(256), 0, st, xp, vp, i32, i64, n, v, k); \
+    else hipLaunchKernelGGL((topk_group_kernel<T, L_, false>), ggrid, dim3(256), 0, st, xp, vp, i32, i64, n, v, k);     \
+  } while (0)
+    if (v <= 64) GOG(8);
+    else if (v <= 128) GOG(16);
+    else if (v <= 256) GOG(32);
+    else GOG(64);
+#undef GOG
+  }
+  else if (v <= kWaveMaxV && !forced) {       // short rows: a wave per row
     int epl = 1;
     while (64 * epl < v) epl *= 2;
     const bool wvec = vec_ok && v % EPV == 0 && epl >= EPV;

@@ -667,6 +667,38 @@ def test_topk_ties_nans_zeros_and_degenerate_rows():
     assert torch.equal(run(x, 4), O.topk(x, 4)[1])
 
 
+def test_topk_lane_group_rows():
+    """Rows of at most 512 elements with k <= 8 take lane groups (several rows per wave): every
+    group width, widths that are not whole vectors, ties, NaNs, signed zeros, -inf, unaligned
+    buffers, and more rows than one workgroup holds."""
+    g = gen(1050)
+
+    def check(x, k):
+        ov, oi = O.topk(x, k)
+        for bits in (torch.int32, torch.int64):
+            vals, idx = _hip.topk(x.to(DEV), k, bits)
+            assert torch.equal(idx.cpu().long(), oi), (tuple(x.shape), x.dtype, k)
+            assert torch.equal(vals.cpu().nan_to_num(7.0), ov.nan_to_num(7.0)), (tuple(x.shape), x.dtype, k)
+    for dt in (BF16, F16, F32):
+        for v in (1, 2, 7, 8, 16, 60, 64, 65, 100, 128, 129, 200, 256, 257, 384, 500, 512):
+            n = 333 if v <= 64 else 77
+            x = (3 * torch.randn(n, v, generator=g)).to(dt)
+            for k in sorted({1, min(v, 2), min(v, 5), min(v, 8)}):
+                check(x, k)
+            t = torch.randint(0, 3, (n, v), generator=g).to(dt)         # heavy ties
+            t[::5, ::3] = float("nan")
+            t[1::5, 1::2] = float("-inf")
+            t[2::5, ::2] = -0.0
+            for k in sorted({1, min(v, 2), min(v, 8)}):
+                check(t, k)
+    z = torch.zeros(1000, 64)
+    check(z, 8)
+    base = (3 * torch.randn(1 + 50 * 128, generator=g)).to(BF16).to(DEV)
+    x = base[1:].view(50, 128)                                          # rows 2 bytes off 16-byte alignment
+    _, idx = _hip.topk(x, 4, torch.int32)
+    assert torch.equal(idx.cpu().long(), O.topk(x.cpu(), 4)[1])
+
+
 def test_topk_two_wave_rows():
     """Rows of 2-24 K elements with k <= 72 take the 128-thread form (512 candidate slots, half
     the work list): random rows around its bounds, then inputs that overflow its slots or its
