@@ -224,6 +224,34 @@ __device__ __forceinline__ int wave_min_i(int v) {
             mn(__builtin_amdgcn_readlane(v, 32), __builtin_amdgcn_readlane(v, 48)));
 }
 
+// The same two over aligned groups of L consecutive lanes (L = 8, 16, 32 or 64); every lane of a
+// group ends with the group's result.
+template <int L>
+__device__ __forceinline__ uint32_t group_max_u(uint32_t v) {
+  static_assert(L == 8 || L == 16 || L == 32 || L == 64, "group of 8, 16, 32 or 64 lanes");
+  if constexpr (L == 64) return wave_max_u(v);
+  auto mx = [](uint32_t a, uint32_t b) { return a > b ? a : b; };
+  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppXor1));
+  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppXor2));
+  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppHalfMirror));
+  if constexpr (L >= 16) v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppMirror));
+  if constexpr (L >= 32) v = mx(v, (uint32_t)__shfl_xor((int)v, 16, 64));
+  return v;
+}
+
+template <int L>
+__device__ __forceinline__ int group_min_i(int v) {
+  static_assert(L == 8 || L == 16 || L == 32 || L == 64, "group of 8, 16, 32 or 64 lanes");
+  if constexpr (L == 64) return wave_min_i(v);
+  auto mn = [](int a, int b) { return a < b ? a : b; };
+  v = mn(v, FM_DPP_I(v, kDppXor1));
+  v = mn(v, FM_DPP_I(v, kDppXor2));
+  v = mn(v, FM_DPP_I(v, kDppHalfMirror));
+  if constexpr (L >= 16) v = mn(v, FM_DPP_I(v, kDppMirror));
+  if constexpr (L >= 32) v = mn(v, __shfl_xor(v, 16, 64));
+  return v;
+}
+
 // Reduce across the T threads that share one row. T <= 64: a lane group inside one wave.
 // T > 64: T/64 whole waves of one workgroup; partials go through LDS and are combined in
 // wave order. `smem` must hold (rows per block) * (T/64) floats; `row_in_block` selects the

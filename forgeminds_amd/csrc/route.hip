@@ -39,32 +39,6 @@ __device__ __forceinline__ uint32_t key_of(float f) {
   return b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);
 }
 
-// Reductions over aligned groups of L consecutive lanes (L = 8, 16 or 32) for the keys and the
-// expert indices; every lane of a group ends with the group's result.
-template <int L>
-__device__ __forceinline__ uint32_t group_max_u(uint32_t v) {
-  if constexpr (L == 64) return wave_max_u(v);
-  auto mx = [](uint32_t a, uint32_t b) { return a > b ? a : b; };
-  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppXor1));
-  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppXor2));
-  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppHalfMirror));
-  if constexpr (L >= 16) v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppMirror));
-  if constexpr (L >= 32) v = mx(v, (uint32_t)__shfl_xor((int)v, 16, 64));
-  return v;
-}
-
-template <int L>
-__device__ __forceinline__ int group_min_i(int v) {
-  if constexpr (L == 64) return wave_min_i(v);
-  auto mn = [](int a, int b) { return a < b ? a : b; };
-  v = mn(v, FM_DPP_I(v, kDppXor1));
-  v = mn(v, FM_DPP_I(v, kDppXor2));
-  v = mn(v, FM_DPP_I(v, kDppHalfMirror));
-  if constexpr (L >= 16) v = mn(v, FM_DPP_I(v, kDppMirror));
-  if constexpr (L >= 32) v = mn(v, __shfl_xor(v, 16, 64));
-  return v;
-}
-
 constexpr int kGroupThreads = 256;    // 4 waves per tile
 constexpr int kGE = 8;                // experts a lane holds
 

@@ -364,30 +364,6 @@ __global__ __launch_bounds__(64) void topk_wave_kernel(const T* __restrict__ x, 
 // with 16-byte loads (VEC: v a multiple of eight, aligned buffer). Each of the k picks is a
 // lane-local first maximum, a group maximum over the keys and a group minimum over the indices
 // that hold it -- the canonical order (value descending, index ascending) by construction.
-template <int L>
-__device__ __forceinline__ uint32_t lanes_max_u(uint32_t v) {
-  if constexpr (L == 64) return wave_max_u(v);
-  auto mx = [](uint32_t a, uint32_t b) { return a > b ? a : b; };
-  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppXor1));
-  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppXor2));
-  v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppHalfMirror));
-  if constexpr (L >= 16) v = mx(v, (uint32_t)FM_DPP_I((int)v, kDppMirror));
-  if constexpr (L >= 32) v = mx(v, (uint32_t)__shfl_xor((int)v, 16, 64));
-  return v;
-}
-
-template <int L>
-__device__ __forceinline__ int lanes_min_i(int v) {
-  if constexpr (L == 64) return wave_min_i(v);
-  auto mn = [](int a, int b) { return a < b ? a : b; };
-  v = mn(v, FM_DPP_I(v, kDppXor1));
-  v = mn(v, FM_DPP_I(v, kDppXor2));
-  v = mn(v, FM_DPP_I(v, kDppHalfMirror));
-  if constexpr (L >= 16) v = mn(v, FM_DPP_I(v, kDppMirror));
-  if constexpr (L >= 32) v = mn(v, __shfl_xor(v, 16, 64));
-  return v;
-}
-
 constexpr int kGroupMaxV = 512;
 constexpr int kGroupMaxK = 8;
 constexpr int kGroupRows = 2;   // rows a lane group works on together (independent chains)
@@ -451,9 +427,9 @@ __global__ __launch_bounds__(256) void topk_group_kernel(const T* __restrict__ x
         }
       }
 #pragma unroll
-      for (int r = 0; r < R; ++r) gk[r] = lanes_max_u<L>(bk[r]);
+      for (int r = 0; r < R; ++r) gk[r] = group_max_u<L>(bk[r]);
 #pragma unroll
-      for (int r = 0; r < R; ++r) gi[r] = lanes_min_i<L>((bk[r] == gk[r]) ? c0 + bq[r] : 0x7fffffff);
+      for (int r = 0; r < R; ++r) gi[r] = group_min_i<L>((bk[r] == gk[r]) ? c0 + bq[r] : 0x7fffffff);
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         const int wl = gi[r] >> 3, wq = gi[r] & 7;
