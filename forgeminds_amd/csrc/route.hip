@@ -217,6 +217,127 @@ __global__ __launch_bounds__(kGroupThreads) void route_group_kernel(const T* __r
   }
 }
 
+// Gradient of the routing outputs wrt the logits, one pass over [n, e] with the lane groups of
+// route_group_kernel (one row per group): the softmax is recomputed, then
+//   through the renormalised top-k weights  w_j = p[idx_j] / S,  S = sum_j p[idx_j]:
+//     g_p[idx_j] = (gw_j - sum_i gw_i w_i) / S
+//   through aux = E * sum_e frac_e * mean_rows(p)_e  (frac = counts / (n k), a constant):
+//     g_p[e] += g_aux * E / n * frac_e
+//   through the softmax:  g_x = (g_p - sum_e g_p p) p
+//   through z = mean(lse^2):  g_x += g_z * 2 / n * lse * p.
+template <typename T, int L, bool VEC>
+__global__ __launch_bounds__(kGroupThreads) void route_bwd_kernel(const T* __restrict__ logits,
+                                                                   const int32_t* __restrict__ idx,
+                                                                   const float* __restrict__ gw,
+                                                                   const int32_t* __restrict__ counts,
+                                                                   const float* __restrict__ g_aux,
+                                                                   const float* __restrict__ g_z,
+                                                                   T* __restrict__ dlogits, int64_t n,
+                                                                   int e, int k) {
+  constexpr int GPW = 64 / L;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g = lane / L, l = lane % L;
+  const int ex0 = l * kGE;
+  const float ca = (g_aux != nullptr && counts != nullptr) ? *g_aux * (float)e / (float)n : 0.f;
+  const float cz = g_z != nullptr ? *g_z * 2.f / (float)n : 0.f;
+  float fr[kGE];
+#pragma unroll
+  for (int q = 0; q < kGE; ++q)
+    fr[q] = (ca != 0.f && ex0 + q < e) ? ca * ((float)counts[ex0 + q] / (float)(n * (int64_t)k)) : 0.f;
+  const int64_t row = ((int64_t)blockIdx.x * (kGroupThreads / 64) + wave) * GPW + g;
+  const bool live = row < n;
+  float p[kGE];
+  if constexpr (VEC) {
+    constexpr int EPV = Elem<T>::kVec;
+    if (live && ex0 < e) {
+#pragma unroll
+      for (int h = 0; h < kGE / EPV; ++h) {
+        float part[EPV];
+        Elem<T>::unpack(load16(logits + row * (int64_t)e + ex0 + h * EPV), part);
+#pragma unroll
+        for (int q = 0; q < EPV; ++q) p[h * EPV + q] = part[q];
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < kGE; ++q) p[q] = -INFINITY;
+    }
+  } else {
+#pragma unroll
+    for (int q = 0; q < kGE; ++q)
+      p[q] = (live && ex0 + q < e) ? Elem<T>::load1(logits + row * (int64_t)e + ex0 + q) : -INFINITY;
+  }
+  float m = p[0];
+#pragma unroll
+  for (int q = 1; q < kGE; ++q) m = fmaxf(m, p[q]);
+  m = group_reduce<L, OpMax>(m);
+  float s = 0.f;
+#pragma unroll
+  for (int q = 0; q < kGE; ++q) {
+    p[q] = fast_exp2((p[q] - m) * kLog2e);
+    s += p[q];
+  }
+  s = group_reduce<L, OpSum>(s);
+  const float inv = 1.f / s;
+  const float lse = m + fast_log2(s) * kLn2;
+#pragma unroll
+  for (int q = 0; q < kGE; ++q) p[q] *= inv;
+  // the selected experts of this row and the gradients of their weights
+  float gsel[kGE];
+  bool sel[kGE];
+#pragma unroll
+  for (int q = 0; q < kGE; ++q) { gsel[q] = 0.f; sel[q] = false; }
+  float s_loc = 0.f, d_loc = 0.f;
+#pragma unroll
+  for (int j = 0; j < kMaxK; ++j) {
+    if (j < k && live) {
+      const int ij = idx[row * (int64_t)k + j];
+      const float gj = gw != nullptr ? gw[row * (int64_t)k + j] : 0.f;
+#pragma unroll
+      for (int q = 0; q < kGE; ++q) {
+        if (ij == ex0 + q) {
+          sel[q] = true;
+          gsel[q] = gj;
+          s_loc += p[q];
+          d_loc += gj * p[q];
+        }
+      }
+    }
+  }
+  const float S = group_reduce<L, OpSum>(s_loc);
+  const float D = group_reduce<L, OpSum>(d_loc);
+  const float inv_s = 1.f / S;
+  const float mean = D * inv_s;
+  float gp[kGE];
+  float dot = 0.f;
+#pragma unroll
+  for (int q = 0; q < kGE; ++q) {
+    gp[q] = (sel[q] ? (gsel[q] - mean) * inv_s : 0.f) + fr[q];
+    dot += gp[q] * p[q];
+  }
+  dot = group_reduce<L, OpSum>(dot);
+  float o[kGE];
+#pragma unroll
+  for (int q = 0; q < kGE; ++q) o[q] = (gp[q] - dot) * p[q] + cz * lse * p[q];
+  if (!live) return;
+  T* op = dlogits + row * (int64_t)e + ex0;
+  if constexpr (VEC) {
+    constexpr int EPV = Elem<T>::kVec;
+    if (ex0 < e) {
+#pragma unroll
+      for (int h = 0; h < kGE / EPV; ++h) {
+        float part[EPV];
+#pragma unroll
+        for (int q = 0; q < EPV; ++q) part[q] = o[h * EPV + q];
+        store16(op + h * EPV, Elem<T>::pack(part));
+      }
+    }
+  } else {
+#pragma unroll
+    for (int q = 0; q < kGE; ++q)
+      if (ex0 + q < e) Elem<T>::store1(op + q, o[q]);
+  }
+}
+
 // Sums the per-tile partial rows [ntiles, e+1]: stats[0..e) = column sums of the probabilities,
 // stats[e] = sum of logsumexp^2. A workgroup owns 64 columns; wave w adds tiles w, w + 16, ...
 // of a column in that order, then the sixteen partial sums are added in wave order. The order
@@ -290,6 +411,29 @@ __global__ __launch_bounds__(1024) void hist_scan_kernel(int32_t* __restrict__ h
     const int t = t0 + u;
     if (col < e && u < per && t < ntiles) hist[(int64_t)t * e + col] = run;
     run += v[u];
+  }
+}
+
+// The two auxiliary losses from the finished sums (forgemind/moe.py:92-95), one workgroup:
+//   stats[e + 1] = aux = E * sum_c counts[c] / (n k) * stats[c] / n
+//   stats[e + 2] = z   = stats[e] / n
+__global__ __launch_bounds__(512) void route_aux_kernel(const int32_t* __restrict__ counts,
+                                                         float* __restrict__ stats, int64_t n, int e,
+                                                         int k) {
+  __shared__ float part[8];
+  const int c = threadIdx.x;
+  const float rows = n > 0 ? (float)n : 1.f;
+  const float slots = n > 0 ? (float)(n * (int64_t)k) : 1.f;
+  float a = c < e ? ((float)counts[c] / slots) * (stats[c] / rows) : 0.f;
+  a = wave_sum(a);
+  if ((c & 63) == 0) part[c >> 6] = a;
+  __syncthreads();
+  if (c == 0) {
+    float t = part[0];
+#pragma unroll
+    for (int w = 1; w < 8; ++w) t += part[w];
+    stats[e + 1] = (float)e * t;
+    stats[e + 2] = stats[e] / rows;
   }
 }
 
@@ -529,6 +673,53 @@ int fm_route(const void* logits, int32_t* idx, float* weights, int32_t* counts, 
                        counts, slot, order, n, e, k, tl.tile_rows, tl.ntiles, emit, scanned);
   }
   FM_CHECK_LAUNCH("fm_route(permute)");
+  if (stats != nullptr) {
+    hipLaunchKernelGGL(route_aux_kernel, dim3(1), dim3(512), 0, st, counts, stats, n, e, k);
+    FM_CHECK_LAUNCH("fm_route(aux)");
+  }
+  return FM_OK;
+}
+
+int fm_route_bwd(const void* logits, const int32_t* idx, const float* gweights, const int32_t* counts,
+                 const float* g_aux, const float* g_z, void* dlogits, int64_t n, int e, int k, int dtype,
+                 fm_stream_t stream) {
+  FM_CHECK_ARG(n >= 0 && e > 0 && k >= 1, "fm_route_bwd: bad shape n=%lld e=%d k=%d", (long long)n, e, k);
+  FM_CHECK_ARG(dtype == FM_F32 || dtype == FM_F16 || dtype == FM_BF16, "fm_route_bwd: bad dtype %d", dtype);
+  FM_CHECK_ARG(k <= e, "fm_route_bwd: selected index k out of range (got %d vs %d)", k, e);
+  if (e > kMaxE || k > kMaxK || n * (int64_t)k >= 0x7fffffffLL) {
+    fm_host::set_error("fm_route_bwd: e <= %d, k <= %d and n*k < 2^31 required (e=%d k=%d n=%lld)", kMaxE,
+                       kMaxK, e, k, (long long)n);
+    return FM_ERR_UNSUPPORTED;
+  }
+  FM_CHECK_ARG(g_aux == nullptr || counts != nullptr, "fm_route_bwd: g_aux needs counts");
+  if (n == 0) return FM_OK;
+  FM_CHECK_ARG(logits && idx && dlogits, "fm_route_bwd: NULL pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool vec = e % kGE == 0 && fm_host::aligned16(logits) && fm_host::aligned16(dlogits);
+#define GOB(T, L_)                                                                                   \
+  do {                                                                                               \
+    constexpr int rows_per_block = (kGroupThreads / 64) * (64 / L_);                                 \
+    const dim3 grid((unsigned)((n + rows_per_block - 1) / rows_per_block));                          \
+    if (vec) hipLaunchKernelGGL((route_bwd_kernel<T, L_, true>), grid, dim3(kGroupThreads), 0, st,   \
+                                static_cast<const T*>(logits), idx, gweights, counts, g_aux, g_z,    \
+                                static_cast<T*>(dlogits), n, e, k);                                  \
+    else hipLaunchKernelGGL((route_bwd_kernel<T, L_, false>), grid, dim3(kGroupThreads), 0, st,      \
+                            static_cast<const T*>(logits), idx, gweights, counts, g_aux, g_z,        \
+                            static_cast<T*>(dlogits), n, e, k);                                      \
+  } while (0)
+#define BY_L(T)                 \
+  do {                          \
+    if (e <= 64) GOB(T, 8);     \
+    else if (e <= 128) GOB(T, 16); \
+    else if (e <= 256) GOB(T, 32); \
+    else GOB(T, 64);            \
+  } while (0)
+  if (dtype == FM_F32) BY_L(float);
+  else if (dtype == FM_BF16) BY_L(bf16_t);
+  else BY_L(f16_t);
+#undef BY_L
+#undef GOB
+  FM_CHECK_LAUNCH("fm_route_bwd");
   return FM_OK;
 }
 

@@ -72,6 +72,7 @@ SIGNATURES = {
     "fm_qk_norm_rope_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64, _i64, _i64,
                                    _int, _int, _vp]),
     "fm_route": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _int, _int, _int, _vp]),
+    "fm_route_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _int, _vp]),
 }
 
 
@@ -464,7 +465,8 @@ def softmax_bwd(y2, dy2):
 
 def route(logits2, k: int, want_permutation: bool = True, want_stats: bool = False):
     """-> (idx int32 [n, k], weights fp32 [n, k], counts int32 [e], slot, order int32 [n*k])
-    and, with want_stats, a sixth item: fp32 [e+1] = column sums of probs, then sum(lse^2)."""
+    and, with want_stats, a sixth item: fp32 [e+3] = column sums of probs, sum(lse^2), then the
+    load-balance loss and the z-loss themselves."""
     _dense(logits2)
     n, e = logits2.shape
     dev = logits2.device
@@ -473,7 +475,7 @@ def route(logits2, k: int, want_permutation: bool = True, want_stats: bool = Fal
     counts = torch.empty(e, device=dev, dtype=torch.int32)
     slot = torch.empty(n * k, device=dev, dtype=torch.int32) if want_permutation else None
     order = torch.empty(n * k, device=dev, dtype=torch.int32) if want_permutation else None
-    stats = torch.empty(e + 1, device=dev, dtype=torch.float32) if want_stats else None
+    stats = torch.empty(e + 3, device=dev, dtype=torch.float32) if want_stats else None
     with _guard(dev):
         nbytes = int(lib().fm_route_workspace(n, e, k))
         ws = torch.empty(max(nbytes, 16), device=dev, dtype=torch.uint8)
@@ -483,6 +485,20 @@ def route(logits2, k: int, want_permutation: bool = True, want_stats: bool = Fal
     if want_stats:
         return idx, wts, counts, slot, order, stats
     return idx, wts, counts, slot, order
+
+
+def route_bwd(logits2, idx, gweights, counts, g_aux, g_z):
+    """-> dlogits like logits2. gweights fp32 [n, k] or None; g_aux / g_z fp32 device scalars or
+    None (g_aux needs counts)."""
+    _dense(logits2, idx, gweights, counts)
+    n, e = logits2.shape
+    k = idx.shape[1]
+    out = torch.empty_like(logits2)
+    with _guard(logits2.device):
+        _check(lib().fm_route_bwd(_ptr(logits2), _ptr(idx), _ptr(gweights), _ptr(counts), _ptr(g_aux),
+                                  _ptr(g_z), _ptr(out), n, e, int(k), dtype_code(logits2.dtype),
+                                  _stream(logits2)), "fm_route_bwd")
+    return out
 
 
 # ------------------------------------------------------------------ token moves around the permutation

@@ -55,24 +55,16 @@ def _torch_route(logits: torch.Tensor, k: int, with_aux: bool = False) -> Routin
                    order.to(torch.int32), aux, z)
 
 
-def _aux_z(counts, stats, n: int, k: int, e: int):
-    """aux = E * sum(frac * mean_rows(probs)), z = mean(logsumexp^2) (reference moe.py:92-95)."""
-    frac = counts.to(torch.float32) / max(n * k, 1)
-    aux = e * (frac * (stats[:e] / max(n, 1))).sum()
-    z = stats[e] / max(n, 1)
-    return aux, z
-
-
 class _RouteFn(torch.autograd.Function):
     """Weights and the two auxiliary losses are differentiable wrt the logits; every integer
-    output is not. The backward recomputes softmax on the small [n, e] tensor with tensor ops."""
+    output is not. The backward is one kernel that recomputes the softmax of the [n, e] logits."""
 
     @staticmethod
     def forward(ctx, logits, k, with_aux):
         n, e = logits.shape
         if with_aux:
             idx, w, counts, slot, order, stats = _hip.route(logits.contiguous(), k, True, True)
-            aux, z = _aux_z(counts, stats, n, k, e)
+            aux, z = stats[e + 1], stats[e + 2]      # both losses come finished from the kernel
         else:
             idx, w, counts, slot, order = _hip.route(logits.contiguous(), k, True)
             aux = z = logits.new_zeros((), dtype=torch.float32)
@@ -84,27 +76,14 @@ class _RouteFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, _gi, gw, _gc, _gs, _go, g_aux, g_z):
         logits, idx, counts = ctx.saved_tensors
-        n, e = logits.shape
-        lf = logits.float()
-        lse = torch.logsumexp(lf, dim=-1, keepdim=True)
-        p = torch.exp(lf - lse)
-        g_p = torch.zeros_like(p)
+        if not ctx.with_aux:
+            g_aux = g_z = None
+
+        def scalar(t):
+            return None if t is None else t.detach().to(torch.float32).reshape(()).contiguous()
         if gw is not None:
-            # through the renormalise and the gather: w = p_top / sum(p_top)
-            pk = torch.gather(p, 1, idx.long())
-            s = pk.sum(dim=-1, keepdim=True)
-            w = pk / s
-            g_pk = (gw - (gw * w).sum(dim=-1, keepdim=True)) / s
-            g_p.scatter_(1, idx.long(), g_pk)
-        g_logits = None
-        if ctx.with_aux and g_aux is not None:
-            # aux = E * sum_e frac_e * mean_rows(p)_e, with frac a constant (no_grad in moe.py:92-93)
-            frac = counts.to(torch.float32) / max(n * ctx.k, 1)
-            g_p = g_p + g_aux * (e / max(n, 1)) * frac
-        g_logits = (g_p - (g_p * p).sum(dim=-1, keepdim=True)) * p          # through the softmax
-        if ctx.with_aux and g_z is not None:
-            g_logits = g_logits + g_z * (2.0 / max(n, 1)) * lse * p          # d mean(lse^2) / dlogits
-        return g_logits.to(logits.dtype), None, None
+            gw = gw.detach().to(torch.float32).contiguous()
+        return _hip.route_bwd(logits.contiguous(), idx, gw, counts, scalar(g_aux), scalar(g_z)), None, None
 
 
 def moe_route(logits: torch.Tensor, k: int, with_aux: bool = False) -> Routing:

@@ -255,14 +255,26 @@ int fm_softmax_bwd(const void* y, const void* dy, void* dx, int64_t n, int64_t v
  *   order[slot[p]] = p  (== torch.sort(flat, stable=True).indices).
  * logits: [n, e] of dtype (fp32 math inside); idx: [n, k] int32; weights: [n, k] fp32;
  * counts: [e] int32; slot, order: [n*k] int32 (either may be NULL: then only routing and
- * counts are produced when both are NULL). stats: fp32 [e+1] or NULL; receives what the
- * auxiliary losses of moe.py:92-95 need without another pass over the logits:
+ * counts are produced when both are NULL). stats: fp32 [e+3] or NULL; receives the auxiliary
+ * losses of moe.py:92-95 and the sums behind them, without another pass over the logits:
  *   stats[j] = sum_rows probs[:, j] (j < e),  stats[e] = sum_rows logsumexp(logits)^2,
+ *   stats[e+1] = aux = E * sum_j counts[j] / (n k) * stats[j] / n,  stats[e+2] = z = stats[e] / n,
  * summed in a fixed order. 1 <= k <= 8, k <= e <= 512, n*k < 2^31. */
 size_t fm_route_workspace(int64_t n, int e, int k);
 int fm_route(const void* logits, int32_t* idx, float* weights, int32_t* counts, int32_t* slot,
              int32_t* order, float* stats, void* workspace, size_t workspace_bytes, int64_t n,
              int e, int k, int dtype, fm_stream_t stream);
+
+/* Gradient of fm_route's differentiable outputs wrt the logits, in one pass. Replaces what
+ * autograd derives from Router.forward (forgemind/moe.py:86-95): through the renormalised top-k
+ * weights (gweights: fp32 [n, k] gradient of `weights`, or NULL), through the load-balance loss
+ * aux = E * sum_e frac_e * mean_rows(probs)_e with frac = counts / (n k) held constant
+ * (moe.py:92-94; g_aux: fp32 device scalar or NULL, needs counts), and through the z-loss
+ * mean_rows(logsumexp^2) (moe.py:95; g_z: fp32 device scalar or NULL). idx, counts: as written
+ * by fm_route. dlogits: [n, e] of dtype. Same limits as fm_route. */
+int fm_route_bwd(const void* logits, const int32_t* idx, const float* gweights, const int32_t* counts,
+                 const float* g_aux, const float* g_z, void* dlogits, int64_t n, int e, int k, int dtype,
+                 fm_stream_t stream);
 
 /* ------------------------------------------------------------------ token moves around the permutation
  * Replaces `xs = x[order // k]` (forgemind/moe.py:234-235): xs[s, :] = scale * x[order[s] / k, :]

@@ -14,7 +14,8 @@ sign here fails there.
 Pinning status (see tests/test_oracle.py): every function below is pinned; none is
 "parity unpinned". The reference's own tests hold no value-level vectors for the router
 (idx / weights / permutation); those are pinned by the integer closed forms instead
-(bincount, stable argsort, inverse permutation) and by brute force on small inputs.
+(bincount, stable argsort, inverse permutation) and by brute force on small inputs; the
+router's gradient is pinned against torch's autograd of the reference expression.
 
 ``acc`` is the accumulation dtype: ``torch.float32`` reproduces the reference's fallback
 (fp32 for half inputs, reference forgemind/kernels/_fallback.py:15-23), ``torch.float64`` is
@@ -254,6 +255,35 @@ def router_aux(logits, idx):
     aux = e * (frac * probs.mean(dim=0)).sum()
     z = torch.logsumexp(lf, dim=-1).pow(2).mean()
     return aux, z
+
+
+def router_bwd(logits, k, gweights=None, g_aux=None, g_z=None, acc=torch.float64):
+    """d(sum(weights * gweights) + g_aux * aux + g_z * z) / d logits, [n, e] in `acc`.
+
+    The closed form of what autograd derives from the reference's Router.forward
+    (forgemind/moe.py:86-95), with the top-k indices and the per-expert fractions held constant
+    (moe.py:92-93 computes `frac` under no_grad; indices carry no gradient):
+      w_j = p[idx_j] / S, S = sum_j p[idx_j]   ->  g_p[idx_j] = (gw_j - sum_i gw_i w_i) / S
+      aux = E * sum_e frac_e * mean_rows(p)_e  ->  g_p[e] += g_aux * E / n * frac_e
+      softmax                                  ->  g_x = (g_p - sum_e g_p p) p
+      z = mean_rows(lse^2)                     ->  g_x += g_z * 2 / n * lse * p."""
+    idx, _w, counts, _slot, _order = router(logits, k)
+    n, e = logits.shape
+    lf = _up(logits, torch.float32).to(acc)
+    lse = torch.logsumexp(lf, dim=-1, keepdim=True)
+    p = torch.exp(lf - lse)
+    g_p = torch.zeros_like(p)
+    if gweights is not None:
+        pk = torch.gather(p, 1, idx)
+        s = pk.sum(dim=-1, keepdim=True)
+        gw = gweights.to(acc)
+        g_p.scatter_(1, idx, (gw - (gw * pk / s).sum(dim=-1, keepdim=True)) / s)
+    if g_aux is not None:
+        g_p = g_p + float(g_aux) * (e / max(n, 1)) * (counts.to(acc) / max(idx.numel(), 1))
+    g = (g_p - (g_p * p).sum(dim=-1, keepdim=True)) * p
+    if g_z is not None:
+        g = g + float(g_z) * (2.0 / max(n, 1)) * lse * p
+    return g
 
 
 # ------------------------------------------------------------------ token moves around the permutation

@@ -36,7 +36,7 @@ def lib():
 
 def test_header_and_binding_agree(lib):
     decl = _declared()
-    assert len(decl) == 37
+    assert len(decl) == 38
     assert set(decl) == set(_hip.SIGNATURES), set(decl) ^ set(_hip.SIGNATURES)
     for name, nargs in decl.items():
         assert hasattr(lib, name), f"{name} is declared in fm_hip.h but not exported"
@@ -76,3 +76,8 @@ def test_argument_validation_happens_before_any_launch(lib):
     assert b"sum or mean" in lib.fm_last_error()
     assert lib.fm_kl_loss_grad_topk(*args, 4, 8, 2, 2, 32, 1.0, 2, None) == 1          # no gradient buffer
     assert lib.fm_rmsnorm_bwd_workspace(0, 8, 2) == 0
+    # the router's backward validates like the router
+    assert lib.fm_route_bwd(None, None, None, None, None, None, None, 4, 8, 9, 0, None) == 1      # k > e
+    assert lib.fm_route_bwd(None, None, None, None, None, None, None, 4, 1024, 2, 0, None) == 2   # e > 512
+    assert lib.fm_route_bwd(None, None, None, None, None, None, None, 0, 8, 2, 0, None) == 0      # no rows
+    assert lib.fm_route_bwd(None, None, None, None, None, None, None, 4, 8, 2, 0, None) == 1      # NULL buffers

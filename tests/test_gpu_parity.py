@@ -853,6 +853,36 @@ def test_route_is_bit_exact(n, e, k):
     aux, z = O.router_aux(lg, oi)
     got_aux = e * ((counts.cpu().float() / (n * k)) * (stats[:e].cpu() / n)).sum()
     assert got_aux.item() == pytest.approx(aux.item(), rel=1e-4) and (stats[e] / n).item() == pytest.approx(z.item(), rel=1e-4)
+    assert stats.shape == (e + 3,)                                   # and finished, as the last two entries
+    assert stats[e + 1].item() == pytest.approx(aux.item(), rel=1e-4) and stats[e + 2].item() == pytest.approx(z.item(), rel=1e-4)
+
+
+ROUTE_BWD_CASES = [(16384, 64, 2, F32), (1000, 8, 2, F32), (513, 128, 4, BF16), (100, 300, 8, F32), (1, 64, 2, F32),
+                   (257, 512, 8, F16), (4099, 60, 6, F32), (3, 2, 2, F32), (700, 65, 2, BF16), (900, 256, 8, F32)]
+
+
+@pytest.mark.parametrize("n,e,k,dt", ROUTE_BWD_CASES)
+def test_route_bwd_matches_the_oracle(n, e, k, dt):
+    """The router's gradient (reference: autograd through moe.py:86-95) from one kernel: through
+    the weights, the load-balance loss and the z-loss, separately and together."""
+    lg = router_inputs(n, e, 1007, dt)
+    g = gen(1008)
+    gw = torch.randn(n, k, generator=g)
+    idx, w, counts, _, _ = _hip.route(lg.to(DEV), k)
+    lgd = lg.to(DEV)
+    for use_w, ga, gz in ((True, None, None), (False, 0.7, None), (False, None, -1.3), (True, 0.01, 0.001)):
+        want = O.router_bwd(lg, k, gw if use_w else None, ga, gz)
+        got = _hip.route_bwd(lgd, idx, gw.to(DEV) if use_w else None, counts,
+                             None if ga is None else torch.tensor(ga, device=DEV),
+                             None if gz is None else torch.tensor(gz, device=DEV))
+        assert got.dtype == dt and got.shape == (n, e)
+        # the terms that cancel inside (g_p - sum g_p p) p set the absolute error, not the result
+        terms = (gw.abs().max().item() if use_w else 0.0) + abs(ga or 0.0) * e / n + abs(gz or 0.0) * 2 / n * 20
+        scale = want.abs().max().item()
+        tol = (1e-2 if dt != F32 else 2e-5) * scale + 1e-6 * terms
+        assert (got.double().cpu() - want).abs().max().item() <= tol, (use_w, ga, gz)
+    # nothing upstream: zeros
+    assert not _hip.route_bwd(lgd, idx, None, None, None, None).any()
 
 
 def test_route_half_precision_logits_and_all_equal_rows():

@@ -392,6 +392,41 @@ def test_router_brute_force_small():
     assert slot.tolist() == [2, 4, 0, 3, 1, 5]
 
 
+def test_router_bwd_matches_autograd_of_the_reference_expression():
+    """Router.forward of the reference (moe.py:86-95) typed out in float64 and differentiated by
+    torch.autograd: weights, load-balance loss and z-loss, separately and together; a dropped
+    term, a wrong sign or a 1/n in the wrong place fails here."""
+    g = torch.Generator().manual_seed(77)
+    for n, e, k in ((9, 8, 2), (33, 64, 6), (5, 3, 3), (17, 130, 1)):
+        logits = torch.round(torch.randn(n, e, generator=g) * 64) / 64
+        idx, *_ = O.router(logits, k)
+        gw = torch.randn(n, k, generator=g)
+        for use_w, ga, gz in ((True, None, None), (False, 0.7, None), (False, None, -1.3), (True, 0.01, 0.001)):
+            lf = logits.double().requires_grad_(True)
+            probs = lf.softmax(-1)
+            w, _ = probs.gather(1, idx), None
+            w = w / w.sum(-1, keepdim=True)
+            with torch.no_grad():
+                frac = torch.bincount(idx.reshape(-1), minlength=e).double() / idx.numel()
+            aux = e * (frac * probs.mean(0)).sum()
+            z = lf.logsumexp(-1).pow(2).mean()
+            total = lf.sum() * 0
+            if use_w:
+                total = total + (w * gw.double()).sum()
+            if ga is not None:
+                total = total + ga * aux
+            if gz is not None:
+                total = total + gz * z
+            (want,) = torch.autograd.grad(total, lf)
+            got = O.router_bwd(logits, k, gw if use_w else None, ga, gz)
+            assert torch.allclose(got, want, rtol=1e-10, atol=1e-12), (n, e, k, use_w, ga, gz)
+    # rows of the weight gradient sum to zero (softmax), and a constant gw gives no gradient
+    # (the renormalised weights sum to one)
+    logits = torch.randn(11, 16, generator=g)
+    assert O.router_bwd(logits, 4, torch.randn(11, 4, generator=g)).sum(-1).abs().max() < 1e-12
+    assert O.router_bwd(logits, 4, torch.full((11, 4), 3.0)).abs().max() < 1e-12
+
+
 def test_router_aux_matches_the_reference_expression():
     # forgemind/moe.py:92-95 written out with library calls
     torch.manual_seed(1)
