@@ -53,8 +53,9 @@ class Router(nn.Module):
         self.last_plan: "Dispatch | None" = None
 
     def forward(self, x: torch.Tensor):
-        logits = self.gate(x).float()
-        plan = dispatch_plan(logits, self.top_k, x.dtype)
+        # the reference casts the gate output to fp32 first (moe.py:87); the routing kernels read
+        # half logits and do the same fp32 math, so the cast (and its backward) is not materialised
+        plan = dispatch_plan(self.gate(x), self.top_k, x.dtype)
         self.last_plan = plan       # MoE.forward reuses order / counts instead of re-sorting
         return plan.weights, plan.idx, plan.aux, plan.z
 
