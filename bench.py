@@ -4,8 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extras] [--no-cpu]
 
 NAME: ce (headline), ce_one_pass, rmsnorm, add_rmsnorm, add_layernorm, kl, kl_one_launch, kl_topk, kl_topk_one_launch, topk,
-route,
-moe_dispatch, swiglu, qk_norm_rope.
+route, route_train, moe_dispatch, swiglu, qk_norm_rope.
 
 A step is one pass of the hot path (forward + backward) over one batch of synthetic,
 seeded input that is already resident in HBM, launched straight through the C ABI of
@@ -52,7 +51,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="ce",
-                    choices=["ce", "ce_one_pass", "rmsnorm", "add_rmsnorm", "add_layernorm", "kl", "kl_one_launch", "kl_topk", "kl_topk_one_launch", "topk", "route", "moe_dispatch", "swiglu", "qk_norm_rope"])
+                    choices=["ce", "ce_one_pass", "rmsnorm", "add_rmsnorm", "add_layernorm", "kl", "kl_one_launch", "kl_topk", "kl_topk_one_launch", "topk", "route", "route_train", "moe_dispatch", "swiglu", "qk_norm_rope"])
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
@@ -452,6 +451,43 @@ def make_workload(name, torch, L, dev):
         w.rows = n
         return w
 
+    if name == "route_train":
+        # what a training step runs around the router: routing with the statistics and the two
+        # auxiliary losses, then the gradient wrt the logits in one kernel
+        n, e, k = 16384, 64, 2
+        g.manual_seed(1003)
+        lg = torch.round(torch.randn(n, e, device=dev, generator=g) * 4096) / 4096
+        idx = torch.empty(n, k, device=dev, dtype=torch.int32)
+        wt = torch.empty(n, k, device=dev)
+        cnt = torch.empty(e, device=dev, dtype=torch.int32)
+        sl = torch.empty(n * k, device=dev, dtype=torch.int32)
+        od = torch.empty(n * k, device=dev, dtype=torch.int32)
+        stats = torch.empty(e + 3, device=dev)
+        gw = torch.randn(n, k, device=dev, generator=g)
+        ga, gz = torch.tensor(0.01, device=dev), torch.tensor(0.001, device=dev)
+        dl = torch.empty_like(lg)
+        nb = L.fm_route_workspace(n, e, k)
+        ws = torch.empty(max(nb, 16), device=dev, dtype=torch.uint8)
+
+        def bwd():
+            _check(L.fm_route_bwd(lg.data_ptr(), idx.data_ptr(), gw.data_ptr(), cnt.data_ptr(), ga.data_ptr(),
+                                  gz.data_ptr(), dl.data_ptr(), n, e, k, F32c, st), "fm_route_bwd")
+
+        def step():
+            _check(L.fm_route(lg.data_ptr(), idx.data_ptr(), wt.data_ptr(), cnt.data_ptr(), sl.data_ptr(),
+                              od.data_ptr(), stats.data_ptr(), ws.data_ptr(), nb, n, e, k, F32c, st), "fm_route")
+            bwd()
+
+        w.step = step
+        w.dominant_launch = bwd
+        w.dominant = "route_bwd_kernel<f32,8>"
+        w.dominant_bytes = n * e * 4 * 2
+        w.bytes = n * (e * 4 + k * 4 * 4) + w.dominant_bytes
+        w.desc = (f"router with statistics and auxiliary losses + its gradient, logits fp32 [{n},{e}], top-{k}")
+        w.unit = "rows/s"
+        w.rows = n
+        return w
+
     if name == "moe_dispatch":
         n, e, k, d = 16384, 64, 2, 4096
         g.manual_seed(1008)
@@ -654,7 +690,7 @@ def main():
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": res["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16" if a.workload != "route" else "f32", "data": "synthetic",
+        "dtype": "bf16" if a.workload not in ("route", "route_train") else "f32", "data": "synthetic",
         "config": {"workload": head.desc, "name": a.workload,
                    "timing": "K steps between two device synchronisations, inputs resident in HBM"},
         "roofline": {
@@ -670,7 +706,7 @@ def main():
     torch.cuda.empty_cache()
     if not a.no_extras:
         extras = {a.workload: res}
-        for name in ["rmsnorm", "add_rmsnorm", "add_layernorm", "ce", "ce_one_pass", "kl", "kl_one_launch", "kl_topk", "kl_topk_one_launch", "topk", "route", "moe_dispatch", "swiglu", "qk_norm_rope"]:
+        for name in ["rmsnorm", "add_rmsnorm", "add_layernorm", "ce", "ce_one_pass", "kl", "kl_one_launch", "kl_topk", "kl_topk_one_launch", "topk", "route", "route_train", "moe_dispatch", "swiglu", "qk_norm_rope"]:
             if name == a.workload:
                 continue
             wl = make_workload(name, torch, L, dev)
