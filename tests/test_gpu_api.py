@@ -448,6 +448,9 @@ def test_loss_selection_and_routing_launches_replay_in_a_graph():
     short = torch.randn(500, 1000, generator=g).to(DEV)
     logits = torch.randn(2048, 64, generator=g).to(DEV)
     xs = torch.randn(2048, 512, generator=g).bfloat16().to(DEV)
+    aligned = torch.randn(700, 512, generator=g).bfloat16().to(DEV)
+    aligned2 = torch.randn(700, 512, generator=g).bfloat16().to(DEV)
+    ya = torch.randint(0, 512, (700,), generator=g).to(DEV)
 
     def step():
         out = []
@@ -462,9 +465,16 @@ def test_loss_selection_and_routing_launches_replay_in_a_graph():
         out += list(_hip.topk(short, 300, torch.int32))
         sm = _hip.softmax_fwd(short)
         out += [sm, _hip.softmax_bwd(sm, short)]
-        idx, wts, counts, slot, order = _hip.route(logits, 2)
+        idx, wts, counts, slot, order, stats = _hip.route(logits, 2, True, True)
         gathered = _hip.moe_gather(xs, order, 2)
-        out += [idx, wts, counts, slot, order, gathered, _hip.moe_combine(gathered, wts, slot, 2048, 2)]
+        out += [idx, wts, counts, slot, order, stats, gathered, _hip.moe_combine(gathered, wts, slot, 2048, 2)]
+        out += [_hip.route_bwd(logits, idx, wts, counts, stats[65], stats[66])]
+        # the lane-group forms: narrow top-k, rows of whole vectors in the loss kernels, and the
+        # two-wave top-k of rows of a few thousand elements
+        out += list(_hip.topk(logits, 2, torch.int32)) + list(_hip.topk(lg, 8, torch.int32))
+        l3, d3, _, r3 = _hip.ce_loss_grad(aligned, ya, -100, "mean")
+        k3, g3, rk3 = _hip.kl_loss_grad(aligned, aligned2, 1.0, "mean", torch.bfloat16)
+        out += [l3, d3, r3, k3, g3, rk3]
         out += [_hip.swiglu_split_fwd(xs), _hip.swiglu_split_bwd(xs, xs[:, :256].contiguous())]
         return out
 
