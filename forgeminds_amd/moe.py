@@ -6,8 +6,6 @@ stay with the caller.
 
 from __future__ import annotations
 
-from typing import NamedTuple
-
 import torch
 import torch.nn as nn
 
@@ -16,30 +14,53 @@ from .kernels import moe_combine, moe_gather, moe_route
 __all__ = ["Router", "Dispatch", "dispatch_plan", "Experts", "MoE"]
 
 
-class Dispatch(NamedTuple):
-    """What ``MoE.forward`` needs after routing (reference ``moe.py:232-241``)."""
+class Dispatch:
+    """What ``MoE.forward`` needs after routing (reference ``moe.py:232-241``).
 
-    weights: torch.Tensor   # [n, k] in the activation dtype
-    idx: torch.Tensor       # [n, k] int64
-    order: torch.Tensor     # [n*k] int64: flat assignments grouped by expert (stable)
-    tok: torch.Tensor       # [n*k] int64: order // k, the token of each grouped assignment
-    slot: torch.Tensor      # [n*k] int32: inverse of `order`
-    order32: torch.Tensor   # [n*k] int32 copy of `order` for the token-move kernels
-    counts: torch.Tensor    # [e] int64
-    offsets: torch.Tensor   # [e] int32 inclusive cumsum of counts (torch._grouped_mm offsets)
-    aux: torch.Tensor       # load-balance loss
-    z: torch.Tensor         # router z-loss
+    The kernels' own outputs are held as they come; the int64 / cumulative forms the reference
+    works with (``order``, ``tok``, ``counts``, ``offsets``) are derived on first use, so a
+    caller that only moves tokens through ``order32`` / ``slot`` pays for none of them."""
+
+    __slots__ = ("weights", "idx", "slot", "order32", "counts32", "aux", "z", "top_k", "_lazy")
+
+    def __init__(self, weights, idx, slot, order32, counts32, aux, z, top_k):
+        self.weights = weights      # [n, k] in the activation dtype
+        self.idx = idx              # [n, k] int64
+        self.slot = slot            # [n*k] int32: inverse of `order`
+        self.order32 = order32      # [n*k] int32: flat assignments grouped by expert (stable)
+        self.counts32 = counts32    # [e] int32
+        self.aux = aux              # load-balance loss
+        self.z = z                  # router z-loss
+        self.top_k = top_k
+        self._lazy = {}
+
+    def _once(self, name, make):
+        if name not in self._lazy:
+            self._lazy[name] = make()
+        return self._lazy[name]
+
+    @property
+    def order(self) -> torch.Tensor:      # [n*k] int64, what torch.sort(flat, stable=True) returns
+        return self._once("order", lambda: self.order32.long())
+
+    @property
+    def tok(self) -> torch.Tensor:        # [n*k] int64: order // k, the token of each grouped assignment
+        return self._once("tok", lambda: self.order // self.top_k)
+
+    @property
+    def counts(self) -> torch.Tensor:     # [e] int64
+        return self._once("counts", lambda: self.counts32.long())
+
+    @property
+    def offsets(self) -> torch.Tensor:    # [e] int32 inclusive cumsum of counts (torch._grouped_mm offsets)
+        return self._once("offsets", lambda: self.counts32.cumsum(0).to(torch.int32))
 
 
 def dispatch_plan(logits: torch.Tensor, top_k: int, out_dtype=None) -> Dispatch:
     """Everything the expert layer needs from ``[n, e]`` router logits."""
     r = moe_route(logits, top_k, with_aux=True)
-    aux, z = r.aux, r.z
-    order = r.order.long()
-    counts = r.counts.long()
     w = r.weights if out_dtype is None else r.weights.to(out_dtype)
-    return Dispatch(w, r.idx.long(), order, order // top_k, r.slot, r.order, counts,
-                    counts.cumsum(0).to(torch.int32), aux, z)
+    return Dispatch(w, r.idx.long(), r.slot, r.order, r.counts, r.aux, r.z, top_k)
 
 
 class Router(nn.Module):
@@ -104,6 +125,6 @@ class MoE(nn.Module):
         plan = self.router.last_plan
         self.last_aux = self.aux_coef * aux + self.z_coef * z
         xs = moe_gather(x2, plan.order32, self.top_k, plan.slot)
-        ys = self.experts(xs, plan.counts.tolist())          # the one host sync of the eager path
+        ys = self.experts(xs, plan.counts32.tolist())        # the one host sync of the eager path
         out = moe_combine(ys, w, plan.slot, plan.order32)
         return out.reshape(shape)
