@@ -69,6 +69,9 @@ def main():
     d.update(route_logits=lr.numpy(), route_idx=ri.numpy().astype(np.int32), route_w=rw.numpy(),
              route_counts=rc.numpy().astype(np.int32), route_slot=rs.numpy().astype(np.int32),
              route_order=ro.numpy().astype(np.int32))
+    # the router's gradient: through the weights, the load-balance loss and the z-loss
+    gw = torch.randn(300, 2, generator=g)
+    d.update(route_gw=gw.numpy(), route_grad=O.router_bwd(lr, 2, gw, 0.01, 0.001, acc=torch.float64).numpy())
     np.savez_compressed(OUT, **d)
     print("wrote", OUT, os.path.getsize(OUT), "bytes,", len(d), "arrays")
 

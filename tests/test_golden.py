@@ -41,6 +41,8 @@ def test_oracle_reproduces_the_vectors(gv):
     ri, rw, rc, rs, ro = O.router(torch.from_numpy(gv["route_logits"]), 2)
     assert np.array_equal(ri.numpy(), gv["route_idx"]) and np.array_equal(ro.numpy(), gv["route_order"])
     assert np.array_equal(rs.numpy(), gv["route_slot"]) and np.array_equal(rc.numpy(), gv["route_counts"])
+    rg = O.router_bwd(torch.from_numpy(gv["route_logits"]), 2, torch.from_numpy(gv["route_gw"]), 0.01, 0.001)
+    assert np.allclose(rg.numpy(), gv["route_grad"], rtol=1e-12, atol=1e-15)
 
 
 @pytest.mark.gpu
@@ -81,3 +83,6 @@ def test_kernels_match_the_vectors(gv):
     assert np.array_equal(idx.cpu().numpy(), gv["route_idx"]) and np.array_equal(counts.cpu().numpy(), gv["route_counts"])
     assert np.array_equal(slot.cpu().numpy(), gv["route_slot"]) and np.array_equal(order.cpu().numpy(), gv["route_order"])
     assert np.allclose(wts.cpu().numpy(), gv["route_w"], rtol=1e-5)
+    rg = _hip.route_bwd(torch.from_numpy(gv["route_logits"]).to(dev), idx, torch.from_numpy(gv["route_gw"]).to(dev),
+                        counts, torch.tensor(0.01, device=dev), torch.tensor(0.001, device=dev))
+    assert np.abs(rg.cpu().numpy() - gv["route_grad"]).max() <= 2e-5 * np.abs(gv["route_grad"]).max() + 1e-9
