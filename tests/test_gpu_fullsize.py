@@ -83,6 +83,19 @@ def test_config3_router_16384x64():
     flat = idx.reshape(-1).long()
     assert torch.equal(slot.long()[order.long()], torch.arange(32768, device=DEV))
     assert (flat[order.long()].diff() >= 0).all()
+    # the gradient at the same size: against the oracle, and through what the softmax fixes --
+    # rows of the weight and load-balance gradients sum to zero, rows of the z-loss gradient to
+    # g_z * 2 / n * logsumexp
+    lgd = lg.to(DEV)
+    gw = torch.randn(16384, 2, generator=g)
+    got = _hip.route_bwd(lgd, idx, gw.to(DEV), counts, torch.tensor(0.01, device=DEV), torch.tensor(0.001, device=DEV))
+    want = O.router_bwd(lg, 2, gw, 0.01, 0.001)
+    assert (got.double().cpu() - want).abs().max().item() <= 2e-5 * want.abs().max().item() + 1e-9
+    only_w = _hip.route_bwd(lgd, idx, gw.to(DEV), counts, torch.tensor(1.0, device=DEV), None)
+    assert only_w.double().sum(-1).abs().max().item() < 1e-5
+    only_z = _hip.route_bwd(lgd, idx, None, None, None, torch.tensor(1.0, device=DEV))
+    lse = torch.logsumexp(lg.double(), -1)
+    assert torch.allclose(only_z.double().sum(-1).cpu(), 2.0 / 16384 * lse, rtol=1e-4, atol=1e-9)
 
 
 def test_config4_add_rmsnorm_16384x8192():
