@@ -463,6 +463,9 @@ def softmax_bwd(y2, dy2):
     return dx
 
 
+_ROUTE_WS: dict = {}     # (rows, experts, k) -> workspace bytes; the answer depends on nothing else
+
+
 def route(logits2, k: int, want_permutation: bool = True, want_stats: bool = False):
     """-> (idx int32 [n, k], weights fp32 [n, k], counts int32 [e], slot, order int32 [n*k])
     and, with want_stats, a sixth item: fp32 [e+3] = column sums of probs, sum(lse^2), then the
@@ -477,7 +480,10 @@ def route(logits2, k: int, want_permutation: bool = True, want_stats: bool = Fal
     order = torch.empty(n * k, device=dev, dtype=torch.int32) if want_permutation else None
     stats = torch.empty(e + 3, device=dev, dtype=torch.float32) if want_stats else None
     with _guard(dev):
-        nbytes = int(lib().fm_route_workspace(n, e, k))
+        key = (n, e, k)
+        nbytes = _ROUTE_WS.get(key)
+        if nbytes is None:
+            nbytes = _ROUTE_WS[key] = int(lib().fm_route_workspace(n, e, k))
         ws = torch.empty(max(nbytes, 16), device=dev, dtype=torch.uint8)
         _check(lib().fm_route(_ptr(logits2), _ptr(idx), _ptr(wts), _ptr(counts), _ptr(slot),
                               _ptr(order), _ptr(stats), _ptr(ws), nbytes, n, e, int(k),
