@@ -565,7 +565,7 @@ __global__ __launch_bounds__(256) void ce_vrows_kernel(const T* logits, const in
   for (int i = 0; i < ITERS; ++i) {
     if (read && i * TPR + t < nvec) {
       float f[EPV];
-      Elem<T>::unpack(r[i], f);
+      unpack_again<T, (ITERS >= 8)>(r[i], f);
 #pragma unroll
       for (int e = 0; e < EPV; ++e) m = fmaxf(m, f[e] * kLog2e);
     }
@@ -579,7 +579,7 @@ __global__ __launch_bounds__(256) void ce_vrows_kernel(const T* logits, const in
     const int c = i * TPR + t;
     if (read && c < nvec) {
       float f[EPV];
-      Elem<T>::unpack(r[i], f);
+      unpack_again<T, (ITERS >= 8)>(r[i], f);
 #pragma unroll
       for (int e = 0; e < EPV; ++e) {
         const float z = f[e] * kLog2e;
@@ -606,7 +606,7 @@ __global__ __launch_bounds__(256) void ce_vrows_kernel(const T* logits, const in
       const int c = i * TPR + t;
       if (valid && c < nvec) {
         float f[EPV], o[EPV];
-        if (!ignored) Elem<T>::unpack(r[i], f);
+        if (!ignored) unpack_again<T, (ITERS >= 8)>(r[i], f);
 #pragma unroll
         for (int e = 0; e < EPV; ++e) {
           float p = ignored ? 0.f : fast_exp2(f[e] * kLog2e - m) * inv;
@@ -627,7 +627,7 @@ bool vrows_fits(int v, int esize, bool bf16, const void* logits, const void* dlo
   const int epv = 16 / esize;
   int lim = fm_host::get_param(fm_host::P_ROWS_VEC_MAX);
   // eight vectors per lane only pay for bf16 (the other types then run at a quarter of the occupancy)
-  const int top = loss && !grad && esize == 2 && bf16 ? kVRowsMaxVec : kVRowsMaxVec / 2;
+  const int top = loss && !grad ? kVRowsMaxVec : kVRowsMaxVec / 2;
   if (lim <= 0 || lim > top) lim = top;
   return v % epv == 0 && v / epv <= lim && fm_host::aligned16(logits) && (!grad || fm_host::aligned16(dlogits));
 }
@@ -654,7 +654,7 @@ bool launch_vrows(const void* logits, const int64_t* labels, const float* n_vali
     return true;                                                                                    \
   }
   GOV(4, 1) GOV(4, 2) GOV(4, 4) GOV(8, 4) GOV(16, 4) GOV(32, 4) GOV(64, 4)
-  if constexpr (std::is_same<T, bf16_t>::value && LOSS && !GRAD) { GOV(64, 8) }
+  if constexpr (LOSS && !GRAD) { GOV(64, 8) }
 #undef GOV
   return false;
 }

@@ -152,6 +152,16 @@ __device__ __forceinline__ void store16_stream(T* p, const u32x4& v) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
 }
 
+// Unpack a vector that is used by several passes without letting the compiler keep the
+// converted floats of the first pass alive for the later ones (fp16 conversions are otherwise
+// hoisted, and eight vectors per lane then take 230 registers instead of 60). FRESH = false is
+// the plain unpack.
+template <typename T, bool FRESH, int N>
+__device__ __forceinline__ void unpack_again(u32x4 raw, float (&f)[N]) {
+  if constexpr (FRESH) asm volatile("" : "+v"(raw.x), "+v"(raw.y), "+v"(raw.z), "+v"(raw.w));
+  Elem<T>::unpack(raw, f);
+}
+
 // ---------------------------------------------------------------- wave reductions (DPP)
 __device__ __forceinline__ int lane_id() {
   return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
