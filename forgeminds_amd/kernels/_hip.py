@@ -181,6 +181,12 @@ def _dense(*ts):
 
 def set_param(name: str, value: int) -> None:
     _check(lib().fm_set_param(name.encode(), int(value)), "fm_set_param")
+    # workspace sizes follow the launch shapes, which the tuning parameters move
+    for cache in _SIZE_CACHES:
+        cache.clear()
+
+
+_SIZE_CACHES: list = []
 
 
 # ------------------------------------------------------------------ norm
@@ -197,7 +203,8 @@ def rmsnorm_fwd(x2: torch.Tensor, w: torch.Tensor, eps: float):
     return y, rstd
 
 
-_WS_BYTES: dict = {}     # (device, rows, width, dtype) -> bytes; the answer depends on nothing else
+_WS_BYTES: dict = {}     # (device, rows, width, dtype) -> bytes, until a tuning parameter changes
+_SIZE_CACHES.append(_WS_BYTES)
 
 
 def _norm_ws(n: int, d: int, x: torch.Tensor, want_dw: bool):
@@ -463,7 +470,8 @@ def softmax_bwd(y2, dy2):
     return dx
 
 
-_ROUTE_WS: dict = {}     # (rows, experts, k) -> workspace bytes; the answer depends on nothing else
+_ROUTE_WS: dict = {}     # (rows, experts, k) -> workspace bytes, until a tuning parameter changes
+_SIZE_CACHES.append(_ROUTE_WS)
 
 
 def route(logits2, k: int, want_permutation: bool = True, want_stats: bool = False):

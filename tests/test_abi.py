@@ -81,3 +81,11 @@ def test_argument_validation_happens_before_any_launch(lib):
     assert lib.fm_route_bwd(None, None, None, None, None, None, None, 4, 1024, 2, 0, None) == 2   # e > 512
     assert lib.fm_route_bwd(None, None, None, None, None, None, None, 0, 8, 2, 0, None) == 0      # no rows
     assert lib.fm_route_bwd(None, None, None, None, None, None, None, 4, 8, 2, 0, None) == 1      # NULL buffers
+
+
+def test_set_param_forgets_cached_workspace_sizes(lib):
+    # the sizes follow the launch shapes, which the tuning parameters move
+    _hip._WS_BYTES[("probe",)] = 1
+    _hip._ROUTE_WS[("probe",)] = 1
+    _hip.set_param("norm_bwd_blocks_per_cu", 0)
+    assert not _hip._WS_BYTES and not _hip._ROUTE_WS
