@@ -80,6 +80,21 @@ int fm_rmsnorm_bwd(const void* x, const void* w, const float* rstd, const void* 
                    void* dw, void* workspace, size_t workspace_bytes, int64_t n, int64_t d,
                    int x_dtype, int w_dtype, fm_stream_t stream);
 
+/* fm_rmsnorm_bwd for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the same kernels and the same results,
+ * with the partial weight gradients in a buffer of FM_RMSNORM_BWD_STATIC_BYTES that is built
+ * into the library (one copy per GPU, held until the process ends) instead of a workspace
+ * argument. No counterpart in the reference. Allocates nothing; the first call on a device
+ * looks the buffer's address up once (make that call before starting a capture). Shapes whose
+ * partial rows need more than the buffer (fm_rmsnorm_bwd_workspace(n, d, x_dtype) >
+ * FM_RMSNORM_BWD_STATIC_BYTES; every shape with d <= 8192 fits) return FM_ERR_UNSUPPORTED. All calls on one
+ * GPU share the buffer: calls that overlap in time on one GPU (two streams) race; calls on one
+ * stream, or on different GPUs, do not. */
+#define FM_RMSNORM_BWD_STATIC_BYTES ((size_t)8 << 20)
+int fm_rmsnorm_bwd_static(const void* x, const void* w, const float* rstd, const void* dy, void* dx,
+                          void* dw, int64_t n, int64_t d, int x_dtype, int w_dtype,
+                          fm_stream_t stream);
+
 /* Replaces _launch_addrms_fwd / _addrms_fwd (norm.py:1118-1131, 1001-1047) with the
  * rounding points of _fallback.add_rms_norm (_fallback.py:33-35):
  *   xn = x + delta rounded to x's dtype; y = rms_norm(xn, w, eps) computed from the rounded xn. */
