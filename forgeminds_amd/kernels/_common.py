@@ -10,9 +10,11 @@ Mirrors the contract of the reference's ``forgemind/kernels/_common.py:47-119``:
 * nothing is counted while ``torch.compile`` traces (a dict update inside a checkpointed
   region would force a graph break, reference ``_common.py:84-96``).
 
-One deliberate difference: tensors on a GPU with the HIP library missing raise instead of
-quietly running torch ops. A GPU box without the extension is a broken install, not a
-supported configuration.
+The library missing or unloadable is the reference's ``"no triton"`` case
+(``_common.py:104-106``): under ``"auto"`` the wrappers run the torch expression and
+``stats()["reasons"]`` counts ``"no extension"``; ``available()`` is False. A forced backend
+(``"triton"`` / ``"hip"``) raises instead, and so do ``bench.py`` and ``smoke()``, which ask for
+the library itself.
 """
 
 from __future__ import annotations
@@ -81,11 +83,17 @@ def _note(why: str) -> None:
 
 
 def fast_ok(*tensors) -> bool:
-    """Can the HIP kernels run on these tensors right now?"""
+    """Can the HIP kernels run on these tensors right now? (Order of the checks as in the
+    reference, ``_common.py:99-119``: backend, extension, then the tensors.)"""
     if _BACKEND == "fallback":
         _note("backend=fallback")
         return False
-    on_gpu = False
+    if not _hip.loaded():
+        if forced():
+            raise RuntimeError(f"kernel backend {_BACKEND!r} is forced but the HIP extension is "
+                               f"unavailable ({_hip.load_error()})")
+        _note("no extension")
+        return False
     for t in tensors:
         if not isinstance(t, torch.Tensor):
             continue
@@ -95,16 +103,9 @@ def fast_ok(*tensors) -> bool:
                                    f"{t.device}; the HIP kernels need GPU tensors")
             _note("not cuda")
             return False
-        on_gpu = True
         if t.dtype not in _FLOATS:
             _note(f"dtype {t.dtype}")
             return False
-    if not _hip.loaded():
-        if on_gpu or forced():
-            raise RuntimeError("forgeminds_amd: tensors are on a GPU but the HIP extension is "
-                               f"unavailable ({_hip.load_error()})")
-        _note("no extension")
-        return False
     if not tracing():
         _STATS["fast"] += 1
     return True

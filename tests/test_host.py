@@ -56,6 +56,32 @@ def test_forced_backend_refuses_cpu_tensors_loudly():
         kernels.rms_norm(torch.randn(4, 8), torch.randn(8), 1e-6)
 
 
+def test_missing_extension_falls_back_with_a_reason(monkeypatch):
+    # reference _common.py:104-106 ("no triton"): no library -> torch expression, counted, no error
+    from forgeminds_amd.kernels import _fallback, _hip
+    monkeypatch.setattr(_hip, "loaded", lambda: False)
+    monkeypatch.setattr(_hip, "load_error", lambda: "libfmhip.so is missing (test)")
+    assert kernels.available() is False
+    g = torch.Generator().manual_seed(5)
+    x, w = torch.randn(6, 32, generator=g), torch.randn(32, generator=g)
+    delta = torch.randn(6, 32, generator=g)
+    s, t = torch.randn(4, 50, generator=g), torch.randn(4, 50, generator=g)
+    kernels.reset_stats()
+    assert torch.equal(kernels.rms_norm(x, w, 1e-6), _fallback.rms_norm(x, w, 1e-6))
+    xn, y = kernels.add_rms_norm(x, delta, w, 1e-6)
+    rxn, ry = _fallback.add_rms_norm(x, delta, w, 1e-6)
+    assert torch.equal(xn, rxn) and torch.equal(y, ry)
+    assert torch.equal(kernels.kl_div_logits(s, t), _fallback.kl_div_logits(s, t))
+    v, i = kernels.topk(s, 3)
+    assert torch.equal(v, torch.topk(s, 3).values)
+    st = kernels.stats()
+    assert st["fast"] == 0 and st["fallback"] == 4 and st["reasons"] == {"no extension": 4}
+    # a forced backend still refuses loudly
+    kernels.set_backend("hip")
+    with pytest.raises(RuntimeError, match="HIP extension is unavailable"):
+        kernels.rms_norm(x, w, 1e-6)
+
+
 def test_stats_are_not_touched_while_tracing():
     # reference tests/test_kernels.py:188-199
     kernels.reset_stats()
