@@ -29,25 +29,51 @@ class _CrossEntropyFn(torch.autograd.Function):
         lg2 = logits.contiguous().view(-1, logits.shape[-1])
         y = labels.contiguous().view(-1)
         ctx.shape = logits.shape
-        ctx.spent = False
+        ctx.mode = "none"
+        ctx.args = (ignore_index, reduction)
         if not ctx.needs_input_grad[0]:
             loss, _lse, _n_valid, _rows = _hip.ce_fwd(lg2, y, ignore_index, reduction)
             return loss.clone()     # `loss` is a view into a 2-element scratch tensor
+        if logits.dtype == torch.float16:
+            # (softmax - onehot) / n_valid stored in fp16 before the upstream gradient is applied
+            # would flush most entries to zero or to subnormals (p / 8192 < 6e-5) and a loss
+            # scaler could no longer bring them back: fp16 keeps the two-pass dataflow, whose
+            # backward applies the upstream gradient in fp32 and rounds once, as autograd does
+            # for F.cross_entropy (reference loss.py:65-70)
+            loss, lse, n_valid, _rows = _hip.ce_fwd(lg2, y, ignore_index, reduction)
+            ctx.mode = "two_pass"
+            ctx.save_for_backward(lg2, y, lse, n_valid.clone())
+            return loss.clone()
         # writing into the caller's storage is only done when asked for and when lg2 is that
         # storage (contiguous() did not copy)
         own = inplace and lg2.data_ptr() == logits.data_ptr()
         loss, dl, _n_valid, _rows = _hip.ce_loss_grad(lg2.detach(), y, ignore_index, reduction, own)
-        ctx.save_for_backward(dl)
+        ctx.mode = "own" if own else "private"
+        ctx.spent = False
+        if own:
+            ctx.save_for_backward(dl)
+        else:
+            ctx.save_for_backward(dl, lg2.detach(), y)   # the logits are intact: a later backward can redo the pass
         return loss.clone()
 
     @staticmethod
     def backward(ctx, g):
-        (dl,) = ctx.saved_tensors
-        if ctx.spent:
-            raise RuntimeError("cross_entropy: the gradient buffer written in the forward was already "
-                               "consumed by a backward pass; run the forward again")
-        ctx.spent = True
         g32 = g.detach().to(torch.float32).contiguous()
+        ignore_index, reduction = ctx.args
+        if ctx.mode == "two_pass":
+            lg2, y, lse, n_valid = ctx.saved_tensors
+            dl = _hip.ce_bwd(lg2, y, lse, n_valid if reduction == "mean" else None, g32, ignore_index)
+            return dl.view(ctx.shape), None, None, None, None
+        if ctx.mode == "own":
+            (dl,) = ctx.saved_tensors
+            if ctx.spent:
+                raise RuntimeError("cross_entropy: the gradient buffer written in the forward was already "
+                                   "consumed by a backward pass; run the forward again")
+        else:
+            dl, lg2, y = ctx.saved_tensors
+            if ctx.spent:   # retain_graph / a second autograd.grad: the first pass scaled `dl` in place
+                _loss, dl, _n, _r = _hip.ce_loss_grad(lg2, y, ignore_index, reduction, False)
+        ctx.spent = True
         _hip.scale_inplace(dl, g32)
         return dl.view(ctx.shape), None, None, None, None
 
@@ -105,7 +131,11 @@ def cross_entropy(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int 
 
     ``inplace=True`` lets the kernel write the gradient over ``logits`` (only for a tensor the
     caller owns and no longer reads, e.g. the output of the head projection): no second
-    ``[N, V]`` buffer exists. The gradient buffer serves one backward pass.
+    ``[N, V]`` buffer exists, and that buffer serves ONE backward pass (a second one raises).
+    Without ``inplace`` the backward may run any number of times (``retain_graph=True``): the
+    first scales the gradient the forward wrote, later ones redo the pass from the logits.
+    fp16 logits always take the two-pass form (forward keeps the log-sum-exps, the backward
+    applies the upstream gradient in fp32 before its one rounding), so a loss scaler works.
     """
     if reduction not in ("mean", "sum"):
         raise ValueError(f"reduction must be mean|sum, got {reduction!r}")

@@ -37,13 +37,20 @@ class _KLDivFn(torch.autograd.Function):
         ctx.meta = (student.shape, reduction, gdt, inv_t)
         ctx.in_forward = False
         ctx.spent = False
-        if reduction != "none" and ctx.needs_input_grad[0]:
+        # fp16 gradients are not written in the forward: (p_s - p_t) / N rounded to fp16 before the
+        # upstream gradient (a loss scale) is applied would flush to zero; the two-pass backward
+        # below scales in fp32 and rounds once
+        if reduction != "none" and ctx.needs_input_grad[0] and gdt != torch.float16:
             # gradient written in the forward (reference kl.py:143-176); `reuse` lets it land in
             # the student's own storage when that is the tensor the caller handed in
-            own = reuse and s2.data_ptr() == student.data_ptr()
+            own = reuse and s2.data_ptr() == student.data_ptr() and gdt == s2.dtype
             loss, grad, _rows = _hip.kl_loss_grad(s2.detach(), t2, inv_t, reduction, gdt, own)
             ctx.in_forward = True
-            ctx.save_for_backward(grad)
+            ctx.own = own
+            if own:
+                ctx.save_for_backward(grad)
+            else:
+                ctx.save_for_backward(grad, s2.detach(), t2)   # inputs intact: a later backward can redo the pass
             return loss
         loss, rows, lse_s, lse_t = _hip.kl_fwd(s2, t2, inv_t, reduction)
         ctx.save_for_backward(s2, t2, lse_s, lse_t)
@@ -55,10 +62,16 @@ class _KLDivFn(torch.autograd.Function):
     def backward(ctx, g):
         shape, reduction, gdt, inv_t = ctx.meta
         if ctx.in_forward:
-            (grad,) = ctx.saved_tensors
-            if ctx.spent:
-                raise RuntimeError("kl_div_logits: the gradient buffer written in the forward was "
-                                   "already consumed by a backward pass; run the forward again")
+            if ctx.own:
+                (grad,) = ctx.saved_tensors
+                if ctx.spent:
+                    raise RuntimeError("kl_div_logits: the gradient buffer written in the forward was "
+                                       "already consumed by a backward pass; run the forward again")
+            else:
+                grad, s2, t2 = ctx.saved_tensors
+                if ctx.spent:   # retain_graph: the first backward scaled `grad` in place (the reference
+                    # multiplies out of place, kl.py:183-191, so repeated backward works there too)
+                    _loss, grad, _rows = _hip.kl_loss_grad(s2, t2, inv_t, reduction, gdt, False)
             ctx.spent = True
             _hip.scale_inplace(grad, g.detach().to(torch.float32).contiguous())
             return grad.view(shape), None, None, None, None, None
@@ -84,7 +97,8 @@ class _KLDivTopkFn(torch.autograd.Function):
         ctx.spent = False
         # KL, the teacher's top-k and (when the student needs it, in its own dtype) the gradient
         # for an upstream gradient of 1, all from one launch
-        with_grad = reduction != "none" and ctx.needs_input_grad[0] and gdt == student.dtype
+        with_grad = (reduction != "none" and ctx.needs_input_grad[0] and gdt == student.dtype
+                     and gdt != torch.float16)
         out = _hip.kl_fwd_topk(s2.detach(), t2, k, inv_t, reduction, index_dtype, want_grad=with_grad)
         if out is None:   # row too wide for the fused kernel: two launches, same results
             with_grad = False
@@ -95,7 +109,7 @@ class _KLDivTopkFn(torch.autograd.Function):
             loss, rows, lse_s, lse_t, _, idx, probs = out[:7]
         if with_grad:
             ctx.in_forward = True
-            ctx.save_for_backward(out[7])
+            ctx.save_for_backward(out[7], s2.detach(), t2)
         else:
             ctx.save_for_backward(s2, t2, lse_s, lse_t)
         ctx.meta = (student.shape, reduction, gdt, inv_t)
@@ -111,10 +125,9 @@ class _KLDivTopkFn(torch.autograd.Function):
     def backward(ctx, g, _gp, _gi):
         shape, reduction, gdt, inv_t = ctx.meta
         if ctx.in_forward:
-            (grad,) = ctx.saved_tensors
-            if ctx.spent:
-                raise RuntimeError("kl_div_logits_topk: the gradient buffer written in the forward was "
-                                   "already consumed by a backward pass; run the forward again")
+            grad, s2, t2 = ctx.saved_tensors
+            if ctx.spent:       # a repeated backward redoes the gradient from the intact inputs
+                _loss, grad, _rows = _hip.kl_loss_grad(s2, t2, inv_t, reduction, gdt, False)
             ctx.spent = True
             _hip.scale_inplace(grad, g.detach().to(torch.float32).contiguous())
             return grad.view(shape), None, None, None, None, None, None

@@ -83,23 +83,50 @@ class Router(nn.Module):
 
 class Experts(nn.Module):
     """Stacked SwiGLU experts run as a per-expert loop over contiguous token groups -- the
-    eager path of the reference's ``Experts`` (``forgemind/moe.py:99-164``). The grouped GEMM
-    and expert parallelism of the reference are outside this build."""
+    eager path of the reference's ``Experts`` (``forgemind/moe.py:99-181``), with its
+    constructor order ``(n_local, dim, hidden)``, its ``normal(std=0.02)`` initialisation and its
+    ``forward(x, counts=None, offsets=None)``. The grouped GEMM (``grouped_mm=True`` is accepted
+    and, as in the reference when ``torch._grouped_mm`` is unusable, runs the loop) and the
+    host-offloaded layout are outside this build."""
 
-    def __init__(self, dim: int, hidden: int, n_experts: int):
+    def __init__(self, n_local: int, dim: int, hidden: int, offload: bool = False, grouped_mm: bool = False):
         super().__init__()
-        scale = dim ** -0.5
-        self.w1 = nn.Parameter(torch.randn(n_experts, dim, hidden) * scale)
-        self.w3 = nn.Parameter(torch.randn(n_experts, dim, hidden) * scale)
-        self.w2 = nn.Parameter(torch.randn(n_experts, hidden, dim) * hidden ** -0.5)
+        if offload:
+            raise ValueError("Experts(offload=True): host-offloaded experts are not part of this build")
+        self.n_local, self.offload, self.grouped = int(n_local), False, False
+        self.w1 = nn.Parameter(torch.empty(n_local, dim, hidden))
+        self.w3 = nn.Parameter(torch.empty(n_local, dim, hidden))
+        self.w2 = nn.Parameter(torch.empty(n_local, hidden, dim))
+        self.reset_parameters(dim, hidden)
 
-    def forward(self, xs: torch.Tensor, counts) -> torch.Tensor:
-        out = torch.empty_like(xs)
+    def reset_parameters(self, dim=None, hidden=None):
+        for w in (self.w1, self.w3, self.w2):
+            nn.init.normal_(w, std=0.02)
+
+    def forward(self, x: torch.Tensor, counts=None, offsets=None) -> torch.Tensor:
+        """``counts``: per-expert group sizes, a python list or a tensor; ``offsets``: cumulative
+        group ends instead (reference ``moe.py:146-159``). Neither: one group."""
+        if counts is None:
+            if offsets is None:
+                counts = [x.size(0)]
+            else:
+                o = offsets.to(torch.int64)
+                counts = torch.diff(o, prepend=o.new_zeros(1)).tolist()
+        elif torch.is_tensor(counts):
+            counts = counts.tolist()
+        sizes = [int(c) for c in counts]
+        if not any(sizes):
+            return x.new_zeros((0,) + tuple(x.shape[1:]))
+        dt = x.dtype
+        out = torch.empty_like(x)
         lo = 0
-        for e, c in enumerate(counts):
+        for e, c in enumerate(sizes):
             if c:
-                seg = xs[lo:lo + c]
-                out[lo:lo + c] = (torch.nn.functional.silu(seg @ self.w1[e]) * (seg @ self.w3[e])) @ self.w2[e]
+                seg = x[lo:lo + c]
+                a, b, o = self.w1[e], self.w3[e], self.w2[e]
+                if a.dtype is not dt:
+                    a, b, o = a.to(dt), b.to(dt), o.to(dt)
+                out[lo:lo + c] = (torch.nn.functional.silu(seg @ a) * (seg @ b)) @ o
             lo += c
         return out
 
@@ -107,14 +134,25 @@ class Experts(nn.Module):
 class MoE(nn.Module):
     """Single-device mixture of experts with the forward of the reference's ``MoE.forward``
     (``forgemind/moe.py:227-251``, ``ep_size == 1``): route, gather tokens by expert, run the
-    experts on contiguous groups, return the weighted outputs to their tokens. Routing and
-    both token moves are fused kernels; ``last_aux`` carries the auxiliary losses."""
+    experts on contiguous groups, return the weighted outputs to their tokens (plus the shared
+    SwiGLU when ``n_shared`` > 0). Routing and both token moves are fused kernels; ``last_aux``
+    carries the auxiliary losses. Constructor arguments in the reference's order
+    (``moe.py:184-186``); expert parallelism and offloaded experts raise."""
 
-    def __init__(self, dim: int, hidden: int, n_experts: int, top_k: int, aux_coef: float = 0.01,
-                 z_coef: float = 1e-3):
+    def __init__(self, dim: int, hidden: int, n_experts: int, top_k: int, n_shared: int = 0, ep_size: int = 1,
+                 ep_group=None, ep_rank: int = 0, offload_experts: bool = False, grouped_mm: bool = False,
+                 aux_coef: float = 1e-2, z_coef: float = 1e-3):
         super().__init__()
+        if ep_size != 1 or ep_group is not None or ep_rank != 0:
+            raise ValueError("MoE: expert parallelism (ep_size > 1) is not part of this one-GPU build")
+        self.dim, self.n_experts = int(dim), int(n_experts)
+        self.ep_size, self.ep_group, self.ep_rank, self.n_local = 1, None, 0, int(n_experts)
         self.router = Router(dim, n_experts, top_k)
-        self.experts = Experts(dim, hidden, n_experts)
+        self.experts = Experts(n_experts, dim, hidden, offload=offload_experts, grouped_mm=grouped_mm)
+        self.shared = None
+        if n_shared:
+            from .nn import SwiGLU
+            self.shared = SwiGLU(dim, hidden * int(n_shared))
         self.top_k, self.aux_coef, self.z_coef = int(top_k), aux_coef, z_coef
         self.last_aux = None
 
@@ -127,4 +165,6 @@ class MoE(nn.Module):
         xs = moe_gather(x2, plan.order32, self.top_k, plan.slot)
         ys = self.experts(xs, plan.counts32.tolist())        # the one host sync of the eager path
         out = moe_combine(ys, w, plan.slot, plan.order32)
+        if self.shared is not None:
+            out = out + self.shared(x2)
         return out.reshape(shape)

@@ -248,6 +248,66 @@ def test_kl_gradient_in_forward_reuse_and_second_backward():
     assert hs.grad is not None and w.grad is not None and hs.grad.abs().sum() > 0
 
 
+def test_fp16_losses_apply_the_upstream_gradient_before_rounding():
+    # a loss scaler multiplies the loss by 65536; (softmax - onehot) / 8192 rounded to fp16 FIRST
+    # would lose most entries (p / 8192 < 6e-5 is subnormal or zero in fp16)
+    g = torch.Generator().manual_seed(77)
+    n, v, scale = 8192, 512, 65536.0
+    lg = (2 * torch.randn(n, v, generator=g)).half()
+    y = torch.randint(0, v, (n,), generator=g)
+    y[::9] = -100
+    ref = lg.double().requires_grad_(True)           # fp64 autograd of the library routine, unrounded
+    (F.cross_entropy(ref, y, ignore_index=-100) * scale).backward()
+    want = ref.grad
+    lgd = lg.to(DEV).requires_grad_(True)
+    (kernels.cross_entropy(lgd, y.to(DEV)) * scale).backward()
+    got = lgd.grad.double().cpu()
+    assert lgd.grad.dtype == torch.float16
+    # one fp16 rounding of the scaled value: half an ulp relative, nothing flushed
+    err = (got - want).abs()
+    assert (err <= want.abs() * 2.0 ** -10 + 2.0 ** -24).all()
+    assert torch.count_nonzero(got) >= 0.99 * torch.count_nonzero(want)
+    # KL with an fp16 gradient: same rule
+    s = (3 * torch.randn(4096, 256, generator=g)).half()
+    t = (s.float() + 0.5 * torch.randn(4096, 256, generator=g)).half()
+    sref = s.double().requires_grad_(True)
+    (F.kl_div(torch.log_softmax(sref, -1), torch.softmax(t.double(), -1), reduction="sum") / 4096 * scale).backward()
+    wantk = sref.grad
+    sd = s.to(DEV).requires_grad_(True)
+    (kernels.kl_div_logits(sd, t.to(DEV)) * scale).backward()
+    errk = (sd.grad.double().cpu() - wantk).abs()
+    # one fp16 rounding, plus the fp32 rounding of the two probabilities (up to 1) whose difference
+    # the gradient is, times the factor scale / rows = 16 they are multiplied by
+    assert (errk <= wantk.abs() * 2.0 ** -10 + (scale / 4096) * 2.0 ** -20).all()
+    assert torch.count_nonzero(sd.grad) >= 0.99 * torch.count_nonzero(wantk)
+
+
+def test_losses_allow_a_second_backward_when_the_gradient_buffer_is_private():
+    # the reference's KL multiplies its stored gradient out of place (kernels/kl.py:183-191), so
+    # retain_graph=True works there; here the first backward scales in place and later ones redo the pass
+    g = torch.Generator().manual_seed(78)
+    lg = (2 * torch.randn(64, 4000, generator=g)).bfloat16()
+    y = torch.randint(0, 4000, (64,), generator=g)
+    _, og = O.cross_entropy(lg, y)
+    lgd = lg.to(DEV).requires_grad_(True)
+    loss = kernels.cross_entropy(lgd, y.to(DEV))
+    (loss * 3.0).backward(retain_graph=True)
+    first = lgd.grad.clone()
+    lgd.grad = None
+    (loss * 5.0).backward()
+    assert close(first, og.float() * 3.0) and close(lgd.grad, og.float() * 5.0)
+    s = (3 * torch.randn(12, 3000, generator=g)).bfloat16()
+    t = (s.float() + 0.5 * torch.randn(12, 3000, generator=g)).bfloat16()
+    _, kg = O.kl_div(s, t, "mean", 1.0)
+    sd = s.to(DEV).requires_grad_(True)
+    kl = kernels.kl_div_logits(sd, t.to(DEV))
+    (kl * 2.0).backward(retain_graph=True)
+    a = sd.grad.clone()
+    sd.grad = None
+    kl.backward()
+    assert close(a, kg.float() * 2.0) and close(sd.grad, kg.float())
+
+
 def test_kl_autograd_reductions_and_temperature():
     g = torch.Generator().manual_seed(4)
     s = (3 * torch.randn(20, 3000, generator=g)).bfloat16()

@@ -513,3 +513,25 @@ def test_layernorm_is_only_patched_on_request():
     ref = model(x).detach().clone()
     assert kernels.enable(model, layer_norm=True)._fm_fused == {"norm": 2, "mlp": 0}
     assert torch.allclose(model(x), ref, atol=2e-6)
+
+
+def test_experts_and_moe_keep_the_reference_constructor_surface():
+    # reference forgemind/moe.py:102, 184-186, 139-159
+    import forgeminds_amd as fm
+    ex = fm.moe.Experts(4, 8, 16)
+    assert ex.w1.shape == (4, 8, 16) and ex.w2.shape == (4, 16, 8)
+    assert float(ex.w1.std()) < 0.05                        # normal(std=0.02), not 1/sqrt(dim)
+    x = torch.randn(10, 8)
+    a = ex(x, counts=[3, 0, 5, 2])
+    b = ex(x, counts=torch.tensor([3, 0, 5, 2]))
+    c = ex(x, offsets=torch.tensor([3, 3, 8, 10], dtype=torch.int32))
+    assert torch.equal(a, b) and torch.equal(a, c)
+    assert ex(x[:0], counts=[0, 0, 0, 0]).shape == (0, 8)
+    with pytest.raises(ValueError):
+        fm.moe.Experts(4, 8, 16, offload=True)
+    layer = fm.moe.MoE(8, 16, 4, 2, 1)                      # fifth positional argument is n_shared
+    assert layer.shared is not None and layer.aux_coef == 1e-2 and layer.n_local == 4
+    with pytest.raises(ValueError):
+        fm.moe.MoE(8, 16, 4, 2, 0, 2)                       # ep_size 2: not in a one-GPU build
+    out = layer(torch.randn(6, 8))                          # CPU: torch expressions end to end
+    assert out.shape == (6, 8) and layer.last_aux is not None
