@@ -3,6 +3,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
+#include <stdlib.h>
+#include <cxxabi.h>
 
 #include <atomic>
 
@@ -10,6 +12,8 @@
 
 namespace {
 thread_local char g_error[512] = "";
+thread_local const void* g_kernel = nullptr;     // host-side handle of the last main kernel
+thread_local char g_kernel_text[384] = "";
 std::atomic<int> g_params[fm_host::P_COUNT];
 const char* const kParamNames[fm_host::P_COUNT] = {
     "norm_bwd_blocks_per_cu",
@@ -35,6 +39,8 @@ void set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
+void note_kernel(const void* host_function) { g_kernel = host_function; }
+
 int get_param(int which) {
   if (which < 0 || which >= P_COUNT) return 0;
   return g_params[which].load(std::memory_order_relaxed);
@@ -59,6 +65,37 @@ extern "C" {
 int fm_version(void) { return 1; }
 
 const char* fm_last_error(void) { return g_error; }
+
+const char* fm_last_kernel(void) {
+  // "void (anonymous namespace)::ce_bwd_kernel<fm::bf16_t, 1024, 4>(fm::bf16_t const*, ...)"
+  //   -> "ce_bwd_kernel<bf16_t, 1024, 4>"
+  g_kernel_text[0] = 0;
+  if (g_kernel == nullptr) return g_kernel_text;
+  const char* mangled = hipKernelNameRefByPtr(g_kernel, nullptr);
+  if (mangled == nullptr) return g_kernel_text;
+  int status = 0;
+  char* full = abi::__cxa_demangle(mangled, nullptr, nullptr, &status);
+  const char* a = (status == 0 && full != nullptr) ? full : mangled;
+  if (strncmp(a, "void ", 5) == 0) a += 5;
+  size_t o = 0;
+  int depth = 0;
+  static const char* const kDrop[] = {"(anonymous namespace)::", "fm::"};
+  while (*a != 0 && o + 1 < sizeof(g_kernel_text)) {
+    bool dropped = false;
+    for (const char* d : kDrop) {
+      const size_t n = strlen(d);
+      if (strncmp(a, d, n) == 0) { a += n; dropped = true; break; }
+    }
+    if (dropped) continue;
+    if (*a == '<') ++depth;
+    if (*a == '>') --depth;
+    if (*a == '(' && depth == 0) break;       // the parameter list
+    g_kernel_text[o++] = *a++;
+  }
+  g_kernel_text[o] = 0;
+  free(full);
+  return g_kernel_text;
+}
 
 int fm_set_param(const char* name, int value) {
   if (name == nullptr) {

@@ -648,7 +648,7 @@ bool launch_vrows(const void* logits, const int64_t* labels, const float* n_vali
   const dim3 grid((unsigned)((n + 256 / tpr - 1) / (256 / tpr)));
 #define GOV(TPR_, IT_)                                                                              \
   if (tpr == TPR_ && iters == IT_) {                                                                \
-    hipLaunchKernelGGL((ce_vrows_kernel<T, TPR_, IT_, LOSS, GRAD>), grid, dim3(256), 0, st,         \
+    FM_LAUNCH((ce_vrows_kernel<T, TPR_, IT_, LOSS, GRAD>), grid, dim3(256), 0, st,         \
                        static_cast<const T*>(logits), labels, n_valid, grad_out, lse, row_loss,     \
                        static_cast<T*>(dlogits), n, v, ignore_index);                               \
     return true;                                                                                    \
@@ -681,7 +681,7 @@ bool launch_rows(const void* logits, const int64_t* labels, const float* n_valid
   const dim3 grid((unsigned)((n + 256 / tpr - 1) / (256 / tpr)));
 #define GOR(TPR_, IT_)                                                                              \
   if (tpr == TPR_ && iters == IT_) {                                                                \
-    hipLaunchKernelGGL((ce_rows_kernel<T, TPR_, IT_, LOSS, GRAD>), grid, dim3(256), 0, st,          \
+    FM_LAUNCH((ce_rows_kernel<T, TPR_, IT_, LOSS, GRAD>), grid, dim3(256), 0, st,          \
                        static_cast<const T*>(logits), labels, n_valid, grad_out, lse, row_loss,     \
                        static_cast<T*>(dlogits), n, v, ignore_index);                               \
     return true;                                                                                    \
@@ -706,7 +706,7 @@ int launch_fwd(const void* logits, const int64_t* labels, float* lse, float* row
   const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 512, 4, 24 * 1024);
   const dim3 grid((unsigned)n);
 #define LAUNCH(TH, UN)                                                                          \
-  hipLaunchKernelGGL((ce_fwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, lp, labels, lse, row_loss, \
+  FM_LAUNCH((ce_fwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, lp, labels, lse, row_loss, \
                      v, ignore_index, vec_ok)
   FM_VOCAB_DISPATCH(sh, LAUNCH);
 #undef LAUNCH
@@ -722,7 +722,7 @@ int launch_bwd(const void* logits, const int64_t* labels, const float* lse, cons
   const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 4);
   const dim3 grid((unsigned)n);
 #define LAUNCH(TH, UN)                                                                         \
-  hipLaunchKernelGGL((ce_bwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, lp, labels, lse, n_valid, \
+  FM_LAUNCH((ce_bwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, lp, labels, lse, n_valid, \
                      grad_out, gp, v, ignore_index, vec_ok)
   FM_VOCAB_DISPATCH(sh, LAUNCH);
 #undef LAUNCH
@@ -841,7 +841,7 @@ int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float
       const bool vec_ok = fm_host::aligned16(logits) && fm_host::aligned16(dlogits);
       const dim3 wgrid((unsigned)n);
 #define WIDE(T)                                                                                   \
-  hipLaunchKernelGGL((ce_loss_grad_wide_kernel<T, 1024, 2>), wgrid, dim3(1024), 0, st,            \
+  FM_LAUNCH((ce_loss_grad_wide_kernel<T, 1024, 2>), wgrid, dim3(1024), 0, st,            \
                      static_cast<const T*>(logits), labels, mean_ ? n_valid : nullptr, lse, row_loss, \
                      static_cast<T*>(dlogits), (int)v, ignore_index, vec_ok)
       FM_CE_BY_DTYPE(dtype, WIDE);
@@ -862,7 +862,7 @@ int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float
   const float* nv = mean ? n_valid : nullptr;
   const dim3 grid((unsigned)n);
 #define LAUNCH(T, TH, IT)                                                                        \
-  hipLaunchKernelGGL((ce_loss_grad_kernel<T, TH, IT>), grid, dim3(TH), 0, st,                    \
+  FM_LAUNCH((ce_loss_grad_kernel<T, TH, IT>), grid, dim3(TH), 0, st,                    \
                      static_cast<const T*>(logits), labels, nv, lse, row_loss,                   \
                      static_cast<T*>(dlogits), (int)v, ignore_index)
 #define BY_ITERS(T, TH)                        \

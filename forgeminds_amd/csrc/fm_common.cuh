@@ -299,6 +299,18 @@ enum Param { P_NORM_BWD_BLOCKS_PER_CU = 0, P_VOCAB_THREADS, P_NORM_TPR, P_TOPK_V
 
 int num_cus();  // compute units of the current device (cached per device)
 
+// Which kernel did the work: every launch of a main kernel (not the small finishing kernels)
+// leaves the kernel's host-side handle for fm_last_kernel(), which asks the runtime for the
+// device function's name and demangles it, so the name (template arguments resolved) cannot
+// drift from what was launched.
+void note_kernel(const void* host_function);
+
+#define FM_LAUNCH(K, grid, block, shmem, st, ...)                    \
+  do {                                                               \
+    fm_host::note_kernel(reinterpret_cast<const void*>(&K));         \
+    hipLaunchKernelGGL(K, grid, block, shmem, st, __VA_ARGS__);      \
+  } while (0)
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 #define FM_CHECK_ARG(cond, ...)                 \

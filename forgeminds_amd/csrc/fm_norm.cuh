@@ -788,12 +788,12 @@ int launch_fwd(const Plan& p, const void* x, const void* delta, const void* w, c
   T* xnp = static_cast<T*>(xn);
   T* yp = static_cast<T*>(y);
   if (p.wide) {
-    hipLaunchKernelGGL((norm_fwd_wide<T, WT, ADD, LN>), dim3((unsigned)n), dim3(kWideThreads), 0, st, xp,
+    FM_LAUNCH((norm_fwd_wide<T, WT, ADD, LN>), dim3((unsigned)n), dim3(kWideThreads), 0, st, xp,
                        dp, wp, bp, xnp, yp, mean, rstd, (int)d, eps);
     return FM_OK;
   }
   if (!p.vec) {
-    hipLaunchKernelGGL((norm_fwd_generic<T, WT, ADD, LN>), dim3((unsigned)n), dim3(256), 0, st, xp, dp,
+    FM_LAUNCH((norm_fwd_generic<T, WT, ADD, LN>), dim3((unsigned)n), dim3(256), 0, st, xp, dp,
                        wp, bp, xnp, yp, mean, rstd, d, eps);
     return FM_OK;
   }
@@ -808,7 +808,7 @@ int launch_fwd(const Plan& p, const void* x, const void* delta, const void* w, c
         o = 2048 / BlockOf<TPR_>::value;                                                        \
       occupancy = o;                                                                            \
     }                                                                                           \
-    hipLaunchKernelGGL((norm_fwd_kernel<T, WT, TPR_, IT_, ADD, LN>),                            \
+    FM_LAUNCH((norm_fwd_kernel<T, WT, TPR_, IT_, ADD, LN>),                            \
                        dim3((unsigned)fwd_grid(p, occupancy)), dim3(BlockOf<TPR_>::value), 0, st, \
                        xp, dp, wp, bp, xnp, yp, mean, rstd, n, (int)d, eps, p.tiles);           \
     return FM_OK;                                                                               \
@@ -832,7 +832,7 @@ int launch_bwd(const Plan& p, const void* x, const void* w, const float* mean, c
   if (dw == nullptr && db == nullptr) partial = nullptr;
   const int pcols = (int)(LN ? 2 * d : d);
   if (p.bwd_wide) {
-    hipLaunchKernelGGL((norm_bwd_wide<T, WT, LN>), dim3((unsigned)n), dim3(kWideThreads), 0, st, xp, wp,
+    FM_LAUNCH((norm_bwd_wide<T, WT, LN>), dim3((unsigned)n), dim3(kWideThreads), 0, st, xp, wp,
                        mean, rstd, dyp, gp, dxp, ddp, (int)d);
     if (partial != nullptr) {
       const int nvec = (int)(d / Elem<T>::kVec);
@@ -841,7 +841,7 @@ int launch_bwd(const Plan& p, const void* x, const void* w, const float* mean, c
                          p.rows_per_chunk);
     }
   } else if (!p.bwd_vec) {
-    hipLaunchKernelGGL((norm_bwd_generic<T, WT, LN>), dim3((unsigned)n), dim3(256), 0, st, xp, wp, mean,
+    FM_LAUNCH((norm_bwd_generic<T, WT, LN>), dim3((unsigned)n), dim3(256), 0, st, xp, wp, mean,
                        rstd, dyp, gp, dxp, ddp, d);
     if (partial != nullptr) {
       dim3 grid((unsigned)((d + 63) / 64), (unsigned)p.bwd_blocks);
@@ -852,7 +852,7 @@ int launch_bwd(const Plan& p, const void* x, const void* w, const float* mean, c
     bool done = false;
 #define X(TPR_, IT_)                                                                           \
   if (!done && p.tpr == TPR_ && p.iters == IT_) {                                              \
-    hipLaunchKernelGGL((norm_bwd_kernel<T, WT, TPR_, IT_, LN>), dim3((unsigned)p.bwd_blocks),  \
+    FM_LAUNCH((norm_bwd_kernel<T, WT, TPR_, IT_, LN>), dim3((unsigned)p.bwd_blocks),  \
                        dim3(kBwdBlock), 0, st, xp, wp, mean, rstd, dyp, gp, dxp, ddp,          \
                        partial, n, (int)d, p.bwd_tiles);                                       \
     done = true;                                                                               \

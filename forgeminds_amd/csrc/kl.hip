@@ -499,7 +499,7 @@ void launch_fwd(const void* s, const void* t, float* lse_s, float* lse_t, float*
   const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 512, 2);
   const dim3 grid((unsigned)n);
 #define LAUNCH(TH, UN)                                                                            \
-  hipLaunchKernelGGL((kl_fwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, sp, tp, lse_s, lse_t, row_kl, \
+  FM_LAUNCH((kl_fwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, sp, tp, lse_s, lse_t, row_kl, \
                      v, inv_temp, vec_ok)
   FM_VOCAB_DISPATCH(sh, LAUNCH);
 #undef LAUNCH
@@ -515,7 +515,7 @@ void launch_bwd(const void* s, const void* t, const float* lse_s, const float* l
   const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 8);
   const dim3 grid((unsigned)n);
 #define LAUNCH(TH, UN)                                                                           \
-  hipLaunchKernelGGL((kl_bwd_kernel<T, GT, TH, UN>), grid, dim3(TH), 0, st, sp, tp, lse_s, lse_t, \
+  FM_LAUNCH((kl_bwd_kernel<T, GT, TH, UN>), grid, dim3(TH), 0, st, sp, tp, lse_s, lse_t, \
                      grad_out, grad_per_row, gp, v, inv_temp, scale, vec_ok)
   FM_VOCAB_DISPATCH(sh, LAUNCH);
 #undef LAUNCH
@@ -773,7 +773,7 @@ bool launch_vrows(const void* student, const void* teacher, float* lse_s, float*
   const dim3 grid((unsigned)((n + 256 / tpr - 1) / (256 / tpr)));
 #define GOV(TPR_, IT_)                                                                             \
   if (tpr == TPR_ && iters == IT_) {                                                               \
-    hipLaunchKernelGGL((kl_vrows_kernel<T, GT, TPR_, IT_, LOSS, GRAD>), grid, dim3(256), 0, st,    \
+    FM_LAUNCH((kl_vrows_kernel<T, GT, TPR_, IT_, LOSS, GRAD>), grid, dim3(256), 0, st,    \
                        static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t, \
                        row_kl, grad_out, grad_per_row, static_cast<GT*>(dstudent), n, v, inv_temp, mul); \
     return true;                                                                                   \
@@ -801,7 +801,7 @@ bool launch_rows(const void* student, const void* teacher, float* lse_s, float* 
   const dim3 grid((unsigned)((n + 256 / tpr - 1) / (256 / tpr)));
 #define GOR(TPR_, IT_)                                                                             \
   if (tpr == TPR_ && iters == IT_) {                                                               \
-    hipLaunchKernelGGL((kl_rows_kernel<T, GT, TPR_, IT_, LOSS, GRAD>), grid, dim3(256), 0, st,     \
+    FM_LAUNCH((kl_rows_kernel<T, GT, TPR_, IT_, LOSS, GRAD>), grid, dim3(256), 0, st,     \
                        static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t, \
                        row_kl, grad_out, grad_per_row, static_cast<GT*>(dstudent), n, v, inv_temp, mul); \
     return true;                                                                                   \
@@ -901,7 +901,7 @@ static int kl_topk_entry(const char* what, const void* student, const void* teac
     // gradient (when asked for) is for an upstream gradient of 1
     const float mul = inv_temperature * ((reduction == FM_REDUCE_MEAN) ? 1.f / (float)n : 1.f);
 #define LAUNCH_AS(T, TH, GRAD_)                                                                     \
-  hipLaunchKernelGGL((kl_fwd_topk_kernel<T, TH, 2, GRAD_>), grid, dim3(TH), lds, st,               \
+  FM_LAUNCH((kl_fwd_topk_kernel<T, TH, 2, GRAD_>), grid, dim3(TH), lds, st,               \
                      static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t, \
                      row_kl, static_cast<T*>(topk_values), i32, i64, topk_probs,                   \
                      static_cast<T*>(dstudent), mul, (int)v, k, inv_temperature, vec_ok)
@@ -1041,7 +1041,7 @@ int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, floa
     const float mul_w = inv_temperature * scale;
     const dim3 wgrid((unsigned)n);
 #define WIDE(T, GT)                                                                                \
-  hipLaunchKernelGGL((kl_loss_grad_wide_kernel<T, GT, 1024, 2>), wgrid, dim3(1024), 0, st,         \
+  FM_LAUNCH((kl_loss_grad_wide_kernel<T, GT, 1024, 2>), wgrid, dim3(1024), 0, st,         \
                      static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t,  \
                      row_kl, static_cast<GT*>(dstudent), (int)v, inv_temperature, mul_w, vec_ok)
     FM_KL_BY_DTYPES(dtype, grad_dtype, WIDE);
@@ -1061,7 +1061,7 @@ int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, floa
   const float mul = inv_temperature * scale;
   const dim3 grid((unsigned)n);
 #define LAUNCH(T, GT, TH, IT)                                                                      \
-  hipLaunchKernelGGL((kl_loss_grad_kernel<T, GT, TH, IT>), grid, dim3(TH), 0, st,                  \
+  FM_LAUNCH((kl_loss_grad_kernel<T, GT, TH, IT>), grid, dim3(TH), 0, st,                  \
                      static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t, \
                      row_kl, static_cast<GT*>(dstudent), (int)v, inv_temperature, mul)
 #define BY_ITERS(T, GT, TH)                       \

@@ -195,10 +195,10 @@ int fm_moe_gather(const void* x, const int32_t* order, const float* scale, void*
     while (g < 256 && g < units) g *= 2;                                                         \
     const dim3 grid((unsigned)((total + 256 / g - 1) / (256 / g)));                              \
     if (vec)                                                                                     \
-      hipLaunchKernelGGL((gather_kernel<T, true>), grid, dim3(256), 0, st, static_cast<const T*>(x), \
+      FM_LAUNCH((gather_kernel<T, true>), grid, dim3(256), 0, st, static_cast<const T*>(x), \
                          order, scale, static_cast<T*>(xs), total, (int)d, k, g);                \
     else                                                                                         \
-      hipLaunchKernelGGL((gather_kernel<T, false>), grid, dim3(256), 0, st, static_cast<const T*>(x), \
+      FM_LAUNCH((gather_kernel<T, false>), grid, dim3(256), 0, st, static_cast<const T*>(x), \
                          order, scale, static_cast<T*>(xs), total, (int)d, k, g);                \
   }
   FM_BY_DTYPE(dtype, CALL);
@@ -217,10 +217,10 @@ int fm_moe_combine(const void* ys, const float* weights, const int32_t* slot, vo
   const dim3 grid((unsigned)n);
 #define CALL(T)                                                                                    \
   if (vec_ok<T>(d, ys, out))                                                                       \
-    hipLaunchKernelGGL((combine_kernel<T, true>), grid, dim3(256), 0, st, static_cast<const T*>(ys), \
+    FM_LAUNCH((combine_kernel<T, true>), grid, dim3(256), 0, st, static_cast<const T*>(ys), \
                        weights, slot, static_cast<T*>(out), (int)d, k);                            \
   else                                                                                             \
-    hipLaunchKernelGGL((combine_kernel<T, false>), grid, dim3(256), 0, st, static_cast<const T*>(ys), \
+    FM_LAUNCH((combine_kernel<T, false>), grid, dim3(256), 0, st, static_cast<const T*>(ys), \
                        weights, slot, static_cast<T*>(out), (int)d, k)
   FM_BY_DTYPE(dtype, CALL);
 #undef CALL
@@ -238,10 +238,10 @@ int fm_moe_combine_dw(const void* ys, const void* dout, const int32_t* slot, flo
   const dim3 grid((unsigned)n);
 #define CALL(T)                                                                                  \
   if (vec_ok<T>(d, ys, dout))                                                                    \
-    hipLaunchKernelGGL((combine_dw_kernel<T, true>), grid, dim3(256), 0, st,                     \
+    FM_LAUNCH((combine_dw_kernel<T, true>), grid, dim3(256), 0, st,                     \
                        static_cast<const T*>(ys), static_cast<const T*>(dout), slot, dweights, (int)d, k); \
   else                                                                                           \
-    hipLaunchKernelGGL((combine_dw_kernel<T, false>), grid, dim3(256), 0, st,                    \
+    FM_LAUNCH((combine_dw_kernel<T, false>), grid, dim3(256), 0, st,                    \
                        static_cast<const T*>(ys), static_cast<const T*>(dout), slot, dweights, (int)d, k)
   FM_BY_DTYPE(dtype, CALL);
 #undef CALL

@@ -293,7 +293,7 @@ int launch(const Shape& sh, bool vec, const void* x, const void* w, const float*
   const int64_t tiles = vec ? sh.vtiles : sh.tiles;
   const int64_t blocks = sh.blocks < tiles ? sh.blocks : tiles;
 #define GO(KERNEL, G)                                                                                 \
-  hipLaunchKernelGGL((KERNEL<T, WT, G, BWD>), dim3((unsigned)blocks), dim3(kBlock), 0, st,            \
+  FM_LAUNCH((KERNEL<T, WT, G, BWD>), dim3((unsigned)blocks), dim3(kBlock), 0, st,            \
                      static_cast<const T*>(x), static_cast<const WT*>(w), c, s,                       \
                      static_cast<const T*>(dout), rstd, static_cast<T*>(out), partial, rows, t_len,   \
                      heads, d, eps, tiles)

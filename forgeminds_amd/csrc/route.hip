@@ -598,9 +598,9 @@ int launch_route(const void* logits, int32_t* idx, float* weights, int32_t* hist
   const dim3 grid((unsigned)tl.ntiles);
 #define GOG(L_)                                                                                       \
   do {                                                                                                \
-    if (vec) hipLaunchKernelGGL((route_group_kernel<T, L_, true>), grid, dim3(kGroupThreads), 0, st,  \
+    if (vec) FM_LAUNCH((route_group_kernel<T, L_, true>), grid, dim3(kGroupThreads), 0, st,  \
                                 lp, idx, weights, hist, fstat, n, e, k, tl.tile_rows);                \
-    else hipLaunchKernelGGL((route_group_kernel<T, L_, false>), grid, dim3(kGroupThreads), 0, st,     \
+    else FM_LAUNCH((route_group_kernel<T, L_, false>), grid, dim3(kGroupThreads), 0, st,     \
                             lp, idx, weights, hist, fstat, n, e, k, tl.tile_rows);                    \
   } while (0)
   const bool vec = e % kGE == 0 && fm_host::aligned16(logits);
@@ -700,10 +700,10 @@ int fm_route_bwd(const void* logits, const int32_t* idx, const float* gweights, 
   do {                                                                                               \
     constexpr int rows_per_block = (kGroupThreads / 64) * (64 / L_);                                 \
     const dim3 grid((unsigned)((n + rows_per_block - 1) / rows_per_block));                          \
-    if (vec) hipLaunchKernelGGL((route_bwd_kernel<T, L_, true>), grid, dim3(kGroupThreads), 0, st,   \
+    if (vec) FM_LAUNCH((route_bwd_kernel<T, L_, true>), grid, dim3(kGroupThreads), 0, st,   \
                                 static_cast<const T*>(logits), idx, gweights, counts, g_aux, g_z,    \
                                 static_cast<T*>(dlogits), n, e, k);                                  \
-    else hipLaunchKernelGGL((route_bwd_kernel<T, L_, false>), grid, dim3(kGroupThreads), 0, st,      \
+    else FM_LAUNCH((route_bwd_kernel<T, L_, false>), grid, dim3(kGroupThreads), 0, st,      \
                             static_cast<const T*>(logits), idx, gweights, counts, g_aux, g_z,        \
                             static_cast<T*>(dlogits), n, e, k);                                      \
   } while (0)

@@ -354,7 +354,7 @@ void launch(const void* x, void* y, int64_t n, int v, bool vec_ok, hipStream_t s
 #define X(TPR_, IT_)                                                                               \
   if (tpr == TPR_ && iters == IT_) {                                                               \
     constexpr int RPB = RowBlock<TPR_>::value / TPR_;                                              \
-    hipLaunchKernelGGL((softmax_rows_kernel<T, TPR_, IT_>), dim3((unsigned)((n + RPB - 1) / RPB)), \
+    FM_LAUNCH((softmax_rows_kernel<T, TPR_, IT_>), dim3((unsigned)((n + RPB - 1) / RPB)), \
                        dim3(RowBlock<TPR_>::value), 0, st, xp, yp, n, v);                          \
     return;                                                                                        \
   }
@@ -367,7 +367,7 @@ void launch(const void* x, void* y, int64_t n, int v, bool vec_ok, hipStream_t s
     const dim3 sgrid((unsigned)((n + 256 / tpr - 1) / (256 / tpr)));
 #define GOS(TPR_, IT_)                                                                             \
   if (tpr == TPR_ && iters == IT_) {                                                               \
-    hipLaunchKernelGGL((softmax_rows_scalar_kernel<T, TPR_, IT_>), sgrid, dim3(256), 0, st, xp, yp, n, v); \
+    FM_LAUNCH((softmax_rows_scalar_kernel<T, TPR_, IT_>), sgrid, dim3(256), 0, st, xp, yp, n, v); \
     return;                                                                                        \
   }
     GOS(1, 1) GOS(1, 2) GOS(1, 4) GOS(2, 4) GOS(4, 4) GOS(8, 4)
@@ -377,7 +377,7 @@ void launch(const void* x, void* y, int64_t n, int v, bool vec_ok, hipStream_t s
   const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 4);
   const dim3 grid((unsigned)n);
 #define LAUNCH(TH, UN) \
-  hipLaunchKernelGGL((softmax_kernel<T, TH, UN>), grid, dim3(TH), 0, st, xp, yp, v, vec_ok)
+  FM_LAUNCH((softmax_kernel<T, TH, UN>), grid, dim3(TH), 0, st, xp, yp, v, vec_ok)
   FM_VOCAB_DISPATCH(sh, LAUNCH);
 #undef LAUNCH
 }
@@ -396,7 +396,7 @@ void launch_bwd(const void* y, const void* dy, void* dx, int64_t n, int v, bool 
 #define X(TPR_, IT_)                                                                               \
   if (tpr == TPR_ && iters == IT_) {                                                               \
     constexpr int RPB = RowBlock<TPR_>::value / TPR_;                                              \
-    hipLaunchKernelGGL((softmax_bwd_rows_kernel<T, TPR_, IT_>), dim3((unsigned)((n + RPB - 1) / RPB)), \
+    FM_LAUNCH((softmax_bwd_rows_kernel<T, TPR_, IT_>), dim3((unsigned)((n + RPB - 1) / RPB)), \
                        dim3(RowBlock<TPR_>::value), 0, st, yp, gp, op, n, v);                      \
     return;                                                                                        \
   }
@@ -409,7 +409,7 @@ void launch_bwd(const void* y, const void* dy, void* dx, int64_t n, int v, bool 
     const dim3 sgrid((unsigned)((n + 256 / tpr - 1) / (256 / tpr)));
 #define GOS(TPR_, IT_)                                                                             \
   if (tpr == TPR_ && iters == IT_) {                                                               \
-    hipLaunchKernelGGL((softmax_bwd_rows_scalar_kernel<T, TPR_, IT_>), sgrid, dim3(256), 0, st, yp, gp, op, n, v); \
+    FM_LAUNCH((softmax_bwd_rows_scalar_kernel<T, TPR_, IT_>), sgrid, dim3(256), 0, st, yp, gp, op, n, v); \
     return;                                                                                        \
   }
     GOS(1, 1) GOS(1, 2) GOS(1, 4) GOS(2, 4) GOS(4, 4) GOS(8, 4)
@@ -419,7 +419,7 @@ void launch_bwd(const void* y, const void* dy, void* dx, int64_t n, int v, bool 
   const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 4);
   const dim3 grid((unsigned)n);
 #define LAUNCH(TH, UN) \
-  hipLaunchKernelGGL((softmax_bwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, yp, gp, op, v, vec_ok)
+  FM_LAUNCH((softmax_bwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, yp, gp, op, v, vec_ok)
   FM_VOCAB_DISPATCH(sh, LAUNCH);
 #undef LAUNCH
 }

@@ -157,10 +157,10 @@ int fm_swiglu_fwd(const void* gate, const void* up, void* y, int64_t n, int dtyp
 #define CALL(T)                                                                                     \
   if (vec) {                                                                                        \
     const int64_t nv = (n + Elem<T>::kVec - 1) / Elem<T>::kVec;                                     \
-    hipLaunchKernelGGL((swiglu_fwd_kernel<T, true>), dim3((unsigned)((nv + 255) / 256)), dim3(256), 0, st, \
+    FM_LAUNCH((swiglu_fwd_kernel<T, true>), dim3((unsigned)((nv + 255) / 256)), dim3(256), 0, st, \
                        static_cast<const T*>(gate), static_cast<const T*>(up), static_cast<T*>(y), n); \
   } else {                                                                                          \
-    hipLaunchKernelGGL((swiglu_fwd_kernel<T, false>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, \
+    FM_LAUNCH((swiglu_fwd_kernel<T, false>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, \
                        static_cast<const T*>(gate), static_cast<const T*>(up), static_cast<T*>(y), n); \
   }
   FM_BY_DTYPE(dtype, CALL);
@@ -182,11 +182,11 @@ int fm_swiglu_bwd(const void* gate, const void* up, const void* dy, void* dgate,
 #define CALL(T)                                                                                     \
   if (vec) {                                                                                        \
     const int64_t nv = (n + Elem<T>::kVec - 1) / Elem<T>::kVec;                                     \
-    hipLaunchKernelGGL((swiglu_bwd_kernel<T, true>), dim3((unsigned)((nv + 255) / 256)), dim3(256), 0, st, \
+    FM_LAUNCH((swiglu_bwd_kernel<T, true>), dim3((unsigned)((nv + 255) / 256)), dim3(256), 0, st, \
                        static_cast<const T*>(gate), static_cast<const T*>(up), static_cast<const T*>(dy), \
                        static_cast<T*>(dgate), static_cast<T*>(dup), n);                            \
   } else {                                                                                          \
-    hipLaunchKernelGGL((swiglu_bwd_kernel<T, false>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, \
+    FM_LAUNCH((swiglu_bwd_kernel<T, false>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, \
                        static_cast<const T*>(gate), static_cast<const T*>(up), static_cast<const T*>(dy), \
                        static_cast<T*>(dgate), static_cast<T*>(dup), n);                            \
   }
@@ -220,10 +220,10 @@ static int split_entry(const char* what, const void* x, const void* dy, void* ou
                      fm_host::aligned16(dy);                                                       \
     const int64_t per = vec ? h / Elem<T>::kVec : h;                                               \
     const dim3 grid((unsigned)((per + 255) / 256), (unsigned)nr);                                  \
-    if (vec && !bwd) hipLaunchKernelGGL((swiglu_split_kernel<T, true, false>), grid, dim3(256), 0, st, xp, dp, op, (int)h); \
-    else if (vec) hipLaunchKernelGGL((swiglu_split_kernel<T, true, true>), grid, dim3(256), 0, st, xp, dp, op, (int)h);     \
-    else if (!bwd) hipLaunchKernelGGL((swiglu_split_kernel<T, false, false>), grid, dim3(256), 0, st, xp, dp, op, (int)h);  \
-    else hipLaunchKernelGGL((swiglu_split_kernel<T, false, true>), grid, dim3(256), 0, st, xp, dp, op, (int)h);             \
+    if (vec && !bwd) FM_LAUNCH((swiglu_split_kernel<T, true, false>), grid, dim3(256), 0, st, xp, dp, op, (int)h); \
+    else if (vec) FM_LAUNCH((swiglu_split_kernel<T, true, true>), grid, dim3(256), 0, st, xp, dp, op, (int)h);     \
+    else if (!bwd) FM_LAUNCH((swiglu_split_kernel<T, false, false>), grid, dim3(256), 0, st, xp, dp, op, (int)h);  \
+    else FM_LAUNCH((swiglu_split_kernel<T, false, true>), grid, dim3(256), 0, st, xp, dp, op, (int)h);             \
   }
     FM_BY_DTYPE(dtype, CALL);
 #undef CALL

@@ -469,9 +469,9 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
   const int64_t nvec = (v + EPV - 1) / EPV + 1;  // upper bound on whole vectors of any row
   const dim3 grid((unsigned)n);
 #define GO(TH, IT, BIG_)                                                                         \
-  hipLaunchKernelGGL((topk_kernel<T, TH, IT, BIG_>), grid, dim3(TH), 0, st, xp, vp, i32, i64, v, k, vec_ok)
+  FM_LAUNCH((topk_kernel<T, TH, IT, BIG_>), grid, dim3(TH), 0, st, xp, vp, i32, i64, v, k, vec_ok)
 #define GOL(TH, UN, BIG_)                                                                        \
-  hipLaunchKernelGGL((topk_lds_kernel<T, TH, UN, BIG_>), grid, dim3(TH), (size_t)(nvec + 8) * 2, st, xp, vp, \
+  FM_LAUNCH((topk_lds_kernel<T, TH, UN, BIG_>), grid, dim3(TH), (size_t)(nvec + 8) * 2, st, xp, vp, \
                      i32, i64, v, k, vec_ok)
   const bool big = k > 256;               // twice the candidate slots (1024-thread forms only)
   int variant = fm_host::get_param(fm_host::P_TOPK_VARIANT);
@@ -512,8 +512,8 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
   do {                                                                                             \
     constexpr int rows_per_block = 4 * (64 / L_) * kGroupRows;                                     \
     const dim3 ggrid((unsigned)((n + rows_per_block - 1) / rows_per_block));                       \
-    if (gvec) hipLaunchKernelGGL((topk_group_kernel<T, L_, true>), ggrid, dim3(256), 0, st, xp, vp, i32, i64, n, v, k); \
-    else hipLaunchKernelGGL((topk_group_kernel<T, L_, false>), ggrid, dim3(256), 0, st, xp, vp, i32, i64, n, v, k);     \
+    if (gvec) FM_LAUNCH((topk_group_kernel<T, L_, true>), ggrid, dim3(256), 0, st, xp, vp, i32, i64, n, v, k); \
+    else FM_LAUNCH((topk_group_kernel<T, L_, false>), ggrid, dim3(256), 0, st, xp, vp, i32, i64, n, v, k);     \
   } while (0)
     if (v <= 64) GOG(8);
     else if (v <= 128) GOG(16);
@@ -526,7 +526,7 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
     while (64 * epl < v) epl *= 2;
     const bool wvec = vec_ok && v % EPV == 0 && epl >= EPV;
 #define GOW(EPL_, VEC_)                                                                            \
-  hipLaunchKernelGGL((topk_wave_kernel<T, EPL_, VEC_>), grid, dim3(64), 0, st, xp, vp, i32, i64, v, k)
+  FM_LAUNCH((topk_wave_kernel<T, EPL_, VEC_>), grid, dim3(64), 0, st, xp, vp, i32, i64, v, k)
 #define GOWV(EPL_)                                                                                 \
   if constexpr (EPL_ % EPV == 0) {                                                                 \
     if (wvec) GOW(EPL_, true);                                                                     \

@@ -32,6 +32,7 @@ _vp, _i64, _int, _f32, _sz = C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_size
 SIGNATURES = {
     "fm_version": (_int, []),
     "fm_last_error": (C.c_char_p, []),
+    "fm_last_kernel": (C.c_char_p, []),
     "fm_set_param": (_int, [C.c_char_p, _int]),
     "fm_stream_probe": (_int, [_vp, _vp, _vp, _sz, _int, _vp]),
     "fm_rmsnorm_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _f32, _vp]),
@@ -178,6 +179,11 @@ def _dense(*ts):
     for t in ts:
         if t is not None and not t.is_contiguous():
             raise RuntimeError("forgeminds_amd: the HIP kernels take contiguous tensors")
+
+
+def last_kernel() -> str:
+    """Name of the last main kernel this thread enqueued (template arguments resolved)."""
+    return lib().fm_last_kernel().decode()
 
 
 def set_param(name: str, value: int) -> None:

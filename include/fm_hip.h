@@ -47,6 +47,12 @@ enum fm_reduction { FM_REDUCE_NONE = 0, FM_REDUCE_SUM = 1, FM_REDUCE_MEAN = 2 };
 int fm_version(void);
 const char* fm_last_error(void);
 
+/* Name of the last main kernel (template arguments resolved, e.g.
+ * "ce_bwd_kernel<bf16_t, 1024, 4>") that an entry point enqueued from the calling thread; empty
+ * before the first launch. A measurement hook: the benchmark keys profiler byte counts by it, so
+ * a figure can never be attached to a kernel that did not run. Not part of the reference surface. */
+const char* fm_last_kernel(void);
+
 /* Tuning hook used by the benchmark sweeps; unknown names return FM_ERR_INVALID.
  * value <= 0 restores the built-in heuristic. Not part of the reference surface. */
 int fm_set_param(const char* name, int value);
