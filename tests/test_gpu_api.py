@@ -248,6 +248,15 @@ def test_kl_gradient_in_forward_reuse_and_second_backward():
     assert hs.grad is not None and w.grad is not None and hs.grad.abs().sum() > 0
 
 
+def test_last_kernel_names_what_ran():
+    x = torch.randn(64, 1024, device=DEV).bfloat16()
+    w = torch.ones(1024, device=DEV)
+    _hip.rmsnorm_fwd(x, w, 1e-6)
+    assert _hip.last_kernel() == "norm_fwd_kernel<bf16_t, float, 64, 2, false, false>"
+    _hip.topk(torch.randn(8, 128256, device=DEV).bfloat16(), 64, torch.int32)
+    assert _hip.last_kernel().startswith("topk_lds_kernel<bf16_t, ")
+
+
 def test_fp16_losses_apply_the_upstream_gradient_before_rounding():
     # a loss scaler multiplies the loss by 65536; (softmax - onehot) / 8192 rounded to fp16 FIRST
     # would lose most entries (p / 8192 < 6e-5 is subnormal or zero in fp16)
