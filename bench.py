@@ -478,8 +478,12 @@ def make_workload(name, torch, L, dev):
             w.dominant_launch = both
             w.dominant = "kl_loss_grad_wide_kernel<bf16,bf16,1024,2>"
             w.dominant_bytes = w.bytes = n * v * 6
-            w.desc = (f"KL loss + gradient in one launch bf16 [{n},{v}], T=2, mean; HBM dataflow read s,t + "
-                      "write g = 6 B/logit pair (each row is swept a second time right after the first, inside the launch)")
+            w.desc = (f"KL loss + gradient in one launch bf16 [{n},{v}], T=2, mean; algorithmic 6 B/logit pair "
+                      "(read s,t + write g). Each row is swept a second time right after the first, inside the "
+                      "launch: the L2-side counters show 10 B/pair (both sweeps fetched); that the second sweep is "
+                      "served by the memory-side cache is an inference from the clock, no counter of this profiler "
+                      "sits behind that cache")
+            w.l2_bytes = n * v * 10
             w.rows = n
             return w
 
@@ -501,8 +505,10 @@ def make_workload(name, torch, L, dev):
             w.dominant_launch = both
             w.dominant = "kl_fwd_topk_kernel<bf16,512,2>"
             w.dominant_bytes = w.bytes = n * v * 6
-            w.desc = (f"KL loss + gradient + teacher top-64 in one launch bf16 [{n},{v}], T=2, mean; HBM "
-                      "dataflow 6 B/logit pair")
+            w.desc = (f"KL loss + gradient + teacher top-64 in one launch bf16 [{n},{v}], T=2, mean; algorithmic "
+                      "6 B/logit pair; two sweeps per row inside the launch, 10 B/pair at the L2 boundary (see "
+                      "kl_one_launch)")
+            w.l2_bytes = n * v * 10
             w.rows = n
             return w
 
@@ -739,9 +745,9 @@ def make_workload(name, torch, L, dev):
         xs = torch.empty(n * k, d, device=dev, dtype=torch.bfloat16)
         out = torch.empty_like(x)
 
-        def gather():
-            _check(L.fm_moe_gather(x.data_ptr(), od.data_ptr(), None, xs.data_ptr(), n, d, k, BF, st),
-                   "fm_moe_gather")
+        def gather():     # from the token's side (fm_route hands out slot as well as order)
+            _check(L.fm_moe_scatter(x.data_ptr(), sl.data_ptr(), None, xs.data_ptr(), n, d, k, BF, st),
+                   "fm_moe_scatter")
 
         def combine():
             _check(L.fm_moe_combine(xs.data_ptr(), wt.data_ptr(), sl.data_ptr(), out.data_ptr(), n, d, k,
@@ -885,6 +891,10 @@ def measure(torch, w, steps, warmup, L, cpu=True):
         out["required_bytes"] = w.required_bytes
         out["required_gbps"] = round(w.required_bytes / ms / 1e6, 1)
         out["required_frac_of_hbm_peak"] = round(w.required_bytes / ms / 1e6 / HBM_PEAK_GBPS, 4)
+    if hasattr(w, "l2_bytes"):       # bytes that cross the L2 boundary (both sweeps of a row), as counted
+        out["l2_boundary_bytes"] = w.l2_bytes
+        out["l2_boundary_gbps"] = round(w.l2_bytes / ms / 1e6, 1)
+        out["l2_boundary_frac_of_hbm_peak"] = round(w.l2_bytes / ms / 1e6 / HBM_PEAK_GBPS, 4)
     if hasattr(w, "warm_step"):      # same buffers every step: served by the memory-side cache
         out["cache"] = "cold (buffer sets rotate through more than the 256 MB memory-side cache)"
         wm = time_steps(torch, w.warm_step, steps, warmup)

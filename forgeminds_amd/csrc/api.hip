@@ -25,6 +25,7 @@ const char* const kParamNames[fm_host::P_COUNT] = {
     "ce_rows_max_v",
     "norm_wide_min_vec",
     "rows_vec_max",
+    "rope_heads",
 };
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cus[kMaxDevices];

@@ -142,7 +142,10 @@ __device__ __forceinline__ void load_w_cols(const WT* p, float (&o)[Elem<T>::kVe
   for (int e = 0; e < EPV; ++e) o[e] = Elem<WT>::load1(p + e);
 }
 
-template <typename T, typename WT, int G, bool BWD>
+// H consecutive heads of one token per lane group and tile: they share the token's cos / sin
+// columns, which are then fetched once per H heads instead of once per head (the tables cost
+// twice the bytes of x at the L1 otherwise), and a lane has H times the bytes in flight.
+template <typename T, typename WT, int G, bool BWD, int H>
 __global__ __launch_bounds__(kBlock) void rope_vec_kernel(const T* __restrict__ x, const WT* __restrict__ w,
                                                            const float* __restrict__ cosv,
                                                            const float* __restrict__ sinv,
@@ -166,76 +169,91 @@ __global__ __launch_bounds__(kBlock) void rope_vec_kernel(const T* __restrict__ 
     load_w_cols<T, WT>(w + half + col, wv2);
   }
   for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-    const int64_t row = tile * RPB + rib;
-    const bool on = lane_on && row < rows;
-    const int t = row < rows ? (int)((row / heads) % t_len) : 0;
-    const T* xp = x + row * (int64_t)d;
-    float x1[EPV], x2[EPV], c[EPV], sn[EPV];
+    // rows is a multiple of H and so is the number of heads of a token: the H rows exist
+    // together and belong to one token
+    const int64_t row0 = (tile * RPB + rib) * H;
+    const bool live = row0 < rows;
+    const bool on = lane_on && live;
+    const int t = live ? (int)((row0 / heads) % t_len) : 0;
+    float c[EPV], sn[EPV];
 #pragma unroll
-    for (int e = 0; e < EPV; ++e) { x1[e] = 0.f; x2[e] = 0.f; c[e] = 0.f; sn[e] = 0.f; }
-    u32x4 r1, r2, q1, q2;
+    for (int e = 0; e < EPV; ++e) { c[e] = 0.f; sn[e] = 0.f; }
+    u32x4 r1[H], r2[H], q1[BWD ? H : 1], q2[BWD ? H : 1];
     if (on) {
-      r1 = load16_stream(xp + col);
-      r2 = load16_stream(xp + half + col);
-      if constexpr (BWD) {
-        const T* gp = dout + row * (int64_t)d;
-        q1 = load16_stream(gp + col);
-        q2 = load16_stream(gp + half + col);
+#pragma unroll
+      for (int j = 0; j < H; ++j) {
+        const T* xp = x + (row0 + j) * (int64_t)d;
+        r1[j] = load16_stream(xp + col);
+        r2[j] = load16_stream(xp + half + col);
+        if constexpr (BWD) {
+          const T* gp = dout + (row0 + j) * (int64_t)d;
+          q1[j] = load16_stream(gp + col);
+          q2[j] = load16_stream(gp + half + col);
+        }
       }
       load_f32_cols<T>(cosv + (int64_t)t * half + col, c);
       load_f32_cols<T>(sinv + (int64_t)t * half + col, sn);
-      Elem<T>::unpack(r1, x1);
-      Elem<T>::unpack(r2, x2);
     }
-    if constexpr (!BWD) {
-      float ss = 0.f;
 #pragma unroll
-      for (int e = 0; e < EPV; ++e) ss += x1[e] * x1[e] + x2[e] * x2[e];
-      ss = group_reduce<G, OpSum>(ss);
-      const float r = rsqrtf(ss / (float)d + eps);
-      if (row < rows && l == 0) rstd[row] = r;
+    for (int j = 0; j < H; ++j) {
+      const int64_t row = row0 + j;
+      float x1[EPV], x2[EPV];
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) { x1[e] = 0.f; x2[e] = 0.f; }
       if (on) {
-        float o1[EPV], o2[EPV];
+        Elem<T>::unpack(r1[j], x1);
+        Elem<T>::unpack(r2[j], x2);
+      }
+      if constexpr (!BWD) {
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) ss += x1[e] * x1[e] + x2[e] * x2[e];
+        ss = group_reduce<G, OpSum>(ss);
+        const float r = rsqrtf(ss / (float)d + eps);
+        if (live && l == 0) rstd[row] = r;
+        if (on) {
+          float o1[EPV], o2[EPV];
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) {
+            const float y1 = (x1[e] * r) * wv1[e], y2 = (x2[e] * r) * wv2[e];
+            o1[e] = y1 * c[e] - y2 * sn[e];
+            o2[e] = y1 * sn[e] + y2 * c[e];
+          }
+          T* op = out + row * (int64_t)d;
+          store16_stream(op + col, Elem<T>::pack(o1));
+          store16_stream(op + half + col, Elem<T>::pack(o2));
+        }
+      } else {
+        const float r = live ? rstd[row] : 0.f;
+        float g1[EPV], g2[EPV];
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) { g1[e] = 0.f; g2[e] = 0.f; }
+        if (on) {
+          Elem<T>::unpack(q1[j], g1);
+          Elem<T>::unpack(q2[j], g2);
+        }
+        float dot = 0.f;
 #pragma unroll
         for (int e = 0; e < EPV; ++e) {
-          const float y1 = (x1[e] * r) * wv1[e], y2 = (x2[e] * r) * wv2[e];
-          o1[e] = y1 * c[e] - y2 * sn[e];
-          o2[e] = y1 * sn[e] + y2 * c[e];
+          const float dy1 = g1[e] * c[e] + g2[e] * sn[e], dy2 = g2[e] * c[e] - g1[e] * sn[e];
+          x1[e] *= r; x2[e] *= r;                       // xhat
+          a1[e] += dy1 * x1[e]; a2[e] += dy2 * x2[e];
+          g1[e] = dy1 * wv1[e]; g2[e] = dy2 * wv2[e];
+          dot += g1[e] * x1[e] + g2[e] * x2[e];
         }
-        T* op = out + row * (int64_t)d;
-        store16_stream(op + col, Elem<T>::pack(o1));
-        store16_stream(op + half + col, Elem<T>::pack(o2));
-      }
-    } else {
-      const float r = row < rows ? rstd[row] : 0.f;
-      float g1[EPV], g2[EPV];
+        dot = group_reduce<G, OpSum>(dot);
+        const float cm = dot / (float)d;
+        if (on) {
+          float o1[EPV], o2[EPV];
 #pragma unroll
-      for (int e = 0; e < EPV; ++e) { g1[e] = 0.f; g2[e] = 0.f; }
-      if (on) {
-        Elem<T>::unpack(q1, g1);
-        Elem<T>::unpack(q2, g2);
-      }
-      float dot = 0.f;
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) {
-        const float dy1 = g1[e] * c[e] + g2[e] * sn[e], dy2 = g2[e] * c[e] - g1[e] * sn[e];
-        x1[e] *= r; x2[e] *= r;                       // xhat
-        a1[e] += dy1 * x1[e]; a2[e] += dy2 * x2[e];
-        g1[e] = dy1 * wv1[e]; g2[e] = dy2 * wv2[e];
-        dot += g1[e] * x1[e] + g2[e] * x2[e];
-      }
-      dot = group_reduce<G, OpSum>(dot);
-      const float cm = dot / (float)d;
-      if (on) {
-        float o1[EPV], o2[EPV];
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) {
-          o1[e] = (g1[e] - x1[e] * cm) * r;
-          o2[e] = (g2[e] - x2[e] * cm) * r;
+          for (int e = 0; e < EPV; ++e) {
+            o1[e] = (g1[e] - x1[e] * cm) * r;
+            o2[e] = (g2[e] - x2[e] * cm) * r;
+          }
+          T* op = out + row * (int64_t)d;
+          store16_stream(op + col, Elem<T>::pack(o1));
+          store16_stream(op + half + col, Elem<T>::pack(o2));
         }
-        T* op = out + row * (int64_t)d;
-        store16_stream(op + col, Elem<T>::pack(o1));
-        store16_stream(op + half + col, Elem<T>::pack(o2));
       }
     }
   }
@@ -290,26 +308,42 @@ template <typename T, typename WT, bool BWD>
 int launch(const Shape& sh, bool vec, const void* x, const void* w, const float* c, const float* s,
            const void* dout, float* rstd, void* out, float* partial, int64_t rows, int t_len, int heads,
            int d, float eps, hipStream_t st) {
-  const int64_t tiles = vec ? sh.vtiles : sh.tiles;
-  const int64_t blocks = sh.blocks < tiles ? sh.blocks : tiles;
-#define GO(KERNEL, G)                                                                                 \
-  FM_LAUNCH((KERNEL<T, WT, G, BWD>), dim3((unsigned)blocks), dim3(kBlock), 0, st,            \
-                     static_cast<const T*>(x), static_cast<const WT*>(w), c, s,                       \
-                     static_cast<const T*>(dout), rstd, static_cast<T*>(out), partial, rows, t_len,   \
-                     heads, d, eps, tiles)
-#define BY_G(KERNEL, g)           \
-  switch (g) {                    \
-    case 1: GO(KERNEL, 1); break; \
-    case 2: GO(KERNEL, 2); break; \
-    case 4: GO(KERNEL, 4); break; \
-    case 8: GO(KERNEL, 8); break; \
-    case 16: GO(KERNEL, 16); break; \
-    case 32: GO(KERNEL, 32); break; \
-    default: GO(KERNEL, 64); break; \
+  // heads of one token that a lane group takes per tile (vector kernel): 2 (4 in the forward is
+  // slower again: fewer waves fit), 1 when the head count is odd
+  int hpg = 1;
+  if (vec) {
+    const int want = fm_host::get_param(fm_host::P_ROPE_HEADS) > 0 ? fm_host::get_param(fm_host::P_ROPE_HEADS)
+                                                                   : 2;
+    if (want >= 4 && !BWD && heads % 4 == 0) hpg = 4;
+    else if (want >= 2 && heads % 2 == 0) hpg = 2;
   }
-  if (vec) { BY_G(rope_vec_kernel, sh.gv) } else { BY_G(rope_kernel, sh.g) }
+  const int rpb = kBlock / (vec ? sh.gv : sh.g);
+  const int64_t tiles = (rows + (int64_t)rpb * hpg - 1) / ((int64_t)rpb * hpg);
+  const int64_t blocks = sh.blocks < tiles ? sh.blocks : tiles;
+#define ARGS static_cast<const T*>(x), static_cast<const WT*>(w), c, s, static_cast<const T*>(dout), rstd, \
+             static_cast<T*>(out), partial, rows, t_len, heads, d, eps, tiles
+#define GO_V(G)                                                                                           \
+  do {                                                                                                    \
+    if (hpg == 1) FM_LAUNCH((rope_vec_kernel<T, WT, G, BWD, 1>), dim3((unsigned)blocks), dim3(kBlock), 0, st, ARGS); \
+    else if (hpg == 2) FM_LAUNCH((rope_vec_kernel<T, WT, G, BWD, 2>), dim3((unsigned)blocks), dim3(kBlock), 0, st, ARGS); \
+    else if constexpr (!BWD) FM_LAUNCH((rope_vec_kernel<T, WT, G, BWD, 4>), dim3((unsigned)blocks), dim3(kBlock), 0, st, ARGS); \
+  } while (0)
+#define GO_S(G) FM_LAUNCH((rope_kernel<T, WT, G, BWD>), dim3((unsigned)blocks), dim3(kBlock), 0, st, ARGS)
+#define BY_G(GO, g)           \
+  switch (g) {                \
+    case 1: GO(1); break;     \
+    case 2: GO(2); break;     \
+    case 4: GO(4); break;     \
+    case 8: GO(8); break;     \
+    case 16: GO(16); break;   \
+    case 32: GO(32); break;   \
+    default: GO(64); break;   \
+  }
+  if (vec) { BY_G(GO_V, sh.gv) } else { BY_G(GO_S, sh.g) }
 #undef BY_G
-#undef GO
+#undef GO_V
+#undef GO_S
+#undef ARGS
   return (int)blocks;
 }
 

@@ -63,6 +63,7 @@ SIGNATURES = {
     "fm_softmax_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _vp]),
     "fm_route_workspace": (_sz, [_i64, _int, _int]),
     "fm_moe_gather": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
+    "fm_moe_scatter": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "fm_moe_combine": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "fm_moe_combine_dw": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _vp]),
     "fm_swiglu_fwd": (_int, [_vp, _vp, _vp, _i64, _int, _vp]),
@@ -531,6 +532,18 @@ def moe_gather(x2, order, k: int, scale_flat=None):
     with _guard(x2.device):
         _check(lib().fm_moe_gather(_ptr(x2), _ptr(order), _ptr(scale_flat), _ptr(xs), n, d, int(k),
                                    dtype_code(x2.dtype), _stream(x2)), "fm_moe_gather")
+    return xs
+
+
+def moe_scatter(x2, slot, k: int, scale_flat=None):
+    """x2 [n, d], slot int32 [n*k] -> xs [n*k, d] with xs[slot[t*k+j]] = scale * x2[t]: the result of
+    ``moe_gather`` from the token's side (each token row is read once)."""
+    _dense(x2, slot, scale_flat)
+    n, d = x2.shape
+    xs = torch.empty((n * k, d), device=x2.device, dtype=x2.dtype)
+    with _guard(x2.device):
+        _check(lib().fm_moe_scatter(_ptr(x2), _ptr(slot), _ptr(scale_flat), _ptr(xs), n, d, int(k),
+                                    dtype_code(x2.dtype), _stream(x2)), "fm_moe_scatter")
     return xs
 
 

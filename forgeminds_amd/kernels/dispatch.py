@@ -27,16 +27,18 @@ def _i32(t: torch.Tensor) -> torch.Tensor:
 
 class _GatherFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, x, order, slot, k):
+    def forward(ctx, x, order, slot, k, have_slot):
         ctx.save_for_backward(slot)
         ctx.k = k
+        if have_slot:     # from the token's side: each row read once, written k times
+            return _hip.moe_scatter(x.contiguous(), slot, k)
         return _hip.moe_gather(x.contiguous(), order, k)
 
     @staticmethod
     def backward(ctx, g):
         (slot,) = ctx.saved_tensors
         n = slot.numel() // ctx.k
-        return _hip.moe_combine(g.contiguous(), None, slot, n, ctx.k), None, None, None
+        return _hip.moe_combine(g.contiguous(), None, slot, n, ctx.k), None, None, None, None
 
 
 class _CombineFn(torch.autograd.Function):
@@ -53,7 +55,7 @@ class _CombineFn(torch.autograd.Function):
         ys, w32, slot, order = ctx.saved_tensors
         n, k = w32.shape
         g = g.contiguous()
-        d_ys = _hip.moe_gather(g, order, k, w32.view(-1)) if ctx.needs_input_grad[0] else None
+        d_ys = _hip.moe_scatter(g, slot, k, w32.view(-1)) if ctx.needs_input_grad[0] else None
         d_w = None
         if ctx.needs_input_grad[1]:
             d_w = _hip.moe_combine_dw(ys.contiguous(), g, slot, n, k).to(ctx.w_dtype)
@@ -75,9 +77,10 @@ def moe_gather(x: torch.Tensor, order: torch.Tensor, k: int,
     if tracing() or not fast_ok(x):      # a traced graph gets the tensor expression
         return x[(order // k).long()]
     order = _i32(order)
+    have_slot = slot is not None or x.requires_grad
     if slot is None:
         slot = _inverse(order) if x.requires_grad else order
-    return _GatherFn.apply(x, order, _i32(slot), int(k))
+    return _GatherFn.apply(x, order, _i32(slot), int(k), have_slot)
 
 
 def moe_combine(ys: torch.Tensor, weights: torch.Tensor, slot: torch.Tensor,

@@ -305,6 +305,12 @@ int fm_route_bwd(const void* logits, const int32_t* idx, const float* gweights, 
 int fm_moe_gather(const void* x, const int32_t* order, const float* scale_flat, void* xs, int64_t n,
                   int64_t d, int k, int dtype, fm_stream_t stream);
 
+/* fm_moe_gather from the token's side, for callers that hold `slot` (the inverse of `order`, also
+ * written by fm_route): xs[slot[t*k + j], :] = scale * x[t, :] for j < k, scale = scale_flat[t*k + j]
+ * or 1. The same xs, bit for bit; a token row is read once instead of k times. */
+int fm_moe_scatter(const void* x, const int32_t* slot, const float* scale_flat, void* xs, int64_t n,
+                   int64_t d, int k, int dtype, fm_stream_t stream);
+
 /* Replaces `ys * w[order]` + `zeros.index_add_(0, order // k, ys)` (moe.py:247-248) by a gather
  * per token through the slot array of fm_route:
  *   out[t, :] = sum_j weights[t, j] * ys[slot[t*k + j], :]   (fp32 sum in j order, one rounding)

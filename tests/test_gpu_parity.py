@@ -923,6 +923,7 @@ def test_moe_gather_and_combine(n, e, k, d, dt):
     o32, s32 = order.to(torch.int32).to(DEV), slot.to(torch.int32).to(DEV)
     xs = _hip.moe_gather(x.to(DEV), o32, k)
     assert torch.equal(xs.cpu(), O.moe_gather(x, order, k))                    # a pure copy: bit-exact
+    assert torch.equal(_hip.moe_scatter(x.to(DEV), s32, k), xs)                # the same move from the token's side
     out = _hip.moe_combine(ys.to(DEV), w.to(DEV), s32, n, k)
     ref = O.moe_combine(ys, w, order, k, n)
     # the reference rounds each w*y product and each partial sum to the activation dtype
@@ -938,6 +939,7 @@ def test_moe_gather_and_combine(n, e, k, d, dt):
     dys = _hip.moe_gather(dout.to(DEV), o32, k, w.reshape(-1).to(DEV))
     want = (dout.float()[(order // k)] * w.reshape(-1)[order][:, None]).to(dt)
     assert_close_lowp(dys, want, dt, "combine backward wrt ys", ulps=2.0)
+    assert torch.equal(_hip.moe_scatter(dout.to(DEV), s32, k, w.reshape(-1).to(DEV)), dys)
     dw = _hip.moe_combine_dw(ys.to(DEV), dout.to(DEV), s32, n, k)
     want_dw = (ys.float()[slot].view(n, k, d) * dout.float()[:, None, :]).sum(-1)
     assert torch.allclose(dw.cpu(), want_dw, rtol=1e-4, atol=1e-4 * float(want_dw.abs().max()))
