@@ -787,8 +787,15 @@ def _close(a, b, rel=1e-2):
 
 
 def time_steps(torch, fn, steps, warmup):
-    for _ in range(warmup):
+    # at least `warmup` untimed steps, and at least 20 ms of them: the self-check that runs before
+    # is CPU work, the GPU idles meanwhile and its first launches afterwards run below full clocks
+    t_warm = time.perf_counter()
+    done = 0
+    while done < warmup or time.perf_counter() - t_warm < 0.02:
         fn()
+        done += 1
+        if done % 16 == 0:
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
