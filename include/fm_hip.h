@@ -179,7 +179,7 @@ int fm_ce_bwd(const void* logits, const int64_t* labels, const float* lse, const
  * (the way the reference's KL writes its gradient into an owned student tensor,
  * kernels/kl.py:146-150, 157-160); lse may be NULL. Rows wider than 128 KiB (or unaligned
  * buffers) are swept twice inside the same launch (the second sweep follows the first at
- * once, while the rows in flight still fit the memory-side cache). lse of ignored rows is written as 0 (those rows are not read). */
+ * once, when the memory-side cache is most likely to still hold the row). lse of ignored rows is written as 0 (those rows are not read). */
 int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float* row_loss,
                     float* loss, float* n_valid, void* dlogits, int64_t n, int64_t v, int dtype,
                     int64_t ignore_index, int reduction, fm_stream_t stream);
@@ -207,7 +207,7 @@ int fm_kl_fwd(const void* student, const void* teacher, float* lse_s, float* lse
  * scale = 1/n (FM_REDUCE_MEAN) or 1 (FM_REDUCE_SUM). Rows of at most 64 KiB stay in
  * registers between the log-sum-exps and the store (4 + 2 bytes per pair of 16-bit logits
  * instead of 4 + 4 + 2); wider rows are swept twice inside the same launch (the second
- * sweep follows the first at once, while the rows in flight fit the memory-side cache). dstudent may be the student buffer itself when
+ * sweep follows the first at once, when the memory-side cache is most likely to still hold the row). dstudent may be the student buffer itself when
  * grad_dtype == dtype (kl.py:146-150, reuse=True); lse_s / lse_t may be NULL.
  * fm_scale_inplace applies an upstream gradient other than 1. */
 int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, float* lse_t,
