@@ -167,8 +167,15 @@ __global__ __launch_bounds__(kBwdBlock) void norm_bwd_kernel(
   constexpr int RPB = BLOCK / TPR;
   constexpr int COVER = TPR * ITERS * EPV;   // columns covered by one row's threads
   constexpr int NB = LN ? ITERS : 1;         // bias-gradient accumulators exist only for LN
+  // Rows of 512 threads: the 8 * ITERS weight registers do not fit next to the packed rows and
+  // the fp32 column sums (the compiler spilled 12-20 bytes per lane to scratch), so the weight
+  // columns live in LDS as fp32 instead, one 16-byte quad per lane and read, laid out so that
+  // neighbouring lanes read neighbouring quads (no bank conflicts).
+  constexpr bool WLDS = TPR >= 512;
+  constexpr int QPV = EPV / 4;
   __shared__ float red[RPB * (TPR > 64 ? TPR / 64 : 1)];
   __shared__ float fold[RPB > 1 ? RPB * COVER : 1];
+  __shared__ f32x4 wsm[WLDS ? ITERS * QPV * TPR : 1];
 
   const int tid = threadIdx.x;
   const int rib = tid / TPR;
@@ -177,21 +184,47 @@ __global__ __launch_bounds__(kBwdBlock) void norm_bwd_kernel(
   const float inv_d = 1.f / (float)d;
   const int pcols = LN ? 2 * d : d;
 
-  float wv[ITERS][EPV];
+  float wv[WLDS ? 1 : ITERS][EPV];
   float acc[ITERS][EPV];
   float accb[NB][EPV];
 #pragma unroll
   for (int i = 0; i < ITERS; ++i) {
     const int c = i * TPR + t;
+    float wl[EPV];
     if (c < nvec) {
-      load_w<T, WT>(w, c * EPV, wv[i]);
+      load_w<T, WT>(w, c * EPV, wl);
     } else {
 #pragma unroll
-      for (int e = 0; e < EPV; ++e) wv[i][e] = 0.f;
+      for (int e = 0; e < EPV; ++e) wl[e] = 0.f;
+    }
+    if constexpr (WLDS) {
+      if (rib == 0) {
+#pragma unroll
+        for (int q = 0; q < QPV; ++q) {
+          const f32x4 v4 = {wl[4 * q], wl[4 * q + 1], wl[4 * q + 2], wl[4 * q + 3]};
+          wsm[(i * QPV + q) * TPR + t] = v4;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) wv[i][e] = wl[e];
     }
 #pragma unroll
     for (int e = 0; e < EPV; ++e) acc[i][e] = 0.f;
   }
+  if constexpr (WLDS) __syncthreads();
+  auto weights = [&](int i, float (&o)[EPV]) {
+    if constexpr (WLDS) {
+#pragma unroll
+      for (int q = 0; q < QPV; ++q) {
+        const f32x4 v4 = wsm[(i * QPV + q) * TPR + t];
+        o[4 * q] = v4.x; o[4 * q + 1] = v4.y; o[4 * q + 2] = v4.z; o[4 * q + 3] = v4.w;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) o[e] = wv[i][e];
+    }
+  };
 #pragma unroll
   for (int i = 0; i < NB; ++i) {
 #pragma unroll
@@ -226,17 +259,18 @@ __global__ __launch_bounds__(kBwdBlock) void norm_bwd_kernel(
     for (int i = 0; i < ITERS; ++i) {
       const int c = i * TPR + t;
       if (valid && c < nvec) {
-        float xv[EPV], gv[EPV];
+        float xv[EPV], gv[EPV], wc[EPV];
         Elem<T>::unpack(rx[i], xv);
         Elem<T>::unpack(rg[i], gv);
+        weights(i, wc);
 #pragma unroll
         for (int e = 0; e < EPV; ++e) {
           const float xh = (xv[e] - mu) * r;
           acc[i][e] += gv[e] * xh;
-          dot += (gv[e] * wv[i][e]) * xh;
+          dot += (gv[e] * wc[e]) * xh;
           if constexpr (LN) {
             accb[i][e] += gv[e];
-            gsum += gv[e] * wv[i][e];
+            gsum += gv[e] * wc[e];
           }
         }
       }
@@ -249,12 +283,13 @@ __global__ __launch_bounds__(kBwdBlock) void norm_bwd_kernel(
     for (int i = 0; i < ITERS; ++i) {
       const int c = i * TPR + t;
       if (valid && c < nvec) {
-        float xv[EPV], gv[EPV], o[EPV];
+        float xv[EPV], gv[EPV], o[EPV], wc[EPV];
         Elem<T>::unpack(rx[i], xv);
         Elem<T>::unpack(rg[i], gv);
+        weights(i, wc);
 #pragma unroll
         for (int e = 0; e < EPV; ++e)
-          o[e] = ((gv[e] * wv[i][e] - gmean) - ((xv[e] - mu) * r) * cmean) * r;
+          o[e] = ((gv[e] * wc[e] - gmean) - ((xv[e] - mu) * r) * cmean) * r;
         if (gxn != nullptr) {
           float rv[EPV];
           if constexpr (EARLY_RES) Elem<T>::unpack(rr[i], rv);
