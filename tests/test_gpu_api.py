@@ -291,6 +291,23 @@ def test_fp16_losses_apply_the_upstream_gradient_before_rounding():
     assert torch.count_nonzero(sd.grad) >= 0.99 * torch.count_nonzero(wantk)
 
 
+def test_fp16_chunked_cross_entropy_under_checkpointing():
+    # fp16 takes the two-pass form, here inside the checkpoint-per-chunk loop of loss.py:23-51
+    g = torch.Generator().manual_seed(79)
+    h = torch.randn(90, 64, generator=g).half().to(DEV).requires_grad_(True)
+    wt = (0.2 * torch.randn(700, 64, generator=g)).half().to(DEV).requires_grad_(True)
+    yy = torch.randint(0, 700, (90,), generator=g).to(DEV)
+    yy[::11] = -100
+    loss = chunked_cross_entropy(h, wt, yy, chunk=32)
+    (loss * 1024.0).backward()
+    hr = h.detach().float().requires_grad_(True)
+    wr = wt.detach().float().requires_grad_(True)
+    ref = F.cross_entropy((hr.half().float() @ wr.t()).half().float(), yy, ignore_index=-100)
+    (ref * 1024.0).backward()
+    assert loss.item() == pytest.approx(ref.item(), rel=2e-3)
+    assert close(h.grad, hr.grad, rel=2e-2) and close(wt.grad, wr.grad, rel=2e-2)
+
+
 def test_losses_allow_a_second_backward_when_the_gradient_buffer_is_private():
     # the reference's KL multiplies its stored gradient out of place (kernels/kl.py:183-191), so
     # retain_graph=True works there; here the first backward scales in place and later ones redo the pass
