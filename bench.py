@@ -45,36 +45,36 @@ METRIC = "HBM GB/s & % roofline: RMSNorm, CE/KL fwd+bwd; MoE top-k rows/s"
 # HBM traffic per launch, keyed by the kernel's full name as fm_last_kernel() reports it:
 # (FETCH_SIZE KiB, WRITE_SIZE KiB) per dispatch from two `rocprofv3 --pmc` runs of this file
 # (profiles/all_workloads_hbm_traffic_pmc.txt). Each counter is scaled by what it reads for the
-# library's own 1 GiB copy (probe_copy_kernel: 524296.1 KiB fetched, 1049373.6 KiB written).
+# library's own 1 GiB copy (probe_copy_kernel: 524296.9 KiB fetched, 1049450.7 KiB written).
 # A kernel that is not in the table (a retune changed its template arguments) reports null.
-TRAFFIC_SCALE = (1048576.0 / 524296.1, 1048576.0 / 1049373.6)
+TRAFFIC_SCALE = (1048576.0 / 524296.9, 1048576.0 / 1049450.7)
 TRAFFIC_KIB = {
-    "ce_bwd_kernel<bf16_t, 1024, 4>": (244178.4, 512255.1),
+    "ce_bwd_kernel<bf16_t, 1024, 4>": (244178.4, 512239.3),
     "ce_fwd_kernel<bf16_t, 512, 4>": (256535.6, 512.2),
-    "ce_loss_grad_kernel<bf16_t, 512, 8>": (243960.2, 512530.6),
+    "ce_loss_grad_kernel<bf16_t, 512, 8>": (243960.2, 512524.2),
     "combine_kernel<bf16_t, true>": (133143.1, 131072.0),
-    "kl_bwd_kernel<bf16_t, bf16_t, 1024, 8>": (1026352.3, 1026488.3),
-    "kl_fwd_kernel<bf16_t, 512, 2>": (1026083.6, 386.5),
-    "kl_fwd_topk_kernel<bf16_t, 512, 2, false>": (1052918.5, 2432.3),
-    "kl_fwd_topk_kernel<bf16_t, 512, 2, true>": (2057243.1, 1028505.3),
-    "kl_loss_grad_wide_kernel<bf16_t, bf16_t, 1024, 2>": (2041075.5, 1026451.7),
-    "norm_bwd_kernel<bf16_t, bf16_t, 256, 2, false>": (65822.1, 69633.0),
-    "norm_bwd_kernel<bf16_t, float, 512, 2, false>": (394398.1, 272384.0),
-    "norm_bwd_kernel<bf16_t, float, 512, 2, true>": (395175.2, 281600.0),
-    "norm_bwd_kernel<bf16_t, float, 64, 2, false>": (16461.5, 17408.0),
-    "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, false, false>": (32820.6, 65848.4),
-    "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, true, false>": (65587.1, 131368.3),
-    "norm_fwd_kernel<bf16_t, float, 512, 2, true, false>": (262295.6, 524835.9),
-    "norm_fwd_kernel<bf16_t, float, 512, 2, true, true>": (262429.3, 525358.4),
-    "norm_fwd_kernel<bf16_t, float, 64, 2, false, false>": (8221.1, 16448.2),
-    "rope_vec_kernel<bf16_t, float, 8, false, 2>": (132141.7, 266248.1),
-    "rope_vec_kernel<bf16_t, float, 8, true, 2>": (265272.2, 263177.2),
+    "kl_bwd_kernel<bf16_t, bf16_t, 1024, 8>": (1026352.3, 1026268.3),
+    "kl_fwd_kernel<bf16_t, 512, 2>": (1026083.8, 386.3),
+    "kl_fwd_topk_kernel<bf16_t, 512, 2, false>": (1052951.3, 2434.7),
+    "kl_fwd_topk_kernel<bf16_t, 512, 2, true>": (2060390.4, 1028521.8),
+    "kl_loss_grad_wide_kernel<bf16_t, bf16_t, 1024, 2>": (2041115.1, 1026451.3),
+    "norm_bwd_kernel<bf16_t, bf16_t, 256, 2, false>": (65815.9, 69634.1),
+    "norm_bwd_kernel<bf16_t, float, 512, 2, false>": (393631.6, 270336.3),
+    "norm_bwd_kernel<bf16_t, float, 512, 2, true>": (393894.8, 278528.0),
+    "norm_bwd_kernel<bf16_t, float, 64, 2, false>": (16461.6, 17408.0),
+    "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, false, false>": (32820.6, 65849.9),
+    "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, true, false>": (65585.1, 131371.5),
+    "norm_fwd_kernel<bf16_t, float, 512, 2, true, false>": (262295.6, 524834.9),
+    "norm_fwd_kernel<bf16_t, float, 512, 2, true, true>": (262429.3, 525356.4),
+    "norm_fwd_kernel<bf16_t, float, 64, 2, false, false>": (8227.6, 16448.2),
+    "rope_vec_kernel<bf16_t, float, 8, false, 2>": (132141.7, 266250.9),
+    "rope_vec_kernel<bf16_t, float, 8, true, 2>": (265272.2, 263182.3),
     "route_bwd_kernel<float, 8, true>": (2270.0, 4096.0),
-    "route_group_kernel<float, 8, true>": (2104.5, 328.0),
-    "scatter_kernel<bf16_t, true>": (66086.0, 262278.5),
-    "swiglu_split_kernel<bf16_t, true, false>": (458769.6, 458752.3),
-    "swiglu_split_kernel<bf16_t, true, true>": (688148.0, 917504.4),
-    "topk_lds_kernel<bf16_t, 1024, 4, 0>": (546136.4, 1024.0),
+    "route_group_kernel<float, 8, true>": (2104.5, 328.7),
+    "scatter_kernel<bf16_t, true>": (66086.1, 262265.5),
+    "swiglu_split_kernel<bf16_t, true, false>": (458769.6, 458752.1),
+    "swiglu_split_kernel<bf16_t, true, true>": (688148.0, 917504.3),
+    "topk_lds_kernel<bf16_t, 1024, 4, 0>": (546078.0, 1024.0),
 }
 TRAFFIC_SOURCE = "profiles/all_workloads_hbm_traffic_pmc.txt"
 
