@@ -116,12 +116,85 @@ __device__ __forceinline__ float fold_vector_max(const u32x4& raw) {
   return bad ? __builtin_nanf("") : m;
 }
 
+// ---- 16-bit stream keys of the half types.
+// The streaming pass of a bf16 / fp16 row needs only the maximum of each 16-byte vector, so it
+// never unpacks to fp32: two elements at a time, the sign-magnitude bit patterns are turned into
+// unsigned 16-bit keys with packed integer instructions and reduced with packed maxima.
+//   skey(b) = (b ^ (b < 0 ? 0x7FFF : 0)) + 0x8000 - off   (mod 2^16),  off = 0x7FFF - bits(+inf)
+// is monotone in the value, puts -inf at 0 and +inf at kNanAbove, and -- because the subtraction
+// wraps -- both NaN signs above kNanAbove. -0.0 lands one below +0.0 (the two tie in the final
+// order), which skey_threshold makes up for.
+template <typename T> struct SKey { static constexpr bool ok = false; };
+template <> struct SKey<bf16_t> { static constexpr bool ok = true; static constexpr uint32_t inf = 0x7F80u; };
+template <> struct SKey<f16_t> { static constexpr bool ok = true; static constexpr uint32_t inf = 0x7C00u; };
+template <typename T> struct SKeyC {
+  static constexpr uint32_t off = 0x7FFFu - SKey<T>::inf;
+  static constexpr uint32_t add = (0x8000u - off) & 0xFFFFu;
+  static constexpr uint32_t kNanAbove = (0x8000u + SKey<T>::inf - off) & 0xFFFFu;
+};
+
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+typedef short i16x2_t __attribute__((ext_vector_type(2)));
+
+// keys of the two elements packed in one 32-bit word
+template <typename T>
+__device__ __forceinline__ u16x2_t skey_pair(uint32_t two) {
+  const i16x2_t sgn = __builtin_bit_cast(i16x2_t, two) >> (short)15;
+  const uint32_t t = two ^ (__builtin_bit_cast(uint32_t, sgn) & 0x7FFF7FFFu);
+  const u16x2_t a = {(unsigned short)SKeyC<T>::add, (unsigned short)SKeyC<T>::add};
+  return __builtin_bit_cast(u16x2_t, t) + a;
+}
+// largest key of a 16-byte vector
+template <typename T>
+__device__ __forceinline__ uint32_t skey_vector_max(const u32x4& raw) {
+  const u16x2_t a = __builtin_elementwise_max(skey_pair<T>(raw[0]), skey_pair<T>(raw[1]));
+  const u16x2_t b = __builtin_elementwise_max(skey_pair<T>(raw[2]), skey_pair<T>(raw[3]));
+  const u16x2_t m = __builtin_elementwise_max(a, b);
+  const uint32_t lo = m[0], hi = m[1];
+  return lo > hi ? lo : hi;
+}
+template <typename T>
+__device__ __forceinline__ uint32_t skey_of_bits(uint32_t b) {
+  return ((b ^ ((b & 0x8000u) ? 0x7FFFu : 0u)) + SKeyC<T>::add) & 0xFFFFu;
+}
+// value of a key that is not above kNanAbove
+template <typename T>
+__device__ __forceinline__ float float_of_skey(uint32_t s) {
+  const uint32_t t = (s - SKeyC<T>::add) & 0xFFFFu;
+  const uint32_t b = t ^ ((t & 0x8000u) ? 0x7FFFu : 0u);
+  if constexpr (Elem<T>::kDtype == FM_BF16) return bf16_bits_to_float((uint16_t)b);
+  else return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
+}
+// Smallest stream key a vector maximum can have when the vector holds an element whose fp32 key
+// reaches tau (tau_f is tau's float image): the key of tau_f rounded DOWN to T. Zero admits -0.0.
+template <typename T>
+__device__ __forceinline__ uint32_t skey_threshold(uint32_t tau, float tau_f, bool only_nan) {
+  // the NaN key, whole or cut down to the bits T can set: vectors that hold a NaN
+  if (only_nan || tau > 0xFF800000u) return SKeyC<T>::kNanAbove + 1u;
+  if (tau <= 0x007FFFFFu) return 0u;   // at or below -inf: everything
+  uint32_t b;
+  float back;
+  if constexpr (Elem<T>::kDtype == FM_BF16) {
+    b = pack_bf16(tau_f, 0.f) & 0xFFFFu;
+    back = bf16_bits_to_float((uint16_t)b);
+  } else {
+    const _Float16 h = (_Float16)tau_f;
+    b = __builtin_bit_cast(uint16_t, h);
+    back = (float)h;
+  }
+  if ((b & 0x7FFFu) == 0u) return skey_of_bits<T>(0x8000u);
+  uint32_t s = skey_of_bits<T>(b);
+  if (back > tau_f && s > 0u) s -= 1u;   // keys are dense in the values: one key down is one value down
+  return s;
+}
+
 // Everything after the streaming read. With kVecMaxRegs `vmax` holds NV vector maxima per
 // thread (vector i * THREADS + tid in slot i); with kVecMaxLds `vhi[c]` holds key_prefix of
 // vector c's maximum for the whole row, padded with zeros to a multiple of four entries and
-// 8-byte aligned; with kVecMaxNone the row is walked a second time. Outputs go to row `orow` of the [rows, k] arrays;
+// 8-byte aligned (with SKEY: the 16-bit stream key of vector c's maximum instead); with
+// kVecMaxNone the row is walked a second time. Outputs go to row `orow` of the [rows, k] arrays;
 // `probs` (optional) receives exp2(x * c1 - lse2) of the selected elements.
-template <typename T, int THREADS, int NV, int VMAX, int BIG = kTopkNormal>
+template <typename T, int THREADS, int NV, int VMAX, int BIG = kTopkNormal, bool SKEY = false>
 __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowSplit& sp, int v, int k,
                                             const float (&vmax)[NV], const uint16_t* vhi, float fm,
                                             bool has_nan,
@@ -233,7 +306,8 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
             if (c < sp.nvec && take_of(vmax[i])) list(c);
           }
         } else {
-          const uint32_t tau_hi = tau >> 16;
+          uint32_t tau_hi = tau >> 16;
+          if constexpr (SKEY) tau_hi = skey_threshold<T>(tau, tau_f, only_nan);
           const uint64_t* quad = reinterpret_cast<const uint64_t*>(vhi);
           for (int q = tid; q * 4 < sp.nvec; q += THREADS) {
             const uint64_t four = quad[q];

@@ -7,7 +7,10 @@
 // One workgroup per row, one streaming read of the row from HBM:
 //   A  every thread folds each 16-byte vector it reads to one maximum and leaves a 16-bit
 //      prefix of that maximum's key in LDS (2 bytes per 16 bytes of row); the maximum over
-//      its vectors is the thread's "group maximum";
+//      its vectors is the thread's "group maximum". bf16 / fp16 rows are never unpacked for
+//      this: packed 16-bit integer instructions turn two elements at a time into 16-bit keys
+//      (about 20 instructions per vector instead of 70; the pass is otherwise bound by
+//      instruction issue as much as by the read);
 //   T  each full wave finds the ceil(k / waves)-th largest of its 64 group maxima with a
 //      ballot search; the minimum over the waves, tau, can never be above the true k-th
 //      value, because at least k group maxima are >= tau;
@@ -24,6 +27,8 @@
 // registers (up to 32 per thread) or make two full passes.
 // Keys are order-preserving integer images of the fp32 value, so no float is ever summed and
 // the result is bit-reproducible.
+#include <type_traits>
+
 #include "fm_topk.cuh"
 
 using namespace fm;
@@ -93,11 +98,12 @@ void topk_kernel(const T* __restrict__ x, T* __restrict__ values, int32_t* __res
 // maxima in registers: few registers, so several workgroups share a compute unit and one
 // row's selection overlaps the next row's streaming read.
 template <typename T, int THREADS, int UNROLL, int BIG>
-__global__ __launch_bounds__(THREADS) void topk_lds_kernel(const T* __restrict__ x, T* __restrict__ values,
+__global__ __launch_bounds__(THREADS, THREADS >= 256 ? 8 : 1) void topk_lds_kernel(const T* __restrict__ x, T* __restrict__ values,
                                                            int32_t* __restrict__ idx32,
                                                            int64_t* __restrict__ idx64, int v, int k,
                                                            bool vec_ok) {
   constexpr int EPV = Elem<T>::kVec;
+  constexpr bool SK = SKey<T>::ok;   // bf16 / fp16: vhi holds 16-bit stream keys
   __shared__ TopkShared<THREADS, kVecMaxLds, BIG> sh;
   extern __shared__ __align__(16) uint16_t vhi[];
   const int64_t row = blockIdx.x;
@@ -111,6 +117,32 @@ __global__ __launch_bounds__(THREADS) void topk_lds_kernel(const T* __restrict__
       const int p = ((sp.nvec + 3) & ~3) - 1 - tid;
       if (tid < 3 && p >= sp.nvec) vhi[p] = 0;
     }
+    if constexpr (SK) {
+      // half types: 16-bit keys from packed integer instructions, no unpacking to fp32
+      uint32_t sm = 0u;   // the key of -inf
+      auto tile = [&](int c0, auto full) {
+        u32x4 raw[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+          const int c = c0 + u * THREADS + tid;
+          if (decltype(full)::value || c < sp.nvec) raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+          const int c = c0 + u * THREADS + tid;
+          if (decltype(full)::value || c < sp.nvec) {
+            const uint32_t m = skey_vector_max<T>(raw[u]);
+            vhi[c] = (uint16_t)m;
+            sm = m > sm ? m : sm;
+          }
+        }
+      };
+      int c0 = 0;
+      for (; c0 + THREADS * UNROLL <= sp.nvec; c0 += THREADS * UNROLL) tile(c0, std::true_type{});
+      if (c0 < sp.nvec) tile(c0, std::false_type{});
+      if (sm > SKeyC<T>::kNanAbove) has_nan = true;
+      else fm = float_of_skey<T>(sm);
+    } else {
     for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
       u32x4 raw[UNROLL];
 #pragma unroll
@@ -130,6 +162,7 @@ __global__ __launch_bounds__(THREADS) void topk_lds_kernel(const T* __restrict__
         }
       }
     }
+    }
     const int ne = edge_count(sp, v);
     for (int e = tid; e < ne; e += THREADS) {
       const float f = Elem<T>::load1(rp + edge_col(sp, e));
@@ -138,8 +171,8 @@ __global__ __launch_bounds__(THREADS) void topk_lds_kernel(const T* __restrict__
     }
   }
   const float none[1] = {0.f};
-  topk_finish<T, THREADS, 1, kVecMaxLds, BIG>(rp, sp, v, k, none, vhi, fm, has_nan, sh, row, values, idx32, idx64,
-                                         nullptr, 0.f, 0.f);
+  topk_finish<T, THREADS, 1, kVecMaxLds, BIG, SK>(rp, sp, v, k, none, vhi, fm, has_nan, sh, row, values, idx32,
+                                                  idx64, nullptr, 0.f, 0.f);
 }
 
 // Rows of up to 2048 elements: one wave per row (a 64-thread workgroup each), the whole row as
