@@ -15,6 +15,8 @@
 // first (k - #greater) ties. Keys are order-preserving integer images of the fp32 value.
 #pragma once
 
+#include <atomic>
+
 #include "fm_vocab.cuh"
 
 namespace fm {
@@ -546,3 +548,28 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
 }
 
 }  // namespace fm
+
+namespace fm_host {
+// Rows of more than 20480 vectors still fit the 160 KB of a compute unit, one 1024-thread
+// workgroup at a time (rows of up to half a million bf16 / a quarter of a million fp32
+// elements). Dynamic LDS beyond 64 KB has to be allowed per kernel and device before the first
+// such launch; K is the kernel's address.
+constexpr int kLdsWideMaxVec = 66560;
+static_assert(sizeof(fm::TopkShared<1024, fm::kVecMaxLds, fm::kTopkBig>) + (size_t)(kLdsWideMaxVec + 8) * 2 <=
+                  160 * 1024 - 256,
+              "prefixes of the widest row plus the selection state must fit one compute unit's LDS");
+template <auto K>
+bool allow_wide_lds() {
+  static std::atomic<uint64_t> allowed{0};   // one bit per device
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+  if ((allowed.load(std::memory_order_acquire) >> dev) & 1u) return true;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(K), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          (kLdsWideMaxVec + 8) * 2) != hipSuccess) {
+    (void)hipGetLastError();   // not fatal: the caller has a form without the prefixes
+    return false;
+  }
+  allowed.fetch_or(1ull << dev, std::memory_order_release);
+  return true;
+}
+}  // namespace fm_host

@@ -235,6 +235,10 @@ __global__ __launch_bounds__(THREADS) void kl_fwd_topk_kernel(
   KLState st{kNegBig, 0.f, kNegBig, 0.f, 0.f};
   float fm = -INFINITY;
   bool has_nan = false;
+  // (with the gradient sweep behind it the float form schedules better: 780 against 795 us at
+  // 4096 x 128256, so only the forward-only kernel takes the packed keys)
+  constexpr bool SK = SKey<T>::ok && !GRAD;
+  uint32_t sm = 0u;   // largest 16-bit stream key of this thread's vectors (0 is -inf)
   {  // zero the padding of the last quad of prefixes
     const int p = ((sp.nvec + 3) & ~3) - 1 - tid;
     if (tid < 3 && p >= sp.nvec) vhi[p] = 0;
@@ -260,13 +264,23 @@ __global__ __launch_bounds__(THREADS) void kl_fwd_topk_kernel(
     for (int u = 0; u < UNROLL; ++u) {
       const int c = c0 + u * THREADS + tid;
       if (c < sp.nvec) {
-        const float m = fold_vector_max<T>(rt[u]);
-        const bool bad = m != m;
-        vhi[c] = (uint16_t)(bad ? 0xFFFFu : key_prefix(key_of(m)));
-        fm = fmaxf(fm, m);
-        has_nan |= bad;
+        if constexpr (SK) {   // half types: 16-bit keys straight from the packed words
+          const uint32_t m = skey_vector_max<T>(rt[u]);
+          vhi[c] = (uint16_t)m;
+          sm = m > sm ? m : sm;
+        } else {
+          const float m = fold_vector_max<T>(rt[u]);
+          const bool bad = m != m;
+          vhi[c] = (uint16_t)(bad ? 0xFFFFu : key_prefix(key_of(m)));
+          fm = fmaxf(fm, m);
+          has_nan |= bad;
+        }
       }
     }
+  }
+  if constexpr (SK) {
+    if (sm > SKeyC<T>::kNanAbove) has_nan = true;
+    else fm = float_of_skey<T>(sm);
   }
   const int ne = edge_count(sp, v);
   for (int e = tid; e < ne; e += THREADS) {
@@ -284,8 +298,8 @@ __global__ __launch_bounds__(THREADS) void kl_fwd_topk_kernel(
     row_kl[row] = kl2 * kLn2;
   }
   const float none[1] = {0.f};
-  topk_finish<T, THREADS, 1, kVecMaxLds>(tp_, sp, v, k, none, vhi, fm, has_nan, sh, row, tk_values,
-                                         tk_idx32, tk_idx64, tk_probs, c1, l2t);
+  topk_finish<T, THREADS, 1, kVecMaxLds, kTopkNormal, SK>(tp_, sp, v, k, none, vhi, fm, has_nan, sh, row,
+                                                          tk_values, tk_idx32, tk_idx64, tk_probs, c1, l2t);
   if constexpr (GRAD)
     kl_grad_sweep<T, T, THREADS, UNROLL>(sp_, tp_, dstudent + row * (int64_t)v, sp, v, c1, l2s, l2t, mul);
 }
@@ -882,9 +896,20 @@ static int kl_topk_entry(const char* what, const void* student, const void* teac
   FM_CHECK_ARG(inv_temperature > 0.f, "%s: the temperature must be positive", what);
   const int esize = dtype == FM_F32 ? 4 : 2;
   const int64_t nvec_max = v / (16 / esize);
-  if (k > kMaxK || nvec_max > kFusedMaxVec) {
+  // rows past kFusedMaxVec vectors: one 1024-thread workgroup per compute unit, more than 64 KB of LDS
+  const bool wide = nvec_max > kFusedMaxVec;
+  bool wide_ok = !wide;
+  if (wide && k <= kMaxK && nvec_max <= fm_host::kLdsWideMaxVec) {
+#define ALLOW(T)                                                                                   \
+  (dstudent != nullptr ? fm_host::allow_wide_lds<&kl_fwd_topk_kernel<T, 1024, 2, true>>()          \
+                       : fm_host::allow_wide_lds<&kl_fwd_topk_kernel<T, 1024, 2, false>>())
+    wide_ok = dtype == FM_F32 ? ALLOW(float) : (dtype == FM_BF16 ? ALLOW(bf16_t) : ALLOW(f16_t));
+#undef ALLOW
+  }
+  if (k > kMaxK || !wide_ok) {
     fm_host::set_error("%s: k <= %d and rows of at most %d bytes are fused (k=%d, v=%lld); "
-                       "call fm_kl_fwd and fm_topk instead", what, kMaxK, kFusedMaxVec * 16, k, (long long)v);
+                       "call fm_kl_fwd and fm_topk instead", what, kMaxK, fm_host::kLdsWideMaxVec * 16, k,
+                       (long long)v);
     return FM_ERR_UNSUPPORTED;
   }
   FM_CHECK_ARG(n == 0 || (student && teacher && lse_s && lse_t && row_kl && topk_indices),
@@ -896,6 +921,7 @@ static int kl_topk_entry(const char* what, const void* student, const void* teac
     int64_t* i64 = index_bits == 64 ? static_cast<int64_t*>(topk_indices) : nullptr;
     int threads = fm_host::get_param(fm_host::P_VOCAB_THREADS);
     if (threads != 256 && threads != 1024) threads = 512;
+    if (wide) threads = 1024;
     const size_t lds = (size_t)((nvec_max + 3) / 4 * 4 + 4) * sizeof(uint16_t);
     const dim3 grid((unsigned)n);
     // gradient (when asked for) is for an upstream gradient of 1

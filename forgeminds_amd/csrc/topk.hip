@@ -576,6 +576,10 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
 #undef GOWV
 #undef GOW
   }
+  else if (nvec > kLdsMaxVec && nvec <= fm_host::kLdsWideMaxVec && !big &&
+           fm_host::allow_wide_lds<&topk_lds_kernel<T, 1024, 4, kTopkNormal>>()) GOL(1024, 4, false);
+  else if (nvec > kLdsMaxVec && nvec <= fm_host::kLdsWideMaxVec && big &&
+           fm_host::allow_wide_lds<&topk_lds_kernel<T, 1024, 4, kTopkBig>>()) GOL(1024, 4, true);
   else if (nvec > kLdsMaxVec) {
     if (nvec <= 1024 * 32) {
       if (big) GO(1024, 32, true);

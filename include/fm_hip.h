@@ -220,7 +220,7 @@ int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, floa
  * teacher twice. Selection follows topk.py:13-19 on the raw teacher logits (softmax and a
  * positive temperature keep the order): topk_values [n, k] (row dtype, may be NULL),
  * topk_indices [n, k] (int32 or int64 by index_bits), topk_probs [n, k] fp32 (may be NULL) =
- * softmax(teacher * inv_temperature) at the selected columns. Rows wider than 320 KiB or
+ * softmax(teacher * inv_temperature) at the selected columns. Rows wider than 1040 KiB or
  * k > 512 return FM_ERR_UNSUPPORTED; the caller then uses fm_kl_fwd + fm_topk. */
 int fm_kl_fwd_topk(const void* student, const void* teacher, float* lse_s, float* lse_t,
                    float* row_kl, float* loss, void* topk_values, void* topk_indices,

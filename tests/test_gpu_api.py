@@ -665,8 +665,8 @@ def test_kl_div_logits_topk_autograd_and_wide_rows():
     assert not probs.requires_grad and idx.dtype == torch.int32
     assert torch.equal(idx.cpu().long(), O.topk(t, 16)[1])
     # a row wider than the fused kernel takes goes through the two kernels, same results
-    s = torch.randn(1, 32 * 1024 * 4 + 40, generator=g)
-    t = torch.randn(1, 32 * 1024 * 4 + 40, generator=g)
+    s = torch.randn(1, 66561 * 4 + 40, generator=g)
+    t = torch.randn(1, 66561 * 4 + 40, generator=g)
     loss, probs, idx = kernels.kl_div_logits_topk(s.to("cuda"), t.to("cuda"), 8, reduction="sum")
     assert torch.equal(idx.cpu(), O.topk(t, 8)[1])
     want = torch.gather(torch.softmax(t.double(), -1), -1, idx.cpu())

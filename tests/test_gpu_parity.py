@@ -509,7 +509,9 @@ def test_kl_known_answers_on_gpu():
 KLTOPK_CASES = [(16, 128256, 64, BF16, 2.0), (6, 32000, 64, BF16, 1.0), (4, 50257, 33, BF16, 2.0),
                 (3, 4096, 8, F32, 1.0), (2, 80000, 64, F32, 2.0), (5, 20000, 100, F16, 1.0),
                 (3, 700, 5, BF16, 1.0), (2, 1025, 512, BF16, 2.0), (4, 1, 1, F32, 1.0),
-                (2, 9000, 512, F32, 1.0)]
+                (2, 9000, 512, F32, 1.0),
+                # rows whose teacher prefixes take more than 64 KB of LDS (one workgroup per compute unit)
+                (2, 262144, 64, BF16, 2.0), (2, 170001, 40, F16, 1.0), (1, 131072, 64, F32, 1.0)]
 
 
 @pytest.mark.parametrize("n,v,k,dt,T", KLTOPK_CASES)
@@ -575,8 +577,8 @@ def test_kl_fwd_topk_ties_unaligned_and_unsupported():
     out = _hip.kl_fwd_topk(s3.to(DEV), t3.to(DEV), 4, 1.0, "none", torch.int64)
     assert torch.equal(out[5].cpu(), O.topk(t3, 4)[1]) and out[5][0, 0].item() == 77
     assert math.isnan(out[1][0].item()) and math.isfinite(out[1][1].item())
-    # rows wider than the fused kernel's register budget: the binding says so
-    wide = torch.zeros(1, 32 * 1024 * 8 + 8, dtype=BF16, device=DEV)
+    # rows wider than the fused kernel's LDS budget: the binding says so
+    wide = torch.zeros(1, 66561 * 8, dtype=BF16, device=DEV)
     assert _hip.kl_fwd_topk(wide, wide, 4, 1.0, "none", torch.int64) is None
 
 
@@ -587,7 +589,10 @@ TOPK_CASES = [(32, 128256, 64, BF16), (8, 4096, 64, F32), (4, 64, 8, F32), (3, 5
               (2, 1025, 3, BF16), (3, 70000, 512, F32), (6, 50257, 64, BF16), (2, 140000, 64, F32),
               (1000, 64, 8, F32), (333, 128, 2, BF16), (77, 200, 200, F16), (50, 1024, 512, BF16),
               (41, 1000, 64, F32), (9, 7, 7, BF16), (130, 513, 100, F16), (5, 1024, 1, F32),
-              (6, 4096, 256, BF16), (5, 8192, 512, F32), (4, 8192, 256, F16), (3, 16384, 512, F32)]
+              (6, 4096, 256, BF16), (5, 8192, 512, F32), (4, 8192, 256, F16), (3, 16384, 512, F32),
+              # rows whose vector prefixes need more than 64 KB of LDS, and one past even that
+              (3, 262144, 64, BF16), (2, 500000, 300, BF16), (2, 262144, 64, F32), (2, 262147, 100, F16),
+              (1, 600000, 8, BF16)]
 
 
 @pytest.mark.parametrize("n,v,k,dt", TOPK_CASES)
