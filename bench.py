@@ -70,7 +70,7 @@ TRAFFIC_KIB = {
     "rope_vec_kernel<bf16_t, float, 8, false, 2>": (132141.7, 266250.9),
     "rope_vec_kernel<bf16_t, float, 8, true, 2>": (265272.2, 263182.3),
     "route_bwd_kernel<float, 8, true>": (2270.0, 4096.0),
-    "route_group_kernel<float, 8, true>": (2104.5, 328.7),
+    "route_group_kernel<float, 8, true, false>": (2104.5, 328.7),
     "scatter_kernel<bf16_t, true>": (66086.1, 262265.5),
     "swiglu_split_kernel<bf16_t, true, false>": (458769.6, 458752.1),
     "swiglu_split_kernel<bf16_t, true, true>": (688148.0, 917504.3),

@@ -26,6 +26,7 @@ const char* const kParamNames[fm_host::P_COUNT] = {
     "norm_wide_min_vec",
     "rows_vec_max",
     "rope_heads",
+    "route_presort",
 };
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cus[kMaxDevices];

@@ -967,6 +967,48 @@ def test_route_half_precision_logits_and_all_equal_rows():
     assert order.cpu().tolist() == list(range(0, 260, 2)) + list(range(1, 260, 2))
 
 
+def test_route_pick_forms_agree():
+    """The router picks either by scanning a lane's eight keys per pick or from lane-sorted keys
+    (the default from five picks on): forced either way, every output keeps its bits (NaN payloads
+    aside), on rows of
+    equal logits, rows with a single finite logit (the other picks tie at probability zero),
+    few distinct values, and NaN / +inf rows (all probabilities NaN: lowest experts win)."""
+    try:
+        for e in (8, 60, 64, 130, 256, 512):
+            lg = router_inputs(400, e, 1021)
+            lg[0] = 0.25
+            lg[1] = float("-inf")
+            lg[1, e // 2] = 1.0
+            lg[2] = torch.randint(0, 3, (e,), generator=gen(e)).float()
+            lg[3, e - 1] = float("nan")
+            lg[4, 1] = float("inf")
+            lg[5] = float("-inf")
+            lg[5, [0, e - 1]] = 2.0
+            finite = torch.ones(400, dtype=torch.bool)
+            finite[3] = finite[4] = False
+            for k in (1, 2, 5, 8):
+                if k > e:
+                    continue
+                outs = {}
+                for form in (1, 2):
+                    _hip.set_param("route_presort", form)
+                    outs[form] = _hip.route(lg.to(DEV), k, want_stats=True)
+                    torch.cuda.synchronize()
+                for a, b in zip(outs[1], outs[2]):
+                    if a.is_floating_point():     # NaN where NaN (payloads aside), bits elsewhere
+                        assert torch.equal(torch.isnan(a), torch.isnan(b)), (e, k)
+                        a, b = a.nan_to_num(nan=-7.0), b.nan_to_num(nan=-7.0)
+                    assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (e, k)
+                idx, w = outs[2][0].cpu().long(), outs[2][1].cpu()
+                oi, ow = O.router(lg[finite], k)[:2]
+                assert torch.equal(idx[finite], oi), (e, k)
+                assert torch.allclose(w[finite], ow, rtol=1e-5, atol=0), (e, k)
+                assert idx[3].tolist() == list(range(k)) and idx[4].tolist() == list(range(k)), (e, k)
+                assert torch.isnan(w[3]).all() and torch.isnan(w[4]).all()
+    finally:
+        _hip.set_param("route_presort", 0)
+
+
 # ------------------------------------------------------------------ gather / combine around the permutation
 @pytest.mark.parametrize("n,e,k,d,dt", [(1000, 8, 2, 1024, BF16), (257, 16, 4, 100, F32), (64, 4, 1, 7, F16),
                                          (2048, 64, 2, 4096, BF16), (33, 8, 8, 256, F32)])
