@@ -190,13 +190,45 @@ __device__ __forceinline__ uint32_t skey_threshold(uint32_t tau, float tau_f, bo
   return s;
 }
 
+// The same for fp32 rows: 32-bit stream keys (three integer instructions an element), of which the
+// LDS keeps the upper 16 bits rounded up.
+constexpr uint32_t kSKey32Add = 0x7F800001u;        // 0x80000000 - (0x7FFFFFFF - bits(+inf))
+constexpr uint32_t kSKey32NanAbove = 0xFF000001u;   // the key of +inf
+__device__ __forceinline__ uint32_t skey32(uint32_t b) {
+  return (b ^ ((uint32_t)((int32_t)b >> 31) & 0x7FFFFFFFu)) + kSKey32Add;
+}
+__device__ __forceinline__ uint32_t skey32_vector_max(const u32x4& raw) {
+  const uint32_t a = skey32(raw[0]), b = skey32(raw[1]), c = skey32(raw[2]), d = skey32(raw[3]);
+  const uint32_t ab = a > b ? a : b, cd = c > d ? c : d;
+  return ab > cd ? ab : cd;
+}
+// upper 16 bits, rounded up: s >= t implies skey32_prefix(s) >= skey32_prefix(t)
+__device__ __forceinline__ uint32_t skey32_prefix(uint32_t s) {
+  const uint32_t c = s < 0xFFFF0000u ? s : 0xFFFF0000u;
+  return (c + 0xFFFFu) >> 16;
+}
+__device__ __forceinline__ float float_of_skey32(uint32_t s) {
+  const uint32_t t = s - kSKey32Add;
+  return __builtin_bit_cast(float, t ^ ((uint32_t)((int32_t)t >> 31) & 0x7FFFFFFFu));
+}
+__device__ __forceinline__ uint32_t skey32_threshold(uint32_t tau, float tau_f, bool only_nan) {
+  if (only_nan) return skey32_prefix(kSKey32NanAbove + 1u);
+  if (tau <= 0x007FFFFFu) return 0u;   // at or below -inf: everything
+  const uint32_t b = __builtin_bit_cast(uint32_t, tau_f);
+  return skey32_prefix(skey32((b & 0x7FFFFFFFu) == 0u ? 0x80000000u : b));   // zero admits -0.0
+}
+
+// how the 16-bit entries of `vhi` were made
+enum VhiKind { kVhiPrefix = 0, kVhiStream16 = 1, kVhiStream32 = 2 };
+
 // Everything after the streaming read. With kVecMaxRegs `vmax` holds NV vector maxima per
 // thread (vector i * THREADS + tid in slot i); with kVecMaxLds `vhi[c]` holds key_prefix of
 // vector c's maximum for the whole row, padded with zeros to a multiple of four entries and
-// 8-byte aligned (with SKEY: the 16-bit stream key of vector c's maximum instead); with
+// 8-byte aligned (with SKEY: the 16-bit stream key of vector c's maximum, or the prefix of its
+// 32-bit stream key, instead); with
 // kVecMaxNone the row is walked a second time. Outputs go to row `orow` of the [rows, k] arrays;
 // `probs` (optional) receives exp2(x * c1 - lse2) of the selected elements.
-template <typename T, int THREADS, int NV, int VMAX, int BIG = kTopkNormal, bool SKEY = false>
+template <typename T, int THREADS, int NV, int VMAX, int BIG = kTopkNormal, int SKEY = kVhiPrefix>
 __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowSplit& sp, int v, int k,
                                             const float (&vmax)[NV], const uint16_t* vhi, float fm,
                                             bool has_nan,
@@ -309,7 +341,8 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
           }
         } else {
           uint32_t tau_hi = tau >> 16;
-          if constexpr (SKEY) tau_hi = skey_threshold<T>(tau, tau_f, only_nan);
+          if constexpr (SKEY == kVhiStream16) tau_hi = skey_threshold<T>(tau, tau_f, only_nan);
+          if constexpr (SKEY == kVhiStream32) tau_hi = skey32_threshold(tau, tau_f, only_nan);
           const uint64_t* quad = reinterpret_cast<const uint64_t*>(vhi);
           for (int q = tid; q * 4 < sp.nvec; q += THREADS) {
             const uint64_t four = quad[q];

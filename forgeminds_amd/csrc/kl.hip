@@ -298,7 +298,7 @@ __global__ __launch_bounds__(THREADS) void kl_fwd_topk_kernel(
     row_kl[row] = kl2 * kLn2;
   }
   const float none[1] = {0.f};
-  topk_finish<T, THREADS, 1, kVecMaxLds, kTopkNormal, SK>(tp_, sp, v, k, none, vhi, fm, has_nan, sh, row,
+  topk_finish<T, THREADS, 1, kVecMaxLds, kTopkNormal, SK ? kVhiStream16 : kVhiPrefix>(tp_, sp, v, k, none, vhi, fm, has_nan, sh, row,
                                                           tk_values, tk_idx32, tk_idx64, tk_probs, c1, l2t);
   if constexpr (GRAD)
     kl_grad_sweep<T, T, THREADS, UNROLL>(sp_, tp_, dstudent + row * (int64_t)v, sp, v, c1, l2s, l2t, mul);

@@ -7,10 +7,11 @@
 // One workgroup per row, one streaming read of the row from HBM:
 //   A  every thread folds each 16-byte vector it reads to one maximum and leaves a 16-bit
 //      prefix of that maximum's key in LDS (2 bytes per 16 bytes of row); the maximum over
-//      its vectors is the thread's "group maximum". bf16 / fp16 rows are never unpacked for
-//      this: packed 16-bit integer instructions turn two elements at a time into 16-bit keys
-//      (about 20 instructions per vector instead of 70; the pass is otherwise bound by
-//      instruction issue as much as by the read);
+//      its vectors is the thread's "group maximum". Rows are never unpacked to fp32 for
+//      this: packed 16-bit integer instructions turn two bf16 / fp16 elements at a time into
+//      16-bit keys, three integer instructions an fp32 element into a 32-bit key (about 20
+//      instructions per vector instead of 70 / 40; the pass is otherwise bound by instruction
+//      issue as much as by the read);
 //   T  each full wave finds the ceil(k / waves)-th largest of its 64 group maxima with a
 //      ballot search; the minimum over the waves, tau, can never be above the true k-th
 //      value, because at least k group maxima are >= tau;
@@ -104,6 +105,7 @@ __global__ __launch_bounds__(THREADS, THREADS >= 256 ? 8 : 1) void topk_lds_kern
                                                            bool vec_ok) {
   constexpr int EPV = Elem<T>::kVec;
   constexpr bool SK = SKey<T>::ok;   // bf16 / fp16: vhi holds 16-bit stream keys
+  constexpr bool SK32 = Elem<T>::kDtype == FM_F32;   // fp32: prefixes of 32-bit stream keys
   __shared__ TopkShared<THREADS, kVecMaxLds, BIG> sh;
   extern __shared__ __align__(16) uint16_t vhi[];
   const int64_t row = blockIdx.x;
@@ -117,51 +119,43 @@ __global__ __launch_bounds__(THREADS, THREADS >= 256 ? 8 : 1) void topk_lds_kern
       const int p = ((sp.nvec + 3) & ~3) - 1 - tid;
       if (tid < 3 && p >= sp.nvec) vhi[p] = 0;
     }
-    if constexpr (SK) {
-      // half types: 16-bit keys from packed integer instructions, no unpacking to fp32
-      uint32_t sm = 0u;   // the key of -inf
-      auto tile = [&](int c0, auto full) {
-        u32x4 raw[UNROLL];
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-          const int c = c0 + u * THREADS + tid;
-          if (decltype(full)::value || c < sp.nvec) raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
-        }
-#pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-          const int c = c0 + u * THREADS + tid;
-          if (decltype(full)::value || c < sp.nvec) {
-            const uint32_t m = skey_vector_max<T>(raw[u]);
-            vhi[c] = (uint16_t)m;
-            sm = m > sm ? m : sm;
-          }
-        }
-      };
-      int c0 = 0;
-      for (; c0 + THREADS * UNROLL <= sp.nvec; c0 += THREADS * UNROLL) tile(c0, std::true_type{});
-      if (c0 < sp.nvec) tile(c0, std::false_type{});
-      if (sm > SKeyC<T>::kNanAbove) has_nan = true;
-      else fm = float_of_skey<T>(sm);
-    } else {
-    for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+    // Integer stream keys, no unpacking to fp32: bf16 / fp16 two elements at a time with packed
+    // 16-bit instructions (the LDS keeps the vector's key), fp32 three instructions an element
+    // (the LDS keeps the upper half of the vector's key, rounded up).
+    static_assert(SK || SK32, "rows are bf16, fp16 or fp32");
+    uint32_t sm = 0u;   // the key of -inf
+    auto tile = [&](int c0, auto full) {
       u32x4 raw[UNROLL];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         const int c = c0 + u * THREADS + tid;
-        if (c < sp.nvec) raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
+        if (decltype(full)::value || c < sp.nvec) raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
       }
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
         const int c = c0 + u * THREADS + tid;
-        if (c < sp.nvec) {
-          const float m = fold_vector_max<T>(raw[u]);
-          const bool bad = m != m;
-          vhi[c] = (uint16_t)(bad ? 0xFFFFu : key_prefix(key_of(m)));
-          fm = fmaxf(fm, m);
-          has_nan |= bad;
+        if (decltype(full)::value || c < sp.nvec) {
+          uint32_t m;
+          if constexpr (SK) {
+            m = skey_vector_max<T>(raw[u]);
+            vhi[c] = (uint16_t)m;
+          } else {
+            m = skey32_vector_max(raw[u]);
+            vhi[c] = (uint16_t)skey32_prefix(m);
+          }
+          sm = m > sm ? m : sm;
         }
       }
-    }
+    };
+    int c0 = 0;
+    for (; c0 + THREADS * UNROLL <= sp.nvec; c0 += THREADS * UNROLL) tile(c0, std::true_type{});
+    if (c0 < sp.nvec) tile(c0, std::false_type{});
+    if constexpr (SK) {
+      if (sm > SKeyC<T>::kNanAbove) has_nan = true;
+      else fm = float_of_skey<T>(sm);
+    } else {
+      if (sm > kSKey32NanAbove) has_nan = true;
+      else fm = float_of_skey32(sm);
     }
     const int ne = edge_count(sp, v);
     for (int e = tid; e < ne; e += THREADS) {
@@ -171,7 +165,7 @@ __global__ __launch_bounds__(THREADS, THREADS >= 256 ? 8 : 1) void topk_lds_kern
     }
   }
   const float none[1] = {0.f};
-  topk_finish<T, THREADS, 1, kVecMaxLds, BIG, SK>(rp, sp, v, k, none, vhi, fm, has_nan, sh, row, values, idx32,
+  topk_finish<T, THREADS, 1, kVecMaxLds, BIG, SK ? kVhiStream16 : (SK32 ? kVhiStream32 : kVhiPrefix)>(rp, sp, v, k, none, vhi, fm, has_nan, sh, row, values, idx32,
                                                   idx64, nullptr, 0.f, 0.f);
 }
 

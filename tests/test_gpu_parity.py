@@ -746,19 +746,23 @@ def test_topk_two_wave_rows():
     assert torch.equal(run(x, 40), O.topk(x.cpu(), 40)[1])
 
 
-def test_topk_half_rows_with_signed_zeros_negative_nans_and_denormals():
-    """bf16 / fp16 rows wide enough for the streaming forms, which fold each 16-byte vector to
-    a 16-bit integer key: inputs where that key and the float order could part ways."""
+def test_topk_rows_with_signed_zeros_negative_nans_and_denormals():
+    """Rows wide enough for the streaming forms, which fold each 16-byte vector to an integer key
+    (16-bit for bf16 / fp16, 32-bit for fp32): inputs where that key and the float order could
+    part ways."""
     g = gen(1013)
+
+    def ints(dt):
+        return torch.int32 if dt == F32 else torch.int16
 
     def check(x, k):
         vals, idx = _hip.topk(x.to(DEV), k, torch.int64)
         oi = O.topk(x, k)[1]
         assert torch.equal(idx.cpu(), oi), (x.dtype, tuple(x.shape), k)
         # the selected elements themselves, bit for bit (NaN payloads and the sign of zero included)
-        want = x.view(torch.int16).gather(1, oi)
-        assert torch.equal(vals.cpu().view(torch.int16), want), (x.dtype, tuple(x.shape), k)
-    for dt in (BF16, F16):
+        want = x.view(ints(x.dtype)).gather(1, oi)
+        assert torch.equal(vals.cpu().view(ints(x.dtype)), want), (x.dtype, tuple(x.shape), k)
+    for dt in (BF16, F16, F32):
         for v in (5000, 40000, 131072):
             # the k-th value is zero; most zeros are -0.0, whole vectors hold nothing above -0.0
             x = -(torch.randn(3, v, generator=g).abs() + 0.5).to(dt)
@@ -768,10 +772,11 @@ def test_topk_half_rows_with_signed_zeros_negative_nans_and_denormals():
                 check(x, k)
             # NaNs of both signs among ordinary values, fewer and more of them than k
             x = (3 * torch.randn(3, v, generator=g)).to(dt)
-            bits = x.view(torch.int16)
-            bits[0, 7::501] = -64 if dt == BF16 else -512       # 0xFFC0 / 0xFE00: NaN with the sign set
-            bits[1, 3::1999] = -1                                # 0xFFFF
-            bits[1, 11::2003] = 0x7FFF
+            bits = x.view(ints(dt))
+            neg_nan = {BF16: -64, F16: -512, F32: -4194304}[dt]     # 0xFFC0 / 0xFE00 / 0xFFC00000
+            bits[0, 7::501] = neg_nan
+            bits[1, 3::1999] = -1                                # all ones
+            bits[1, 11::2003] = 0x7FFFFFFF if dt == F32 else 0x7FFF
             bits[2, 5::97] = -3
             for k in (5, 64, 512):
                 check(x, k)
@@ -781,14 +786,21 @@ def test_topk_half_rows_with_signed_zeros_negative_nans_and_denormals():
             x[2, 19::4001] = float("inf")
             for k in (3, 64, 257):
                 check(x, k)
-            # denormals of both signs (fp16: below 6.1e-5; bf16: below 1.2e-38) around zero
-            tiny = 2.0 ** -24 if dt == F16 else 2.0 ** -133
-            x = (torch.randint(-40, 41, (3, v), generator=g).float() * tiny).to(dt)
+            # denormals of both signs around zero (fp16: below 6.1e-5; bf16 / fp32: below 1.2e-38)
+            tiny = {F16: 2.0 ** -24, BF16: 2.0 ** -133, F32: 2.0 ** -149}[dt]
+            x = (torch.randint(-40, 41, (3, v), generator=g).double() * tiny).to(dt)
             for k in (8, 64, 400):
                 check(x, k)
             # few distinct negative values: long tie runs below zero
             x = (-torch.randint(1, 4, (2, v), generator=g).float()).to(dt)
             check(x, 100)
+        # values that differ only in their last mantissa bit (below the 16 bits the LDS keeps of an
+        # fp32 key): the threshold must not cut between them
+        step = torch.finfo(dt).eps
+        x = (1.0 + torch.randint(0, 3, (3, 30000), generator=g).double() * step).to(dt)
+        x[1] = -x[1]
+        for k in (10, 200):
+            check(x, k)
     # the largest finite values and one step below (fp16 65504, 65472)
     x = torch.full((2, 30000), 65472.0).to(F16)
     x[:, 5::7] = 65504.0
