@@ -280,7 +280,10 @@ int fm_softmax_bwd(const void* y, const void* dy, void* dx, int64_t n, int64_t v
  * losses of moe.py:92-95 and the sums behind them, without another pass over the logits:
  *   stats[j] = sum_rows probs[:, j] (j < e),  stats[e] = sum_rows logsumexp(logits)^2,
  *   stats[e+1] = aux = E * sum_j counts[j] / (n k) * stats[j] / n,  stats[e+2] = z = stats[e] / n,
- * summed in a fixed order. 1 <= k <= 8, k <= e <= 512, n*k < 2^31. */
+ * summed in a fixed order. 1 <= k <= 8, k <= e <= 512, n*k < 2^31.
+ * Probabilities below the smallest normal fp32 (a logit more than 87 below the row maximum) come
+ * out as zero and tie by expert index; a row holding a NaN or +inf, or only -inf, has NaN
+ * probabilities throughout, selects experts 0..k-1 and gets NaN weights. */
 size_t fm_route_workspace(int64_t n, int e, int k);
 int fm_route(const void* logits, int32_t* idx, float* weights, int32_t* counts, int32_t* slot,
              int32_t* order, float* stats, void* workspace, size_t workspace_bytes, int64_t n,
