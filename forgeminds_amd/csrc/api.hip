@@ -27,6 +27,7 @@ const char* const kParamNames[fm_host::P_COUNT] = {
     "rows_vec_max",
     "rope_heads",
     "route_presort",
+    "norm_wide_acc",
 };
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cus[kMaxDevices];

@@ -677,6 +677,123 @@ __global__ __launch_bounds__(kWideThreads) void norm_bwd_wide(
   }
 }
 
+// Rows just past the register path (up to ITERS vectors per thread of a 1024-thread workgroup,
+// ITERS * EPV <= 32: 32768 columns): the per-thread fp32 column sums of the weight gradient still
+// fit the registers, so one persistent kernel does the whole backward. A workgroup walks a
+// contiguous chunk of rows and holds the packed x and dy of a row in registers between the
+// reduction and the output sweep (2 reads + 1 write from HBM, as on the register path; re-reading
+// them through the caches instead was 1.5 times slower). The weight comes from cache each time,
+// not from registers or LDS. The widest forms spill a few registers and still beat two kernels
+// that read the row three times; only fp32 LayerNorm past six vectors per thread does not.
+template <typename T, typename WT, bool LN, int ITERS>
+__global__ __launch_bounds__(kWideThreads) void norm_bwd_wide_acc(
+    const T* __restrict__ x, const WT* __restrict__ w, const float* __restrict__ mean,
+    const float* __restrict__ rstd, const T* __restrict__ dy, const T* __restrict__ gxn,
+    T* __restrict__ dx, T* __restrict__ dd, float* __restrict__ partial, int64_t n, int d,
+    int64_t rows_per_chunk) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int NB = LN ? ITERS : 1;
+  __shared__ float smem[kWideThreads / 64];
+  const int tid = threadIdx.x;
+  const int nvec = d / EPV;
+  const float inv_d = 1.f / (float)d;
+  float acc[ITERS][EPV], accb[NB][EPV];
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) acc[i][e] = 0.f;
+  }
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) accb[i][e] = 0.f;
+  }
+  const int64_t r0 = (int64_t)blockIdx.x * rows_per_chunk;
+  const int64_t r1 = (r0 + rows_per_chunk < n) ? r0 + rows_per_chunk : n;
+  for (int64_t row = r0; row < r1; ++row) {
+    const int64_t base = row * (int64_t)d;
+    const float r = rstd[row];
+    float mu = 0.f;
+    if constexpr (LN) mu = mean[row];
+    u32x4 rx[ITERS], rg[ITERS];
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = i * kWideThreads + tid;
+      if (c < nvec) {
+        rx[i] = load16_stream(x + base + (int64_t)c * EPV);
+        rg[i] = load16_stream(dy + base + (int64_t)c * EPV);
+      }
+    }
+    float dot = 0.f, gsum = 0.f;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = i * kWideThreads + tid;
+      if (c < nvec) {
+        float xv[EPV], gv[EPV], wv[EPV];
+        Elem<T>::unpack(rx[i], xv);
+        Elem<T>::unpack(rg[i], gv);
+        load_w<T, WT>(w, c * EPV, wv);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+          const float xh = (xv[e] - mu) * r;
+          acc[i][e] += gv[e] * xh;
+          dot += (gv[e] * wv[e]) * xh;
+          if constexpr (LN) {
+            accb[i][e] += gv[e];
+            gsum += gv[e] * wv[e];
+          }
+        }
+      }
+    }
+    dot = row_reduce<kWideThreads, OpSum>(dot, smem, 0, tid);
+    const float cmean = dot * inv_d;
+    float gmean = 0.f;
+    if constexpr (LN) gmean = row_reduce<kWideThreads, OpSum>(gsum, smem, 0, tid) * inv_d;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int c = i * kWideThreads + tid;
+      if (c < nvec) {
+        float xv[EPV], gv[EPV], wv[EPV], o[EPV];
+        Elem<T>::unpack(rx[i], xv);
+        Elem<T>::unpack(rg[i], gv);
+        load_w<T, WT>(w, c * EPV, wv);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] = ((gv[e] * wv[e] - gmean) - ((xv[e] - mu) * r) * cmean) * r;
+        if (gxn != nullptr) {
+          float rv[EPV];
+          Elem<T>::unpack(load16_stream(gxn + base + (int64_t)c * EPV), rv);
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) o[e] += rv[e];
+        }
+        const u32x4 packed = Elem<T>::pack(o);
+        store16_stream(dx + base + (int64_t)c * EPV, packed);
+        if (dd != nullptr) store16_stream(dd + base + (int64_t)c * EPV, packed);
+      }
+    }
+  }
+  if (partial == nullptr) return;
+  const int64_t pcols = LN ? 2 * (int64_t)d : d;
+  float* prow = partial + (int64_t)blockIdx.x * pcols;
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * kWideThreads + tid;
+    if (c < nvec) {
+#pragma unroll
+      for (int q = 0; q < EPV / 4; ++q) {
+        float o4[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o4[j] = acc[i][4 * q + j];
+        store16(prow + c * EPV + 4 * q, Elem<float>::pack(o4));
+        if constexpr (LN) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) o4[j] = accb[i][4 * q + j];
+          store16(prow + d + c * EPV + 4 * q, Elem<float>::pack(o4));
+        }
+      }
+    }
+  }
+}
+
 // dW (and, for LN, db) partials of the wide path: grid (ceil(nvec / 64), chunks); a workgroup
 // owns 64 vector columns and the rows of its chunk, four row lanes of 64 threads each; the
 // four are folded in a fixed order. Partial rows as in dw_generic.
@@ -866,7 +983,21 @@ int launch_bwd(const Plan& p, const void* x, const void* w, const float* mean, c
   T* ddp = static_cast<T*>(dd);
   if (dw == nullptr && db == nullptr) partial = nullptr;
   const int pcols = (int)(LN ? 2 * d : d);
-  if (p.bwd_wide) {
+  const int wide_iters = (int)((d / Elem<T>::kVec + kWideThreads - 1) / kWideThreads);
+  const bool acc_fits = wide_iters * Elem<T>::kVec <= 32 && !(LN && sizeof(T) == 4 && wide_iters > 6);
+  if (p.bwd_wide && acc_fits && fm_host::get_param(fm_host::P_NORM_WIDE_ACC) != 1) {
+    // the column sums fit the registers: one persistent kernel, a chunk of rows per workgroup
+    const dim3 grid((unsigned)p.bwd_blocks);
+#define GOA(IT_)                                                                                  \
+  FM_LAUNCH((norm_bwd_wide_acc<T, WT, LN, IT_>), grid, dim3(kWideThreads), 0, st, xp, wp, mean, rstd, dyp, \
+            gp, dxp, ddp, partial, n, (int)d, p.rows_per_chunk)
+    constexpr int kMaxIt = 32 / Elem<T>::kVec;
+    if (wide_iters <= 3 && kMaxIt >= 3) GOA(3);
+    else if (wide_iters <= 4 || kMaxIt < 8) GOA(4);
+    else if (wide_iters <= 6) GOA((kMaxIt >= 6 ? 6 : 4));
+    else GOA((kMaxIt >= 8 ? 8 : 4));
+#undef GOA
+  } else if (p.bwd_wide) {
     FM_LAUNCH((norm_bwd_wide<T, WT, LN>), dim3((unsigned)n), dim3(kWideThreads), 0, st, xp, wp,
                        mean, rstd, dyp, gp, dxp, ddp, (int)d);
     if (partial != nullptr) {

@@ -69,6 +69,10 @@ NORM_CASES = [
     # rows past the register path: streamed 16-byte vectors (and, one row wider, scalars)
     (5, 40960, BF16, F32, 1e-6), (3, 65536, F16, F16, 1e-5), (6, 20480, F32, F32, 1e-6),
     (300, 32768, BF16, BF16, 1e-6), (2, 131080, BF16, F32, 1e-6), (3, 40961, BF16, F32, 1e-6),
+    # 2049-4096 vectors (fp32: up to 8192): the backward is one persistent kernel with the column
+    # sums in registers; more rows than workgroups, uneven chunks
+    (700, 18432, BF16, F32, 1e-6), (513, 28672, F32, F32, 1e-6), (257, 32768, F16, F16, 1e-5),
+    (300, 16392, BF16, BF16, 1e-6),
 ]
 
 
@@ -160,7 +164,8 @@ LN_CASES = [
     (9, 16384, BF16, F32, 1e-5, True), (4, 40000, F16, F32, 1e-5, True), (130, 3072, F32, F32, 1e-5, True),
     (7, 12288, BF16, BF16, 1e-5, True), (2, 24576, BF16, F32, 1e-5, False), (40, 4096, BF16, F32, 1e-5, True),
     (5, 40960, BF16, F32, 1e-5, True), (3, 65536, F16, F16, 1e-5, False), (6, 20480, F32, F32, 1e-5, True),
-    (270, 32768, BF16, BF16, 1e-5, True),
+    (270, 32768, BF16, BF16, 1e-5, True), (700, 18432, BF16, F32, 1e-5, True), (300, 24576, F32, F32, 1e-5, True),
+    (260, 32768, F32, F32, 1e-5, True),
 ]
 
 
