@@ -976,8 +976,20 @@ def kbench_style(torch):
         lambda: [torch.randn(8192, 4096, device=dev).bfloat16(), torch.randn(8192, 4096, device=dev).bfloat16(),
                  torch.ones(4096, device=dev).bfloat16()],
         lambda t: sum(fm.kernels.add_rms_norm(t[0], t[1], t[2], 1e-6)), 8192 * 4096 * 16)
-    out["note"] = ("reference PERF.md:775-782 lists 0.591 / 1.239 ms for its Triton kernels and 0.276 / 0.436 ms "
-                   "for inductor at these two shapes on an unrecorded NVIDIA GPU")
+    out["swiglu gate,up [8192,11008] bf16"] = run(
+        lambda: [torch.randn(8192, 11008, device=dev).bfloat16(), torch.randn(8192, 11008, device=dev).bfloat16()],
+        lambda t: fm.kernels.swiglu(t[0], t[1]), 8192 * 11008 * 16)
+    out["swiglu_split [8192,22016] bf16"] = run(
+        lambda: [torch.randn(8192, 22016, device=dev).bfloat16()],
+        lambda t: fm.kernels.swiglu_split(t[0]), 8192 * 11008 * 16)
+    ang = torch.randn(2048, 64, device=dev)
+    out["qk_norm_rope [8,2048,32,128] bf16"] = run(
+        lambda: [torch.randn(8, 2048, 32, 128, device=dev).bfloat16(), torch.ones(128, device=dev), ang.cos(), ang.sin()],
+        lambda t: fm.kernels.qk_norm_rope(t[0], t[1], t[2].detach(), t[3].detach(), 1e-6), 8 * 2048 * 32 * 128 * 10)
+    out["note"] = ("reference PERF.md:775-782 lists, in this order, 0.591 / 1.239 / 2.466 / 2.436 / 1.394 ms for its "
+                   "Triton kernels and 0.276 / 0.436 / 1.314 / 1.563 / - ms for inductor at these shapes on an "
+                   "unrecorded NVIDIA GPU; the timed region holds the input clones and autograd as there, so "
+                   "gbps_on_algorithmic_bytes undercounts what moves")
     return out
 
 
