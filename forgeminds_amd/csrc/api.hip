@@ -28,6 +28,7 @@ const char* const kParamNames[fm_host::P_COUNT] = {
     "rope_heads",
     "route_presort",
     "norm_wide_acc",
+    "colsum16",
 };
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cus[kMaxDevices];

@@ -529,6 +529,49 @@ __global__ __launch_bounds__(256) void dw_generic(const T* __restrict__ x,
   }
 }
 
+// The same sum for narrow weights (few column blocks of 64 would leave most of the device idle and
+// each workgroup with a long serial tail): 16 columns per workgroup, four lanes per partial row,
+// 256 partial rows at a time, then a two-level fold in LDS whose order depends only on (p, d).
+template <typename WT>
+__global__ __launch_bounds__(1024) void colsum16_kernel(const float* __restrict__ partial,
+                                                         WT* __restrict__ dw, int p, int d,
+                                                         int stride) {
+  __shared__ float s[256][16 + 1];
+  __shared__ float s2[16][16 + 1];
+  const int q = threadIdx.x & 3;
+  const int g = threadIdx.x >> 2;
+  const int col = blockIdx.x * 16 + q * 4;
+  float a[4] = {0.f, 0.f, 0.f, 0.f};
+  if (col < d) {
+    for (int r = g; r < p; r += 256) {
+      float v[4];
+      Elem<float>::unpack(load16(partial + (int64_t)r * stride + col), v);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) a[c] += v[c];
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) s[g][q * 4 + c] = a[c];
+  __syncthreads();
+  if (threadIdx.x < 256) {   // thread (gg, c): row groups gg * 16 .. gg * 16 + 15 of column c, in order
+    const int gg = threadIdx.x >> 4, c = threadIdx.x & 15;
+    float t = s[gg * 16][c];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) t += s[gg * 16 + i][c];
+    s2[gg][c] = t;
+  }
+  __syncthreads();
+  if (threadIdx.x < 16) {
+    const int cc = blockIdx.x * 16 + threadIdx.x;
+    if (cc < d) {
+      float tot = s2[0][threadIdx.x];
+#pragma unroll
+      for (int i = 1; i < 16; ++i) tot += s2[i][threadIdx.x];
+      Elem<WT>::store1(dw + cc, tot);
+    }
+  }
+}
+
 // ---------------------------------------------------------------- wide rows (16-byte vectors, streamed)
 // Rows too wide for the register path (more than 4096 vectors) whose width is a whole number
 // of vectors and whose buffers are aligned: one 1024-thread workgroup per row, the row read
@@ -1036,7 +1079,12 @@ int launch_bwd(const Plan& p, const void* x, const void* w, const float* mean, c
     for (int which = 0; which < (LN ? 2 : 1); ++which) {
       if (outs[which] == nullptr) continue;
       const float* src = partial + (int64_t)which * d;
-      if (d % 4 == 0)
+      int lim16 = fm_host::get_param(fm_host::P_COLSUM16);   // widest weight the 16-column form takes (1: never)
+      if (lim16 <= 0) lim16 = 4096;
+      if (d % 4 == 0 && d <= lim16)
+        hipLaunchKernelGGL((colsum16_kernel<WT>), dim3((unsigned)((d + 15) / 16)), dim3(1024), 0, st, src,
+                           static_cast<WT*>(outs[which]), p.bwd_blocks, (int)d, pcols);
+      else if (d % 4 == 0)
         hipLaunchKernelGGL((colsum_kernel<WT>), grid, dim3(1024), 0, st, src, static_cast<WT*>(outs[which]),
                            p.bwd_blocks, (int)d, pcols);
       else
