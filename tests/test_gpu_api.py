@@ -537,9 +537,17 @@ def test_loss_selection_and_routing_launches_replay_in_a_graph():
     aligned = torch.randn(700, 512, generator=g).bfloat16().to(DEV)
     aligned2 = torch.randn(700, 512, generator=g).bfloat16().to(DEV)
     ya = torch.randint(0, 512, (700,), generator=g).to(DEV)
+    huge = (3 * torch.randn(2, 262144, generator=g)).bfloat16().to(DEV)      # prefixes past 64 KB of LDS
+    logits256 = torch.randn(600, 256, generator=g).to(DEV)
+    xw = torch.randn(300, 18432, generator=g).bfloat16().to(DEV)             # backward just past the register path
+    ww = torch.randn(18432, generator=g).to(DEV)
 
     def step():
         out = []
+        out += list(_hip.topk(huge, 64, torch.int32))
+        out += list(_hip.route(logits256, 8, True, True))                    # picks from lane-sorted keys
+        yw, rw = _hip.rmsnorm_fwd(xw, ww, 1e-6)
+        out += [yw, rw] + list(_hip.rmsnorm_bwd(xw, ww, rw, xw))
         loss, dl, nv, rows = _hip.ce_loss_grad(lg, y, -100, "mean")
         out += [loss, dl, nv, rows]
         loss2, lse, nv2, rows2 = _hip.ce_fwd(narrow, yn, -100, "mean")
