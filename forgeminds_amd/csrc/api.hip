@@ -29,6 +29,7 @@ const char* const kParamNames[fm_host::P_COUNT] = {
     "route_presort",
     "norm_wide_acc",
     "colsum16",
+    "route_stats_late",
 };
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cus[kMaxDevices];

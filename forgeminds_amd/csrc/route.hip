@@ -496,6 +496,62 @@ __global__ __launch_bounds__(512) void route_aux_kernel(const int32_t* __restric
   }
 }
 
+// route_stats_kernel and route_aux_kernel in one launch for small problems (at most two column
+// blocks and 256 tiles): one workgroup folds the column blocks one after the other, in the same
+// order and with the same additions as route_stats_kernel, keeps the sums in LDS and finishes
+// with route_aux_kernel's arithmetic. Same bits as the two kernels, one launch fewer.
+__global__ __launch_bounds__(1024) void route_stats_aux_kernel(const float* __restrict__ fstat,
+                                                                const int32_t* __restrict__ counts,
+                                                                float* __restrict__ stats, int64_t n,
+                                                                int e, int k, int ntiles) {
+  __shared__ float part[16][64];
+  __shared__ float sums[2 * 64];
+  __shared__ float apart[8];
+  const int cols = e + 1;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int cb = 0; cb * 64 < cols; ++cb) {
+    const int c = cb * 64 + lane;
+    float a = 0.f;
+    if (c < cols) {
+      int t = wave;
+      for (; t + 15 * 16 < ntiles; t += 16 * 16) {
+        float v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) v[u] = fstat[(int64_t)(t + u * 16) * cols + c];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) a += v[u];
+      }
+      for (; t < ntiles; t += 16) a += fstat[(int64_t)t * cols + c];
+    }
+    part[wave][lane] = a;
+    __syncthreads();
+    if (wave == 0 && c < cols) {
+      float r = part[0][lane];
+#pragma unroll
+      for (int w = 1; w < 16; ++w) r += part[w][lane];
+      stats[c] = r;
+      sums[c] = r;
+    }
+    __syncthreads();
+  }
+  const int c = threadIdx.x;
+  const float rows = n > 0 ? (float)n : 1.f;
+  const float slots = n > 0 ? (float)(n * (int64_t)k) : 1.f;
+  if (c < 512) {
+    float a = c < e ? ((float)counts[c] / slots) * (sums[c] / rows) : 0.f;
+    a = wave_sum(a);
+    if ((c & 63) == 0) apart[c >> 6] = a;
+  }
+  __syncthreads();
+  if (c == 0) {
+    float t = apart[0];
+#pragma unroll
+    for (int w = 1; w < 8; ++w) t += apart[w];
+    stats[e + 1] = (float)e * t;
+    stats[e + 2] = sums[e] / rows;
+  }
+}
+
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(256) void permute_kernel(const int32_t* __restrict__ idx,
@@ -719,7 +775,10 @@ int fm_route(const void* logits, int32_t* idx, float* weights, int32_t* counts, 
   else if (dtype == FM_BF16) launch_route<bf16_t>(logits, idx, weights, hist, fstat, n, e, k, tl, st);
   else launch_route<f16_t>(logits, idx, weights, hist, fstat, n, e, k, tl, st);
   FM_CHECK_LAUNCH("fm_route");
-  if (stats != nullptr) {
+  // few columns and tiles: the statistics are folded by the kernel that also finishes the losses
+  const bool stats_late = stats != nullptr && e + 1 <= 128 && tl.ntiles <= 256 &&
+                          fm_host::get_param(fm_host::P_ROUTE_STATS_LATE) != 1;
+  if (stats != nullptr && !stats_late) {
     hipLaunchKernelGGL(route_stats_kernel, dim3((unsigned)((e + 1 + 63) / 64)), dim3(1024), 0, st, fstat, stats,
                        e, tl.ntiles);
     FM_CHECK_LAUNCH("fm_route(stats)");
@@ -738,7 +797,11 @@ int fm_route(const void* logits, int32_t* idx, float* weights, int32_t* counts, 
                        counts, slot, order, n, e, k, tl.tile_rows, tl.ntiles, emit, scanned);
   }
   FM_CHECK_LAUNCH("fm_route(permute)");
-  if (stats != nullptr) {
+  if (stats_late) {
+    hipLaunchKernelGGL(route_stats_aux_kernel, dim3(1), dim3(1024), 0, st, fstat, counts, stats, n, e, k,
+                       tl.ntiles);
+    FM_CHECK_LAUNCH("fm_route(stats + aux)");
+  } else if (stats != nullptr) {
     hipLaunchKernelGGL(route_aux_kernel, dim3(1), dim3(512), 0, st, counts, stats, n, e, k);
     FM_CHECK_LAUNCH("fm_route(aux)");
   }

@@ -1026,6 +1026,23 @@ def test_route_pick_forms_agree():
         _hip.set_param("route_presort", 0)
 
 
+def test_route_statistics_from_one_or_two_kernels_keep_their_bits():
+    """Small problems fold the statistics inside the kernel that finishes the auxiliary losses;
+    forced back to the two kernels, every output keeps its bits."""
+    try:
+        for n, e, k in ((16384, 64, 2), (1000, 8, 2), (513, 127, 4), (3, 2, 2), (9000, 100, 8), (1, 64, 1)):
+            lg = router_inputs(n, e, 1031).to(DEV)
+            _hip.set_param("route_stats_late", 1)
+            two = _hip.route(lg, k, True, True)
+            _hip.set_param("route_stats_late", 0)
+            one = _hip.route(lg, k, True, True)
+            torch.cuda.synchronize()
+            for a, b in zip(one, two):
+                assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (n, e, k)
+    finally:
+        _hip.set_param("route_stats_late", 0)
+
+
 # ------------------------------------------------------------------ gather / combine around the permutation
 @pytest.mark.parametrize("n,e,k,d,dt", [(1000, 8, 2, 1024, BF16), (257, 16, 4, 100, F32), (64, 4, 1, 7, F16),
                                          (2048, 64, 2, 4096, BF16), (33, 8, 8, 256, F32)])
