@@ -30,6 +30,7 @@ const char* const kParamNames[fm_host::P_COUNT] = {
     "norm_wide_acc",
     "colsum16",
     "route_stats_late",
+    "rope_pair",
 };
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cus[kMaxDevices];

@@ -297,7 +297,7 @@ int get_param(int which);
 enum Param { P_NORM_BWD_BLOCKS_PER_CU = 0, P_VOCAB_THREADS, P_NORM_TPR, P_TOPK_VARIANT, P_VOCAB_UNROLL,
              P_NORM_FWD_BLOCKS_PER_CU, P_CE_ROWS_MAX_V, P_NORM_WIDE_MIN_VEC, P_ROWS_VEC_MAX,
              P_ROPE_HEADS, P_ROUTE_PRESORT, P_NORM_WIDE_ACC, P_COLSUM16,
-             P_ROUTE_STATS_LATE, P_COUNT };
+             P_ROUTE_STATS_LATE, P_ROPE_PAIR, P_COUNT };
 
 int num_cus();  // compute units of the current device (cached per device)
 

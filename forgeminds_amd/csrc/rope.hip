@@ -276,6 +276,133 @@ __global__ __launch_bounds__(kBlock) void rope_vec_kernel(const T* __restrict__ 
   }
 }
 
+// Heads of four or eight 16-byte vectors (64 bf16 / fp16 elements and below). With one vector of
+// each half per lane a load instruction of the kernel above touches only half of every 128-byte
+// line (the halves of such a head are 64 bytes or less). Here a head is owned by G = d / EPV lanes,
+// one vector per lane, so a group's load is the head's contiguous bytes; the rotation partner
+// (the same columns of the other half) lives G / 2 lanes away and is fetched with lane-permute
+// instructions: the packed input vector in the forward (the partner's normalised value is then
+// recomputed from it and the partner's weights), the packed incoming gradient in the backward.
+template <int HG>
+__device__ __forceinline__ uint32_t lane_xor(uint32_t v) {
+  static_assert(HG == 2 || HG == 4, "partner two or four lanes away");
+  if constexpr (HG == 2) return (uint32_t)FM_DPP_I((int)v, kDppXor2);
+  // i ^ 4 inside eight lanes: mirror the eight (i -> 7 - i), then reverse each quad (quad_perm:[3,2,1,0])
+  return (uint32_t)FM_DPP_I(FM_DPP_I((int)v, kDppHalfMirror), 0x1B);
+}
+
+template <typename T, typename WT, int G, bool BWD, int H>
+__global__ __launch_bounds__(kBlock) void rope_pair_kernel(const T* __restrict__ x, const WT* __restrict__ w,
+                                                            const float* __restrict__ cosv,
+                                                            const float* __restrict__ sinv,
+                                                            const T* __restrict__ dout,
+                                                            float* __restrict__ rstd, T* __restrict__ out,
+                                                            float* __restrict__ partial, int64_t rows,
+                                                            int t_len, int heads, int d, float eps,
+                                                            int64_t tiles) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int RPB = kBlock / G;
+  constexpr int HG = G / 2;
+  __shared__ float fold[BWD ? RPB * G * EPV : 1];
+  const int tid = threadIdx.x, rib = tid / G, l = tid % G;
+  const int half = d / 2;                 // == HG * EPV
+  const bool first = l < HG;              // this lane holds columns of the first half
+  const int col = l * EPV;                // its columns inside the head
+  const int hcol = (l % HG) * EPV;        // the same columns inside a half: cos / sin
+  float wo[EPV], wp[BWD ? 1 : EPV], a[BWD ? EPV : 1];
+  load_w_cols<T, WT>(w + col, wo);
+  if constexpr (!BWD) load_w_cols<T, WT>(w + (first ? col + half : col - half), wp);
+  if constexpr (BWD) {
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) a[e] = 0.f;
+  }
+  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    // rows is a multiple of H and so is the number of heads of a token: the H rows exist
+    // together and belong to one token
+    const int64_t row0 = (tile * RPB + rib) * H;
+    const bool live = row0 < rows;
+    const int t = live ? (int)((row0 / heads) % t_len) : 0;
+    float c[EPV], sn[EPV];
+    u32x4 rx[H], rg[BWD ? H : 1];
+#pragma unroll
+    for (int j = 0; j < H; ++j) rx[j] = u32x4{0u, 0u, 0u, 0u};
+    if constexpr (BWD) {
+#pragma unroll
+      for (int j = 0; j < H; ++j) rg[j] = u32x4{0u, 0u, 0u, 0u};
+    }
+    if (live) {
+#pragma unroll
+      for (int j = 0; j < H; ++j) {
+        rx[j] = load16_stream(x + (row0 + j) * (int64_t)d + col);
+        if constexpr (BWD) rg[j] = load16_stream(dout + (row0 + j) * (int64_t)d + col);
+      }
+    }
+    load_f32_cols<T>(cosv + (int64_t)t * half + hcol, c);
+    load_f32_cols<T>(sinv + (int64_t)t * half + hcol, sn);
+#pragma unroll
+    for (int j = 0; j < H; ++j) {
+      const int64_t row = row0 + j;
+      float xv[EPV], o[EPV];
+      Elem<T>::unpack(rx[j], xv);
+      if constexpr (!BWD) {
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) ss += xv[e] * xv[e];
+        ss = group_reduce<G, OpSum>(ss);
+        const float r = rsqrtf(ss / (float)d + eps);
+        if (live && l == 0) rstd[row] = r;
+        u32x4 pr;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) pr[q] = lane_xor<HG>(rx[j][q]);
+        float pv[EPV];
+        Elem<T>::unpack(pr, pv);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+          const float y = (xv[e] * r) * wo[e], py = (pv[e] * r) * wp[e];
+          // first half: y1 * cos - y2 * sin; second half: y1 * sin + y2 * cos
+          o[e] = first ? y * c[e] - py * sn[e] : py * sn[e] + y * c[e];
+        }
+      } else {
+        const float r = live ? rstd[row] : 0.f;
+        u32x4 pq;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) pq[q] = lane_xor<HG>(rg[j][q]);
+        float gv[EPV], pg[EPV];
+        Elem<T>::unpack(rg[j], gv);
+        Elem<T>::unpack(pq, pg);
+        float dot = 0.f;
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+          // rotate back: dy1 = do1 * cos + do2 * sin, dy2 = do2 * cos - do1 * sin
+          const float dy = first ? gv[e] * c[e] + pg[e] * sn[e] : gv[e] * c[e] - pg[e] * sn[e];
+          xv[e] *= r;                                   // xhat
+          a[e] += dy * xv[e];
+          o[e] = dy * wo[e];
+          dot += o[e] * xv[e];
+        }
+        dot = group_reduce<G, OpSum>(dot);
+        const float cm = dot / (float)d;
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] = (o[e] - xv[e] * cm) * r;
+      }
+      if (live) store16_stream(out + row * (int64_t)d + col, Elem<T>::pack(o));
+    }
+  }
+  if constexpr (BWD) {
+    if (partial == nullptr) return;
+    // fold the rows of this workgroup in row order, then write one partial row
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) fold[rib * G * EPV + col + e] = a[e];
+    __syncthreads();
+    float* prow = partial + (int64_t)blockIdx.x * d;
+    for (int j = tid; j < d; j += kBlock) {
+      float acc = 0.f;
+      for (int rr = 0; rr < RPB; ++rr) acc += fold[rr * G * EPV + j];
+      prow[j] = acc;
+    }
+  }
+}
+
 struct Shape { int g; int gv; int64_t tiles; int64_t vtiles; int blocks; };
 
 // g: lanes per head of the scalar kernel; gv: of the vector kernel (0 when the head does not
@@ -311,13 +438,19 @@ int launch(const Shape& sh, bool vec, const void* x, const void* w, const float*
   // heads of one token that a lane group takes per tile (vector kernel): 2 (4 in the forward is
   // slower again: fewer waves fit), 1 when the head count is odd
   int hpg = 1;
+  // heads of exactly four or eight vectors: one vector per lane, partner by lane permute
+  const bool pair = vec && (sh.gv == 2 || sh.gv == 4) && (int64_t)sh.gv * 2 * Elem<T>::kVec == d &&
+                    fm_host::get_param(fm_host::P_ROPE_PAIR) != 1;
   if (vec) {
+    // the one-vector-per-lane kernel: eight-lane groups take four heads forward and two backward;
+    // four-lane groups one (with more, a wave's load instruction skips between 64-byte heads)
+    const int dflt = !pair ? 2 : (sh.gv == 2 ? 1 : (BWD ? 2 : 4));
     const int want = fm_host::get_param(fm_host::P_ROPE_HEADS) > 0 ? fm_host::get_param(fm_host::P_ROPE_HEADS)
-                                                                   : 2;
-    if (want >= 4 && !BWD && heads % 4 == 0) hpg = 4;
+                                                                   : dflt;
+    if (want >= 4 && (!BWD || pair) && heads % 4 == 0) hpg = 4;
     else if (want >= 2 && heads % 2 == 0) hpg = 2;
   }
-  const int rpb = kBlock / (vec ? sh.gv : sh.g);
+  const int rpb = kBlock / (pair ? 2 * sh.gv : (vec ? sh.gv : sh.g));
   const int64_t tiles = (rows + (int64_t)rpb * hpg - 1) / ((int64_t)rpb * hpg);
   const int64_t blocks = sh.blocks < tiles ? sh.blocks : tiles;
 #define ARGS static_cast<const T*>(x), static_cast<const WT*>(w), c, s, static_cast<const T*>(dout), rstd, \
@@ -339,7 +472,19 @@ int launch(const Shape& sh, bool vec, const void* x, const void* w, const float*
     case 32: GO(32); break;   \
     default: GO(64); break;   \
   }
-  if (vec) { BY_G(GO_V, sh.gv) } else { BY_G(GO_S, sh.g) }
+  if (pair) {
+#define GO_P(G, H_) FM_LAUNCH((rope_pair_kernel<T, WT, G, BWD, H_>), dim3((unsigned)blocks), dim3(kBlock), 0, st, ARGS)
+#define GO_PH(G)                  \
+  do {                            \
+    if (hpg == 4) GO_P(G, 4);     \
+    else if (hpg == 2) GO_P(G, 2);\
+    else GO_P(G, 1);              \
+  } while (0)
+    if (sh.gv == 2) GO_PH(4);
+    else GO_PH(8);
+#undef GO_PH
+#undef GO_P
+  } else if (vec) { BY_G(GO_V, sh.gv) } else { BY_G(GO_S, sh.g) }
 #undef BY_G
 #undef GO_V
 #undef GO_S

@@ -1111,7 +1111,11 @@ def test_swiglu_split_fwd_bwd(rows, h, dt):
 
 # ------------------------------------------------------------------ per-head RMSNorm + RoPE
 @pytest.mark.parametrize("b,t,h,hd,dt,wdt", [(2, 5, 3, 4, F32, F32), (1, 7, 2, 8, F32, F32), (2, 3, 4, 6, F32, F32),
-                                              (2, 64, 8, 64, BF16, F32), (1, 33, 4, 32, F16, F16), (2, 16, 2, 256, BF16, BF16)])
+                                              (2, 64, 8, 64, BF16, F32), (1, 33, 4, 32, F16, F16), (2, 16, 2, 256, BF16, BF16),
+                                              # heads of four or eight vectors (one vector per lane, partner by lane
+                                              # permute): 1, 2 and 4 heads per lane group, several tiles
+                                              (2, 9, 6, 32, BF16, F32), (1, 5, 3, 32, BF16, BF16), (2, 7, 8, 16, BF16, F32),
+                                              (3, 4, 5, 16, F32, F32), (2, 300, 8, 32, BF16, F32), (1, 130, 2, 8, F32, F32)])
 def test_qk_norm_rope_fwd_bwd(b, t, h, hd, dt, wdt):
     # shapes of reference tests/kernel_interp_check.py:82-89, then realistic head sizes
     g = gen(41)
