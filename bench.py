@@ -12,19 +12,26 @@ libfmhip.so with pre-allocated outputs (no allocator, no autograd in the timed r
 The headline workload is the fused cross entropy of the reference's loss path at
 logits bf16 [8192, 32000]; `value` is algorithmic bytes per step / time per step.
 
-Prints ONE JSON line. Besides the headline it carries
+Prints ONE JSON line of a few KB (numbers only; `--detail PATH` writes the long form with the
+descriptions, warm-cache, graph-replay, torch-eager and CPU columns to a file). The line carries
   checked       one step's output compared with the CPU oracle on a bounded row sample before
                 anything is timed (per workload too);
   roofline      the dominant kernel of the headline workload against the 8 TB/s HBM peak, timed
                 with HIP events around that kernel's launches, on the bytes it has to move;
                 `traffic` = that kernel's HBM bytes from the committed profiler counter runs,
                 looked up by the name of the kernel that actually ran (null when unknown);
+                `configs` = one row per BASELINE configuration (cfg1 RMSNorm, cfg2 CE, cfg3 router,
+                cfg4 add-RMSNorm, cfg5 KL, cfg5b top-k): ms per step, fraction of the 8 TB/s peak
+                on the algorithmic bytes, rows/s, the dominant kernel with its average and minimum
+                launch time, and `floor_ms` = the best bare sweep (fm_stream_probe_mix: same
+                buffers, same read / write mix per launch, no arithmetic), `of_floor` = floor / ms;
   cpu_baseline  the CPU oracle (the reference's torch expression) on the host's cores -- a
                 reported baseline, never a target;
-  workloads     the same measurement for the other shapes of the hot path; launch-sized ones
-                add a HIP-graph replay and a warm-cache figure, the BASELINE configurations add
-                `torch_eager_gpu_ms` (the reference's torch expression on this GPU) and
-                `cpu_ms` / `cpu_gbps` (the oracle on a bounded sample, scaled, sample stated).
+  workloads     ms / GB/s / fraction for the other shapes of the hot path;
+  kbench        the reference's own protocol (public API, clones + autograd timed), ms per op.
+
+Inputs follow one recipe: torch.Generator(device="cpu").manual_seed(1000 + config number), values
+drawn on the CPU in row chunks, converted to the storage type and moved to the GPU.
 """
 
 from __future__ import annotations
@@ -100,6 +107,8 @@ def parse():
                     choices=WORKLOADS)
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--detail", default="", metavar="PATH",
+                    help="also write the long form (descriptions, warm / graph / eager / CPU columns) here")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="only run a plain device copy of this many MiB (counter calibration)")
     return ap.parse_args()
@@ -127,23 +136,45 @@ def _check(rc, what):
         raise RuntimeError(f"{what}: status {rc}: {_hip.lib().fm_last_error().decode()}")
 
 
+_SHARED = {}        # big inputs that several workloads use (the KL pair): drawn once
+
+
 def make_workload(name, torch, L, dev):
     from forgeminds_amd.kernels import _hip
     st = torch.cuda.current_stream().cuda_stream
-    g = torch.Generator(device=dev)
+    g = torch.Generator(device="cpu")
     BF, F32c = _hip.BF16, _hip.F32
     w = Workload()
     w.name = name
+
+    def rn(*shape, scale=1.0, dtype=torch.bfloat16, base=None):
+        """scale * N(0,1) (+ base, added in fp32) drawn from the CPU generator in row chunks,
+        rounded once to `dtype`, resident on the GPU."""
+        out = torch.empty(*shape, device=dev, dtype=dtype)
+        flat = out.view(shape[0], -1) if len(shape) > 1 else out.view(1, -1)
+        rows, width = flat.shape
+        step = max(1, (1 << 25) // max(1, width))
+        for r0 in range(0, rows, step):
+            r1 = min(rows, r0 + step)
+            c = torch.randn(r1 - r0, width, generator=g)
+            if scale != 1.0:
+                c.mul_(scale)
+            if base is None:
+                flat[r0:r1] = c.to(dtype)
+            else:
+                bf = base.view(rows, width)[r0:r1].float()
+                flat[r0:r1] = (bf + c.to(dev)).to(dtype)
+        return out
 
     if name == "rmsnorm":
         n, d = 8192, 1024
         g.manual_seed(1001)
         sets = 8     # rotate through > 256 MB so the Infinity Cache cannot serve a step
-        xs = [torch.randn(n, d, device=dev, generator=g).bfloat16() for _ in range(sets)]
-        dys = [torch.randn(n, d, device=dev, generator=g).bfloat16() for _ in range(sets)]
+        xs = [rn(n, d) for _ in range(sets)]
+        dys = [rn(n, d) for _ in range(sets)]
         ys = [torch.empty_like(xs[0]) for _ in range(sets)]
         dxs = [torch.empty_like(xs[0]) for _ in range(sets)]
-        wt = (1 + 0.02 * torch.randn(d, device=dev, generator=g))
+        wt = 1 + 0.02 * rn(d, dtype=torch.float32)
         rstd = torch.empty(n, device=dev)
         dw = torch.empty_like(wt)
         nb = L.fm_rmsnorm_bwd_workspace(n, d, BF)
@@ -197,16 +228,15 @@ def make_workload(name, torch, L, dev):
         w.bytes = n * d * 10
         w.desc = f"RMSNorm fwd+bwd x bf16 [{n},{d}], w fp32, eps 1e-6 (rotating {sets} buffer sets)"
         w.rows = n
+        w.sets = sets
+        w.floor = [lambda i: ((xs[i],), (ys[i],)), lambda i: ((xs[i], dys[i]), (dxs[i],))]
         return w
 
     if name == "add_rmsnorm":
         n, d = 16384, 8192
         g.manual_seed(1004)
-        x = torch.randn(n, d, device=dev, generator=g).bfloat16()
-        dl = torch.randn(n, d, device=dev, generator=g).bfloat16()
-        gy = torch.randn(n, d, device=dev, generator=g).bfloat16()
-        gxn = torch.randn(n, d, device=dev, generator=g).bfloat16()
-        wt = (1 + 0.02 * torch.randn(d, device=dev, generator=g))
+        x, dl, gy, gxn = rn(n, d), rn(n, d), rn(n, d), rn(n, d)
+        wt = 1 + 0.02 * rn(d, dtype=torch.float32)
         xn, y, dx = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
         rstd = torch.empty(n, device=dev)
         dw = torch.empty_like(wt)
@@ -259,17 +289,15 @@ def make_workload(name, torch, L, dev):
         w.bytes = n * d * 16
         w.desc = f"add-RMSNorm fwd+bwd x,delta bf16 [{n},{d}], w fp32, eps 1e-5, with residual grad"
         w.rows = n
+        w.floor = [lambda i: ((x, dl), (xn, y)), lambda i: ((xn, gy, gxn), (dx,))]
         return w
 
     if name == "add_layernorm":
         n, d = 16384, 8192
         g.manual_seed(1034)
-        x = torch.randn(n, d, device=dev, generator=g).bfloat16()
-        dl = torch.randn(n, d, device=dev, generator=g).bfloat16()
-        gy = torch.randn(n, d, device=dev, generator=g).bfloat16()
-        gxn = torch.randn(n, d, device=dev, generator=g).bfloat16()
-        wt = (1 + 0.02 * torch.randn(d, device=dev, generator=g))
-        bs = 0.1 * torch.randn(d, device=dev, generator=g)
+        x, dl, gy, gxn = rn(n, d), rn(n, d), rn(n, d), rn(n, d)
+        wt = 1 + 0.02 * rn(d, dtype=torch.float32)
+        bs = 0.1 * rn(d, dtype=torch.float32)
         xn, y, dx = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
         mean, rstd = torch.empty(n, device=dev), torch.empty(n, device=dev)
         dw, db = torch.empty_like(wt), torch.empty_like(wt)
@@ -312,9 +340,10 @@ def make_workload(name, torch, L, dev):
     if name in ("ce", "ce_one_pass"):
         n, v = 8192, 32000
         g.manual_seed(1002)
-        lg = (2 * torch.randn(n, v, device=dev, generator=g)).bfloat16()
-        y = torch.randint(0, v, (n,), device=dev, generator=g)
-        y[torch.rand(n, device=dev, generator=g) < 0.05] = -100
+        lg = rn(n, v, scale=2.0)
+        y = torch.randint(0, v, (n,), generator=g)
+        y[torch.rand(n, generator=g) < 0.05] = -100
+        y = y.to(dev)
         lse, rl = torch.empty(n, device=dev), torch.empty(n, device=dev)
         sc = torch.empty(2, device=dev)
         dlg = torch.empty_like(lg)
@@ -376,6 +405,7 @@ def make_workload(name, torch, L, dev):
                       "dataflow read + write = 4 B/logit")
             w.rows = n
             w.tensors = (lg, y)
+            w.floor = [lambda i: ((lg,), (dlg,))]
             return w
 
         def step():
@@ -393,15 +423,17 @@ def make_workload(name, torch, L, dev):
                   "dataflow fwd(read) + bwd(read, write) = 6 B/logit")
         w.rows = n
         w.tensors = (lg, y)
+        w.floor = [lambda i: ((lg,), ()), lambda i: ((lg,), (dlg,))]
         return w
 
     if name in ("kl", "kl_one_launch", "kl_topk", "kl_topk_one_launch", "topk"):
         n, v = 4096, 128256
-        g.manual_seed(1005)
-        s = (3 * torch.randn(n, v, device=dev, generator=g)).bfloat16()
-        t = (s.float() + 0.5 * torch.randn(n, v, device=dev, generator=g)).bfloat16()
+        if "kl_st" not in _SHARED:
+            g.manual_seed(1005)
+            s_ = rn(n, v, scale=3.0)
+            _SHARED["kl_st"] = (s_, rn(n, v, scale=0.5, base=s_))
+        s, t = _SHARED["kl_st"]
         if name == "topk":
-            del s
             idx = torch.empty(n, 64, device=dev, dtype=torch.int32)
 
             def step():
@@ -426,6 +458,7 @@ def make_workload(name, torch, L, dev):
             w.dominant_bytes = w.bytes = n * v * 2
             w.desc = f"top-64 of teacher logits bf16 [{n},{v}], int32 indices (separate launch)"
             w.rows = n
+            w.floor = [lambda i: ((t,), ())]
             return w
         b3 = torch.empty(3, n, device=dev)
         ls = torch.empty((), device=dev)
@@ -488,6 +521,7 @@ def make_workload(name, torch, L, dev):
                       "sits behind that cache")
             w.l2_bytes = n * v * 10
             w.rows = n
+            w.floor = [lambda i: ((s, t), (gs,))]
             return w
 
         if name == "kl_topk_one_launch":
@@ -537,13 +571,14 @@ def make_workload(name, torch, L, dev):
         if name == "kl_topk":
             w.desc += "; the forward also returns the teacher's top-64 (int32 indices, fp32 probabilities)"
         w.rows = n
+        w.floor = [lambda i: ((s, t), ()), lambda i: ((s, t), (gs,))]
         return w
 
     if name == "swiglu":
         rows, h = 16384, 14336
         g.manual_seed(1041)
-        x = torch.randn(rows, 2 * h, device=dev, generator=g).bfloat16()
-        dy = torch.randn(rows, h, device=dev, generator=g).bfloat16()
+        x = rn(rows, 2 * h)
+        dy = rn(rows, h)
         y = torch.empty(rows, h, device=dev, dtype=torch.bfloat16)
         dx = torch.empty_like(x)
 
@@ -580,10 +615,10 @@ def make_workload(name, torch, L, dev):
     if name == "qk_norm_rope":
         b, t, hh, d = 8, 4096, 32, 128
         g.manual_seed(1042)
-        x = torch.randn(b, t, hh, d, device=dev, generator=g).bfloat16()
-        do = torch.randn(b, t, hh, d, device=dev, generator=g).bfloat16()
-        wt = 1 + 0.02 * torch.randn(d, device=dev, generator=g)
-        ang = torch.rand(t, d // 2, device=dev, generator=g) * 6.28
+        x = rn(b, t, hh, d)
+        do = rn(b, t, hh, d)
+        wt = 1 + 0.02 * rn(d, dtype=torch.float32)
+        ang = (torch.rand(t, d // 2, generator=g) * 6.28).to(dev)
         cs, sn = torch.cos(ang), torch.sin(ang)
         out, dx = torch.empty_like(x), torch.empty_like(x)
         rstd = torch.empty(b * t * hh, device=dev)
@@ -629,15 +664,15 @@ def make_workload(name, torch, L, dev):
         sets = 80    # 80 x 4 MiB of logits: a step's input is never in the 256 MB memory-side cache
         lgs = []
         for i in range(sets):
-            lg = torch.round(torch.randn(n, e, device=dev, generator=g) * 4096) / 4096
+            lg = torch.round(torch.randn(n, e, generator=g) * 4096) / 4096
             if i == 0:
                 # 1 % of the rows get ties at the top and a second group of equal values
-                rows = torch.randperm(n, device=dev, generator=g)[: n // 100]
-                cols = torch.stack([torch.randperm(e, device=dev, generator=g)[:8] for _ in range(rows.numel())])
+                rows = torch.randperm(n, generator=g)[: n // 100]
+                cols = torch.stack([torch.randperm(e, generator=g)[:8] for _ in range(rows.numel())])
                 top = lg[rows].max(dim=1, keepdim=True).values
                 lg[rows[:, None], cols[:, :4]] = top
                 lg[rows[:, None], cols[:, 4:]] = lg[rows, cols[:, 4]][:, None]
-            lgs.append(lg)
+            lgs.append(lg.to(dev))
         idx = torch.empty(n, k, device=dev, dtype=torch.int32)
         wt = torch.empty(n, k, device=dev)
         cnt = torch.empty(e, device=dev, dtype=torch.int32)
@@ -688,6 +723,8 @@ def make_workload(name, torch, L, dev):
                   f"(rotating {sets} logit sets: cold)")
         w.unit = "rows/s"
         w.rows = n
+        w.sets = sets
+        w.floor = [lambda i: ((lgs[i],), ()), lambda i: ((idx.view(-1),), (sl,))]
         return w
 
     if name == "route_train":
@@ -695,14 +732,14 @@ def make_workload(name, torch, L, dev):
         # auxiliary losses, then the gradient wrt the logits in one kernel
         n, e, k = 16384, 64, 2
         g.manual_seed(1003)
-        lg = torch.round(torch.randn(n, e, device=dev, generator=g) * 4096) / 4096
+        lg = (torch.round(torch.randn(n, e, generator=g) * 4096) / 4096).to(dev)
         idx = torch.empty(n, k, device=dev, dtype=torch.int32)
         wt = torch.empty(n, k, device=dev)
         cnt = torch.empty(e, device=dev, dtype=torch.int32)
         sl = torch.empty(n * k, device=dev, dtype=torch.int32)
         od = torch.empty(n * k, device=dev, dtype=torch.int32)
         stats = torch.empty(e + 3, device=dev)
-        gw = torch.randn(n, k, device=dev, generator=g)
+        gw = torch.randn(n, k, generator=g).to(dev)
         ga, gz = torch.tensor(0.01, device=dev), torch.tensor(0.001, device=dev)
         dl = torch.empty_like(lg)
         nb = L.fm_route_workspace(n, e, k)
@@ -742,8 +779,8 @@ def make_workload(name, torch, L, dev):
     if name == "moe_dispatch":
         n, e, k, d = 16384, 64, 2, 4096
         g.manual_seed(1008)
-        lg = torch.round(torch.randn(n, e, device=dev, generator=g) * 4096) / 4096
-        x = torch.randn(n, d, device=dev, generator=g).bfloat16()
+        lg = (torch.round(torch.randn(n, e, generator=g) * 4096) / 4096).to(dev)
+        x = rn(n, d)
         idx, wt, cnt, sl, od = _hip.route(lg, k)
         xs = torch.empty(n * k, d, device=dev, dtype=torch.bfloat16)
         out = torch.empty_like(x)
@@ -820,6 +857,21 @@ def time_kernel_events(torch, fn, steps):
     torch.cuda.synchronize()
     times = sorted(a.elapsed_time(b) for a, b in pairs)
     return sum(times) / len(times), times[0], times[len(times) // 2]
+
+
+def time_back_to_back(torch, fn, reps, batches=2):
+    """ms per launch of `reps` launches enqueued back to back between one pair of events (no event,
+    hence no cache write-back, between the launches): best of `batches`."""
+    best = float("inf")
+    for _ in range(batches):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        best = min(best, a.elapsed_time(b) / reps)
+    return best
 
 
 def time_graph(torch, step_fns, steps):
@@ -923,39 +975,122 @@ def measure(torch, w, steps, warmup, L, cpu=True):
         out["cpu_ms"] = round(sec * 1e3, 1)
         out["cpu_gbps"] = round(w.bytes / sec / 1e9, 3)
         out["cpu_sample"] = sample
+    if hasattr(w, "floor"):          # last: the sweeps overwrite the workload's outputs
+        out.update(measure_floor(torch, w, steps, warmup, L, ms))
     return out
 
 
+# ---------------------------------------------------------------------------- floors
+# (threads, vectors per thread) of fm_stream_probe_mix and the persistent grids tried with each
+FLOOR_SHAPES = ((256, 2), (256, 4), (512, 2), (1024, 4))
+FLOOR_GRIDS = (0, 2048, 1024)       # 0: one workgroup per tile
+
+
+def measure_floor(torch, w, steps, warmup, L, ms):
+    """The workload's step as bare data movement: for each of its launches the best
+    fm_stream_probe_mix variant over tile shapes, grids and store kinds, on the workload's own
+    buffers with that launch's reads and writes; then those best sweeps timed back to back with
+    the protocol the real step was timed with."""
+    st = torch.cuda.current_stream().cuda_stream
+    dev = torch.device("cuda:0")
+    sink = torch.zeros(1, device=dev, dtype=torch.int32)
+    sets = getattr(w, "sets", 1)
+
+    def launcher(spec, kind, thr, vec, grid):
+        def go(i):
+            rd, wr = spec(i)
+            nbytes = rd[0].numel() * rd[0].element_size()
+            ptr = [t.data_ptr() for t in rd] + [None] * (3 - len(rd))
+            out = [t.data_ptr() for t in wr] + [None] * (2 - len(wr))
+            _check(L.fm_stream_probe_mix(ptr[0], ptr[1], ptr[2], out[0], out[1], sink.data_ptr(), nbytes,
+                                         len(rd), len(wr), kind, thr, vec, grid, st), "fm_stream_probe_mix")
+        return go
+
+    chosen, names = [], []
+    for spec in w.floor:
+        rd, wr = spec(0)
+        nbytes = rd[0].numel() * rd[0].element_size()
+        kinds = (0,) if not wr else ((0, 1) if len(wr) == 1 else (0, 1, 2))
+        best = None
+        for thr, vec in FLOOR_SHAPES:
+            if nbytes % (thr * vec * 16):
+                continue
+            tiles = nbytes // (thr * vec * 16)
+            for grid in FLOOR_GRIDS:
+                if grid >= tiles and grid != 0:
+                    continue
+                for kind in kinds:
+                    go = launcher(spec, kind, thr, vec, grid)
+                    state = {"i": 0}
+
+                    def one():
+                        state["i"] = (state["i"] + 1) % sets
+                        go(state["i"])
+                    for _ in range(3):
+                        one()
+                    avg = time_back_to_back(torch, one, 10)
+                    if best is None or avg < best[0]:
+                        best = (avg, go, f"{len(rd)}r{len(wr)}w {thr}x{vec} grid {grid or tiles} store {kind}")
+        if best is None:
+            return {"floor_ms": None}
+        chosen.append(best[1])
+        names.append(f"{best[2]}: {best[0] * 1e3:.1f} us")
+    state = {"i": 0}
+
+    def floor_step():
+        i = state["i"] = (state["i"] + 1) % sets
+        for go in chosen:
+            go(i)
+    fms = time_steps(torch, floor_step, steps, warmup)
+    return {"floor_ms": round(fms, 5), "of_floor": round(fms / ms, 4), "floor_sweeps": names}
+
+
 def stream_ceiling(torch, L, dev):
-    """What a plain read sweep and a plain copy reach on this GPU (1 GiB, min of 10)."""
+    """What a plain read sweep and a plain copy reach on this GPU (1 GiB, ten launches back to back,
+    best of two such batches; the copy over both store kinds, two tile shapes and two grids)."""
     n = 1 << 30
     src = torch.empty(n, device=dev, dtype=torch.uint8).fill_(1)
     dst = torch.empty_like(src)
     sink = torch.zeros(1, device=dev, dtype=torch.int32)
     st = torch.cuda.current_stream().cuda_stream
     out = {}
-    for mode, name, moved in ((0, "read_gbps", n), (1, "copy_gbps", 2 * n)):
-        fn = lambda: _check(L.fm_stream_probe(src.data_ptr(), dst.data_ptr(), sink.data_ptr(), n, mode, st),
-                            "fm_stream_probe")
-        _, best, _ = time_kernel_events(torch, fn, 12)
-        out[name] = round(moved / best / 1e6, 1)
-    out["note"] = "fm_stream_probe, 16-byte non-temporal accesses, one 64 KiB chunk per workgroup"
+    fn = lambda: _check(L.fm_stream_probe(src.data_ptr(), dst.data_ptr(), sink.data_ptr(), n, 0, st),
+                        "fm_stream_probe")
+    fn()
+    best = time_back_to_back(torch, fn, 10)
+    out["read_gbps"] = round(n / best / 1e6, 1)
+    best_copy = None
+    for thr, vec in ((512, 2), (1024, 4)):
+        for grid in (0, 2048):
+            for kind in (0, 1):
+                fn = lambda: _check(L.fm_stream_probe_mix(src.data_ptr(), None, None, dst.data_ptr(), None,
+                                                          sink.data_ptr(), n, 1, 1, kind, thr, vec, grid, st),
+                                    "fm_stream_probe_mix")
+                fn()
+                b = time_back_to_back(torch, fn, 10)
+                if best_copy is None or b < best_copy[0]:
+                    best_copy = (b, f"{thr}x{vec} grid {grid or 'tiles'} store {'nt' if kind else 'plain'}")
+    out["copy_gbps"] = round(2 * n / best_copy[0] / 1e6, 1)
+    out["copy_form"] = best_copy[1]
     return out
 
 
 def kbench_style(torch):
     """The reference's own protocol (forgemind/cli/kbench.py:122-158): public API, fresh
     detach().clone().requires_grad_() inputs and autograd inside the timed region, warm-up 5,
-    min of 20. Reported next to the kernel-only numbers, never instead of them."""
+    min of 20; shapes and forward-only cases as forgemind/cli/kbench.py:55-116 builds them.
+    Reported next to the kernel-only numbers, never instead of them. ms per call."""
     import forgeminds_amd as fm
     dev = "cuda:0"
     out = {}
 
-    def run(make, fn, algorithmic_bytes):
+    def run(make, fn, backward=True):
         tensors = make()
         def step():
-            ins = [t.detach().clone().requires_grad_(t.is_floating_point()) for t in tensors]
-            fn(ins).float().sum().backward()
+            ins = [t.detach().clone().requires_grad_(t.is_floating_point() and backward) for t in tensors]
+            o = fn(ins)
+            if backward:
+                o.float().sum().backward()
         for _ in range(5):
             step()
         torch.cuda.synchronize()
@@ -967,30 +1102,33 @@ def kbench_style(torch):
             b.record()
             torch.cuda.synchronize()
             best = min(best, a.elapsed_time(b))
-        return {"ms": round(best, 4), "gbps_on_algorithmic_bytes": round(algorithmic_bytes / best / 1e6, 1)}
+        return round(best, 4)
 
-    out["rms_norm [8192,4096] bf16"] = run(
-        lambda: [torch.randn(8192, 4096, device=dev).bfloat16(), torch.ones(4096, device=dev).bfloat16()],
-        lambda t: fm.kernels.rms_norm(t[0], t[1], 1e-6), 8192 * 4096 * 10)
-    out["add_rms_norm [8192,4096] bf16"] = run(
-        lambda: [torch.randn(8192, 4096, device=dev).bfloat16(), torch.randn(8192, 4096, device=dev).bfloat16(),
-                 torch.ones(4096, device=dev).bfloat16()],
-        lambda t: sum(fm.kernels.add_rms_norm(t[0], t[1], t[2], 1e-6)), 8192 * 4096 * 16)
-    out["swiglu gate,up [8192,11008] bf16"] = run(
-        lambda: [torch.randn(8192, 11008, device=dev).bfloat16(), torch.randn(8192, 11008, device=dev).bfloat16()],
-        lambda t: fm.kernels.swiglu(t[0], t[1]), 8192 * 11008 * 16)
-    out["swiglu_split [8192,22016] bf16"] = run(
-        lambda: [torch.randn(8192, 22016, device=dev).bfloat16()],
-        lambda t: fm.kernels.swiglu_split(t[0]), 8192 * 11008 * 16)
+    rnd = lambda *sh: torch.randn(*sh, device=dev).bfloat16()
+    out["rms_norm [8192,4096]"] = run(lambda: [rnd(8192, 4096), torch.ones(4096, device=dev).bfloat16()],
+                                      lambda t: fm.kernels.rms_norm(t[0], t[1], 1e-6))
+    out["add_rms_norm [8192,4096]"] = run(
+        lambda: [rnd(8192, 4096), rnd(8192, 4096), torch.ones(4096, device=dev).bfloat16()],
+        lambda t: sum(fm.kernels.add_rms_norm(t[0], t[1], t[2], 1e-6)))
+    out["swiglu [8192,11008]"] = run(lambda: [rnd(8192, 11008), rnd(8192, 11008)],
+                                     lambda t: fm.kernels.swiglu(t[0], t[1]))
+    out["swiglu_split [8192,22016]"] = run(lambda: [rnd(8192, 22016)], lambda t: fm.kernels.swiglu_split(t[0]))
     ang = torch.randn(2048, 64, device=dev)
-    out["qk_norm_rope [8,2048,32,128] bf16"] = run(
-        lambda: [torch.randn(8, 2048, 32, 128, device=dev).bfloat16(), torch.ones(128, device=dev), ang.cos(), ang.sin()],
-        lambda t: fm.kernels.qk_norm_rope(t[0], t[1], t[2].detach(), t[3].detach(), 1e-6), 8 * 2048 * 32 * 128 * 10)
-    out["note"] = ("reference PERF.md:775-782 lists, in this order, 0.591 / 1.239 / 2.466 / 2.436 / 1.394 ms for its "
-                   "Triton kernels and 0.276 / 0.436 / 1.314 / 1.563 / - ms for inductor at these shapes on an "
-                   "unrecorded NVIDIA GPU; the timed region holds the input clones and autograd as there, so "
-                   "gbps_on_algorithmic_bytes undercounts what moves")
+    out["qk_norm_rope [8,2048,32,128]"] = run(
+        lambda: [rnd(8, 2048, 32, 128), torch.ones(128, device=dev), ang.cos(), ang.sin()],
+        lambda t: fm.kernels.qk_norm_rope(t[0], t[1], t[2].detach(), t[3].detach(), 1e-6))
+    out["kl_div_logits [512,32000] fwd"] = run(lambda: [rnd(512, 32000), rnd(512, 32000)],
+                                               lambda t: fm.kernels.kl_div_logits(t[0], t[1]), backward=False)
+    out["topk [512,32000] k=64"] = run(lambda: [rnd(512, 32000)], lambda t: fm.kernels.topk(t[0], 64)[0])
+    out["softmax [8192,128]"] = run(lambda: [rnd(8192, 128)], lambda t: fm.kernels.softmax(t[0], -1))
+    out["softmax [8192,4096]"] = run(lambda: [rnd(8192, 4096)], lambda t: fm.kernels.softmax(t[0], -1))
     return out
+
+
+KBENCH_NOTE = ("reference PERF.md:775-782 lists 0.591 / 1.239 / 2.466 / 2.436 / 1.394 ms for its Triton kernels and "
+               "0.276 / 0.436 / 1.314 / 1.563 / - ms for inductor at the first five shapes on an unrecorded NVIDIA "
+               "GPU, PERF.md:761-766 85 ms (topk) and 2.6 ms (softmax [8192,128]) on a CPU; the timed region holds "
+               "the input clones and autograd as there")
 
 
 # ---------------------------------------------------------------------------- CPU baseline
@@ -1007,6 +1145,38 @@ def cpu_baseline(torch, w):
         "sample": f"oracle (CPU restatement of the reference's torch expression) on {sample}, "
                   f"min of up to 3 passes, {sec * 1e3:.1f} ms for the whole workload, same byte accounting",
     }
+
+
+# BASELINE.json's configurations, in its order, and the workload that measures each
+CONFIGS = (("cfg1", "rmsnorm"), ("cfg2", "ce"), ("cfg3", "route"), ("cfg4", "add_rmsnorm"), ("cfg5", "kl"),
+           ("cfg5b", "topk"))
+
+
+def config_row(r, rows_unit):
+    """One BASELINE configuration as numbers only."""
+    row = {
+        "ms": r["ms_per_step"],
+        "frac": None if rows_unit else r.get("required_frac_of_hbm_peak", r["frac_of_hbm_peak"]),
+        "frac_per_element_accounting": None if rows_unit else r["frac_of_hbm_peak"],
+        "rows_per_s": r["rows_per_s"], "checked": r["checked"],
+        "dom_kernel": r["dominant_kernel"].split("<")[0],
+        "dom_us": round(r["dominant_ms_avg"] * 1e3, 2), "dom_us_min": round(r["dominant_ms_min"] * 1e3, 2),
+        "floor_ms": r.get("floor_ms"), "of_floor": r.get("of_floor"),
+    }
+    if "warm_cache_ms_per_step" in r:
+        row["warm_ms"] = r["warm_cache_ms_per_step"]
+    if "graph_replay_ms_per_step" in r:
+        row["graph_ms"] = r["graph_replay_ms_per_step"]
+    return row
+
+
+def short_row(r):
+    row = {"ms": r["ms_per_step"], "gbps": r["gbps"], "frac": r["frac_of_hbm_peak"], "checked": r["checked"]}
+    if "l2_boundary_frac_of_hbm_peak" in r:
+        row["frac_l2_boundary"] = r["l2_boundary_frac_of_hbm_peak"]
+    if "floor_ms" in r and r["floor_ms"] is not None:
+        row["floor_ms"], row["of_floor"] = r["floor_ms"], r["of_floor"]
+    return row
 
 
 def main():
@@ -1059,7 +1229,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if a.workload not in ("route", "route_train") else "f32", "data": "synthetic",
         "config": {"workload": head.desc, "name": a.workload,
-                   "timing": "K steps between two device synchronisations, inputs resident in HBM"},
+                   "timing": "K steps between two device synchronisations, inputs resident in HBM",
+                   "inputs": "torch.Generator(cpu).manual_seed(1000 + config number), drawn in row chunks"},
         "checked": res["checked"],
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -1073,26 +1244,41 @@ def main():
         "frac_of_hbm_peak": res["frac_of_hbm_peak"],
     }
     line["cpu_baseline"] = None if (a.no_cpu or not hasattr(head, "cpu")) else cpu_baseline(torch, head)
+    head_unit_rows = head.unit == "rows/s"
     del head
     torch.cuda.empty_cache()
+    detail = {a.workload: res}
+    units = {a.workload: head_unit_rows}
     if not a.no_extras:
-        extras = {a.workload: res}
         for name in WORKLOADS:
             if name == a.workload:
                 continue
             wl = make_workload(name, torch, L, dev)
-            extras[name] = measure(torch, wl, a.steps, a.warmup, L, cpu=not a.no_cpu)
+            detail[name] = measure(torch, wl, a.steps, a.warmup, L, cpu=not a.no_cpu)
+            units[name] = wl.unit == "rows/s"
             del wl
             torch.cuda.empty_cache()
         if line["cpu_baseline"] is not None:     # the headline's CPU column, in the table's units
             cb = line["cpu_baseline"]
             if cb["unit"] == "GB/s":
-                extras[a.workload]["cpu_gbps"] = cb["value"]
-                extras[a.workload]["cpu_ms"] = round(extras[a.workload]["algorithmic_bytes"] / cb["value"] / 1e6, 1)
-        line["workloads"] = extras
-        line["kbench_style"] = kbench_style(torch)
+                detail[a.workload]["cpu_gbps"] = cb["value"]
+                detail[a.workload]["cpu_ms"] = round(detail[a.workload]["algorithmic_bytes"] / cb["value"] / 1e6, 1)
+    _SHARED.clear()
+    torch.cuda.empty_cache()
+    by_workload = dict(CONFIGS)
+    line["roofline"]["configs"] = {c: config_row(detail[wn], units[wn]) for c, wn in CONFIGS if wn in detail}
+    named = set(by_workload.values())
+    line["workloads"] = {n: short_row(r) for n, r in detail.items() if n not in named}
+    kb = None
+    if not a.no_extras:
+        kb = kbench_style(torch)
+        line["kbench"] = kb
     line["hbm_ceiling_measured"] = stream_ceiling(torch, L, dev)
-    print(json.dumps(line))
+    if a.detail:
+        os.makedirs(os.path.dirname(os.path.abspath(a.detail)), exist_ok=True)
+        with open(a.detail, "w") as f:
+            json.dump({"line": line, "workloads": detail, "kbench_note": KBENCH_NOTE}, f, indent=1)
+    print(json.dumps(line, separators=(",", ":")))
     return 0
 
 

@@ -8,7 +8,7 @@
 
 #include <atomic>
 
-#include "fm_common.cuh"
+#include "fm_common.hip.h"
 
 namespace {
 thread_local char g_error[512] = "";

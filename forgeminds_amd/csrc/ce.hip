@@ -9,7 +9,7 @@
 // being stored, so the whole fwd+bwd moves 2 + 2 + 2 bytes per bf16 logit. A second form
 // (ce_loss_grad_kernel) produces the loss and the gradient from one read of rows that fit the
 // register file: 2 + 2 bytes per logit.
-#include "fm_vocab.cuh"
+#include "fm_vocab.hip.h"
 
 using namespace fm;
 

@@ -11,7 +11,7 @@
 // one partial row; a second kernel sums the partial rows in a fixed order.
 #pragma once
 
-#include "fm_common.cuh"
+#include "fm_common.hip.h"
 
 using namespace fm;
 

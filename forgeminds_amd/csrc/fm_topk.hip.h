@@ -17,7 +17,7 @@
 
 #include <atomic>
 
-#include "fm_vocab.cuh"
+#include "fm_vocab.hip.h"
 
 namespace fm {
 

@@ -8,7 +8,7 @@
 // the element offset, the same split is valid for all of them, whatever their dtypes.
 #pragma once
 
-#include "fm_common.cuh"
+#include "fm_common.hip.h"
 
 namespace fm {
 

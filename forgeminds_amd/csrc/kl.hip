@@ -11,7 +11,7 @@
 // Two more forms: kl_loss_grad_kernel writes the gradient in the forward from one read of rows
 // that fit the register file, and kl_fwd_topk_kernel also selects the teacher's top-k.
 // All exponentials run in the base-2 domain; the temperature is folded into the scale.
-#include "fm_topk.cuh"
+#include "fm_topk.hip.h"
 
 using namespace fm;
 

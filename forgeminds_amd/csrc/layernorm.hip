@@ -6,8 +6,8 @@
 //   mean = sum(x)/d, rstd = rsqrt(sum((x-mean)^2)/d + eps), y = ((x-mean)*rstd)*w + b
 //   dx = ((g - mean(g)) - xhat*mean(g*xhat))*rstd with g = dy*w; dw = sum_rows dy*xhat;
 //   db = sum_rows dy.
-// Kernels: fm_norm.cuh with LN = true.
-#include "fm_norm.cuh"
+// Kernels: fm_norm.hip.h with LN = true.
+#include "fm_norm.hip.h"
 
 extern "C" {
 

@@ -9,7 +9,7 @@
 // gather is a combine with unit weights, the gradient of the combine is a weighted gather.
 //
 // Pure HBM-bound row moves: one workgroup per destination row, 16-byte vectors.
-#include "fm_common.cuh"
+#include "fm_common.hip.h"
 
 using namespace fm;
 

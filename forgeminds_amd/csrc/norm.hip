@@ -2,8 +2,8 @@
 //
 // Reference semantics: forgemind/kernels/_fallback.py:26-35 (forward, rounding points),
 // forgemind/kernels/norm.py:179-231 (backward row math), norm.py:571-593 (fixed-order
-// column sum of the fp32 weight-gradient partials). Kernels: fm_norm.cuh with LN = false.
-#include "fm_norm.cuh"
+// column sum of the fp32 weight-gradient partials). Kernels: fm_norm.hip.h with LN = false.
+#include "fm_norm.hip.h"
 
 #include <atomic>
 

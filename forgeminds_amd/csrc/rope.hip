@@ -13,7 +13,7 @@
 // vectors per half, or unaligned buffers, use a scalar variant (four elements of each half per
 // lane). Grids are persistent: the weight columns stay in registers, cos/sin rows are shared by
 // the heads of a token and come from cache.
-#include "fm_norm.cuh"   // colsum_kernel / colsum_scalar_kernel: fixed-order column sums of partial rows
+#include "fm_norm.hip.h"   // colsum_kernel / colsum_scalar_kernel: fixed-order column sums of partial rows
 
 using namespace fm;
 

@@ -22,7 +22,7 @@
 //                   flat position and gives each assignment the slot
 //                     base[e] + (#assignments to e in earlier tiles) + (rank inside the tile),
 //                   which is exactly the position a stable sort by expert would assign.
-#include "fm_common.cuh"
+#include "fm_common.hip.h"
 
 using namespace fm;
 

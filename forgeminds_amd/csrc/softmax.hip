@@ -10,7 +10,7 @@
 //
 // Backward (forgemind/kernels/softmax.py:108-115: dx = (dy - sum(dy * y)) * y): the same three
 // shapes over two inputs, fp32 math on the stored y and dy, one rounding at the store.
-#include "fm_vocab.cuh"
+#include "fm_vocab.hip.h"
 
 using namespace fm;
 

@@ -5,7 +5,7 @@
 // forgemind/kernels/swiglu.py:48-120 (the derivative: with s = sigmoid(g),
 // d/dg [g*s*u] = u * s * (1 + g*(1 - s)), d/du = g*s).
 // Flat element-wise streams: 16-byte vectors, one-shot grid, scalar tail / unaligned path.
-#include "fm_common.cuh"
+#include "fm_common.hip.h"
 
 using namespace fm;
 

@@ -30,7 +30,7 @@
 // the result is bit-reproducible.
 #include <type_traits>
 
-#include "fm_topk.cuh"
+#include "fm_topk.hip.h"
 
 using namespace fm;
 

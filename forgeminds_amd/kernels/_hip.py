@@ -35,6 +35,7 @@ SIGNATURES = {
     "fm_last_kernel": (C.c_char_p, []),
     "fm_set_param": (_int, [C.c_char_p, _int]),
     "fm_stream_probe": (_int, [_vp, _vp, _vp, _sz, _int, _vp]),
+    "fm_stream_probe_mix": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _int, _int, _int, _int, _int, _i64, _vp]),
     "fm_rmsnorm_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _f32, _vp]),
     "fm_rmsnorm_bwd_workspace": (_sz, [_i64, _i64, _int]),
     "fm_rmsnorm_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64, _int, _int, _vp]),

@@ -65,6 +65,20 @@ int fm_set_param(const char* name, int value);
 int fm_stream_probe(const void* src, void* dst, uint32_t* sink, size_t bytes, int mode,
                     fm_stream_t stream);
 
+/* The floor of a row kernel: `reads` (1-3) input streams a, b, c and `writes` (0-2) output streams
+ * o1, o2 of `bytes` each are swept once with 16-byte accesses and no arithmetic beyond an xor
+ * (read-only sweeps keep their loads alive through `sink`, one uint32 on the device that ordinary
+ * data never reaches). Loads are non-temporal like the row kernels'; store_kind 0 = plain,
+ * 1 = non-temporal, 2 = o1 plain and o2 non-temporal. A workgroup of `threads` threads moves tiles
+ * of threads * vecs_per_thread vectors (256x1, 256x2, 256x4, 512x2, 512x4, 1024x1, 1024x4); `grid`
+ * workgroups walk the tiles (<= 0: one workgroup per tile). bytes must be a whole number of tiles.
+ * bench.py times it on each workload's own buffers, with that workload's read / write mix, and
+ * reports the workload's step as a fraction of the best such sweep. No counterpart in the
+ * reference. */
+int fm_stream_probe_mix(const void* a, const void* b, const void* c, void* o1, void* o2,
+                        uint32_t* sink, size_t bytes, int reads, int writes, int store_kind,
+                        int threads, int vecs_per_thread, int64_t grid, fm_stream_t stream);
+
 /* ------------------------------------------------------------------ RMSNorm
  * Replaces _launch_rms_fwd / _rms_layernorm_forward (forgemind/kernels/norm.py:1095-1101,
  * 133-175); semantics of _fallback.rms_norm (forgemind/kernels/_fallback.py:26-30):

@@ -36,7 +36,7 @@ def lib():
 
 def test_header_and_binding_agree(lib):
     decl = _declared()
-    assert len(decl) == 41
+    assert len(decl) == 42
     assert set(decl) == set(_hip.SIGNATURES), set(decl) ^ set(_hip.SIGNATURES)
     for name, nargs in decl.items():
         assert hasattr(lib, name), f"{name} is declared in fm_hip.h but not exported"
