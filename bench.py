@@ -106,6 +106,7 @@ def parse():
     ap.add_argument("--workload", default="ce",
                     choices=WORKLOADS)
     ap.add_argument("--no-extras", action="store_true", help="only the headline workload")
+    ap.add_argument("--only", default="", metavar="A,B", help="besides the headline, only these workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--detail", default="", metavar="PATH",
                     help="also write the long form (descriptions, warm / graph / eager / CPU columns) here")
@@ -1250,7 +1251,8 @@ def main():
     detail = {a.workload: res}
     units = {a.workload: head_unit_rows}
     if not a.no_extras:
-        for name in WORKLOADS:
+        chosen = [n for n in a.only.split(",") if n] or WORKLOADS
+        for name in chosen:
             if name == a.workload:
                 continue
             wl = make_workload(name, torch, L, dev)
@@ -1269,10 +1271,8 @@ def main():
     line["roofline"]["configs"] = {c: config_row(detail[wn], units[wn]) for c, wn in CONFIGS if wn in detail}
     named = set(by_workload.values())
     line["workloads"] = {n: short_row(r) for n, r in detail.items() if n not in named}
-    kb = None
-    if not a.no_extras:
-        kb = kbench_style(torch)
-        line["kbench"] = kb
+    if not a.no_extras and not a.only:
+        line["kbench"] = kbench_style(torch)
     line["hbm_ceiling_measured"] = stream_ceiling(torch, L, dev)
     if a.detail:
         os.makedirs(os.path.dirname(os.path.abspath(a.detail)), exist_ok=True)

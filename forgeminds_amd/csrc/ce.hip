@@ -43,8 +43,8 @@ __global__ __launch_bounds__(THREADS) void ce_fwd_kernel(const T* __restrict__ l
     u32x4 raw[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
     }
     // the maximum is taken on the raw logits and scaled once per batch, so each element costs
     // one max, one fma and one exp2
@@ -160,24 +160,22 @@ __global__ __launch_bounds__(THREADS) void ce_bwd_kernel(const T* __restrict__ l
     u32x4 raw[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const int c = c0 + u * THREADS + tid;
+      touch(raw[u]);
       if (c < sp.nvec) {
         float z[EPV], o[EPV];
         Elem<T>::unpack(raw[u], z);
         const int col0 = sp.head + c * EPV;
 #pragma unroll
-        for (int e = 0; e < EPV; ++e) o[e] = fast_exp2(z[e] * kLog2e - l2);
-        if (y >= col0 && y < col0 + EPV) {
-#pragma unroll
-          for (int e = 0; e < EPV; ++e) o[e] -= (col0 + e == y) ? 1.f : 0.f;
+        for (int e = 0; e < EPV; ++e) {
+          o[e] = fast_exp2(z[e] * kLog2e - l2);
+          o[e] = (col0 + e == y ? o[e] - 1.f : o[e]) * scale;
         }
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) o[e] *= scale;
         store16_stream(gp + col0, Elem<T>::pack(o));
       }
     }
@@ -233,8 +231,8 @@ __global__ __launch_bounds__(THREADS) void ce_loss_grad_wide_kernel(const T* log
     u32x4 raw[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) raw[u] = load16(rp + sp.head + (int64_t)c * EPV);
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      raw[u] = load16(rp + sp.head + (int64_t)c * EPV);
     }
     float z[UNROLL][EPV];
     float raw_max = -INFINITY;
@@ -278,24 +276,22 @@ __global__ __launch_bounds__(THREADS) void ce_loss_grad_wide_kernel(const T* log
     u32x4 raw[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const int c = c0 + u * THREADS + tid;
+      touch(raw[u]);
       if (c < sp.nvec) {
         float z[EPV], o[EPV];
         Elem<T>::unpack(raw[u], z);
         const int col0 = sp.head + c * EPV;
 #pragma unroll
-        for (int e = 0; e < EPV; ++e) o[e] = fast_exp2(z[e] * kLog2e - l2);
-        if (y >= col0 && y < col0 + EPV) {
-#pragma unroll
-          for (int e = 0; e < EPV; ++e) o[e] -= (col0 + e == y) ? 1.f : 0.f;
+        for (int e = 0; e < EPV; ++e) {
+          o[e] = fast_exp2(z[e] * kLog2e - l2);
+          o[e] = (col0 + e == y ? o[e] - 1.f : o[e]) * scale;
         }
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) o[e] *= scale;
         store16_stream(gp + col0, Elem<T>::pack(o));
       }
     }

@@ -162,6 +162,14 @@ __device__ __forceinline__ void unpack_again(u32x4 raw, float (&f)[N]) {
   Elem<T>::unpack(raw, f);
 }
 
+// Marks the point where a loaded vector is taken into use, unconditionally. Without it the
+// compiler sinks a load whose only use sits behind a lane-dependent branch into that branch, and
+// then has to wait for every outstanding load before the next one may reuse the register; with it
+// the wait for vector u sits in straight-line code and counts exactly the loads issued after it.
+__device__ __forceinline__ void touch(u32x4& raw) {
+  asm volatile("" : "+v"(raw.x), "+v"(raw.y), "+v"(raw.z), "+v"(raw.w));
+}
+
 // ---------------------------------------------------------------- wave reductions (DPP)
 __device__ __forceinline__ int lane_id() {
   return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));

@@ -39,6 +39,13 @@ __device__ __forceinline__ int edge_col(const RowSplit& s, int e) {
   return e < s.head ? e : s.tail0 + (e - s.head);
 }
 
+// Column a lane fetches when its own column `c` may lie past the row's last vector: such lanes
+// re-read the last vector and discard it. The load then needs no branch. A load behind a
+// lane-dependent branch makes the compiler wait for every earlier load of the wave before it
+// issues the next one (it cannot prove that the register's previous load was consumed), which
+// leaves one 16-byte load per wave in flight however far the loop is unrolled.
+__device__ __forceinline__ int clamp_col(int c, int nvec) { return c < nvec ? c : nvec - 1; }
+
 // Online-softmax state in the base-2 domain: sum = sum_j exp2(z_j - m).
 struct MaxSum {
   float m, s;

@@ -128,11 +128,9 @@ __device__ __forceinline__ void kl_grad_sweep(const T* sp_, const T* tp_, GT* gp
     u32x4 rs[UNROLL], rt[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) {
-        rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
-        rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
-      }
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
+      rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
@@ -187,11 +185,9 @@ __global__ __launch_bounds__(THREADS) void kl_fwd_kernel(const T* __restrict__ s
     u32x4 rs[UNROLL], rt[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) {
-        rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
-        rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
-      }
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
+      rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
     }
     kl_update<T, UNROLL>(k, rs, rt, c0 + tid, THREADS, sp.nvec, c1);
   }
@@ -248,15 +244,13 @@ __global__ __launch_bounds__(THREADS) void kl_fwd_topk_kernel(
     u32x4 rs[UNROLL], rt[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) {
-        if constexpr (GRAD) {   // a gradient sweep follows: leave the row to the caches
-          rs[u] = load16(sp_ + sp.head + (int64_t)c * EPV);
-          rt[u] = load16(tp_ + sp.head + (int64_t)c * EPV);
-        } else {
-          rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
-          rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
-        }
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      if constexpr (GRAD) {   // a gradient sweep follows: leave the row to the caches
+        rs[u] = load16(sp_ + sp.head + (int64_t)c * EPV);
+        rt[u] = load16(tp_ + sp.head + (int64_t)c * EPV);
+      } else {
+        rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
+        rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
       }
     }
     kl_update<T, UNROLL>(st, rs, rt, c0 + tid, THREADS, sp.nvec, c1);
@@ -356,15 +350,15 @@ __global__ __launch_bounds__(THREADS) void kl_bwd_kernel(const T* __restrict__ s
     u32x4 rs[UNROLL], rt[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) {
-        rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
-        rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
-      }
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
+      rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const int c = c0 + u * THREADS + tid;
+      touch(rs[u]);
+      touch(rt[u]);
       if (c < sp.nvec) {
         float zs[EPV], zt[EPV], o[EPV];
         Elem<T>::unpack(rs[u], zs);
@@ -567,11 +561,9 @@ __global__ __launch_bounds__(THREADS) void kl_loss_grad_wide_kernel(const T* stu
     u32x4 rs[UNROLL], rt[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) {
-        rs[u] = load16(sp_ + sp.head + (int64_t)c * EPV);
-        rt[u] = load16(tp_ + sp.head + (int64_t)c * EPV);
-      }
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      rs[u] = load16(sp_ + sp.head + (int64_t)c * EPV);
+      rt[u] = load16(tp_ + sp.head + (int64_t)c * EPV);
     }
     kl_update<T, UNROLL>(k, rs, rt, c0 + tid, THREADS, sp.nvec, c1);
   }

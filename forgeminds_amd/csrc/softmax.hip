@@ -34,8 +34,8 @@ __global__ __launch_bounds__(THREADS) void softmax_kernel(const T* __restrict__ 
     u32x4 raw[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) raw[u] = load16(rp + sp.head + (int64_t)c * EPV);
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      raw[u] = load16(rp + sp.head + (int64_t)c * EPV);
     }
     float z[UNROLL][EPV];
     float cm = st.m;
@@ -69,12 +69,25 @@ __global__ __launch_bounds__(THREADS) void softmax_kernel(const T* __restrict__ 
   const MaxSum tot = block_merge<NW>(st, smem);
   // a row whose maximum is -inf has sum 0: 0 * inf = NaN, which is what torch returns
   const float inv = 1.f / tot.s;
-  for (int c = tid; c < sp.nvec; c += THREADS) {
-    float z[EPV], o[EPV];
-    Elem<T>::unpack(load16(rp + sp.head + (int64_t)c * EPV), z);
+  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+    u32x4 raw[UNROLL];
 #pragma unroll
-    for (int e = 0; e < EPV; ++e) o[e] = fast_exp2(z[e] * kLog2e - tot.m) * inv;
-    store16_stream(op + sp.head + (int64_t)c * EPV, Elem<T>::pack(o));
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      raw[u] = load16(rp + sp.head + (int64_t)c * EPV);
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      touch(raw[u]);
+      if (c < sp.nvec) {
+        float z[EPV], o[EPV];
+        Elem<T>::unpack(raw[u], z);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] = fast_exp2(z[e] * kLog2e - tot.m) * inv;
+        store16_stream(op + sp.head + (int64_t)c * EPV, Elem<T>::pack(o));
+      }
+    }
   }
   for (int e = tid; e < ne; e += THREADS) {
     const int col = edge_col(sp, e);
@@ -198,11 +211,9 @@ __global__ __launch_bounds__(THREADS) void softmax_bwd_kernel(const T* __restric
     u32x4 ry[UNROLL], rg[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int c = c0 + u * THREADS + tid;
-      if (c < sp.nvec) {
-        ry[u] = load16(yp + sp.head + (int64_t)c * EPV);
-        rg[u] = load16(gp + sp.head + (int64_t)c * EPV);
-      }
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      ry[u] = load16(yp + sp.head + (int64_t)c * EPV);
+      rg[u] = load16(gp + sp.head + (int64_t)c * EPV);
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
@@ -221,13 +232,28 @@ __global__ __launch_bounds__(THREADS) void softmax_bwd_kernel(const T* __restric
     dot += Elem<T>::load1(yp + col) * Elem<T>::load1(gp + col);
   }
   dot = block_sum<NW>(dot, smem);
-  for (int c = tid; c < sp.nvec; c += THREADS) {
-    float a[EPV], b[EPV], o[EPV];
-    Elem<T>::unpack(load16(yp + sp.head + (int64_t)c * EPV), a);
-    Elem<T>::unpack(load16(gp + sp.head + (int64_t)c * EPV), b);
+  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+    u32x4 ry[UNROLL], rg[UNROLL];
 #pragma unroll
-    for (int e = 0; e < EPV; ++e) o[e] = (b[e] - dot) * a[e];
-    store16_stream(op + sp.head + (int64_t)c * EPV, Elem<T>::pack(o));
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      ry[u] = load16(yp + sp.head + (int64_t)c * EPV);
+      rg[u] = load16(gp + sp.head + (int64_t)c * EPV);
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      touch(ry[u]);
+      touch(rg[u]);
+      if (c < sp.nvec) {
+        float a[EPV], b[EPV], o[EPV];
+        Elem<T>::unpack(ry[u], a);
+        Elem<T>::unpack(rg[u], b);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] = (b[e] - dot) * a[e];
+        store16_stream(op + sp.head + (int64_t)c * EPV, Elem<T>::pack(o));
+      }
+    }
   }
   for (int e = tid; e < ne; e += THREADS) {
     const int col = edge_col(sp, e);

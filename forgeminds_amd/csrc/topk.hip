@@ -128,8 +128,8 @@ __global__ __launch_bounds__(THREADS, THREADS >= 256 ? 8 : 1) void topk_lds_kern
       u32x4 raw[UNROLL];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {
-        const int c = c0 + u * THREADS + tid;
-        if (decltype(full)::value || c < sp.nvec) raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
+        const int c = decltype(full)::value ? c0 + u * THREADS + tid : clamp_col(c0 + u * THREADS + tid, sp.nvec);
+        raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
       }
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) {

@@ -16,7 +16,8 @@ import threading
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_HERE), "_lib", "libfmhip.so")
+# FORGEMINDS_AMD_LIB points at another build of the library (a release next to a debug build)
+LIB_PATH = os.environ.get("FORGEMINDS_AMD_LIB") or os.path.join(os.path.dirname(_HERE), "_lib", "libfmhip.so")
 
 F32, F16, BF16 = 0, 1, 2
 REDUCE = {"none": 0, "sum": 1, "mean": 2}
