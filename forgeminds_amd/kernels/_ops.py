@@ -60,17 +60,18 @@ def wanted() -> bool:
         return False
 
 
-def _new_op(name: str, impl, fake):
+def _new_op(name: str, impl, fake, mutates=()):
     qual = f"{NAMESPACE}::{name}"
     try:
-        op = torch.library.custom_op(qual, mutates_args=())(impl)
+        op = torch.library.custom_op(qual, mutates_args=mutates)(impl)
     except (RuntimeError, ValueError) as exc:  # module imported twice in one process
         text = str(exc)
         packet = getattr(getattr(torch.ops, NAMESPACE, None), name, None)
         if packet is None or not ("already" in text or "overriding" in text):
             raise
         return packet.default
-    op.register_fake(fake)
+    if fake is not None:
+        op.register_fake(fake)
     return op
 
 
@@ -91,4 +92,12 @@ def define_backward(name: str, impl, fake):
     return _new_op(f"{name}_backward", impl, fake)
 
 
-__all__ = ["AVAILABLE", "available", "use_custom_ops", "wanted", "define", "define_backward"]
+def define_inplace(name: str, impl, mutates):
+    """Op ``forgemind::<name>`` that returns nothing and writes into the arguments named in
+    ``mutates`` (the in-place multiply behind the losses whose forward already wrote the gradient)."""
+    if not AVAILABLE:  # pragma: no cover
+        return None
+    return _new_op(name, impl, lambda *a, **k: None, mutates=tuple(mutates))
+
+
+__all__ = ["AVAILABLE", "available", "use_custom_ops", "wanted", "define", "define_backward", "define_inplace"]

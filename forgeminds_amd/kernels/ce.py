@@ -25,7 +25,7 @@ from ._common import _note, fast_ok
 
 class _CrossEntropyFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, logits, labels, ignore_index, reduction, inplace):
+    def forward(ctx, logits, labels, ignore_index, reduction, inplace, retain):
         lg2 = logits.contiguous().view(-1, logits.shape[-1])
         y = labels.contiguous().view(-1)
         ctx.shape = logits.shape
@@ -48,12 +48,12 @@ class _CrossEntropyFn(torch.autograd.Function):
         # storage (contiguous() did not copy)
         own = inplace and lg2.data_ptr() == logits.data_ptr()
         loss, dl, _n_valid, _rows = _hip.ce_loss_grad(lg2.detach(), y, ignore_index, reduction, own)
-        ctx.mode = "own" if own else "private"
+        ctx.mode = "retain" if (retain and not own) else "once"
         ctx.spent = False
-        if own:
+        if ctx.mode == "retain":    # asked for: keep the (intact) logits so that a later backward can redo the pass
+            ctx.save_for_backward(dl, lg2.detach(), y)
+        else:                       # only the gradient buffer lives on, as in the reference (kernels/kl.py:171)
             ctx.save_for_backward(dl)
-        else:
-            ctx.save_for_backward(dl, lg2.detach(), y)   # the logits are intact: a later backward can redo the pass
         return loss.clone()
 
     @staticmethod
@@ -63,24 +63,29 @@ class _CrossEntropyFn(torch.autograd.Function):
         if ctx.mode == "two_pass":
             lg2, y, lse, n_valid = ctx.saved_tensors
             dl = _hip.ce_bwd(lg2, y, lse, n_valid if reduction == "mean" else None, g32, ignore_index)
-            return dl.view(ctx.shape), None, None, None, None
-        if ctx.mode == "own":
+            return dl.view(ctx.shape), None, None, None, None, None
+        if ctx.mode == "once":
             (dl,) = ctx.saved_tensors
             if ctx.spent:
                 raise RuntimeError("cross_entropy: the gradient buffer written in the forward was already "
-                                   "consumed by a backward pass; run the forward again")
+                                   "consumed by a backward pass; run the forward again, or pass retain=True "
+                                   "to keep the logits for repeated backward passes")
         else:
             dl, lg2, y = ctx.saved_tensors
             if ctx.spent:   # retain_graph / a second autograd.grad: the first pass scaled `dl` in place
                 _loss, dl, _n, _r = _hip.ce_loss_grad(lg2, y, ignore_index, reduction, False)
         ctx.spent = True
         _hip.scale_inplace(dl, g32)
-        return dl.view(ctx.shape), None, None, None, None
+        return dl.view(ctx.shape), None, None, None, None, None
 
 
 # ------------------------------------------------------------------ traced: custom ops
-# While tracing, the two-pass dataflow is used (forward keeps the per-row log-sum-exp, backward
-# recomputes the softmax): it is purely functional, which is what a traced graph needs.
+# Two op pairs. bf16 / fp32 logits take the dataflow of the eager path: the forward op returns the
+# loss and, as extra outputs (the way the reference's ops carry rstd and xn,
+# forgemind/kernels/_ops.py:44-48), the gradient for an upstream gradient of 1; the backward is an
+# op that multiplies that buffer in place (mutates_args) and hands it on. fp16 logits keep the
+# two-pass dataflow (forward keeps the per-row log-sum-exp, backward recomputes the softmax and
+# applies the upstream gradient in fp32), which is purely functional.
 def _ce_impl(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int,
              mean: bool) -> typing.Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     lg2 = logits.contiguous().view(-1, logits.shape[-1])
@@ -114,13 +119,42 @@ def _ce_autograd(ctx, g, _glse, _gn):
     return _CE_BWD_OP(logits, labels, lse, n_valid, g, ctx.ignore_index, ctx.mean), None, None, None
 
 
+def _ce1_impl(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int,
+              mean: bool) -> typing.Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    lg2 = logits.contiguous().view(-1, logits.shape[-1])
+    loss, dl, n_valid, _rows = _hip.ce_loss_grad(lg2, labels.contiguous().view(-1), ignore_index,
+                                                 "mean" if mean else "sum", False)
+    return loss.clone(), dl.view(logits.shape), n_valid.clone()
+
+
+def _ce1_fake(logits, labels, ignore_index, mean):
+    f32 = dict(device=logits.device, dtype=torch.float32)
+    return torch.empty((), **f32), torch.empty_like(logits, memory_format=torch.contiguous_format), torch.empty((), **f32)
+
+
+def _scale_impl(grad: torch.Tensor, g: torch.Tensor) -> None:
+    _hip.scale_inplace(grad, g.detach().to(torch.float32).contiguous())
+
+
+def _ce1_setup(ctx, inputs, output):
+    ctx.save_for_backward(output[1])
+
+
+def _ce1_autograd(ctx, g, _gdl, _gn):
+    (dl,) = ctx.saved_tensors
+    SCALE_OP(dl, g)
+    return dl, None, None, None
+
+
+SCALE_OP = _ops.define_inplace("scale_grad_", _scale_impl, ("grad",))
+_CE1_OP = _ops.define("cross_entropy_grad", _ce1_impl, _ce1_fake, _ce1_setup, _ce1_autograd)
 _CE_BWD_OP = _ops.define_backward("cross_entropy", _ce_bwd_impl,
                                   lambda logits, labels, lse, n_valid, g, ignore_index, mean: torch.empty_like(logits))
 _CE_OP = _ops.define("cross_entropy", _ce_impl, _ce_fake, _ce_setup, _ce_autograd)
 
 
 def cross_entropy(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int = -100,
-                  reduction: str = "mean", inplace: bool = False) -> torch.Tensor:
+                  reduction: str = "mean", inplace: bool = False, retain: bool = False) -> torch.Tensor:
     """fp32 scalar CE over the last dim of ``logits``.
 
     ``reduction="mean"`` divides the sum over valid rows by ``max(1, #valid)`` (all-ignored
@@ -132,8 +166,11 @@ def cross_entropy(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int 
     ``inplace=True`` lets the kernel write the gradient over ``logits`` (only for a tensor the
     caller owns and no longer reads, e.g. the output of the head projection): no second
     ``[N, V]`` buffer exists, and that buffer serves ONE backward pass (a second one raises).
-    Without ``inplace`` the backward may run any number of times (``retain_graph=True``): the
-    first scales the gradient the forward wrote, later ones redo the pass from the logits.
+    Without ``inplace`` the gradient goes to a buffer of its own, which is all that is kept for
+    the backward (the logits are not pinned), and it too serves one backward pass;
+    ``retain=True`` also keeps the logits so that the backward may run any number of times
+    (``retain_graph=True``): the first scales the gradient the forward wrote, later ones redo
+    the pass.
     fp16 logits always take the two-pass form (forward keeps the log-sum-exps, the backward
     applies the upstream gradient in fp32 before its one rounding), so a loss scaler works.
     """
@@ -148,8 +185,10 @@ def cross_entropy(logits: torch.Tensor, labels: torch.Tensor, ignore_index: int 
     if not fast_ok(logits):
         return fb.cross_entropy(logits, labels, ignore_index, reduction)
     if _CE_OP is not None and _ops.wanted():
+        if logits.dtype != torch.float16 and logits.requires_grad and torch.is_grad_enabled():
+            return _CE1_OP(logits, labels, int(ignore_index), reduction == "mean")[0]
         return _CE_OP(logits, labels, int(ignore_index), reduction == "mean")[0]
-    return _CrossEntropyFn.apply(logits, labels, int(ignore_index), reduction, bool(inplace))
+    return _CrossEntropyFn.apply(logits, labels, int(ignore_index), reduction, bool(inplace), bool(retain))
 
 
 __all__ = ["cross_entropy"]

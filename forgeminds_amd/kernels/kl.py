@@ -28,7 +28,7 @@ _REDUCTIONS = ("mean", "sum", "none")
 
 class _KLDivFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, student, teacher, reduction, grad_dtype, temperature, reuse):
+    def forward(ctx, student, teacher, reduction, grad_dtype, temperature, reuse, retain):
         v = student.shape[-1]
         s2 = student.contiguous().view(-1, v)
         t2 = teacher.contiguous().view(-1, v)
@@ -46,11 +46,11 @@ class _KLDivFn(torch.autograd.Function):
             own = reuse and s2.data_ptr() == student.data_ptr() and gdt == s2.dtype
             loss, grad, _rows = _hip.kl_loss_grad(s2.detach(), t2, inv_t, reduction, gdt, own)
             ctx.in_forward = True
-            ctx.own = own
-            if own:
+            ctx.once = own or not retain
+            if ctx.once:     # only the gradient buffer lives on (reference kl.py:171)
                 ctx.save_for_backward(grad)
-            else:
-                ctx.save_for_backward(grad, s2.detach(), t2)   # inputs intact: a later backward can redo the pass
+            else:            # asked for: the intact inputs stay too, so that a later backward can redo the pass
+                ctx.save_for_backward(grad, s2.detach(), t2)
             return loss
         loss, rows, lse_s, lse_t = _hip.kl_fwd(s2, t2, inv_t, reduction)
         ctx.save_for_backward(s2, t2, lse_s, lse_t)
@@ -62,11 +62,12 @@ class _KLDivFn(torch.autograd.Function):
     def backward(ctx, g):
         shape, reduction, gdt, inv_t = ctx.meta
         if ctx.in_forward:
-            if ctx.own:
+            if ctx.once:
                 (grad,) = ctx.saved_tensors
                 if ctx.spent:
                     raise RuntimeError("kl_div_logits: the gradient buffer written in the forward was "
-                                       "already consumed by a backward pass; run the forward again")
+                                       "already consumed by a backward pass; run the forward again, or pass "
+                                       "retain=True to keep the inputs for repeated backward passes")
             else:
                 grad, s2, t2 = ctx.saved_tensors
                 if ctx.spent:   # retain_graph: the first backward scaled `grad` in place (the reference
@@ -74,20 +75,20 @@ class _KLDivFn(torch.autograd.Function):
                     _loss, grad, _rows = _hip.kl_loss_grad(s2, t2, inv_t, reduction, gdt, False)
             ctx.spent = True
             _hip.scale_inplace(grad, g.detach().to(torch.float32).contiguous())
-            return grad.view(shape), None, None, None, None, None
+            return grad.view(shape), None, None, None, None, None, None
         s2, t2, lse_s, lse_t = ctx.saved_tensors
         n = s2.shape[0]
         g32 = g.detach().to(torch.float32).contiguous().view(-1)
         scale = 1.0 / n if reduction == "mean" else 1.0
         grad = _hip.kl_bwd(s2, t2, lse_s, lse_t, g32, reduction == "none", gdt, inv_t, scale)
-        return grad.view(shape), None, None, None, None, None
+        return grad.view(shape), None, None, None, None, None, None
 
 
 class _KLDivTopkFn(torch.autograd.Function):
     """KL forward that also hands back the teacher's top-k (indices and probabilities)."""
 
     @staticmethod
-    def forward(ctx, student, teacher, k, reduction, grad_dtype, temperature, index_dtype):
+    def forward(ctx, student, teacher, k, reduction, grad_dtype, temperature, index_dtype, retain):
         v = student.shape[-1]
         s2 = student.contiguous().view(-1, v)
         t2 = teacher.contiguous().view(-1, v)
@@ -109,7 +110,11 @@ class _KLDivTopkFn(torch.autograd.Function):
             loss, rows, lse_s, lse_t, _, idx, probs = out[:7]
         if with_grad:
             ctx.in_forward = True
-            ctx.save_for_backward(out[7], s2.detach(), t2)
+            ctx.once = not retain
+            if ctx.once:
+                ctx.save_for_backward(out[7])
+            else:
+                ctx.save_for_backward(out[7], s2.detach(), t2)
         else:
             ctx.save_for_backward(s2, t2, lse_s, lse_t)
         ctx.meta = (student.shape, reduction, gdt, inv_t)
@@ -125,23 +130,34 @@ class _KLDivTopkFn(torch.autograd.Function):
     def backward(ctx, g, _gp, _gi):
         shape, reduction, gdt, inv_t = ctx.meta
         if ctx.in_forward:
-            grad, s2, t2 = ctx.saved_tensors
-            if ctx.spent:       # a repeated backward redoes the gradient from the intact inputs
-                _loss, grad, _rows = _hip.kl_loss_grad(s2, t2, inv_t, reduction, gdt, False)
+            if ctx.once:
+                (grad,) = ctx.saved_tensors
+                if ctx.spent:
+                    raise RuntimeError("kl_div_logits_topk: the gradient buffer written in the forward was "
+                                       "already consumed by a backward pass; run the forward again, or pass "
+                                       "retain=True to keep the inputs for repeated backward passes")
+            else:
+                grad, s2, t2 = ctx.saved_tensors
+                if ctx.spent:       # a repeated backward redoes the gradient from the intact inputs
+                    _loss, grad, _rows = _hip.kl_loss_grad(s2, t2, inv_t, reduction, gdt, False)
             ctx.spent = True
             _hip.scale_inplace(grad, g.detach().to(torch.float32).contiguous())
-            return grad.view(shape), None, None, None, None, None, None
+            return grad.view(shape), None, None, None, None, None, None, None
         s2, t2, lse_s, lse_t = ctx.saved_tensors
         n = s2.shape[0]
         g32 = g.detach().to(torch.float32).contiguous().view(-1)
         scale = 1.0 / n if reduction == "mean" else 1.0
         grad = _hip.kl_bwd(s2, t2, lse_s, lse_t, g32, reduction == "none", gdt, inv_t, scale)
-        return grad.view(shape), None, None, None, None, None, None
+        return grad.view(shape), None, None, None, None, None, None, None
 
 
 # ------------------------------------------------------------------ traced: custom ops
-# While tracing, the functional two-pass dataflow: the forward keeps the two per-row
-# log-sum-exps, the backward recomputes both softmaxes.
+# Two op pairs, as for the cross entropy. Sum / mean over bf16 or fp32 logits: the forward op
+# returns the loss and, as an extra output, the student's gradient for an upstream gradient of 1
+# (the reference's dataflow, kl.py:143-191; aux outputs as in its _ops.py:44-48); the backward is
+# the op that multiplies that buffer in place. reduction="none" and fp16 keep the functional
+# two-pass dataflow: the forward keeps the two per-row log-sum-exps, the backward recomputes both
+# softmaxes.
 _RED = ("none", "sum", "mean")
 
 
@@ -186,6 +202,31 @@ def _kl_autograd(ctx, g, _g1, _g2):
     return _KL_BWD_OP(student, teacher, lse_s, lse_t, g, ctx.reduction, ctx.inv_t, False), None, None, None
 
 
+def _kl1_impl(student: torch.Tensor, teacher: torch.Tensor, reduction: int,
+              inv_t: float) -> typing.Tuple[torch.Tensor, torch.Tensor]:
+    v = student.shape[-1]
+    s2, t2 = student.contiguous().view(-1, v), teacher.contiguous().view(-1, v)
+    loss, grad, _rows = _hip.kl_loss_grad(s2, t2, inv_t, _RED[reduction], student.dtype, False)
+    return loss, grad.view(student.shape)
+
+
+def _kl1_fake(student, teacher, reduction, inv_t):
+    return (torch.empty((), device=student.device, dtype=torch.float32),
+            torch.empty_like(student, memory_format=torch.contiguous_format))
+
+
+def _kl1_setup(ctx, inputs, output):
+    ctx.save_for_backward(output[1])
+
+
+def _kl1_autograd(ctx, g, _ggrad):
+    from .ce import SCALE_OP
+    (grad,) = ctx.saved_tensors
+    SCALE_OP(grad, g)
+    return grad, None, None, None
+
+
+_KL1_OP = _ops.define("kl_div_grad", _kl1_impl, _kl1_fake, _kl1_setup, _kl1_autograd)
 _KL_BWD_OP = _ops.define_backward("kl_div", _kl_bwd_impl, _kl_bwd_fake)
 _KL_OP = _ops.define("kl_div", _kl_impl, _kl_fake, _kl_setup, _kl_autograd)
 
@@ -199,7 +240,7 @@ def _kernel_ok(*tensors) -> bool:
 
 def kl_div_logits(student: torch.Tensor, teacher: torch.Tensor, reduction: str = "mean",
                   grad_dtype: "torch.dtype | None" = None,
-                  temperature: float = 1.0, reuse: bool = False) -> torch.Tensor:
+                  temperature: float = 1.0, reuse: bool = False, retain: bool = False) -> torch.Tensor:
     """``KL(softmax(teacher / T) || softmax(student / T))`` over the last dim.
 
     ``mean`` divides by the number of rows (there is no ignore mask, reference
@@ -207,6 +248,8 @@ def kl_div_logits(student: torch.Tensor, teacher: torch.Tensor, reduction: str =
     ``grad_dtype`` (the student's dtype by default, or ``torch.float32``) is the dtype the
     kernel writes the student gradient in. ``reuse=True`` (reference ``kl.py:146-150``) lets
     the gradient overwrite ``student``: only for a tensor the caller owns and no longer reads.
+    The gradient written in the forward serves one backward pass; ``retain=True`` also keeps the
+    two logit tensors so that the backward may run again (``retain_graph=True``).
     """
     if reduction not in _REDUCTIONS:
         raise ValueError(f"reduction must be mean|sum|none, got {reduction!r}")
@@ -220,13 +263,17 @@ def kl_div_logits(student: torch.Tensor, teacher: torch.Tensor, reduction: str =
     if not _kernel_ok(student, teacher):
         return fb.kl_div_logits(student, teacher, reduction, temperature)
     if _KL_OP is not None and _ops.wanted() and grad_dtype in (None, student.dtype):
+        if (reduction != "none" and student.dtype != torch.float16 and student.requires_grad
+                and torch.is_grad_enabled()):
+            return _KL1_OP(student, teacher, _RED.index(reduction), 1.0 / float(temperature))[0]
         return _KL_OP(student, teacher, _RED.index(reduction), 1.0 / float(temperature))[0]
-    return _KLDivFn.apply(student, teacher, reduction, grad_dtype, float(temperature), bool(reuse))
+    return _KLDivFn.apply(student, teacher, reduction, grad_dtype, float(temperature), bool(reuse), bool(retain))
 
 
 def kl_div_logits_topk(student: torch.Tensor, teacher: torch.Tensor, k: int,
                        reduction: str = "mean", grad_dtype: "torch.dtype | None" = None,
-                       temperature: float = 1.0, index_dtype: torch.dtype = torch.int64):
+                       temperature: float = 1.0, index_dtype: torch.dtype = torch.int64,
+                       retain: bool = False):
     """``kl_div_logits`` plus the teacher's exact top-``k`` from the same pass over the logits.
 
     Returns ``(loss, probs, idx)``: ``idx [..., k]`` are the columns ``topk(teacher, k)`` would
@@ -256,7 +303,7 @@ def kl_div_logits_topk(student: torch.Tensor, teacher: torch.Tensor, k: int,
             probs = torch.gather(logp, -1, idx).exp()
         return loss, probs, idx.to(index_dtype)
     return _KLDivTopkFn.apply(student, teacher, int(k), reduction, grad_dtype, float(temperature),
-                              index_dtype)
+                              index_dtype, bool(retain))
 
 
 def kl_distill_loss(hs: torch.Tensor, ht: torch.Tensor, w: torch.Tensor, teacher_head,

@@ -308,15 +308,24 @@ def test_fp16_chunked_cross_entropy_under_checkpointing():
     assert close(h.grad, hr.grad, rel=2e-2) and close(wt.grad, wr.grad, rel=2e-2)
 
 
-def test_losses_allow_a_second_backward_when_the_gradient_buffer_is_private():
+def test_losses_allow_a_second_backward_when_asked_to_retain():
     # the reference's KL multiplies its stored gradient out of place (kernels/kl.py:183-191), so
-    # retain_graph=True works there; here the first backward scales in place and later ones redo the pass
+    # retain_graph=True works there; here the first backward scales in place, and with retain=True
+    # (which keeps the inputs alive) later ones redo the pass. Without it only the gradient buffer
+    # is saved and a second backward says so.
     g = torch.Generator().manual_seed(78)
     lg = (2 * torch.randn(64, 4000, generator=g)).bfloat16()
     y = torch.randint(0, 4000, (64,), generator=g)
     _, og = O.cross_entropy(lg, y)
     lgd = lg.to(DEV).requires_grad_(True)
-    loss = kernels.cross_entropy(lgd, y.to(DEV))
+    once = kernels.cross_entropy(lgd, y.to(DEV))
+    saved = [t for t in (once.grad_fn.saved_tensors if hasattr(once.grad_fn, "saved_tensors") else ())]
+    assert len(saved) == 1 and saved[0].shape == (64, 4000)      # the gradient buffer only: the logits are not pinned
+    once.backward(retain_graph=True)
+    with pytest.raises(RuntimeError, match="already consumed"):
+        once.backward()
+    lgd.grad = None
+    loss = kernels.cross_entropy(lgd, y.to(DEV), retain=True)
     (loss * 3.0).backward(retain_graph=True)
     first = lgd.grad.clone()
     lgd.grad = None
@@ -326,12 +335,68 @@ def test_losses_allow_a_second_backward_when_the_gradient_buffer_is_private():
     t = (s.float() + 0.5 * torch.randn(12, 3000, generator=g)).bfloat16()
     _, kg = O.kl_div(s, t, "mean", 1.0)
     sd = s.to(DEV).requires_grad_(True)
-    kl = kernels.kl_div_logits(sd, t.to(DEV))
+    kl1 = kernels.kl_div_logits(sd, t.to(DEV))
+    kl1.backward(retain_graph=True)
+    with pytest.raises(RuntimeError, match="already consumed"):
+        kl1.backward()
+    sd.grad = None
+    kl = kernels.kl_div_logits(sd, t.to(DEV), retain=True)
     (kl * 2.0).backward(retain_graph=True)
     a = sd.grad.clone()
     sd.grad = None
     kl.backward()
     assert close(a, kg.float() * 2.0) and close(sd.grad, kg.float())
+
+
+def test_compiled_losses_write_the_gradient_in_the_forward():
+    # under torch.compile the bf16 / fp32 losses are ONE op whose extra output is the gradient for an
+    # upstream gradient of 1 (aux outputs as in the reference's forgemind/kernels/_ops.py:44-48), and the
+    # backward is an op that scales that buffer in place: same kernels, same bits as the eager path
+    g = torch.Generator().manual_seed(91)
+    lg = (2 * torch.randn(96, 4000, generator=g)).bfloat16().to(DEV)
+    y = torch.randint(0, 4000, (96,), generator=g)
+    y[::9] = -100
+    y = y.to(DEV)
+    s = (3 * torch.randn(24, 3000, generator=g)).bfloat16().to(DEV)
+    t = (s.float() + 0.5 * torch.randn(24, 3000, generator=g).to(DEV)).bfloat16()
+
+    def ce(x):
+        return kernels.cross_entropy(x * 1.0, y) * 3.0
+
+    def kl(x):
+        return kernels.kl_div_logits(x * 1.0, t, temperature=2.0) * 0.5
+
+    for fn, x0, kernel in ((ce, lg, "ce_loss_grad"), (kl, s, "kl_loss_grad")):
+        xe = x0.clone().requires_grad_(True)
+        le = fn(xe)
+        le.backward()
+        xc = x0.clone().requires_grad_(True)
+        compiled = torch.compile(fn, backend="aot_eager", fullgraph=True)
+        lc = compiled(xc)
+        assert kernel in _hip.last_kernel(), _hip.last_kernel()      # the one-pass kernel ran in the compiled forward
+        lc.backward()
+        assert torch.equal(le, lc) and torch.equal(xe.grad, xc.grad)
+        # a second compiled step (the graph is cached; the buffer of the first step was consumed, not reused)
+        xc2 = x0.clone().requires_grad_(True)
+        lc2 = compiled(xc2)
+        lc2.backward()
+        assert torch.equal(lc2, le) and torch.equal(xc2.grad, xe.grad)
+    # one node per loss in the traced graph
+    class M(nn.Module):
+        def forward(self, x):
+            return kernels.cross_entropy(x, y)
+    ep = torch.export.export(M(), (lg.clone().requires_grad_(True),))
+    targets = [str(n.target) for n in ep.graph.nodes if n.op == "call_function"]
+    assert sum("forgemind.cross_entropy" in t_ for t_ in targets) == 1, targets
+    # fp16 keeps the two-pass ops (the upstream gradient is applied in fp32 before the one rounding)
+    lh = lg.half().clone().requires_grad_(True)
+    out = torch.compile(lambda x: kernels.cross_entropy(x, y) * 1024.0, backend="aot_eager", fullgraph=True)(lh)
+    fwd_kernel = _hip.last_kernel()          # (the backward runs on autograd's thread; this is the forward's)
+    out.backward()
+    assert "loss_grad" not in fwd_kernel and fwd_kernel.endswith("true, false>"), fwd_kernel   # loss only, no gradient
+    lr = lg.half().clone().requires_grad_(True)
+    (kernels.cross_entropy(lr, y) * 1024.0).backward()
+    assert torch.equal(lr.grad, lh.grad)
 
 
 def test_kl_autograd_reductions_and_temperature():
