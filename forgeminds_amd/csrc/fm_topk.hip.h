@@ -52,6 +52,19 @@ __device__ __forceinline__ int block_sum_int(int v, int* smem, int nw) {
   return s;
 }
 
+// Sum of a 64-bit value over the workgroup (smem: nw words).
+__device__ __forceinline__ unsigned long long block_sum_u64(unsigned long long v, unsigned long long* smem, int nw) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) smem[wave] = v;
+  __syncthreads();
+  unsigned long long s = 0ull;
+  for (int i = 0; i < nw; ++i) s += smem[i];
+  __syncthreads();
+  return s;
+}
+
 // Exclusive scan of a small per-thread count in thread order; *total gets the block sum.
 __device__ __forceinline__ int block_excl_scan(int v, int* smem, int nw, int* total) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -254,6 +267,81 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
   const int ne = edge_count(sp, v);
   const int64_t row = orow;
 
+  // Sorting or ranking of the C candidates in ccomp and the output of the best k.
+  auto rank_and_write = [&](int C) {
+  // ---- many candidates for the size of the workgroup: a bitonic sort of the slots (key
+  // descending, then column ascending; zero padding sorts last) puts output slot r at position
+  // r for log^2 steps of work, where counting costs one read of every candidate per candidate
+  if (C > kSortFrom && C * C > 256 * THREADS) {
+    int cp = 2 * kSortFrom;
+    while (cp < C) cp <<= 1;
+    for (int s = C + tid; s < cp; s += THREADS) ccomp[s] = 0ull;
+    __syncthreads();
+    for (int size = 2; size <= cp; size <<= 1) {
+      for (int stride = size >> 1; stride > 0; stride >>= 1) {
+        for (int t = tid; t < cp / 2; t += THREADS) {
+          const int lo = 2 * t - (t & (stride - 1));
+          const int hi = lo + stride;
+          const bool desc = (lo & size) == 0;
+          const unsigned long long a = ccomp[lo], b = ccomp[hi];
+          if ((a < b) == desc) { ccomp[lo] = b; ccomp[hi] = a; }
+        }
+        __syncthreads();
+      }
+    }
+    for (int r = tid; r < k; r += THREADS) {
+      const int col = (int)(~(uint32_t)(ccomp[r] & 0xFFFFFFFFull));
+      const int64_t o = row * (int64_t)k + r;
+      if (idx32 != nullptr) idx32[o] = col;
+      if (idx64 != nullptr) idx64[o] = col;
+      if (values != nullptr) values[o] = rp[col];
+      if (probs != nullptr) probs[o] = fast_exp2(Elem<T>::load1(rp + col) * c1 - lse2);
+    }
+    return;
+  }
+
+  // ---- rank the C candidates by counting; rank r < k goes to output slot r
+  int cpad = 64;
+  while (cpad < C) cpad <<= 1;
+  const int parts = THREADS / cpad > 1 ? THREADS / cpad : 1;
+  for (int jx = tid; jx < C; jx += THREADS) crank[jx] = 0;
+  __syncthreads();
+  const int per = (C + parts - 1) / parts;
+  for (int wk = tid; wk < cpad * parts; wk += THREADS) {
+    const int jx = wk % cpad, part = wk / cpad;
+    if (jx < C) {
+      const unsigned long long me = ccomp[jx];
+      const int i0 = part * per;
+      const int i1 = i0 + per < C ? i0 + per : C;
+      // every lane reads the same candidate (an LDS broadcast); eight reads in flight hide
+      // the LDS latency that a one-at-a-time loop would pay per candidate
+      int r = 0;
+      int i = i0;
+      for (; i + 8 <= i1; i += 8) {
+        unsigned long long o[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) o[u] = ccomp[i + u];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) r += o[u] > me ? 1 : 0;
+      }
+      for (; i < i1; ++i) r += ccomp[i] > me ? 1 : 0;
+      if (parts == 1) crank[jx] = r; else atomicAdd(&crank[jx], r);
+    }
+  }
+  __syncthreads();
+  for (int jx = tid; jx < C; jx += THREADS) {
+    const int r = crank[jx];
+    if (r < k) {
+      const int col = (int)(~(uint32_t)(ccomp[jx] & 0xFFFFFFFFull));
+      const int64_t o = row * (int64_t)k + r;
+      if (idx32 != nullptr) idx32[o] = col;
+      if (idx64 != nullptr) idx64[o] = col;
+      if (values != nullptr) values[o] = rp[col];
+      if (probs != nullptr) probs[o] = fast_exp2(Elem<T>::load1(rp + col) * c1 - lse2);
+    }
+  }
+  };
+
   int C = 0;
   bool overflow = false;
   if (v <= CAP) {
@@ -329,6 +417,8 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
       };
       if constexpr (VMAX != kVecMaxNone) {
         // B1: vectors that can hold a candidate go to the work list
+        // (once the list has overflowed the row goes to the exact path anyway: the remaining
+        // vectors are not appended, which spares a row of equal values 16 K atomics on one word)
         auto list = [&](int c) {
           const int slot = atomicAdd(&s_nwork, 1);
           if (slot < WORK) work[slot] = c;
@@ -344,12 +434,17 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
           if constexpr (SKEY == kVhiStream16) tau_hi = skey_threshold<T>(tau, tau_f, only_nan);
           if constexpr (SKEY == kVhiStream32) tau_hi = skey32_threshold(tau, tau_f, only_nan);
           const uint64_t* quad = reinterpret_cast<const uint64_t*>(vhi);
-          for (int q = tid; q * 4 < sp.nvec; q += THREADS) {
-            const uint64_t four = quad[q];
+          bool full = false;   // this thread has seen the list overflow: the row takes the exact path
+          for (int q = tid; q * 4 < sp.nvec && !full; q += THREADS) {   // anyway, and a row of equal values
+            const uint64_t four = quad[q];                              // is spared 16 K atomics on one word
   #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const int c = q * 4 + e;
-              if (c < sp.nvec && (uint32_t)((four >> (16 * e)) & 0xFFFFu) >= tau_hi) list(c);
+              if (c < sp.nvec && (uint32_t)((four >> (16 * e)) & 0xFFFFu) >= tau_hi) {
+                const int slot = atomicAdd(&s_nwork, 1);
+                if (slot < WORK) work[slot] = c;
+                else full = true;
+              }
             }
           }
         }
@@ -375,6 +470,139 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
       __syncthreads();
       if (overflow) C = CAP + 1;
 
+    }
+    // ---- runs of equal values at the k-th place, rows whose vector maxima sit in LDS as exact
+    // 16-bit keys (bf16 / fp16): the k-th largest VECTOR maximum, tau_v, is found by a bit search
+    // over those 2 bytes per vector in LDS, no row read. At least k vectors hold an element
+    // >= tau_v, and elements > tau_v can only sit in the fewer than k vectors whose maximum is
+    // above it: those are revisited through the work list. Either they are k or more -- then the
+    // top k are among them -- or the k-th value IS tau_v and the remaining places go to the first
+    // elements equal to it in column order, which a scan of the row's head finds (it stops as soon
+    // as it has them: with long runs that is the first few thousand columns).
+    if constexpr (VMAX == kVecMaxLds && SKEY == kVhiStream16) {
+      if (C > CAP && sp.nvec >= k) {
+        constexpr uint32_t NANK = SKeyC<T>::kNanAbove + 1u;
+        const uint32_t negz = skey_of_bits<T>(0x8000u);
+        auto nsk = [&](int c) -> uint32_t {   // -0.0 ties with +0.0, every NaN with every other
+          uint32_t sk = vhi[c];
+          sk = sk == negz ? sk + 1u : sk;
+          return sk < NANK ? sk : NANK;
+        };
+        uint32_t tsk = 0u;
+        for (int shift = 14; shift >= 0; shift -= 2) {   // two bits a step: three counts, one reduction
+          int c1 = 0, c2 = 0, c3 = 0;
+          const uint32_t t1 = tsk | (1u << shift), t2 = tsk | (2u << shift), t3 = tsk | (3u << shift);
+          for (int c = tid; c < sp.nvec; c += THREADS) {
+            const uint32_t sk = nsk(c);
+            c1 += sk >= t1 ? 1 : 0;
+            c2 += sk >= t2 ? 1 : 0;
+            c3 += sk >= t3 ? 1 : 0;
+          }
+          // counts are below 2^20 (a row holds at most 2^16.1 vectors): three fit one 64-bit sum
+          const unsigned long long packed = block_sum_u64(((unsigned long long)c3 << 42) |
+                                                          ((unsigned long long)c2 << 21) | (unsigned long long)c1,
+                                                          reinterpret_cast<unsigned long long*>(ccomp), NW);
+          const int n1 = (int)(packed & 0x1FFFFFull), n2 = (int)((packed >> 21) & 0x1FFFFFull), n3 = (int)(packed >> 42);
+          tsk = n3 >= k ? t3 : (n2 >= k ? t2 : (n1 >= k ? t1 : tsk));
+        }
+        const uint32_t kth_c = tsk >= NANK ? (0xFFFFFFFFu & KMASK) : (key_of(float_of_skey<T>(tsk)) & KMASK);
+        if (tid == 0) { s_count = 0; s_nwork = 0; }
+        __syncthreads();
+        for (int c = tid; c < sp.nvec; c += THREADS) {
+          if (nsk(c) > tsk) {
+            const int slot = atomicAdd(&s_nwork, 1);
+            if (slot < WORK) work[slot] = c;
+          }
+        }
+        auto above = [&](float f, int col) {
+          const uint32_t key = key_of(f);
+          if ((key & KMASK) > kth_c) {
+            const int slot = atomicAdd(&s_count, 1);
+            if (slot < CAP) ccomp[slot] = ((unsigned long long)key << 32) | (uint32_t)(~col);
+          }
+        };
+        for (int e = tid; e < ne; e += THREADS) {
+          const int col = edge_col(sp, e);
+          above(Elem<T>::load1(rp + col), col);
+        }
+        __syncthreads();
+        const int nwork = s_nwork;   // fewer than k, so it fits the list
+        for (int w = tid; w < nwork && nwork <= WORK; w += THREADS) {
+          const int c = work[w];
+          float f[EPV];
+          Elem<T>::unpack(load16(rp + sp.head + (int64_t)c * EPV), f);
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) above(f[e], sp.head + c * EPV + e);
+        }
+        __syncthreads();
+        const int got = s_count;
+        __syncthreads();
+        if (nwork <= WORK && got <= CAP) {
+          if (got >= k) {   // the top k are among them
+            rank_and_write(got);
+            return;
+          }
+          // the k-th key is tau_v's: places [got, k) go to the first elements equal to it, in
+          // column order (head edge, vectors, tail edge), found by a scan that stops when it has them
+          const int need = k - got;
+          int base = 0;
+          auto place = [&](float f, int col, int pos) {
+            ccomp[got + pos] = ((unsigned long long)key_of(f) << 32) | (uint32_t)(~col);
+          };
+          {
+            float f0 = 0.f;
+            int mine = 0;
+            if (tid < sp.head) {
+              f0 = Elem<T>::load1(rp + tid);
+              mine = ((key_of(f0) & KMASK) == kth_c) ? 1 : 0;
+            }
+            int tot;
+            const int ex = block_excl_scan(mine, s_int, NW, &tot);
+            if (mine && base + ex < need) place(f0, tid, base + ex);
+            base += tot;
+          }
+          const int niter = (sp.nvec + THREADS - 1) / THREADS;
+          for (int i = 0; i < niter && base < need; ++i) {   // base is uniform
+            const int c = i * THREADS + tid;
+            float f[EPV];
+            int mine = 0;
+            if (c < sp.nvec) {
+              Elem<T>::unpack(load16(rp + sp.head + (int64_t)c * EPV), f);
+#pragma unroll
+              for (int e = 0; e < EPV; ++e) mine += ((key_of(f[e]) & KMASK) == kth_c) ? 1 : 0;
+            }
+            int tot;
+            int pos = base + block_excl_scan(mine, s_int, NW, &tot);
+            if (mine && pos < need) {
+#pragma unroll
+              for (int e = 0; e < EPV; ++e) {
+                if ((key_of(f[e]) & KMASK) == kth_c) {
+                  if (pos < need) place(f[e], sp.head + c * EPV + e, pos);
+                  ++pos;
+                }
+              }
+            }
+            base += tot;
+          }
+          const int ntail = v - sp.tail0;
+          for (int t0 = 0; t0 < ntail && base < need; t0 += THREADS) {
+            const int col = sp.tail0 + t0 + tid;
+            float f0 = 0.f;
+            int mine = 0;
+            if (col < v) {
+              f0 = Elem<T>::load1(rp + col);
+              mine = ((key_of(f0) & KMASK) == kth_c) ? 1 : 0;
+            }
+            int tot;
+            const int ex = block_excl_scan(mine, s_int, NW, &tot);
+            if (mine && base + ex < need) place(f0, col, base + ex);
+            base += tot;
+          }
+          __syncthreads();
+          rank_and_write(k);
+          return;
+        }
+      }
     }
     if (C > CAP) {
       // ---- exact path: k-th key by bitwise search over the whole row. Rows of up to RK vectors
@@ -422,12 +650,83 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
         return block_sum_int(cnt, s_int, NW);
       };
       uint32_t kth = 0u;
-      for (int bit = 31; bit >= KeyBits<T>::low; --bit) {
-        const uint32_t trial = kth | (1u << bit);
-        const int cnt = count_if([&](uint32_t key) { return key >= trial; });
-        if (cnt >= k) kth = trial;
+      int c_gt = 0;
+      if (cached) {
+        for (int bit = 31; bit >= KeyBits<T>::low; --bit) {
+          const uint32_t trial = kth | (1u << bit);
+          const int cnt = count_if([&](uint32_t key) { return key >= trial; });
+          if (cnt >= k) kth = trial;
+        }
+        c_gt = count_if([&](uint32_t key) { return key > kth; });
+      } else {
+        // Rows that do not fit the registers: radix select, eight key bits per sweep of the row
+        // (two sweeps for bf16, three for fp16, four for fp32) instead of one sweep per bit. A
+        // sweep counts, in a 256-bin LDS histogram, the next key byte of the elements whose
+        // higher bytes equal the prefix found so far. Rows come here because of runs of equal
+        // values, so the lanes of a wave mostly hold the same bin: equal bins are found with a
+        // ballot and added once by one lane (a plain LDS atomic per element would serialise the
+        // whole wave on one address). The bin that holds the k-th largest follows from suffix sums.
+        int* hist = crank;
+        uint32_t prefix = 0u, pmask = 0u;
+        int kk = k;   // rank still wanted inside the current prefix
+        for (int shift = 24; shift + 8 > KeyBits<T>::low; shift -= 8) {
+          for (int i = tid; i < 256; i += THREADS) hist[i] = 0;
+          __syncthreads();
+          auto tally = [&](uint32_t key, bool live) {   // called by whole waves
+            const bool ok = live && (key & pmask) == prefix;
+            const uint32_t bin = (key >> shift) & 255u;
+            unsigned long long todo = __ballot(ok);
+            while (todo != 0ull) {
+              const int leader = __builtin_ctzll(todo);
+              const uint32_t b = (uint32_t)__builtin_amdgcn_readlane((int)bin, leader);
+              const unsigned long long same = __ballot(ok && bin == b);
+              if (lane == leader) atomicAdd(&hist[b], (int)__builtin_popcountll(same));
+              todo &= ~same;
+            }
+          };
+          for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * 4) {
+            u32x4 raw[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+              raw[u] = load16(rp + sp.head + (int64_t)clamp_col(c0 + u * THREADS + tid, sp.nvec) * EPV);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              touch(raw[u]);
+              const bool live = c0 + u * THREADS + tid < sp.nvec;
+              float f[EPV];
+              Elem<T>::unpack(raw[u], f);
+#pragma unroll
+              for (int e = 0; e < EPV; ++e) tally(key_of(f[e]) & KMASK, live);
+            }
+          }
+          for (int e0 = 0; e0 < ne; e0 += THREADS) {
+            const int e = e0 + tid;
+            const bool live = e < ne;
+            tally(key_of(Elem<T>::load1(rp + edge_col(sp, live ? e : ne - 1))) & KMASK, live);
+          }
+          __syncthreads();
+          // bins from the top: thread t of a round owns bin 255 - (round + t); the exclusive scan
+          // in thread order is the number of elements in higher bins
+          int carry = 0;
+          for (int round = 0; round < 256; round += THREADS) {
+            const int bin = 255 - (round + tid);
+            const int mine = bin >= 0 ? hist[bin] : 0;
+            int tot;
+            const int above = carry + block_excl_scan(mine, s_int, NW, &tot);
+            if (bin >= 0 && above < kk && kk <= above + mine) { s_tau[0] = (uint32_t)bin; s_count = above; }
+            carry += tot;
+          }
+          __syncthreads();
+          const uint32_t sel = s_tau[0];
+          const int above = s_count;
+          __syncthreads();
+          prefix |= sel << shift;
+          pmask |= 255u << shift;
+          kk -= above;
+        }
+        kth = prefix;
+        c_gt = k - kk;
       }
-      const int c_gt = count_if([&](uint32_t key) { return key > kth; });
       const int need = k - c_gt;  // ties admitted, in ascending index order
       if (tid == 0) s_count = 0;
       __syncthreads();
@@ -507,77 +806,7 @@ __device__ __forceinline__ void topk_finish(const T* __restrict__ rp, const RowS
     }
   }
 
-  // ---- many candidates for the size of the workgroup: a bitonic sort of the slots (key
-  // descending, then column ascending; zero padding sorts last) puts output slot r at position
-  // r for log^2 steps of work, where counting costs one read of every candidate per candidate
-  if (C > kSortFrom && C * C > 256 * THREADS) {
-    int cp = 2 * kSortFrom;
-    while (cp < C) cp <<= 1;
-    for (int s = C + tid; s < cp; s += THREADS) ccomp[s] = 0ull;
-    __syncthreads();
-    for (int size = 2; size <= cp; size <<= 1) {
-      for (int stride = size >> 1; stride > 0; stride >>= 1) {
-        for (int t = tid; t < cp / 2; t += THREADS) {
-          const int lo = 2 * t - (t & (stride - 1));
-          const int hi = lo + stride;
-          const bool desc = (lo & size) == 0;
-          const unsigned long long a = ccomp[lo], b = ccomp[hi];
-          if ((a < b) == desc) { ccomp[lo] = b; ccomp[hi] = a; }
-        }
-        __syncthreads();
-      }
-    }
-    for (int r = tid; r < k; r += THREADS) {
-      const int col = (int)(~(uint32_t)(ccomp[r] & 0xFFFFFFFFull));
-      const int64_t o = row * (int64_t)k + r;
-      if (idx32 != nullptr) idx32[o] = col;
-      if (idx64 != nullptr) idx64[o] = col;
-      if (values != nullptr) values[o] = rp[col];
-      if (probs != nullptr) probs[o] = fast_exp2(Elem<T>::load1(rp + col) * c1 - lse2);
-    }
-    return;
-  }
-
-  // ---- rank the C candidates by counting; rank r < k goes to output slot r
-  int cpad = 64;
-  while (cpad < C) cpad <<= 1;
-  const int parts = THREADS / cpad > 1 ? THREADS / cpad : 1;
-  for (int jx = tid; jx < C; jx += THREADS) crank[jx] = 0;
-  __syncthreads();
-  const int per = (C + parts - 1) / parts;
-  for (int wk = tid; wk < cpad * parts; wk += THREADS) {
-    const int jx = wk % cpad, part = wk / cpad;
-    if (jx < C) {
-      const unsigned long long me = ccomp[jx];
-      const int i0 = part * per;
-      const int i1 = i0 + per < C ? i0 + per : C;
-      // every lane reads the same candidate (an LDS broadcast); eight reads in flight hide
-      // the LDS latency that a one-at-a-time loop would pay per candidate
-      int r = 0;
-      int i = i0;
-      for (; i + 8 <= i1; i += 8) {
-        unsigned long long o[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) o[u] = ccomp[i + u];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) r += o[u] > me ? 1 : 0;
-      }
-      for (; i < i1; ++i) r += ccomp[i] > me ? 1 : 0;
-      if (parts == 1) crank[jx] = r; else atomicAdd(&crank[jx], r);
-    }
-  }
-  __syncthreads();
-  for (int jx = tid; jx < C; jx += THREADS) {
-    const int r = crank[jx];
-    if (r < k) {
-      const int col = (int)(~(uint32_t)(ccomp[jx] & 0xFFFFFFFFull));
-      const int64_t o = row * (int64_t)k + r;
-      if (idx32 != nullptr) idx32[o] = col;
-      if (idx64 != nullptr) idx64[o] = col;
-      if (values != nullptr) values[o] = rp[col];
-      if (probs != nullptr) probs[o] = fast_exp2(Elem<T>::load1(rp + col) * c1 - lse2);
-    }
-  }
+  rank_and_write(C);
 }
 
 }  // namespace fm

@@ -174,3 +174,44 @@ def test_config5_kl_and_topk_4096x128256():
     assert torch.allclose(rows_f, rows, rtol=2e-4, atol=1e-7) and torch.allclose(lt_f, lt, rtol=1e-6, atol=2e-6)
     want = torch.exp(vals.double() / T - lt.double()[:, None])
     assert torch.allclose(probs_f.double(), want, rtol=1e-5, atol=1e-12)
+
+
+def test_topk_rows_of_long_equal_runs_at_config5_width():
+    # [4096, 128256] bf16 whose rows hold 2 (then 50) distinct values: tens of thousands of ties at the
+    # k-th place, so no candidate list can hold them and the kernels select by radix counting. The
+    # answer has a closed form: the columns of the largest value(s) in ascending order.
+    n, v, k = 4096, 128256, 64
+    g = gen(1055)
+    for distinct in (2, 50):
+        vals = (3 * torch.randn(n, distinct, generator=g)).to(BF16)
+        pick = torch.randint(0, distinct, (n, v), generator=g)
+        x = torch.gather(vals, 1, pick)
+        xd = x.to(DEV)
+        tv, ti = _hip.topk(xd, k, torch.int32)
+        sample = torch.arange(0, n, 257)
+        assert torch.equal(ti[sample.to(DEV)].cpu().long(), O.topk(x[sample], k)[1]), distinct
+        ii = ti.long()
+        assert torch.equal(torch.gather(xd, 1, ii), tv)
+        vf = tv.float()
+        assert (vf[:, :-1] >= vf[:, 1:]).all()
+        tie = vf[:, :-1] == vf[:, 1:]
+        assert (ii[:, :-1][tie] < ii[:, 1:][tie]).all()
+        kth = vf[:, -1:]
+        for lo in range(0, n, 512):
+            xf = xd[lo:lo + 512].float()
+            k_lo = kth[lo:lo + 512]
+            assert torch.equal((xf > k_lo).sum(-1), (vf[lo:lo + 512] > k_lo).sum(-1))
+            chosen = torch.zeros_like(xf, dtype=torch.bool).scatter_(1, ii[lo:lo + 512], True)
+            left = (xf == k_lo) & ~chosen
+            pos = torch.arange(v, device=DEV).expand_as(xf)
+            first_left = torch.where(left, pos, torch.full_like(pos, v)).min(-1).values
+            last_taken = torch.where(chosen & (xf == k_lo), pos, torch.full_like(pos, -1)).max(-1).values
+            assert (last_taken < first_left).all()
+        # the fused KL forward selects the same columns from the same teacher
+        out = _hip.kl_fwd_topk(xd, xd, k, 1.0, "mean", torch.int32, want_values=False, want_probs=False)
+        assert torch.equal(out[5], ti)
+        del xd, tv, ti, ii, vf
+    # fp32 rows take four sweeps of eight bits
+    xf32 = torch.gather((3 * torch.randn(512, 3, generator=g)), 1, torch.randint(0, 3, (512, 40000), generator=g))
+    ti = _hip.topk(xf32.to(DEV), 100, torch.int32)[1]
+    assert torch.equal(ti.cpu().long(), O.topk(xf32, 100)[1])
