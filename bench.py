@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extras] [--no-cpu]
 
 NAME: ce (headline), ce_one_pass, rmsnorm, add_rmsnorm, add_layernorm, kl, kl_one_launch, kl_topk, kl_topk_one_launch, topk,
-route, route_train, moe_dispatch, swiglu, qk_norm_rope.
+route, route_256x8, route_train, moe_dispatch, swiglu, qk_norm_rope.
 
 A step is one pass of the hot path (forward + backward) over one batch of synthetic,
 seeded input that is already resident in HBM, launched straight through the C ABI of
@@ -95,7 +95,7 @@ def measured_traffic(kernel):
 
 
 WORKLOADS = ["ce", "ce_one_pass", "rmsnorm", "add_rmsnorm", "add_layernorm", "kl", "kl_one_launch", "kl_topk",
-             "kl_topk_one_launch", "topk", "route", "route_train", "moe_dispatch", "swiglu", "qk_norm_rope"]
+             "kl_topk_one_launch", "topk", "route", "route_256x8", "route_train", "moe_dispatch", "swiglu", "qk_norm_rope"]
 
 
 def parse():
@@ -659,10 +659,12 @@ def make_workload(name, torch, L, dev):
         w.rows = b * t * hh
         return w
 
-    if name == "route":
-        n, e, k = 16384, 64, 2
-        g.manual_seed(1003)
-        sets = 80    # 80 x 4 MiB of logits: a step's input is never in the 256 MB memory-side cache
+    if name in ("route", "route_256x8"):
+        big = name == "route_256x8"     # the common MoE shape of today: 256 experts, eight picks, with statistics
+        n, e, k = (65536, 256, 8) if big else (16384, 64, 2)
+        g.manual_seed(1013 if big else 1003)
+        # 80 x 4 MiB (8 x 64 MiB) of logits: a step's input is never in the 256 MB memory-side cache
+        sets = 8 if big else 80
         lgs = []
         for i in range(sets):
             lg = torch.round(torch.randn(n, e, generator=g) * 4096) / 4096
@@ -681,11 +683,13 @@ def make_workload(name, torch, L, dev):
         od = torch.empty(n * k, device=dev, dtype=torch.int32)
         nb = L.fm_route_workspace(n, e, k)
         ws = torch.empty(max(nb, 16), device=dev, dtype=torch.uint8)
+        stats = torch.empty(e + 3, device=dev) if big else None
         state = {"i": 0}
 
         def run(i):
             _check(L.fm_route(lgs[i].data_ptr(), idx.data_ptr(), wt.data_ptr(), cnt.data_ptr(), sl.data_ptr(),
-                              od.data_ptr(), None, ws.data_ptr(), nb, n, e, k, F32c, st), "fm_route")
+                              od.data_ptr(), None if stats is None else stats.data_ptr(), ws.data_ptr(), nb, n, e, k,
+                              F32c, st), "fm_route")
 
         def step():
             i = state["i"] = (state["i"] + 1) % sets
@@ -720,8 +724,8 @@ def make_workload(name, torch, L, dev):
         w.dominant_launch = step
         w.dominant = "route_group_kernel + permute_kernel"
         w.dominant_bytes = w.bytes = n * (e * 4 + k * 4 * 4)
-        w.desc = (f"router softmax + top-{k} + counts + stable permutation, logits fp32 [{n},{e}], 1% tie rows "
-                  f"(rotating {sets} logit sets: cold)")
+        w.desc = (f"router softmax + top-{k} + counts + stable permutation" + (" + statistics and auxiliary losses" if big else "")
+                  + f", logits fp32 [{n},{e}], 1% tie rows (rotating {sets} logit sets: cold)")
         w.unit = "rows/s"
         w.rows = n
         w.sets = sets
@@ -947,6 +951,7 @@ def measure(torch, w, steps, warmup, L, cpu=True):
         "dominant_ms_median": round(med, 5),
         "dominant_gbps": round(w.dominant_bytes / avg / 1e6, 1),
         "dominant_traffic_bytes": measured_traffic(kernel),
+        "unit": w.unit,
     }
     if hasattr(w, "required_bytes"):
         # bytes the dataflow must move (rows with an ignored label are never read), next to the
@@ -1173,6 +1178,8 @@ def config_row(r, rows_unit):
 
 def short_row(r):
     row = {"ms": r["ms_per_step"], "gbps": r["gbps"], "frac": r["frac_of_hbm_peak"], "checked": r["checked"]}
+    if r.get("unit") == "rows/s":
+        row["rows_per_s"] = r["rows_per_s"]
     if "l2_boundary_frac_of_hbm_peak" in r:
         row["frac_l2_boundary"] = r["l2_boundary_frac_of_hbm_peak"]
     if "floor_ms" in r and r["floor_ms"] is not None:
@@ -1228,7 +1235,7 @@ def main():
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": res["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16" if a.workload not in ("route", "route_train") else "f32", "data": "synthetic",
+        "dtype": "bf16" if a.workload not in ("route", "route_256x8", "route_train") else "f32", "data": "synthetic",
         "config": {"workload": head.desc, "name": a.workload,
                    "timing": "K steps between two device synchronisations, inputs resident in HBM",
                    "inputs": "torch.Generator(cpu).manual_seed(1000 + config number), drawn in row chunks"},

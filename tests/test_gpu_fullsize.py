@@ -215,3 +215,33 @@ def test_topk_rows_of_long_equal_runs_at_config5_width():
     xf32 = torch.gather((3 * torch.randn(512, 3, generator=g)), 1, torch.randint(0, 3, (512, 40000), generator=g))
     ti = _hip.topk(xf32.to(DEV), 100, torch.int32)[1]
     assert torch.equal(ti.cpu().long(), O.topk(xf32, 100)[1])
+
+
+def test_router_65536x256_top8_with_statistics():
+    # the common shape of current MoE layers (128-256 experts, six to eight picks): indices, counts and the
+    # permutation bit for bit, weights and statistics to fp32 rounding, on every row
+    n, e, k = 65536, 256, 8
+    g = gen(1013)
+    lg = torch.round(torch.randn(n, e, generator=g) * 4096) / 4096
+    rows = torch.randperm(n, generator=g)[: n // 100]
+    for r in rows.tolist():
+        cols = torch.randperm(e, generator=g)[:12]
+        lg[r, cols[:6]] = lg[r].max().clone()          # six equal maxima: picks 1-6 tie, lowest expert first
+        lg[r, cols[6:]] = lg[r, cols[11]].clone()      # and a second run of equal values further down
+    oi, ow, oc, oslot, oorder = O.router(lg, k)
+    idx, w, counts, slot, order, stats = _hip.route(lg.to(DEV), k, want_stats=True)
+    assert torch.equal(idx.cpu().long(), oi) and torch.equal(counts.cpu().long(), oc)
+    assert torch.equal(slot.cpu().long(), oslot) and torch.equal(order.cpu().long(), oorder)
+    assert torch.allclose(w.cpu(), ow, rtol=1e-5, atol=0)
+    assert torch.equal(slot.long()[order.long()], torch.arange(n * k, device=DEV))
+    aux, z = O.router_aux(lg, oi)
+    probs = torch.softmax(lg.double(), -1)
+    assert torch.allclose(stats[:e].double().cpu(), probs.sum(0), rtol=1e-5)
+    assert stats[e + 1].item() == pytest.approx(aux.item(), rel=1e-5)
+    assert stats[e + 2].item() == pytest.approx(z.item(), rel=1e-5)
+    # six picks of 128 experts take the same kernels with sixteen lanes a row
+    lg2 = lg[:, :128].contiguous()
+    oi2, _, oc2, _, oorder2 = O.router(lg2, 6)
+    idx2, _, counts2, _, order2 = _hip.route(lg2.to(DEV), 6)
+    assert torch.equal(idx2.cpu().long(), oi2) and torch.equal(counts2.cpu().long(), oc2)
+    assert torch.equal(order2.cpu().long(), oorder2)

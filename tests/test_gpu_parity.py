@@ -1137,3 +1137,34 @@ def test_qk_norm_rope_fwd_bwd(b, t, h, hd, dt, wdt):
     assert_close_lowp(out, ref.detach(), dt, "qk_norm_rope", ulps=3.0, cancel=scale)
     assert_close_lowp(dx, xr.grad, dt, "dx", ulps=4.0, cancel=float(xr.grad.abs().max()) * 4)
     assert rel_max(dw, wr.grad) <= (1e-2 if wdt != F32 else 1e-4)
+
+
+def test_router_where_probabilities_leave_the_normal_range():
+    """A pick whose probability is below 2^-126 (its logit more than 87.3 under the row maximum):
+    the hardware exponential flushes it to zero, so such picks tie and go to the lowest expert
+    index, where a CPU softmax still tells denormals apart (and rounds them to a grid of 1.4e-45,
+    so its own order there is an artefact of the rounding as well). Pinned here: rows whose k-th
+    largest logit is within 86 of the maximum match the oracle bit for bit; beyond 88 the picks
+    follow the flush-to-zero model exactly (the deviation is confined to that window and to the
+    places after the last normal probability)."""
+    g = torch.Generator().manual_seed(5150)
+    n, e, k = 512, 64, 4
+    for gap, exact in ((60.0, True), (80.0, True), (86.0, True), (88.0, False), (95.0, False), (120.0, False)):
+        lg = -torch.round(torch.rand(n, e, generator=g) * 256) / 256   # the field: (-1, 0] on a 1/256 grid
+        top2 = torch.stack([torch.randperm(e, generator=g)[:2] for _ in range(n)])
+        lg.scatter_(1, top2, torch.tensor([gap, gap - 0.5]).expand(n, 2).contiguous())   # picks 3, 4 sit gap .. gap + 1 below the maximum
+        idx, w, counts, slot, order = _hip.route(lg.to(DEV), k)
+        oi, ow, oc, oslot, oorder = O.router(lg, k)
+        if exact:
+            assert torch.equal(idx.cpu().long(), oi), gap
+            assert torch.allclose(w.cpu(), ow, rtol=1e-5, atol=1e-37)
+        else:
+            # flush-to-zero model: probabilities below 2^-126 are zero, ties to the lowest index
+            p = torch.softmax(lg.double(), -1)
+            p = torch.where(p < 2.0 ** -126, torch.zeros_like(p), p).float()
+            mi = O.topk(p, k)[1]
+            assert torch.equal(idx.cpu().long(), mi), gap
+            assert torch.equal(idx.cpu().long()[:, :2], oi[:, :2])          # the normal picks agree with the oracle
+        flat = idx.reshape(-1).long().cpu()
+        assert torch.equal(counts.cpu().long(), torch.bincount(flat, minlength=e))
+        assert torch.equal(order.cpu().long(), torch.from_numpy(np.argsort(flat.numpy(), kind="stable")))
