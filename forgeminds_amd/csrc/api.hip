@@ -17,20 +17,9 @@ thread_local char g_kernel_text[384] = "";
 std::atomic<int> g_params[fm_host::P_COUNT];
 const char* const kParamNames[fm_host::P_COUNT] = {
     "norm_bwd_blocks_per_cu",
-    "vocab_threads",
-    "norm_tpr",
-    "topk_variant",
-    "vocab_unroll",
     "norm_fwd_blocks_per_cu",
-    "ce_rows_max_v",
-    "norm_wide_min_vec",
-    "rows_vec_max",
-    "rope_heads",
-    "route_presort",
-    "norm_wide_acc",
-    "colsum16",
-    "route_stats_late",
-    "rope_pair",
+    "vocab_threads",
+    "vocab_unroll",
 };
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cus[kMaxDevices];

@@ -615,16 +615,14 @@ __global__ __launch_bounds__(256) void ce_vrows_kernel(const T* logits, const in
   }
 }
 
-// Widest row, in 16-byte vectors, of the vector lane-group kernel (tunable downwards with
-// "rows_vec_max"; the forward alone takes twice the width of the forms that write a gradient).
+// Widest row, in 16-byte vectors, of the vector lane-group kernel (the forward alone takes twice
+// the width of the forms that write a gradient).
 constexpr int kVRowsMaxVec = 512;
 
 bool vrows_fits(int v, int esize, bool bf16, const void* logits, const void* dlogits, bool loss, bool grad) {
   const int epv = 16 / esize;
-  int lim = fm_host::get_param(fm_host::P_ROWS_VEC_MAX);
   // eight vectors per lane only pay for bf16 (the other types then run at a quarter of the occupancy)
-  const int top = loss && !grad ? kVRowsMaxVec : kVRowsMaxVec / 2;
-  if (lim <= 0 || lim > top) lim = top;
+  const int lim = loss && !grad ? kVRowsMaxVec : kVRowsMaxVec / 2;
   return v % epv == 0 && v / epv <= lim && fm_host::aligned16(logits) && (!grad || fm_host::aligned16(dlogits));
 }
 
@@ -656,11 +654,8 @@ bool launch_vrows(const void* logits, const int64_t* labels, const float* n_vali
 }
 
 // rows of up to 1024 logits go to ce_rows_kernel; returns false for wider rows
-// Widest row the lane-group kernel takes (tunable downwards with "ce_rows_max_v").
-inline int rows_max_v() {
-  const int p = fm_host::get_param(fm_host::P_CE_ROWS_MAX_V);
-  return p > 0 && p < 64 * 16 ? p : 64 * 16;
-}
+// Widest row the lane-group kernel takes.
+inline int rows_max_v() { return 64 * 16; }
 
 template <typename T, bool LOSS, bool GRAD>
 bool launch_rows(const void* logits, const int64_t* labels, const float* n_valid, const float* grad_out,

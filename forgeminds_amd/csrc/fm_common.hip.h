@@ -302,10 +302,9 @@ namespace fm_host {
 void set_error(const char* fmt, ...);
 int get_param(int which);
 
-enum Param { P_NORM_BWD_BLOCKS_PER_CU = 0, P_VOCAB_THREADS, P_NORM_TPR, P_TOPK_VARIANT, P_VOCAB_UNROLL,
-             P_NORM_FWD_BLOCKS_PER_CU, P_CE_ROWS_MAX_V, P_NORM_WIDE_MIN_VEC, P_ROWS_VEC_MAX,
-             P_ROPE_HEADS, P_ROUTE_PRESORT, P_NORM_WIDE_ACC, P_COLSUM16,
-             P_ROUTE_STATS_LATE, P_ROPE_PAIR, P_COUNT };
+// Launch-shape parameters a caller may move for another part or shape (fm_set_param); none of
+// them selects between code paths, the results do not depend on them.
+enum Param { P_NORM_BWD_BLOCKS_PER_CU = 0, P_NORM_FWD_BLOCKS_PER_CU, P_VOCAB_THREADS, P_VOCAB_UNROLL, P_COUNT };
 
 int num_cus();  // compute units of the current device (cached per device)
 

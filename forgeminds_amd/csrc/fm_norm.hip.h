@@ -909,9 +909,8 @@ Plan make_plan(int64_t n, int64_t d, int x_dtype, bool aligned) {
   Plan p{};
   const int epv = 16 / elem_size(x_dtype);
   const int64_t nvec = d / epv;
-  // rows of more than `reg_max` vectors are streamed (tunable downwards with "norm_wide_min_vec")
-  int64_t reg_max = fm_host::get_param(fm_host::P_NORM_WIDE_MIN_VEC);
-  if (reg_max <= 0 || reg_max > 4096) reg_max = 4096;
+  // rows of more than `reg_max` vectors are streamed
+  const int64_t reg_max = 4096;
   p.vec = aligned && (d % epv == 0) && nvec <= reg_max;
   p.wide = aligned && (d % epv == 0) && nvec > reg_max;
   // the backward of half types keeps x, dy and two fp32 column sets per thread: past 2048
@@ -931,10 +930,6 @@ Plan make_plan(int64_t n, int64_t d, int x_dtype, bool aligned) {
       for (auto& pr : kPairs) {
         if (nvec <= pr[0]) { p.tpr = pr[1]; p.iters = pr[2]; break; }
       }
-      // experiment hook: trade threads per row against vectors per thread
-      const int want = fm_host::get_param(fm_host::P_NORM_TPR);
-      if (want == 256 && nvec > 768 && nvec <= 1024) { p.tpr = 256; p.iters = 4; }
-      if (want == 128 && nvec > 64 && nvec <= 128) { p.tpr = 128; p.iters = 1; }
     }
     const int block = p.tpr > kMinBlock ? p.tpr : kMinBlock;
     p.rpb = block / p.tpr;
@@ -959,8 +954,8 @@ Plan make_plan(int64_t n, int64_t d, int x_dtype, bool aligned) {
 }
 
 #define FM_FOR_EACH_SHAPE(X) \
-  X(4, 1) X(8, 1) X(16, 1) X(32, 1) X(64, 1) X(128, 1) X(64, 2) X(64, 3) X(128, 2) X(128, 3)    \
-  X(256, 2) X(256, 3) X(256, 4) X(512, 2) X(512, 3) X(1024, 2) X(1024, 3) X(1024, 4)
+  X(4, 1) X(8, 1) X(16, 1) X(32, 1) X(64, 1) X(64, 2) X(64, 3) X(128, 2) X(128, 3)    \
+  X(256, 2) X(256, 3) X(512, 2) X(512, 3) X(1024, 2) X(1024, 3) X(1024, 4)
 
 // Persistent grid of the forward: every workgroup slot of the device exactly once, so the
 // hardware places the same number of workgroups on every compute unit.
@@ -1028,7 +1023,7 @@ int launch_bwd(const Plan& p, const void* x, const void* w, const float* mean, c
   const int pcols = (int)(LN ? 2 * d : d);
   const int wide_iters = (int)((d / Elem<T>::kVec + kWideThreads - 1) / kWideThreads);
   const bool acc_fits = wide_iters * Elem<T>::kVec <= 32 && !(LN && sizeof(T) == 4 && wide_iters > 6);
-  if (p.bwd_wide && acc_fits && fm_host::get_param(fm_host::P_NORM_WIDE_ACC) != 1) {
+  if (p.bwd_wide && acc_fits) {
     // the column sums fit the registers: one persistent kernel, a chunk of rows per workgroup
     const dim3 grid((unsigned)p.bwd_blocks);
 #define GOA(IT_)                                                                                  \
@@ -1079,9 +1074,9 @@ int launch_bwd(const Plan& p, const void* x, const void* w, const float* mean, c
     for (int which = 0; which < (LN ? 2 : 1); ++which) {
       if (outs[which] == nullptr) continue;
       const float* src = partial + (int64_t)which * d;
-      int lim16 = fm_host::get_param(fm_host::P_COLSUM16);   // widest weight the 16-column form takes (1: never)
-      if (lim16 <= 0) lim16 = 4096;
-      if (d % 4 == 0 && d <= lim16)
+      // narrow weights: 16 columns a workgroup, so that a column sum of few columns still spreads
+      // over the device (no difference from 8192 columns on)
+      if (d % 4 == 0 && d <= 4096)
         hipLaunchKernelGGL((colsum16_kernel<WT>), dim3((unsigned)((d + 15) / 16)), dim3(1024), 0, st, src,
                            static_cast<WT*>(outs[which]), p.bwd_blocks, (int)d, pcols);
       else if (d % 4 == 0)

@@ -764,9 +764,7 @@ bool launch_vrows(const void* student, const void* teacher, float* lse_s, float*
                   const float* grad_out, int grad_per_row, void* dstudent, int64_t n, int v, float inv_temp,
                   float mul, hipStream_t st) {
   constexpr int EPV = Elem<T>::kVec;
-  int lim = fm_host::get_param(fm_host::P_ROWS_VEC_MAX);
-  if (lim <= 0 || lim > kVRowsMaxVec) lim = kVRowsMaxVec;
-  if (v % EPV != 0 || v / EPV > lim || !fm_host::aligned16(student) || !fm_host::aligned16(teacher) ||
+  if (v % EPV != 0 || v / EPV > kVRowsMaxVec || !fm_host::aligned16(student) || !fm_host::aligned16(teacher) ||
       (GRAD && !fm_host::aligned16(dstudent)))
     return false;
   // two vectors of each row a lane where the rows have them: a wave then keeps 4 KiB in

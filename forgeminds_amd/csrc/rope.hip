@@ -439,14 +439,11 @@ int launch(const Shape& sh, bool vec, const void* x, const void* w, const float*
   // slower again: fewer waves fit), 1 when the head count is odd
   int hpg = 1;
   // heads of exactly four or eight vectors: one vector per lane, partner by lane permute
-  const bool pair = vec && (sh.gv == 2 || sh.gv == 4) && (int64_t)sh.gv * 2 * Elem<T>::kVec == d &&
-                    fm_host::get_param(fm_host::P_ROPE_PAIR) != 1;
+  const bool pair = vec && (sh.gv == 2 || sh.gv == 4) && (int64_t)sh.gv * 2 * Elem<T>::kVec == d;
   if (vec) {
     // the one-vector-per-lane kernel: eight-lane groups take four heads forward and two backward;
     // four-lane groups one (with more, a wave's load instruction skips between 64-byte heads)
-    const int dflt = !pair ? 2 : (sh.gv == 2 ? 1 : (BWD ? 2 : 4));
-    const int want = fm_host::get_param(fm_host::P_ROPE_HEADS) > 0 ? fm_host::get_param(fm_host::P_ROPE_HEADS)
-                                                                   : dflt;
+    const int want = !pair ? 2 : (sh.gv == 2 ? 1 : (BWD ? 2 : 4));
     if (want >= 4 && (!BWD || pair) && heads % 4 == 0) hpg = 4;
     else if (want >= 2 && heads % 2 == 0) hpg = 2;
   }

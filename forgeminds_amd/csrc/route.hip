@@ -723,8 +723,7 @@ int launch_route(const void* logits, int32_t* idx, float* weights, int32_t* hist
                    lp, idx, weights, hist, fstat, n, e, k, tl.tile_rows);                            \
   } while (0)
   const bool vec = e % kGE == 0 && fm_host::aligned16(logits);
-  int ps = fm_host::get_param(fm_host::P_ROUTE_PRESORT);   // 0: by k, 1: never, 2: always
-  const bool presort = ps == 2 || (ps == 0 && k >= 5);
+  const bool presort = k >= 5;   // at four picks the two forms tie, below that the sort does not pay
   if (e <= 64) GOG(8);
   else if (e <= 128) GOG(16);
   else if (e <= 256) GOG(32);
@@ -776,8 +775,7 @@ int fm_route(const void* logits, int32_t* idx, float* weights, int32_t* counts, 
   else launch_route<f16_t>(logits, idx, weights, hist, fstat, n, e, k, tl, st);
   FM_CHECK_LAUNCH("fm_route");
   // few columns and tiles: the statistics are folded by the kernel that also finishes the losses
-  const bool stats_late = stats != nullptr && e + 1 <= 128 && tl.ntiles <= 256 &&
-                          fm_host::get_param(fm_host::P_ROUTE_STATS_LATE) != 1;
+  const bool stats_late = stats != nullptr && e + 1 <= 128 && tl.ntiles <= 256;
   if (stats != nullptr && !stats_late) {
     hipLaunchKernelGGL(route_stats_kernel, dim3((unsigned)((e + 1 + 63) / 64)), dim3(1024), 0, st, fstat, stats,
                        e, tl.ntiles);

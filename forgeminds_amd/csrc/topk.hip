@@ -501,10 +501,8 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
   FM_LAUNCH((topk_lds_kernel<T, TH, UN, BIG_>), grid, dim3(TH), (size_t)(nvec + 8) * 2, st, xp, vp, \
                      i32, i64, v, k, vec_ok)
   const bool big = k > 256;               // twice the candidate slots (1024-thread forms only)
-  int variant = fm_host::get_param(fm_host::P_TOPK_VARIANT);
-  const bool forced = variant != 0;       // a forced variant also bypasses the wave-per-row kernel
-  if (variant == 0) variant = nvec <= 3072 ? 1 : (nvec <= 12288 ? 2 : 3);
-  if (!forced) {
+  int variant = nvec <= 3072 ? 1 : (nvec <= 12288 ? 2 : 3);
+  {
     // The threshold search needs k <= 63 x (full waves of the row); more threads give more of
     // them while the row has a vector for each, and it pays while k stays within half of that
     // bound (past it the candidates mostly overflow anyway). Otherwise the exact path runs for
@@ -533,7 +531,7 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
   // narrow rows, few picks: lane groups. A pick costs a lane group as much as it costs the
   // wave-per-row kernel, which pays it once per candidate set instead: past 256 columns that is
   // cheaper from the third pick on.
-  if (v <= kGroupMaxV && k <= (v <= 256 ? kGroupMaxK : 2) && !forced) {
+  if (v <= kGroupMaxV && k <= (v <= 256 ? kGroupMaxK : 2)) {
     const bool gvec = vec_ok && v % 8 == 0;
 #define GOG(L_)                                                                                    \
   do {                                                                                             \
@@ -548,7 +546,7 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
     else GOG(64);
 #undef GOG
   }
-  else if (v <= kWaveMaxV && !forced) {       // short rows: a wave per row
+  else if (v <= kWaveMaxV) {       // short rows: a wave per row
     int epl = 1;
     while (64 * epl < v) epl *= 2;
     const bool wvec = vec_ok && v % EPV == 0 && epl >= EPV;

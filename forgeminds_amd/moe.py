@@ -115,6 +115,8 @@ class Experts(nn.Module):
         elif torch.is_tensor(counts):
             counts = counts.tolist()
         sizes = [int(c) for c in counts]
+        if sum(sizes) != x.size(0):    # the reference's x.split(sizes) raises here (moe.py:160)
+            raise RuntimeError(f"Experts.forward: group sizes sum to {sum(sizes)}, but x has {x.size(0)} rows")
         if not any(sizes):
             return x.new_zeros((0,) + tuple(x.shape[1:]))
         dt = x.dtype
@@ -155,6 +157,19 @@ class MoE(nn.Module):
             self.shared = SwiGLU(dim, hidden * int(n_shared))
         self.top_k, self.aux_coef, self.z_coef = int(top_k), aux_coef, z_coef
         self.last_aux = None
+
+    @property
+    def compile_friendly(self) -> bool:
+        """Reference ``moe.py:199-201``: true only with working grouped GEMM experts; here the
+        experts always run the per-expert loop (``Experts.grouped`` stays False)."""
+        return self.ep_size == 1 and self.experts.grouped
+
+    def probe_grouped(self, device, dtype) -> bool:
+        """Reference ``moe.py:203-225`` checks ``torch._grouped_mm`` once before compilation; the
+        grouped GEMM is outside this build, so the answer is always no (callers such as the
+        reference's ``models/gpt.py:261`` then keep the loop)."""
+        self.experts.grouped = False
+        return False
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         shape = x.shape

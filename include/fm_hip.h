@@ -53,8 +53,13 @@ const char* fm_last_error(void);
  * a figure can never be attached to a kernel that did not run. Not part of the reference surface. */
 const char* fm_last_kernel(void);
 
-/* Tuning hook used by the benchmark sweeps; unknown names return FM_ERR_INVALID.
- * value <= 0 restores the built-in heuristic. Not part of the reference surface. */
+/* Launch-shape parameters for another part or shape: "norm_fwd_blocks_per_cu" and
+ * "norm_bwd_blocks_per_cu" (workgroups of the persistent norm grids per compute unit; the second
+ * also sizes the backward's workspace, so ask fm_*_bwd_workspace again after changing it),
+ * "vocab_threads" (256 / 512 / 1024) and "vocab_unroll" (2 / 4 / 8) for the kernels that give a
+ * workgroup a whole vocabulary row. None selects between code paths and no result depends on
+ * them. Process-wide. value <= 0 restores the built-in choice; unknown names return
+ * FM_ERR_INVALID. Not part of the reference surface. */
 int fm_set_param(const char* name, int value);
 
 /* STREAM-style probe with the kernels' own access pattern (16-byte non-temporal accesses, one
@@ -106,8 +111,11 @@ int fm_rmsnorm_bwd(const void* x, const void* w, const float* rstd, const void* 
  * into the library (one copy per GPU, held until the process ends) instead of a workspace
  * argument. No counterpart in the reference. Allocates nothing; the first call on a device
  * looks the buffer's address up once (make that call before starting a capture). Shapes whose
- * partial rows need more than the buffer (fm_rmsnorm_bwd_workspace(n, d, x_dtype) >
- * FM_RMSNORM_BWD_STATIC_BYTES; every shape with d <= 8192 fits) return FM_ERR_UNSUPPORTED. All calls on one
+ * partial rows need more than the buffer return FM_ERR_UNSUPPORTED: the condition is
+ * fm_rmsnorm_bwd_workspace(n, d, x_dtype) <= FM_RMSNORM_BWD_STATIC_BYTES, i.e. (partial rows) x d
+ * x 4 bytes with one partial row per workgroup of the persistent grid -- compute units x
+ * "norm_bwd_blocks_per_cu" (1 unless changed with fm_set_param). On a 256-unit part with the
+ * default that is every d <= 8192; with two workgroups per unit, d <= 4096. All calls on one
  * GPU share the buffer: calls that overlap in time on one GPU (two streams) race; calls on one
  * stream, or on different GPUs, do not. */
 #define FM_RMSNORM_BWD_STATIC_BYTES ((size_t)8 << 20)

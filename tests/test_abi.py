@@ -48,6 +48,7 @@ def test_version_and_error_channel(lib):
     assert lib.fm_set_param(b"no_such_knob", 1) == 1
     assert b"unknown parameter" in lib.fm_last_error()
     assert lib.fm_set_param(b"vocab_threads", 0) == 0
+    assert lib.fm_set_param(b"route_presort", 1) == 1      # switches between code paths are not parameters
 
 
 def test_argument_validation_happens_before_any_launch(lib):

@@ -325,8 +325,8 @@ def test_ce_loss_and_gradient_in_one_pass(n, v, dt, reduction):
 
 def test_ce_kl_vector_rows_agree_with_the_scalar_form():
     """Narrow rows of whole aligned vectors take 16-byte loads; the same rows one element per
-    load (the form for other widths and alignments, forced here through the tuning knob) must
-    give the same answers, special values included."""
+    load (the form for other widths and alignments, reached here by buffers that start one element
+    off a 16-byte line) must give the same answers, special values included."""
     g = gen(1040)
     for dt, v in ((BF16, 512), (F16, 1024), (F32, 256), (BF16, 2048)):
         n = 37
@@ -340,10 +340,14 @@ def test_ce_kl_vector_rows_agree_with_the_scalar_form():
         y[4] = v + 5                       # out of range: the loss of that row is NaN, as in torch
         y[1] = 7
         t = (lg.float() + 0.5 * torch.randn(n, v, generator=g)).to(dt)
-        lgd, yd, td = lg.to(DEV), y.to(DEV), t.to(DEV)
+        yd = y.to(DEV)
         res = []
-        for limit in (0, 1):
-            _hip.set_param("rows_vec_max", limit)
+        for shift in (0, 1):
+            def place(x):       # the tensor, or a copy of it that starts `shift` elements into an allocation
+                buf = torch.empty(x.numel() + shift, device=DEV, dtype=x.dtype)
+                buf[shift:] = x.reshape(-1).to(DEV)
+                return buf[shift:].view(x.shape)
+            lgd, td = place(lg), place(t)
             loss, lse, nv, rows = _hip.ce_fwd(lgd, yd, -100, "sum")
             dl = _hip.ce_bwd(lgd, yd, lse, nv, None, -100)
             l1, d1, _, r1 = _hip.ce_loss_grad(lgd, yd, -100, "mean")
@@ -351,7 +355,6 @@ def test_ce_kl_vector_rows_agree_with_the_scalar_form():
             kg = _hip.kl_bwd(lgd, td, ls, lt, None, False, dt, 0.5, 1.0)
             torch.cuda.synchronize()
             res.append([x.float().cpu() for x in (lse, rows, dl, d1, r1, krows, ls, lt, kg)])
-        _hip.set_param("rows_vec_max", 0)
         names = ("lse", "rows", "dl", "d1", "r1", "krows", "ls", "lt", "kg")
         for name, a, b in zip(names, *res):
             assert torch.equal(a.isnan(), b.isnan()), (dt, v, name)
@@ -984,13 +987,12 @@ def test_route_half_precision_logits_and_all_equal_rows():
     assert order.cpu().tolist() == list(range(0, 260, 2)) + list(range(1, 260, 2))
 
 
-def test_route_pick_forms_agree():
-    """The router picks either by scanning a lane's eight keys per pick or from lane-sorted keys
-    (the default from five picks on): forced either way, every output keeps its bits (NaN payloads
-    aside), on rows of
-    equal logits, rows with a single finite logit (the other picks tie at probability zero),
-    few distinct values, and NaN / +inf rows (all probabilities NaN: lowest experts win)."""
-    try:
+def test_route_pick_forms_on_special_rows():
+    """The router picks either by scanning a lane's eight keys per pick (up to four picks) or from
+    lane-sorted keys (from five picks on): both against the oracle on rows of equal logits, rows
+    with a single finite logit (the other picks tie at probability zero), few distinct values, and
+    NaN / +inf rows (all probabilities NaN: lowest experts win)."""
+    if True:
         for e in (8, 60, 64, 130, 256, 512):
             lg = router_inputs(400, e, 1021)
             lg[0] = 0.25
@@ -1006,41 +1008,29 @@ def test_route_pick_forms_agree():
             for k in (1, 2, 5, 8):
                 if k > e:
                     continue
-                outs = {}
-                for form in (1, 2):
-                    _hip.set_param("route_presort", form)
-                    outs[form] = _hip.route(lg.to(DEV), k, want_stats=True)
-                    torch.cuda.synchronize()
-                for a, b in zip(outs[1], outs[2]):
-                    if a.is_floating_point():     # NaN where NaN (payloads aside), bits elsewhere
-                        assert torch.equal(torch.isnan(a), torch.isnan(b)), (e, k)
-                        a, b = a.nan_to_num(nan=-7.0), b.nan_to_num(nan=-7.0)
-                    assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (e, k)
-                idx, w = outs[2][0].cpu().long(), outs[2][1].cpu()
+                out = _hip.route(lg.to(DEV), k, want_stats=True)
+                idx, w = out[0].cpu().long(), out[1].cpu()
                 oi, ow = O.router(lg[finite], k)[:2]
                 assert torch.equal(idx[finite], oi), (e, k)
                 assert torch.allclose(w[finite], ow, rtol=1e-5, atol=0), (e, k)
                 assert idx[3].tolist() == list(range(k)) and idx[4].tolist() == list(range(k)), (e, k)
                 assert torch.isnan(w[3]).all() and torch.isnan(w[4]).all()
-    finally:
-        _hip.set_param("route_presort", 0)
 
 
-def test_route_statistics_from_one_or_two_kernels_keep_their_bits():
-    """Small problems fold the statistics inside the kernel that finishes the auxiliary losses;
-    forced back to the two kernels, every output keeps its bits."""
-    try:
-        for n, e, k in ((16384, 64, 2), (1000, 8, 2), (513, 127, 4), (3, 2, 2), (9000, 100, 8), (1, 64, 1)):
-            lg = router_inputs(n, e, 1031).to(DEV)
-            _hip.set_param("route_stats_late", 1)
-            two = _hip.route(lg, k, True, True)
-            _hip.set_param("route_stats_late", 0)
-            one = _hip.route(lg, k, True, True)
-            torch.cuda.synchronize()
-            for a, b in zip(one, two):
-                assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (n, e, k)
-    finally:
-        _hip.set_param("route_stats_late", 0)
+def test_route_statistics_from_one_or_two_kernels():
+    """Small problems (up to 127 experts, 256 tiles) fold the statistics inside the kernel that
+    finishes the auxiliary losses, larger ones in a kernel of their own: both against the oracle."""
+    for n, e, k in ((16384, 64, 2), (1000, 8, 2), (513, 127, 4), (3, 2, 2), (9000, 100, 8), (1, 64, 1),
+                    (4000, 128, 2), (70000, 200, 6)):
+        lg = router_inputs(n, e, 1031)
+        idx, w, counts, slot, order, stats = _hip.route(lg.to(DEV), k, True, True)
+        oi = O.router(lg, k)[0]
+        assert torch.equal(idx.cpu().long(), oi), (n, e, k)
+        aux, z = O.router_aux(lg, oi)
+        probs = torch.softmax(lg.double(), -1)
+        assert torch.allclose(stats[:e].double().cpu(), probs.sum(0), rtol=2e-5, atol=1e-6), (n, e, k)
+        assert stats[e + 1].item() == pytest.approx(aux.item(), rel=2e-5), (n, e, k)
+        assert stats[e + 2].item() == pytest.approx(z.item(), rel=2e-5), (n, e, k)
 
 
 # ------------------------------------------------------------------ gather / combine around the permutation

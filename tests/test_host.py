@@ -527,11 +527,16 @@ def test_experts_and_moe_keep_the_reference_constructor_surface():
     c = ex(x, offsets=torch.tensor([3, 3, 8, 10], dtype=torch.int32))
     assert torch.equal(a, b) and torch.equal(a, c)
     assert ex(x[:0], counts=[0, 0, 0, 0]).shape == (0, 8)
+    with pytest.raises(RuntimeError, match="group sizes"):   # the reference's x.split(sizes) raises too
+        ex(x, counts=[3, 0, 5, 1])
     with pytest.raises(ValueError):
         fm.moe.Experts(4, 8, 16, offload=True)
     layer = fm.moe.MoE(8, 16, 4, 2, 1)                      # fifth positional argument is n_shared
     assert layer.shared is not None and layer.aux_coef == 1e-2 and layer.n_local == 4
     with pytest.raises(ValueError):
         fm.moe.MoE(8, 16, 4, 2, 0, 2)                       # ep_size 2: not in a one-GPU build
+    grouped = fm.moe.MoE(8, 16, 4, 2, grouped_mm=True)      # accepted; the experts keep the loop
+    assert grouped.compile_friendly is False and grouped.probe_grouped(torch.device("cpu"), torch.bfloat16) is False
+    assert layer.compile_friendly is False
     out = layer(torch.randn(6, 8))                          # CPU: torch expressions end to end
     assert out.shape == (6, 8) and layer.last_aux is not None

@@ -96,3 +96,24 @@ def test_static_scratch_backward_rejects_shapes_past_its_buffer():
     # 256 partial rows of 16384 floats = 16 MiB > the 8 MiB the library holds: refused before any launch
     assert lib.fm_rmsnorm_bwd_static(None, None, None, None, None, 1, 4096, 16384, _hip.BF16, _hip.F32, None) == 2
     assert b"built-in buffer" in lib.fm_last_error()
+
+
+def test_static_scratch_limit_follows_the_backward_grid():
+    # the buffer holds (partial rows) x d x 4 bytes and there is one partial row per workgroup of the
+    # persistent grid: with two workgroups per compute unit a [4096, 8192] problem needs twice the
+    # bytes and is refused, where the default grid fits exactly
+    lib = _hip.lib()
+    n, d = 4096, 8192
+    limit = 8 << 20
+    try:
+        need1 = int(lib.fm_rmsnorm_bwd_workspace(n, d, _hip.BF16))
+        _hip.set_param("norm_bwd_blocks_per_cu", 2)
+        need2 = int(lib.fm_rmsnorm_bwd_workspace(n, d, _hip.BF16))
+        assert need2 == 2 * need1
+        rc = lib.fm_rmsnorm_bwd_static(None, None, None, None, None, 1, n, d, _hip.BF16, _hip.F32, None)
+        assert (rc == 2) == (need2 > limit), (need1, need2)
+        if need2 > limit:
+            assert b"built-in buffer" in lib.fm_last_error()
+    finally:
+        _hip.set_param("norm_bwd_blocks_per_cu", 0)
+    assert need1 <= limit
