@@ -136,19 +136,24 @@ __global__ __launch_bounds__(THREADS) void ce_bwd_kernel(const T* __restrict__ l
                                                           const float* __restrict__ n_valid,
                                                           const float* __restrict__ grad_out,
                                                           T* __restrict__ dlogits, int v,
-                                                          int64_t ignore_index, bool vec_ok) {
+                                                          int64_t ignore_index, bool vec_ok, int chunks) {
   constexpr int EPV = Elem<T>::kVec;
-  const int64_t row = blockIdx.x;
+  // chunks > 1: a workgroup takes one tile of THREADS * UNROLL vectors of a row, not the whole row
+  // (the backward needs nothing from the rest of the row but the saved log-sum-exp)
+  const int64_t row = chunks > 1 ? (int64_t)(blockIdx.x / (unsigned)chunks) : (int64_t)blockIdx.x;
+  const int chunk = chunks > 1 ? (int)(blockIdx.x % (unsigned)chunks) : 0;
   const T* rp = logits + row * (int64_t)v;
   T* gp = dlogits + row * (int64_t)v;
   const RowSplit sp = split_row<EPV>(row, v, vec_ok);
   const int tid = threadIdx.x;
   const int64_t y64 = labels[row];
-  const int ne = edge_count(sp, v);
+  const int ne = chunk == 0 ? edge_count(sp, v) : 0;   // the row's unaligned ends go with its first tile
+  const int c_begin = chunks > 1 ? chunk * THREADS * UNROLL : 0;
+  const int c_end = chunks > 1 ? (c_begin + THREADS * UNROLL < sp.nvec ? c_begin + THREADS * UNROLL : sp.nvec) : sp.nvec;
 
   if (y64 == ignore_index) {  // ignored row: zeros, and the logits are never read
     const u32x4 zero = {0u, 0u, 0u, 0u};
-    for (int c = tid; c < sp.nvec; c += THREADS) store16_stream(gp + sp.head + (int64_t)c * EPV, zero);
+    for (int c = c_begin + tid; c < c_end; c += THREADS) store16_stream(gp + sp.head + (int64_t)c * EPV, zero);
     for (int e = tid; e < ne; e += THREADS) Elem<T>::store1(gp + edge_col(sp, e), 0.f);
     return;
   }
@@ -156,7 +161,7 @@ __global__ __launch_bounds__(THREADS) void ce_bwd_kernel(const T* __restrict__ l
   const float scale = (grad_out != nullptr ? *grad_out : 1.f) / (n_valid != nullptr ? *n_valid : 1.f);
   const float l2 = lse[row] * kLog2e;
 
-  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+  for (int c0 = c_begin; c0 < c_end; c0 += THREADS * UNROLL) {
     u32x4 raw[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
@@ -711,10 +716,14 @@ int launch_bwd(const void* logits, const int64_t* labels, const float* lse, cons
   const T* lp = static_cast<const T*>(logits);
   T* gp = static_cast<T*>(dlogits);
   const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 4);
-  const dim3 grid((unsigned)n);
+  // rows longer than one tile (threads x unroll vectors): a workgroup per tile
+  const int64_t tile = (int64_t)sh.threads * sh.unroll;
+  int64_t chunks = (v / Elem<T>::kVec + 1 + tile - 1) / tile;
+  if (chunks < 1 || n * chunks > 0x7fffffffLL) chunks = 1;
+  const dim3 grid((unsigned)(n * chunks));
 #define LAUNCH(TH, UN)                                                                         \
   FM_LAUNCH((ce_bwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, lp, labels, lse, n_valid, \
-                     grad_out, gp, v, ignore_index, vec_ok)
+                     grad_out, gp, v, ignore_index, vec_ok, (int)chunks)
   FM_VOCAB_DISPATCH(sh, LAUNCH);
 #undef LAUNCH
   return FM_OK;
