@@ -1012,12 +1012,12 @@ def measure_floor(torch, w, steps, warmup, L, ms):
                                          len(rd), len(wr), kind, thr, vec, grid, st), "fm_stream_probe_mix")
         return go
 
-    chosen, names = [], []
+    per_launch = []      # for every launch: {store kind: (ms, launcher, label)}, the best shape and grid of that kind
     for spec in w.floor:
         rd, wr = spec(0)
         nbytes = rd[0].numel() * rd[0].element_size()
         kinds = (0,) if not wr else ((0, 1) if len(wr) == 1 else (0, 1, 2))
-        best = None
+        best = {}
         for thr, vec in FLOOR_SHAPES:
             if nbytes % (thr * vec * 16):
                 continue
@@ -1035,19 +1035,27 @@ def measure_floor(torch, w, steps, warmup, L, ms):
                     for _ in range(3):
                         one()
                     avg = time_back_to_back(torch, one, 10)
-                    if best is None or avg < best[0]:
-                        best = (avg, go, f"{len(rd)}r{len(wr)}w {thr}x{vec} grid {grid or tiles} store {kind}")
-        if best is None:
+                    if kind not in best or avg < best[kind][0]:
+                        best[kind] = (avg, go, f"{len(rd)}r{len(wr)}w {thr}x{vec} grid {grid or tiles} store {kind}")
+        if not best:
             return {"floor_ms": None}
-        chosen.append(best[1])
-        names.append(f"{best[2]}: {best[0] * 1e3:.1f} us")
-    state = {"i": 0}
+        per_launch.append(best)
+    # the store kinds are chosen for the step as a whole (what one launch leaves in the caches is
+    # what the next one finds): every combination of kinds, each launch in its best shape for that kind
+    import itertools
+    fms, names = None, None
+    for combo in itertools.product(*[sorted(b) for b in per_launch]):
+        chosen = [per_launch[j][kind][1] for j, kind in enumerate(combo)]
+        state = {"i": 0}
 
-    def floor_step():
-        i = state["i"] = (state["i"] + 1) % sets
-        for go in chosen:
-            go(i)
-    fms = time_steps(torch, floor_step, steps, warmup)
+        def floor_step():
+            i = state["i"] = (state["i"] + 1) % sets
+            for go in chosen:
+                go(i)
+        t = time_steps(torch, floor_step, steps, warmup)
+        if fms is None or t < fms:
+            fms = t
+            names = [f"{per_launch[j][kind][2]}: {per_launch[j][kind][0] * 1e3:.1f} us" for j, kind in enumerate(combo)]
     return {"floor_ms": round(fms, 5), "of_floor": round(fms / ms, 4), "floor_sweeps": names}
 
 

@@ -509,7 +509,7 @@ void launch_fwd(const void* s, const void* t, float* lse_s, float* lse_t, float*
                 int v, float inv_temp, bool vec_ok, hipStream_t st) {
   const T* sp = static_cast<const T*>(s);
   const T* tp = static_cast<const T*>(t);
-  const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 512, 2);
+  const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 512, 4);
   const dim3 grid((unsigned)n);
 #define LAUNCH(TH, UN)                                                                            \
   FM_LAUNCH((kl_fwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, sp, tp, lse_s, lse_t, row_kl, \
