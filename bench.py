@@ -52,36 +52,38 @@ METRIC = "HBM GB/s & % roofline: RMSNorm, CE/KL fwd+bwd; MoE top-k rows/s"
 # HBM traffic per launch, keyed by the kernel's full name as fm_last_kernel() reports it:
 # (FETCH_SIZE KiB, WRITE_SIZE KiB) per dispatch from two `rocprofv3 --pmc` runs of this file
 # (profiles/all_workloads_hbm_traffic_pmc.txt). Each counter is scaled by what it reads for the
-# library's own 1 GiB copy (probe_copy_kernel: 524295.9 KiB fetched, 1049434.5 KiB written).
+# library's own 1 GiB copy (probe_copy_kernel, `bench.py --copy-probe 1024` under the same counters).
 # A kernel that is not in the table (a retune changed its template arguments) reports null.
-TRAFFIC_SCALE = (1048576.0 / 524295.9, 1048576.0 / 1049434.5)
+TRAFFIC_SCALE = (1048576.0 / 524303.3, 1048576.0 / 1049376.6)
 TRAFFIC_KIB = {
-    "ce_bwd_kernel<bf16_t, 1024, 4>": (244178.2, 512240.8),
-    "ce_fwd_kernel<bf16_t, 512, 4>": (256535.5, 512.2),
-    "ce_loss_grad_kernel<bf16_t, 512, 8>": (243960.2, 512528.3),
+    "ce_bwd_kernel<bf16_t, 1024, 4>": (244206.7, 512065.2),
+    "ce_fwd_kernel<bf16_t, 512, 4>": (256685.1, 512.9),
+    "ce_loss_grad_kernel<bf16_t, 512, 8>": (243968.6, 512548.1),
     "combine_kernel<bf16_t, true>": (133143.1, 131072.0),
-    "kl_bwd_kernel<bf16_t, bf16_t, 1024, 8>": (1026352.3, 1026350.2),
-    "kl_fwd_kernel<bf16_t, 512, 2>": (1026083.7, 386.6),
-    "kl_fwd_topk_kernel<bf16_t, 512, 2, false>": (1052904.3, 2432.6),
-    "kl_fwd_topk_kernel<bf16_t, 512, 2, true>": (2057675.9, 1028504.1),
-    "kl_loss_grad_wide_kernel<bf16_t, bf16_t, 1024, 2>": (2040992.4, 1026451.2),
-    "norm_bwd_kernel<bf16_t, bf16_t, 256, 2, false>": (65812.9, 69632.7),
-    "norm_bwd_kernel<bf16_t, float, 512, 2, false>": (393631.6, 270336.1),
-    "norm_bwd_kernel<bf16_t, float, 512, 2, true>": (393894.8, 278528.0),
-    "norm_bwd_kernel<bf16_t, float, 64, 2, false>": (16459.1, 17408.0),
+    "kl_bwd_kernel<bf16_t, bf16_t, 1024, 8>": (1026900.0, 1026058.1),
+    "kl_fwd_kernel<bf16_t, 512, 4>": (1026890.9, 385.2),
+    "kl_fwd_topk_kernel<bf16_t, 512, 2, false>": (1054167.0, 2433.9),
+    "kl_fwd_topk_kernel<bf16_t, 512, 2, true>": (2057714.4, 1028506.4),
+    "kl_loss_grad_wide_kernel<bf16_t, bf16_t, 1024, 2>": (2041391.9, 1026451.9),
+    "norm_bwd_kernel<bf16_t, bf16_t, 256, 2, false>": (65853.4, 69632.9),
+    "norm_bwd_kernel<bf16_t, float, 512, 2, false>": (393631.7, 270336.0),
+    "norm_bwd_kernel<bf16_t, float, 512, 2, true>": (393891.4, 278528.0),
+    "norm_bwd_kernel<bf16_t, float, 64, 2, false>": (16461.7, 17408.0),
     "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, false, false>": (32820.6, 65846.5),
-    "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, true, false>": (65587.1, 131372.5),
-    "norm_fwd_kernel<bf16_t, float, 512, 2, true, false>": (262295.6, 524836.1),
-    "norm_fwd_kernel<bf16_t, float, 512, 2, true, true>": (262429.4, 525353.4),
-    "norm_fwd_kernel<bf16_t, float, 64, 2, false, false>": (8221.1, 16448.5),
-    "rope_vec_kernel<bf16_t, float, 8, false, 2>": (105932.1, 213459.0),
-    "rope_vec_kernel<bf16_t, float, 8, true, 2>": (216519.2, 214989.4),
-    "route_bwd_kernel<float, 8, true>": (2273.0, 4096.0),
-    "route_group_kernel<float, 8, true, false>": (2107.7, 328.3),
-    "scatter_kernel<bf16_t, true>": (66086.0, 262270.7),
-    "swiglu_split_kernel<bf16_t, true, false>": (346617.2, 346599.8),
-    "swiglu_split_kernel<bf16_t, true, true>": (532289.2, 709692.8),
-    "topk_lds_kernel<bf16_t, 1024, 4, 0>": (546459.6, 1024.0),
+    "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, true, false>": (65585.1, 131361.4),
+    "norm_fwd_kernel<bf16_t, float, 512, 2, true, false>": (262295.9, 524841.5),
+    "norm_fwd_kernel<bf16_t, float, 512, 2, true, true>": (262429.8, 525347.6),
+    "norm_fwd_kernel<bf16_t, float, 64, 2, false, false>": (8227.7, 16448.3),
+    "permute_kernel": (1578.5, 10806.2),
+    "rope_vec_kernel<bf16_t, float, 8, false, 2>": (105932.2, 213459.8),
+    "rope_vec_kernel<bf16_t, float, 8, true, 2>": (216521.7, 215000.3),
+    "route_bwd_kernel<float, 8, true>": (2273.5, 4096.0),
+    "route_group_kernel<float, 32, true, true>": (32841.1, 6176.0),
+    "route_group_kernel<float, 8, true, false>": (2106.0, 328.3),
+    "scatter_kernel<bf16_t, true>": (66086.3, 262271.0),
+    "swiglu_split_kernel<bf16_t, true, false>": (458770.2, 458752.0),
+    "swiglu_split_kernel<bf16_t, true, true>": (688148.4, 917504.8),
+    "topk_lds_kernel<bf16_t, 1024, 4, 0>": (546659.6, 1024.0),
 }
 TRAFFIC_SOURCE = "profiles/all_workloads_hbm_traffic_pmc.txt"
 

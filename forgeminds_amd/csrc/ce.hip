@@ -177,10 +177,13 @@ __global__ __launch_bounds__(THREADS) void ce_bwd_kernel(const T* __restrict__ l
         Elem<T>::unpack(raw[u], z);
         const int col0 = sp.head + c * EPV;
 #pragma unroll
-        for (int e = 0; e < EPV; ++e) {
-          o[e] = fast_exp2(z[e] * kLog2e - l2);
-          o[e] = (col0 + e == y ? o[e] - 1.f : o[e]) * scale;
+        for (int e = 0; e < EPV; ++e) o[e] = fast_exp2(z[e] * kLog2e - l2);
+        if (y >= col0 && y < col0 + EPV) {   // the one vector of the row that holds the label
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) o[e] -= (col0 + e == y) ? 1.f : 0.f;
         }
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] *= scale;
         store16_stream(gp + col0, Elem<T>::pack(o));
       }
     }
@@ -293,10 +296,13 @@ __global__ __launch_bounds__(THREADS) void ce_loss_grad_wide_kernel(const T* log
         Elem<T>::unpack(raw[u], z);
         const int col0 = sp.head + c * EPV;
 #pragma unroll
-        for (int e = 0; e < EPV; ++e) {
-          o[e] = fast_exp2(z[e] * kLog2e - l2);
-          o[e] = (col0 + e == y ? o[e] - 1.f : o[e]) * scale;
+        for (int e = 0; e < EPV; ++e) o[e] = fast_exp2(z[e] * kLog2e - l2);
+        if (y >= col0 && y < col0 + EPV) {   // the one vector of the row that holds the label
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) o[e] -= (col0 + e == y) ? 1.f : 0.f;
         }
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] *= scale;
         store16_stream(gp + col0, Elem<T>::pack(o));
       }
     }
