@@ -10,13 +10,15 @@
 //   route_group_kernel  L lanes per row (8, 16, 32 or 64 for up to 64, 128, 256, 512 experts),
 //                   eight neighbouring experts per lane, so a wave works on 64 / L rows at once
 //                   and reads whole rows with 16-byte loads. Group max / sum give the softmax;
-//                   each of the k picks is a group max over order-preserving integer keys
-//                   followed by a group min over the tied expert indices. Each 4-wave workgroup
+//                   the k picks come from order-preserving integer keys in one of three ways
+//                   (kSelScan, kSelSorted, kSelCands below). Each 4-wave workgroup
 //                   owns a contiguous tile of rows and leaves its expert histogram in
 //                   `hist[tile][e]` (and, when asked, a partial row of the statistics).
 //   route_stats_kernel  folds the statistics partials in a fixed order (only when asked for).
 //   hist_scan_kernel    only for many tiles x many experts: exclusive scan of the histograms
-//                   over the tiles, in place, and the expert totals.
+//                   over the tiles, in place, and the expert totals. With statistics the two run
+//                   as one launch (route_scan_stats_kernel), and the two auxiliary losses are then
+//                   finished by one more workgroup of the permute_kernel launch.
 //   permute_kernel  every workgroup takes (or, without the scan, sums) the histograms of the
 //                   tiles before it and the expert totals, then walks its own tile in ascending
 //                   flat position and gives each assignment the slot
@@ -35,17 +37,110 @@ constexpr int kMaxTiles = 1024;
 constexpr int kGroupThreads = 256;    // 4 waves per tile
 constexpr int kGE = 8;                // experts a lane holds
 
+// How route_group_kernel selects a row's k experts.
+constexpr int kSelScan = 0;     // every pick scans the lane's eight keys afresh (up to four picks)
+constexpr int kSelSorted = 1;   // lanes sort their eight pairs first; a pick is the maximum over the lanes' heads
+constexpr int kSelCands = 2;    // threshold, then a sort of the few candidates across the lanes
+
+constexpr int kDppXor3 = 0x1B;      // quad_perm:[3,2,1,0]
+constexpr int kDppRor8 = 0x128;     // row_ror:8 (lane ^ 8 inside a row of 16)
+constexpr int kSwzXor4 = 0x101F;    // ds_swizzle, bit mode: lane ^ 4
+constexpr int kSwzXor16 = 0x401F;   // lane ^ 16
+constexpr int kSwzXor31 = 0x7C1F;   // lane ^ 31
+
+template <int CTRL>
+__device__ __forceinline__ unsigned long long dpp64(unsigned long long v) {
+  // (every lane of these patterns has a source lane: no value for missing ones to set up)
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_mov_dpp((int)(uint32_t)v, CTRL, 0xf, 0xf, true);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_mov_dpp((int)(uint32_t)(v >> 32), CTRL, 0xf, 0xf, true);
+  return ((unsigned long long)hi << 32) | lo;
+}
+template <int PATTERN>
+__device__ __forceinline__ unsigned long long swz64(unsigned long long v) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_swizzle((int)(uint32_t)v, PATTERN);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_swizzle((int)(uint32_t)(v >> 32), PATTERN);
+  return ((unsigned long long)hi << 32) | lo;
+}
+__device__ __forceinline__ unsigned long long xor64(unsigned long long v, int mask) {
+  const uint32_t lo = (uint32_t)__shfl_xor((int)(uint32_t)v, mask, 64);
+  const uint32_t hi = (uint32_t)__shfl_xor((int)(uint32_t)(v >> 32), mask, 64);
+  return ((unsigned long long)hi << 32) | lo;
+}
+// one exchange of the network below: the lower lane of a pair keeps the larger value
+__device__ __forceinline__ unsigned long long keep(unsigned long long mine, unsigned long long other, bool lower) {
+  return ((other > mine) == lower) ? other : mine;
+}
+// Sorts one 64-bit value per lane over groups of L lanes, largest in the group's first lane: the
+// bitonic network in its mirrored form (a merge of 2m lanes starts with lane ^ (2m - 1), then
+// lane ^ m/2 ... lane ^ 1), whose exchanges all point the same way, so that every step is one of the
+// lane patterns the hardware moves data by (quad permutes, row mirrors, a row rotation, swizzles).
+template <int L>
+__device__ __forceinline__ unsigned long long group_sort_desc(unsigned long long c, int l) {
+  static_assert(L == 16 || L == 32 || L == 64, "groups of 16, 32 or 64 lanes");
+  const bool u1 = (l & 1) == 0, u2 = (l & 2) == 0, u4 = (l & 4) == 0, u8 = (l & 8) == 0;
+  c = keep(c, dpp64<kDppXor1>(c), u1);
+  c = keep(c, dpp64<kDppXor3>(c), u2);
+  c = keep(c, dpp64<kDppXor1>(c), u1);
+  c = keep(c, dpp64<kDppHalfMirror>(c), u4);
+  c = keep(c, dpp64<kDppXor2>(c), u2);
+  c = keep(c, dpp64<kDppXor1>(c), u1);
+  c = keep(c, dpp64<kDppMirror>(c), u8);
+  c = keep(c, swz64<kSwzXor4>(c), u4);
+  c = keep(c, dpp64<kDppXor2>(c), u2);
+  c = keep(c, dpp64<kDppXor1>(c), u1);
+  if constexpr (L >= 32) {
+    const bool u16 = (l & 16) == 0;
+    c = keep(c, swz64<kSwzXor31>(c), u16);
+    c = keep(c, dpp64<kDppRor8>(c), u8);
+    c = keep(c, swz64<kSwzXor4>(c), u4);
+    c = keep(c, dpp64<kDppXor2>(c), u2);
+    c = keep(c, dpp64<kDppXor1>(c), u1);
+  }
+  if constexpr (L == 64) {
+    const bool u16 = (l & 16) == 0, u32 = (l & 32) == 0;
+    c = keep(c, xor64(c, 63), u32);
+    c = keep(c, swz64<kSwzXor16>(c), u16);
+    c = keep(c, dpp64<kDppRor8>(c), u8);
+    c = keep(c, swz64<kSwzXor4>(c), u4);
+    c = keep(c, dpp64<kDppXor2>(c), u2);
+    c = keep(c, dpp64<kDppXor1>(c), u1);
+  }
+  return c;
+}
+
+// Maximum of a float over a group of L lanes, through the integers: the bits of a float, with the
+// magnitude of the negative ones inverted, order as signed integers the way the floats do, and an
+// integer maximum takes its lane pattern in the same instruction, where the float maximum needs
+// three more to fetch and quiet its operand. (A positive NaN wins, a negative one loses: the row
+// is a NaN row either way, through its sum.)
+template <int L>
+__device__ __forceinline__ float group_max_f(float v) {
+  auto flip = [](int i) { return i ^ ((i >> 31) & 0x7fffffff); };
+  auto mx = [](int a, int b) { return a > b ? a : b; };
+  int i = flip(__builtin_bit_cast(int, v));
+  i = mx(i, FM_DPP_I(i, kDppXor1));
+  i = mx(i, FM_DPP_I(i, kDppXor2));
+  i = mx(i, FM_DPP_I(i, kDppHalfMirror));
+  if constexpr (L >= 16) i = mx(i, FM_DPP_I(i, kDppMirror));
+  if constexpr (L >= 32) i = mx(i, __builtin_amdgcn_ds_swizzle(i, kSwzXor16));
+  if constexpr (L == 64) i = mx(i, __shfl_xor(i, 32, 64));
+  return __builtin_bit_cast(float, flip(i));
+}
+
 // L lanes per row, eight neighbouring experts per lane: a wave works on 64 / L rows at once, reads
 // whole rows with 16-byte loads (VEC: e a multiple of eight, aligned buffer) and reduces over L
 // lanes only. Ties go to the lowest expert index: the lane keeps its first maximum, the group
 // takes the smallest index among the lanes that hold the group's maximum.
-// PRESORT (five picks or more): every lane first sorts its eight (key, expert) pairs with a
-// 19-exchange network, so that a pick is the group maximum over the lanes' heads and a shift in
-// the winning lane, instead of a fresh scan of the lane's eight keys and three selects by position
-// -- about 30 instead of 75 instructions a pick. The probability of a pick is read back from its
-// key (they are the same bits above the sign), so both forms give identical results (a NaN row's
+// kSelSorted: every lane first sorts its eight (key, expert) pairs with a 19-exchange network, so
+// that a pick is the group maximum over the lanes' heads, a ballot for the first lane that holds it
+// and a shift in that lane, instead of a fresh scan of the lane's eight keys, a second reduction
+// over the tied experts and three selects by position -- about 30 instead of 75 instructions a
+// pick. kSelCands (129-256 experts, five picks or more): a cheap lower bound of the k-th key, the
+// twenty or so experts at or above it compacted into LDS, one of them per lane, and ONE sort
+// across the lanes in place of k rounds. The probability of a pick is read back from its key
+// (they are the same bits above the sign), so all forms give identical results (a NaN row's
 // weights are NaN either way, with whatever payload).
-template <typename T, int L, bool VEC, bool PRESORT>
+template <typename T, int L, bool VEC, int SEL>
 __global__ __launch_bounds__(kGroupThreads) void route_group_kernel(const T* __restrict__ logits,
                                                                      int32_t* __restrict__ idx,
                                                                      float* __restrict__ weights,
@@ -57,6 +152,10 @@ __global__ __launch_bounds__(kGroupThreads) void route_group_kernel(const T* __r
   __shared__ int lh[L * kGE];
   __shared__ float wstat[NW][L * kGE];  // per-wave column sums of the probabilities
   __shared__ float wz[NW];              // per-wave sums of logsumexp^2
+  constexpr int R = 2;                  // rows per lane group in flight
+  // candidate lists (one per row in flight) and their lengths
+  __shared__ unsigned long long cand[SEL == kSelCands ? NW * R : 1][SEL == kSelCands ? 64 * kGE : 1];
+  __shared__ int ccount[SEL == kSelCands ? NW * R : 1][SEL == kSelCands ? GPW : 1];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int g = lane / L, l = lane % L;
   const int ex0 = l * kGE;              // this lane's first expert
@@ -69,7 +168,6 @@ __global__ __launch_bounds__(kGroupThreads) void route_group_kernel(const T* __r
   const int64_t row0 = (int64_t)blockIdx.x * tile_rows;
   const int64_t row1 = row0 + tile_rows < n ? row0 + tile_rows : n;
   // R rows per lane group are in flight at once so that their dependent reduction chains overlap
-  constexpr int R = 2;
   for (int64_t rb = row0 + wave * GPW; rb < row1; rb += (int64_t)NW * GPW * R) {
     int64_t row[R];
     bool live[R];
@@ -106,7 +204,7 @@ __global__ __launch_bounds__(kGroupThreads) void route_group_kernel(const T* __r
       for (int q = 1; q < kGE; ++q) m[r] = fmaxf(m[r], p[r][q]);
     }
 #pragma unroll
-    for (int r = 0; r < R; ++r) m[r] = group_reduce<L, OpMax>(m[r]);
+    for (int r = 0; r < R; ++r) m[r] = group_max_f<L>(m[r]);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       s[r] = 0.f;
@@ -148,7 +246,81 @@ __global__ __launch_bounds__(kGroupThreads) void route_group_kernel(const T* __r
     float my_p[R], wsum[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) { my_i[r] = 0; my_p[r] = 0.f; wsum[r] = 0.f; }
-    if constexpr (PRESORT) {
+    if constexpr (SEL == kSelCands) {
+      // Threshold: the lanes with equal l % 8 form eight disjoint sets of experts, none empty (the
+      // launcher takes this form only when the row has more than 64 experts); the smallest of the
+      // eight set maxima has eight different experts at or above it, so it is a lower bound of
+      // the k-th largest key. On rows without long runs of equal keys some twenty experts reach it.
+      uint32_t tau[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        uint32_t hm = key[r][0];
+#pragma unroll
+        for (int q = 1; q < kGE; ++q) hm = hm > key[r][q] ? hm : key[r][q];
+        auto mx = [](uint32_t a, uint32_t b) { return a > b ? a : b; };
+        auto mn = [](uint32_t a, uint32_t b) { return a < b ? a : b; };
+        hm = mx(hm, (uint32_t)FM_DPP_I((int)hm, kDppRor8));
+        if constexpr (L >= 32) hm = mx(hm, (uint32_t)__builtin_amdgcn_ds_swizzle((int)hm, kSwzXor16));
+        if constexpr (L == 64) hm = mx(hm, (uint32_t)__shfl_xor((int)hm, 32, 64));
+        hm = mn(hm, (uint32_t)FM_DPP_I((int)hm, kDppXor1));
+        hm = mn(hm, (uint32_t)FM_DPP_I((int)hm, kDppXor2));
+        hm = mn(hm, (uint32_t)FM_DPP_I((int)hm, kDppHalfMirror));
+        tau[r] = hm;
+      }
+      // The experts at or above the threshold go to the group's list in LDS, in any order, as
+      // (key, 65535 - expert): larger is better, equal keys keep the lower expert in front.
+      const int gbase = lane & ~(L - 1);
+      const int wr0 = wave * R;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        if (l == 0) ccount[wr0 + r][g] = 0;
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        int at[kGE];
+#pragma unroll
+        for (int q = 0; q < kGE; ++q)
+          at[q] = (live[r] && key[r][q] >= tau[r]) ? atomicAdd(&ccount[wr0 + r][g], 1) : -1;
+#pragma unroll
+        for (int q = 0; q < kGE; ++q) {
+          if (at[q] >= 0)
+            cand[wr0 + r][gbase * kGE + at[q]] =
+                ((unsigned long long)key[r][q] << 32) | (uint32_t)(0xFFFF - (ex0 + q));
+        }
+      }
+      // One candidate per lane, sorted across the group: its first k lanes then hold the picks in
+      // order. A longer list is taken L - 8 at a time next to the best eight so far.
+      int cn[R];
+      unsigned long long c[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        cn[r] = ccount[wr0 + r][g];
+        c[r] = l < cn[r] ? cand[wr0 + r][gbase * kGE + l] : 0ull;
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) c[r] = group_sort_desc<L>(c[r], l);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        for (int base = L; __builtin_amdgcn_ballot_w64(base < cn[r]) != 0ull; base += L - 8) {
+          const int src = base + l - 8;
+          const unsigned long long nx = (l >= 8 && src < cn[r]) ? cand[wr0 + r][gbase * kGE + src] : 0ull;
+          c[r] = l < 8 ? c[r] : nx;
+          c[r] = group_sort_desc<L>(c[r], l);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        // a probability is never negative: its key is its bit pattern with the top bit set
+        // (the all-ones NaN key reads back as a NaN)
+        const float pv = __builtin_bit_cast(float, (uint32_t)(c[r] >> 32) & 0x7FFFFFFFu);
+        my_p[r] = pv;
+        my_i[r] = 0xFFFF - (int)((uint32_t)c[r] & 0xFFFFu);
+#pragma unroll
+        for (int j = 0; j < kMaxK; ++j) {
+          if (j < k) wsum[r] += __shfl(pv, gbase + j, 64);   // in pick order, as the other forms add them
+        }
+      }
+    } else if constexpr (SEL == kSelSorted) {
       // (key, kGE - 1 - position) as one 64-bit value: larger is better, equal keys keep the
       // lower expert in front
       unsigned long long c[R][kGE];
@@ -169,30 +341,60 @@ __global__ __launch_bounds__(kGroupThreads) void route_group_kernel(const T* __r
         cx(2, 4); cx(3, 5);
         cx(1, 2); cx(3, 4); cx(5, 6);
       }
+      // After the sort the keys stay in registers, head first; the positions are packed four bits
+      // apiece into one register (head in the low bits), so that a winning lane moves its list up
+      // with eight selects and one shift.
+      uint32_t ck[R][kGE], ord[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        ord[r] = 0u;
+#pragma unroll
+        for (int q = 0; q < kGE; ++q) {
+          ck[r][q] = (uint32_t)(c[r][q] >> 32);
+          ord[r] |= ((uint32_t)c[r][q] & 7u) << (4 * q);
+        }
+      }
+      const int gbase = lane & ~(L - 1);
 #pragma unroll
       for (int j = 0; j < kMaxK; ++j) {
         if (j < k) {
           uint32_t gk[R];
-          int gi[R];
 #pragma unroll
-          for (int r = 0; r < R; ++r) gk[r] = group_max_u<L>((uint32_t)(c[r][0] >> 32));
-#pragma unroll
-          for (int r = 0; r < R; ++r)
-            gi[r] = group_min_i<L>(((uint32_t)(c[r][0] >> 32) == gk[r]) ? ex0 + (kGE - 1 - (int)(uint32_t)c[r][0])
-                                                                        : 0x7fffffff);
+          for (int r = 0; r < R; ++r) gk[r] = group_max_u<L>(ck[r][0]);
 #pragma unroll
           for (int r = 0; r < R; ++r) {
-            if (j + 1 < k) {   // the winning lane moves its next pair to the front
-              const bool won = (gi[r] >> 3) == l;
-#pragma unroll
-              for (int q = 0; q + 1 < kGE; ++q) c[r][q] = won ? c[r][q + 1] : c[r][q];
-              c[r][kGE - 1] = won ? 0ull : c[r][kGE - 1];
+            // The lanes of a group hold ascending blocks of experts and a lane's equal keys are in
+            // ascending order of expert, so the FIRST lane whose head is the group's maximum holds
+            // the lowest expert among the tied ones: one ballot instead of a second reduction.
+            const unsigned long long tied = __builtin_amdgcn_ballot_w64(ck[r][0] == gk[r]);
+            int first;
+            if constexpr (L == 64) {
+              first = __builtin_ctzll(tied);
+            } else {
+              const uint32_t half = gbase >= 32 ? (uint32_t)(tied >> 32) : (uint32_t)tied;
+              const uint32_t mine = L == 32 ? half : ((half >> (gbase & 31)) & ((1u << (L & 31)) - 1u));
+              first = __builtin_ctz(mine);
             }
+            const bool won = first == l;
             // a probability is never negative: its key is its bit pattern with the top bit set
             // (the all-ones NaN key reads back as a NaN)
             const float pv = __builtin_bit_cast(float, gk[r] & 0x7FFFFFFFu);
             wsum[r] += pv;
-            if (l == j) { my_i[r] = gi[r]; my_p[r] = pv; }
+            if (l == j) my_p[r] = pv;
+            if (won) {
+              // the winner itself records the pick: no other lane needs to learn the expert
+              const int ex = ex0 + (kGE - 1) - (int)(ord[r] & 7u);
+              if (live[r]) {
+                idx[row[r] * (int64_t)k + j] = ex;
+                atomicAdd(&lh[ex], 1);
+              }
+            }
+            if (j + 1 < k) {   // the winning lane moves its next pair to the front
+#pragma unroll
+              for (int q = 0; q + 1 < kGE; ++q) ck[r][q] = won ? ck[r][q + 1] : ck[r][q];
+              ck[r][kGE - 1] = won ? 0u : ck[r][kGE - 1];
+              ord[r] = won ? (ord[r] >> 4) : ord[r];
+            }
           }
         }
       }
@@ -235,9 +437,11 @@ __global__ __launch_bounds__(kGroupThreads) void route_group_kernel(const T* __r
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       if (live[r] && l < k) {
-        idx[row[r] * (int64_t)k + l] = my_i[r];
         weights[row[r] * (int64_t)k + l] = my_p[r] / wsum[r];
-        atomicAdd(&lh[my_i[r]], 1);
+        if constexpr (SEL != kSelSorted) {   // (the sorted form's winners have stored these themselves)
+          idx[row[r] * (int64_t)k + l] = my_i[r];
+          atomicAdd(&lh[my_i[r]], 1);
+        }
       }
     }
   }
@@ -401,13 +605,11 @@ __global__ __launch_bounds__(kGroupThreads) void route_bwd_kernel(const T* __res
 // stats[e] = sum of logsumexp^2. A workgroup owns 64 columns; wave w adds tiles w, w + 16, ...
 // of a column in that order, then the sixteen partial sums are added in wave order. The order
 // depends on ntiles only, so equal inputs give equal bits.
-__global__ __launch_bounds__(1024) void route_stats_kernel(const float* __restrict__ fstat,
-                                                            float* __restrict__ stats, int e,
-                                                            int ntiles) {
-  __shared__ float part[16][64];
+__device__ __forceinline__ void stats_fold_block(const float* __restrict__ fstat, float* __restrict__ stats,
+                                                 int e, int ntiles, int block, float (*part)[64]) {
   const int cols = e + 1;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int c = blockIdx.x * 64 + lane;
+  const int c = block * 64 + lane;
   float a = 0.f;
   if (c < cols) {
     // sixteen loads in flight; the additions stay in tile order
@@ -431,15 +633,20 @@ __global__ __launch_bounds__(1024) void route_stats_kernel(const float* __restri
   }
 }
 
+__global__ __launch_bounds__(1024) void route_stats_kernel(const float* __restrict__ fstat,
+                                                            float* __restrict__ stats, int e,
+                                                            int ntiles) {
+  __shared__ float part[16][64];
+  stats_fold_block(fstat, stats, e, ntiles, (int)blockIdx.x, part);
+}
+
 // Exclusive scan of the tile histograms over the tiles, in place: hist[t][c] becomes the number
 // of assignments to expert c in tiles before t, counts[c] their total. A workgroup owns 16
 // experts; thread (s, c) walks tiles s * per, ..., (s + 1) * per - 1 of expert c.
-__global__ __launch_bounds__(1024) void hist_scan_kernel(int32_t* __restrict__ hist,
-                                                          int32_t* __restrict__ counts, int e,
-                                                          int ntiles) {
-  __shared__ int seg[64][17];
+__device__ __forceinline__ void hist_scan_block(int32_t* __restrict__ hist, int32_t* __restrict__ counts,
+                                                int e, int ntiles, int block, int (*seg)[17]) {
   const int c = threadIdx.x & 15, sgm = threadIdx.x >> 4;
-  const int col = blockIdx.x * 16 + c;
+  const int col = block * 16 + c;
   constexpr int kPer = kMaxTiles / 64;   // tiles per segment at most
   const int per = (ntiles + 63) / 64;
   const int t0 = sgm * per;
@@ -461,7 +668,7 @@ __global__ __launch_bounds__(1024) void hist_scan_kernel(int32_t* __restrict__ h
       seg[q][threadIdx.x] = run;
       run += w;
     }
-    if (blockIdx.x * 16 + (int)threadIdx.x < e) counts[blockIdx.x * 16 + threadIdx.x] = run;
+    if (block * 16 + (int)threadIdx.x < e) counts[block * 16 + threadIdx.x] = run;
   }
   __syncthreads();
   int run = seg[sgm][c];
@@ -471,6 +678,26 @@ __global__ __launch_bounds__(1024) void hist_scan_kernel(int32_t* __restrict__ h
     if (col < e && u < per && t < ntiles) hist[(int64_t)t * e + col] = run;
     run += v[u];
   }
+}
+
+__global__ __launch_bounds__(1024) void hist_scan_kernel(int32_t* __restrict__ hist,
+                                                          int32_t* __restrict__ counts, int e,
+                                                          int ntiles) {
+  __shared__ int seg[64][17];
+  hist_scan_block(hist, counts, e, ntiles, (int)blockIdx.x, seg);
+}
+
+// The scan of the histograms and the fold of the statistics need nothing of each other: one
+// launch, the first `scan_blocks` workgroups scan, the others fold.
+__global__ __launch_bounds__(1024) void route_scan_stats_kernel(int32_t* __restrict__ hist,
+                                                                 int32_t* __restrict__ counts,
+                                                                 const float* __restrict__ fstat,
+                                                                 float* __restrict__ stats, int e,
+                                                                 int ntiles, int scan_blocks) {
+  __shared__ int seg[64][17];
+  __shared__ float part[16][64];
+  if ((int)blockIdx.x < scan_blocks) hist_scan_block(hist, counts, e, ntiles, (int)blockIdx.x, seg);
+  else stats_fold_block(fstat, stats, e, ntiles, (int)blockIdx.x - scan_blocks, part);
 }
 
 // The two auxiliary losses from the finished sums (forgemind/moe.py:92-95), one workgroup:
@@ -488,6 +715,31 @@ __global__ __launch_bounds__(512) void route_aux_kernel(const int32_t* __restric
   if ((c & 63) == 0) part[c >> 6] = a;
   __syncthreads();
   if (c == 0) {
+    float t = part[0];
+#pragma unroll
+    for (int w = 1; w < 8; ++w) t += part[w];
+    stats[e + 1] = (float)e * t;
+    stats[e + 2] = stats[e] / rows;
+  }
+}
+
+// route_aux_kernel's arithmetic from a workgroup of 256 threads (the extra workgroup of a
+// permute_kernel launch): every wave stands in for two of that kernel's eight, so the sums are
+// formed from the same values in the same order.
+__device__ __forceinline__ void aux_block_256(const int32_t* counts, float* __restrict__ stats, int64_t n,
+                                              int e, int k) {
+  __shared__ float part[8];
+  const float rows = n > 0 ? (float)n : 1.f;
+  const float slots = n > 0 ? (float)(n * (int64_t)k) : 1.f;
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    const int c = half * 256 + (int)threadIdx.x;
+    float a = c < e ? ((float)counts[c] / slots) * (stats[c] / rows) : 0.f;
+    a = wave_sum(a);
+    if ((c & 63) == 0) part[c >> 6] = a;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
     float t = part[0];
 #pragma unroll
     for (int w = 1; w < 8; ++w) t += part[w];
@@ -560,7 +812,7 @@ __global__ __launch_bounds__(256) void permute_kernel(const int32_t* __restrict_
                                                        int32_t* __restrict__ slot,
                                                        int32_t* __restrict__ order, int64_t n, int e,
                                                        int k, int tile_rows, int ntiles, int emit,
-                                                       int scanned) {
+                                                       int scanned, float* aux_stats) {
   // partial sums of the tile histograms: [group][expert], "before my tile" and "all tiles"
   __shared__ int part_b[4 * kMaxE];   // flat [group][e]; groups * e <= 4 * kMaxE on every path
   __shared__ int part_t[4 * kMaxE];
@@ -569,6 +821,12 @@ __global__ __launch_bounds__(256) void permute_kernel(const int32_t* __restrict_
   __shared__ unsigned long long wmask[4][kMaxE];   // per wave and expert: the lanes assigned to it (current chunk)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int me = blockIdx.x;
+  if (aux_stats != nullptr && me == (int)gridDim.x - 1) {
+    // one workgroup past the tiles finishes the two losses (the scanned totals and the folded
+    // statistics are both complete before this launch starts)
+    aux_block_256(counts, aux_stats, n, e, k);
+    return;
+  }
 
   // the first chunk of this tile's assignments is fetched now, under the histogram loads
   const int64_t p0 = (int64_t)me * tile_rows * k;
@@ -711,23 +969,31 @@ int launch_route(const void* logits, int32_t* idx, float* weights, int32_t* hist
                  int64_t n, int e, int k, const Tiling& tl, hipStream_t st) {
   const T* lp = static_cast<const T*>(logits);
   const dim3 grid((unsigned)tl.ntiles);
+#define GOS(L_, VEC_, SEL_)                                                                           \
+  FM_LAUNCH((route_group_kernel<T, L_, VEC_, SEL_>), grid, dim3(kGroupThreads), 0, st, lp, idx, weights, \
+            hist, fstat, n, e, k, tl.tile_rows)
 #define GOG(L_)                                                                                       \
   do {                                                                                                \
-    if (vec && presort) FM_LAUNCH((route_group_kernel<T, L_, true, true>), grid, dim3(kGroupThreads), 0, st,   \
-                                  lp, idx, weights, hist, fstat, n, e, k, tl.tile_rows);             \
-    else if (vec) FM_LAUNCH((route_group_kernel<T, L_, true, false>), grid, dim3(kGroupThreads), 0, st,        \
-                            lp, idx, weights, hist, fstat, n, e, k, tl.tile_rows);                   \
-    else if (presort) FM_LAUNCH((route_group_kernel<T, L_, false, true>), grid, dim3(kGroupThreads), 0, st,    \
-                                lp, idx, weights, hist, fstat, n, e, k, tl.tile_rows);               \
-    else FM_LAUNCH((route_group_kernel<T, L_, false, false>), grid, dim3(kGroupThreads), 0, st,      \
-                   lp, idx, weights, hist, fstat, n, e, k, tl.tile_rows);                            \
+    if (vec && sel == kSelSorted) GOS(L_, true, kSelSorted);                                          \
+    else if (vec) GOS(L_, true, kSelScan);                                                            \
+    else if (sel == kSelSorted) GOS(L_, false, kSelSorted);                                           \
+    else GOS(L_, false, kSelScan);                                                                    \
   } while (0)
   const bool vec = e % kGE == 0 && fm_host::aligned16(logits);
-  const bool presort = k >= 5;   // at four picks the two forms tie, below that the sort does not pay
+  // Kernel time at 65536 rows, fp32, by picks (1 / 2 / 4 / 8), in microseconds:
+  //   128 experts: scan 15 / 17 / 21 / 27, sorted heads 17 / 18 / 20 / 22, candidates 24 at all four
+  //   256 experts: scan 22 / 26 / 33 / 46, sorted heads 27 / 28 / 31 / 35, candidates 31 at all four
+  //   512 experts (32768 rows): scan 25 / 29 / 38 / 56, sorted heads 30 / 32 / 35 / 43, candidates 42-44
+  // Up to 64 experts the scan and the sorted heads tie at four picks.
+  const int sel = k >= (e > 64 ? 4 : 5) ? kSelSorted : kSelScan;
   if (e <= 64) GOG(8);
   else if (e <= 128) GOG(16);
-  else if (e <= 256) GOG(32);
-  else GOG(64);
+  else if (e <= 256) {
+    if (k >= 5 && vec) GOS(32, true, kSelCands);
+    else if (k >= 5) GOS(32, false, kSelCands);
+    else GOG(32);
+  } else GOG(64);
+#undef GOS
 #undef GOG
   return FM_OK;
 }
@@ -776,30 +1042,37 @@ int fm_route(const void* logits, int32_t* idx, float* weights, int32_t* counts, 
   FM_CHECK_LAUNCH("fm_route");
   // few columns and tiles: the statistics are folded by the kernel that also finishes the losses
   const bool stats_late = stats != nullptr && e + 1 <= 128 && tl.ntiles <= 256;
-  if (stats != nullptr && !stats_late) {
-    hipLaunchKernelGGL(route_stats_kernel, dim3((unsigned)((e + 1 + 63) / 64)), dim3(1024), 0, st, fstat, stats,
-                       e, tl.ntiles);
-    FM_CHECK_LAUNCH("fm_route(stats)");
-  }
   const int emit = (slot != nullptr || order != nullptr) && n > 0 ? 1 : 0;
   // Many tiles times many experts: every permutation workgroup summing all histograms before
   // its own would read ntiles^2 * e integers in total; scan them once instead.
   const int scanned = (int64_t)tl.ntiles * e > 32768 ? 1 : 0;
-  if (scanned) {
-    hipLaunchKernelGGL(hist_scan_kernel, dim3((unsigned)((e + 15) / 16)), dim3(1024), 0, st, hist, counts, e,
-                       tl.ntiles);
+  const bool fold = stats != nullptr && !stats_late;
+  const unsigned scan_blocks = (unsigned)((e + 15) / 16), fold_blocks = (unsigned)((e + 1 + 63) / 64);
+  if (fold && scanned) {
+    hipLaunchKernelGGL(route_scan_stats_kernel, dim3(scan_blocks + fold_blocks), dim3(1024), 0, st, hist, counts,
+                       fstat, stats, e, tl.ntiles, (int)scan_blocks);
+    FM_CHECK_LAUNCH("fm_route(scan + stats)");
+  } else if (fold) {
+    hipLaunchKernelGGL(route_stats_kernel, dim3(fold_blocks), dim3(1024), 0, st, fstat, stats, e, tl.ntiles);
+    FM_CHECK_LAUNCH("fm_route(stats)");
+  } else if (scanned) {
+    hipLaunchKernelGGL(hist_scan_kernel, dim3(scan_blocks), dim3(1024), 0, st, hist, counts, e, tl.ntiles);
     FM_CHECK_LAUNCH("fm_route(scan)");
   }
+  // after a scan the totals are final before the permutation starts: its launch takes one more
+  // workgroup for the two losses
+  const bool aux_inside = fold && scanned && emit;
   if (emit || !scanned) {
-    hipLaunchKernelGGL(permute_kernel, dim3(emit ? (unsigned)tl.ntiles : 1u), dim3(256), 0, st, idx, hist,
-                       counts, slot, order, n, e, k, tl.tile_rows, tl.ntiles, emit, scanned);
+    hipLaunchKernelGGL(permute_kernel, dim3((emit ? (unsigned)tl.ntiles : 1u) + (aux_inside ? 1u : 0u)), dim3(256), 0,
+                       st, idx, hist, counts, slot, order, n, e, k, tl.tile_rows, tl.ntiles, emit, scanned,
+                       aux_inside ? stats : nullptr);
   }
   FM_CHECK_LAUNCH("fm_route(permute)");
   if (stats_late) {
     hipLaunchKernelGGL(route_stats_aux_kernel, dim3(1), dim3(1024), 0, st, fstat, counts, stats, n, e, k,
                        tl.ntiles);
     FM_CHECK_LAUNCH("fm_route(stats + aux)");
-  } else if (stats != nullptr) {
+  } else if (stats != nullptr && !aux_inside) {
     hipLaunchKernelGGL(route_aux_kernel, dim3(1), dim3(512), 0, st, counts, stats, n, e, k);
     FM_CHECK_LAUNCH("fm_route(aux)");
   }

@@ -988,12 +988,15 @@ def test_route_half_precision_logits_and_all_equal_rows():
 
 
 def test_route_pick_forms_on_special_rows():
-    """The router picks either by scanning a lane's eight keys per pick (up to four picks) or from
-    lane-sorted keys (from five picks on): both against the oracle on rows of equal logits, rows
-    with a single finite logit (the other picks tie at probability zero), few distinct values, and
-    NaN / +inf rows (all probabilities NaN: lowest experts win)."""
+    """The router picks by scanning a lane's eight keys per pick (few picks), from lane-sorted keys
+    (more picks), or, for 129-256 experts and five picks or more, by sorting the experts that reach a
+    lower bound of the k-th key across the lanes: all against the oracle on rows of equal logits
+    (every expert is a candidate: the list is taken in several rounds), rows with a single finite
+    logit (the other picks tie at probability zero), few distinct values, runs of equal logits of
+    every length around the row width, and NaN / +inf rows (all probabilities NaN: lowest experts
+    win)."""
     if True:
-        for e in (8, 60, 64, 130, 256, 512):
+        for e in (8, 60, 64, 130, 136, 200, 256, 512):
             lg = router_inputs(400, e, 1021)
             lg[0] = 0.25
             lg[1] = float("-inf")
@@ -1003,9 +1006,14 @@ def test_route_pick_forms_on_special_rows():
             lg[4, 1] = float("inf")
             lg[5] = float("-inf")
             lg[5, [0, e - 1]] = 2.0
+            # rows 6..: the m largest logits are equal, for m around 8, 24, 32, 56 and the row width
+            runs = [m for m in (7, 8, 9, 23, 24, 25, 31, 32, 33, 55, 56, 57, e - 1, e) if m <= e]
+            for i, m in enumerate(runs):
+                perm = torch.randperm(e, generator=gen(100 + i))
+                lg[6 + i, perm[:m]] = 9.0
             finite = torch.ones(400, dtype=torch.bool)
             finite[3] = finite[4] = False
-            for k in (1, 2, 5, 8):
+            for k in (1, 2, 4, 5, 8):
                 if k > e:
                     continue
                 out = _hip.route(lg.to(DEV), k, want_stats=True)
@@ -1015,6 +1023,7 @@ def test_route_pick_forms_on_special_rows():
                 assert torch.allclose(w[finite], ow, rtol=1e-5, atol=0), (e, k)
                 assert idx[3].tolist() == list(range(k)) and idx[4].tolist() == list(range(k)), (e, k)
                 assert torch.isnan(w[3]).all() and torch.isnan(w[4]).all()
+                assert torch.equal(out[2].cpu().long(), torch.bincount(idx.flatten(), minlength=e)), (e, k)
 
 
 def test_route_statistics_from_one_or_two_kernels():
