@@ -22,6 +22,13 @@ namespace {
 constexpr int kEH = 4;        // elements per lane per half
 constexpr int kBlock = 256;
 
+// Position of a row's token in its sequence. The entry points refuse more than 2^31 - 1 rows, so the
+// two divisions are 32-bit ones (a 64-bit division is some two hundred dependent instructions, paid
+// by every tile of every wave).
+__device__ __forceinline__ int token_of(int64_t row, int heads, int t_len) {
+  return (int)(((uint32_t)row / (uint32_t)heads) % (uint32_t)t_len);
+}
+
 template <typename T, typename WT, int G, bool BWD>
 __global__ __launch_bounds__(kBlock) void rope_kernel(const T* __restrict__ x, const WT* __restrict__ w,
                                                        const float* __restrict__ cosv,
@@ -45,7 +52,7 @@ __global__ __launch_bounds__(kBlock) void rope_kernel(const T* __restrict__ x, c
   for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
     const int64_t row = tile * RPB + rib;
     const bool valid = row < rows;
-    const int t = valid ? (int)((row / heads) % t_len) : 0;
+    const int t = valid ? token_of(row, heads, t_len) : 0;
     const T* xp = x + row * (int64_t)d;
     float x1[kEH], x2[kEH], c[kEH], s[kEH];
     float ss = 0.f;
@@ -174,7 +181,7 @@ __global__ __launch_bounds__(kBlock) void rope_vec_kernel(const T* __restrict__ 
     const int64_t row0 = (tile * RPB + rib) * H;
     const bool live = row0 < rows;
     const bool on = lane_on && live;
-    const int t = live ? (int)((row0 / heads) % t_len) : 0;
+    const int t = live ? token_of(row0, heads, t_len) : 0;
     float c[EPV], sn[EPV];
 #pragma unroll
     for (int e = 0; e < EPV; ++e) { c[e] = 0.f; sn[e] = 0.f; }
@@ -283,6 +290,22 @@ __global__ __launch_bounds__(kBlock) void rope_vec_kernel(const T* __restrict__ 
 // (the same columns of the other half) lives G / 2 lanes away and is fetched with lane-permute
 // instructions: the packed input vector in the forward (the partner's normalised value is then
 // recomputed from it and the partner's weights), the packed incoming gradient in the backward.
+// Sum over the g lanes of a group that starts at lane `base` (any g: the groups of a wave need not
+// be a power of two wide), in lane order; four fetches from other lanes in flight at a time.
+__device__ __forceinline__ float group_sum_any(float v, int base, int g) {
+  float t = 0.f;
+  const int last = base + g - 1;
+  for (int i = 0; i < g; i += 4) {
+    const int s0 = base + i;
+    float a[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) a[u] = __shfl(v, s0 + u < last ? s0 + u : last, 64);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) t += (i + u < g) ? a[u] : 0.f;
+  }
+  return t;
+}
+
 template <int HG>
 __device__ __forceinline__ uint32_t lane_xor(uint32_t v) {
   static_assert(HG == 2 || HG == 4, "partner two or four lanes away");
@@ -291,6 +314,10 @@ __device__ __forceinline__ uint32_t lane_xor(uint32_t v) {
   return (uint32_t)FM_DPP_I(FM_DPP_I((int)v, kDppHalfMirror), 0x1B);
 }
 
+// G = 0: the group width comes at run time (`g_any`, any even number up to 64: heads of 6, 10, 12,
+// 14, 20, 24 ... vectors, head sizes 48, 80, 96, 112, 160, 192 ... in bf16). A wave then holds
+// 64 / g heads, its last 64 % g lanes stay idle, the partner is fetched with ds_bpermute and the
+// sums over a head run over its lanes in order.
 template <typename T, typename WT, int G, bool BWD, int H>
 __global__ __launch_bounds__(kBlock) void rope_pair_kernel(const T* __restrict__ x, const WT* __restrict__ w,
                                                             const float* __restrict__ cosv,
@@ -299,12 +326,16 @@ __global__ __launch_bounds__(kBlock) void rope_pair_kernel(const T* __restrict__
                                                             float* __restrict__ rstd, T* __restrict__ out,
                                                             float* __restrict__ partial, int64_t rows,
                                                             int t_len, int heads, int d, float eps,
-                                                            int64_t tiles) {
+                                                            int64_t tiles, int g_any) {
   constexpr int EPV = Elem<T>::kVec;
-  constexpr int RPB = kBlock / G;
-  constexpr int HG = G / 2;
-  __shared__ float fold[BWD ? RPB * G * EPV : 1];
-  const int tid = threadIdx.x, rib = tid / G, l = tid % G;
+  __shared__ float fold[BWD ? kBlock * EPV : 1];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int g = G ? G : g_any;
+  const int gpw = 64 / g;                 // heads per wave
+  const int RPB = (kBlock / 64) * gpw;
+  const int HG = g / 2;
+  const bool used = lane < gpw * g;       // (every lane when g is a power of two)
+  const int rib = (tid >> 6) * gpw + (used ? lane / g : 0), l = used ? lane % g : 0;
   const int half = d / 2;                 // == HG * EPV
   const bool first = l < HG;              // this lane holds columns of the first half
   const int col = l * EPV;                // its columns inside the head
@@ -319,9 +350,19 @@ __global__ __launch_bounds__(kBlock) void rope_pair_kernel(const T* __restrict__
   for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
     // rows is a multiple of H and so is the number of heads of a token: the H rows exist
     // together and belong to one token
-    const int64_t row0 = (tile * RPB + rib) * H;
-    const bool live = row0 < rows;
-    const int t = live ? (int)((row0 / heads) % t_len) : 0;
+    // Power-of-two groups: the H rows of a group are consecutive heads of one token and share its
+    // cos / sin columns (rows and the heads of a token are multiples of H there). Other widths:
+    // the H rows lie RPB apart, so that each load instruction of a wave covers consecutive rows
+    // (whole 128-byte lines although a row is not a whole number of them), and every row fetches
+    // the columns of its own token.
+    constexpr bool SHARED = G != 0;
+    int64_t rowj[H];
+    bool livej[H];
+#pragma unroll
+    for (int j = 0; j < H; ++j) {
+      rowj[j] = SHARED ? (tile * RPB + rib) * H + j : (tile * H + j) * RPB + rib;
+      livej[j] = used && rowj[j] < rows;
+    }
     float c[EPV], sn[EPV];
     u32x4 rx[H], rg[BWD ? H : 1];
 #pragma unroll
@@ -330,30 +371,43 @@ __global__ __launch_bounds__(kBlock) void rope_pair_kernel(const T* __restrict__
 #pragma unroll
       for (int j = 0; j < H; ++j) rg[j] = u32x4{0u, 0u, 0u, 0u};
     }
-    if (live) {
-#pragma unroll
-      for (int j = 0; j < H; ++j) {
-        rx[j] = load16_stream(x + (row0 + j) * (int64_t)d + col);
-        if constexpr (BWD) rg[j] = load16_stream(dout + (row0 + j) * (int64_t)d + col);
-      }
-    }
-    load_f32_cols<T>(cosv + (int64_t)t * half + hcol, c);
-    load_f32_cols<T>(sinv + (int64_t)t * half + hcol, sn);
 #pragma unroll
     for (int j = 0; j < H; ++j) {
-      const int64_t row = row0 + j;
+      if (livej[j]) {
+        rx[j] = load16_stream(x + rowj[j] * (int64_t)d + col);
+        if constexpr (BWD) rg[j] = load16_stream(dout + rowj[j] * (int64_t)d + col);
+      }
+    }
+    if constexpr (SHARED) {
+      const int t = livej[0] ? token_of(rowj[0], heads, t_len) : 0;
+      load_f32_cols<T>(cosv + (int64_t)t * half + hcol, c);
+      load_f32_cols<T>(sinv + (int64_t)t * half + hcol, sn);
+    }
+#pragma unroll
+    for (int j = 0; j < H; ++j) {
+      const int64_t row = rowj[j];
+      const bool live = livej[j];
+      if constexpr (!SHARED) {
+        const int t = live ? token_of(row, heads, t_len) : 0;
+        load_f32_cols<T>(cosv + (int64_t)t * half + hcol, c);
+        load_f32_cols<T>(sinv + (int64_t)t * half + hcol, sn);
+      }
       float xv[EPV], o[EPV];
       Elem<T>::unpack(rx[j], xv);
       if constexpr (!BWD) {
         float ss = 0.f;
 #pragma unroll
         for (int e = 0; e < EPV; ++e) ss += xv[e] * xv[e];
-        ss = group_reduce<G, OpSum>(ss);
+        if constexpr (G != 0) ss = group_reduce<(G ? G : 2), OpSum>(ss);
+        else ss = group_sum_any(ss, lane - l, g);
         const float r = rsqrtf(ss / (float)d + eps);
         if (live && l == 0) rstd[row] = r;
         u32x4 pr;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) pr[q] = lane_xor<HG>(rx[j][q]);
+        for (int q = 0; q < 4; ++q) {
+          if constexpr (G != 0) pr[q] = lane_xor<(G ? G / 2 : 2)>(rx[j][q]);
+          else pr[q] = (uint32_t)__shfl((int)rx[j][q], first ? lane + HG : lane - HG, 64);
+        }
         float pv[EPV];
         Elem<T>::unpack(pr, pv);
 #pragma unroll
@@ -366,7 +420,10 @@ __global__ __launch_bounds__(kBlock) void rope_pair_kernel(const T* __restrict__
         const float r = live ? rstd[row] : 0.f;
         u32x4 pq;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) pq[q] = lane_xor<HG>(rg[j][q]);
+        for (int q = 0; q < 4; ++q) {
+          if constexpr (G != 0) pq[q] = lane_xor<(G ? G / 2 : 2)>(rg[j][q]);
+          else pq[q] = (uint32_t)__shfl((int)rg[j][q], first ? lane + HG : lane - HG, 64);
+        }
         float gv[EPV], pg[EPV];
         Elem<T>::unpack(rg[j], gv);
         Elem<T>::unpack(pq, pg);
@@ -380,7 +437,8 @@ __global__ __launch_bounds__(kBlock) void rope_pair_kernel(const T* __restrict__
           o[e] = dy * wo[e];
           dot += o[e] * xv[e];
         }
-        dot = group_reduce<G, OpSum>(dot);
+        if constexpr (G != 0) dot = group_reduce<(G ? G : 2), OpSum>(dot);
+        else dot = group_sum_any(dot, lane - l, g);
         const float cm = dot / (float)d;
 #pragma unroll
         for (int e = 0; e < EPV; ++e) o[e] = (o[e] - xv[e] * cm) * r;
@@ -391,13 +449,15 @@ __global__ __launch_bounds__(kBlock) void rope_pair_kernel(const T* __restrict__
   if constexpr (BWD) {
     if (partial == nullptr) return;
     // fold the rows of this workgroup in row order, then write one partial row
+    if (used) {
 #pragma unroll
-    for (int e = 0; e < EPV; ++e) fold[rib * G * EPV + col + e] = a[e];
+      for (int e = 0; e < EPV; ++e) fold[rib * g * EPV + col + e] = a[e];
+    }
     __syncthreads();
     float* prow = partial + (int64_t)blockIdx.x * d;
     for (int j = tid; j < d; j += kBlock) {
       float acc = 0.f;
-      for (int rr = 0; rr < RPB; ++rr) acc += fold[rr * G * EPV + j];
+      for (int rr = 0; rr < RPB; ++rr) acc += fold[rr * g * EPV + j];
       prow[j] = acc;
     }
   }
@@ -447,18 +507,42 @@ int launch(const Shape& sh, bool vec, const void* x, const void* w, const float*
     if (want >= 4 && (!BWD || pair) && heads % 4 == 0) hpg = 4;
     else if (want >= 2 && heads % 2 == 0) hpg = 2;
   }
-  const int rpb = kBlock / (pair ? 2 * sh.gv : (vec ? sh.gv : sh.g));
+  // other heads of up to fourteen vectors (head sizes 48, 80, 96, 112 in bf16): the same kernel with
+  // groups of exactly that many lanes. bf16 [.., 32, d], 2^27 elements, forward / backward in TB/s,
+  // against the vector kernel with the next power of two of lanes: d = 48: 3.8 / 4.4 against
+  // 2.0 / 2.6; 80: 3.7 / 4.4 against 3.0 / 3.6; 96: 3.9 / 4.6 against 3.9 / 4.4; 112: 3.6 / 4.3
+  // against 3.3 / 3.9; wider heads (160, 192) are faster there (4.3 / 4.3 and 4.9 / 4.9).
+  const int hv = vec ? (int)(d / Elem<T>::kVec) : 0;
+  const int g_any = (vec && !pair && hv <= 14 && (hv & (hv - 1)) != 0) ? hv : 0;
+  if (g_any) hpg = 2;
+  const int rpb = g_any ? (kBlock / 64) * (64 / g_any) : kBlock / (pair ? 2 * sh.gv : (vec ? sh.gv : sh.g));
   const int64_t tiles = (rows + (int64_t)rpb * hpg - 1) / ((int64_t)rpb * hpg);
   const int64_t blocks = sh.blocks < tiles ? sh.blocks : tiles;
+  int64_t used_blocks = blocks;
+  // The grid is persistent: no more workgroups than the device holds at once (a kernel whose
+  // registers allow seven per compute unit, launched with eight, runs the eighth after the others
+  // have finished their whole share: twice the time).
+#define GO_K(K, ...)                                                                                  \
+  do {                                                                                                \
+    static int occupancy = 0; /* workgroups of this kernel one compute unit holds, at most 8 */       \
+    if (occupancy == 0) {                                                                             \
+      int o = 0;                                                                                      \
+      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&o, K, kBlock, 0) != hipSuccess || o < 1) o = 8; \
+      occupancy = o > 8 ? 8 : o;                                                                      \
+    }                                                                                                 \
+    const int64_t fit = (int64_t)fm_host::num_cus() * occupancy;                                      \
+    used_blocks = blocks < fit ? blocks : fit;                                                        \
+    FM_LAUNCH(K, dim3((unsigned)used_blocks), dim3(kBlock), 0, st, __VA_ARGS__);                      \
+  } while (0)
 #define ARGS static_cast<const T*>(x), static_cast<const WT*>(w), c, s, static_cast<const T*>(dout), rstd, \
              static_cast<T*>(out), partial, rows, t_len, heads, d, eps, tiles
 #define GO_V(G)                                                                                           \
   do {                                                                                                    \
-    if (hpg == 1) FM_LAUNCH((rope_vec_kernel<T, WT, G, BWD, 1>), dim3((unsigned)blocks), dim3(kBlock), 0, st, ARGS); \
-    else if (hpg == 2) FM_LAUNCH((rope_vec_kernel<T, WT, G, BWD, 2>), dim3((unsigned)blocks), dim3(kBlock), 0, st, ARGS); \
-    else if constexpr (!BWD) FM_LAUNCH((rope_vec_kernel<T, WT, G, BWD, 4>), dim3((unsigned)blocks), dim3(kBlock), 0, st, ARGS); \
+    if (hpg == 1) GO_K((rope_vec_kernel<T, WT, G, BWD, 1>), ARGS);                                          \
+    else if (hpg == 2) GO_K((rope_vec_kernel<T, WT, G, BWD, 2>), ARGS);                                     \
+    else if constexpr (!BWD) GO_K((rope_vec_kernel<T, WT, G, BWD, 4>), ARGS);                               \
   } while (0)
-#define GO_S(G) FM_LAUNCH((rope_kernel<T, WT, G, BWD>), dim3((unsigned)blocks), dim3(kBlock), 0, st, ARGS)
+#define GO_S(G) GO_K((rope_kernel<T, WT, G, BWD>), ARGS)
 #define BY_G(GO, g)           \
   switch (g) {                \
     case 1: GO(1); break;     \
@@ -469,15 +553,16 @@ int launch(const Shape& sh, bool vec, const void* x, const void* w, const float*
     case 32: GO(32); break;   \
     default: GO(64); break;   \
   }
-  if (pair) {
-#define GO_P(G, H_) FM_LAUNCH((rope_pair_kernel<T, WT, G, BWD, H_>), dim3((unsigned)blocks), dim3(kBlock), 0, st, ARGS)
+  if (pair || g_any) {
+#define GO_P(G, H_) GO_K((rope_pair_kernel<T, WT, G, BWD, H_>), ARGS, g_any)
 #define GO_PH(G)                  \
   do {                            \
     if (hpg == 4) GO_P(G, 4);     \
     else if (hpg == 2) GO_P(G, 2);\
     else GO_P(G, 1);              \
   } while (0)
-    if (sh.gv == 2) GO_PH(4);
+    if (g_any) GO_PH(0);
+    else if (sh.gv == 2) GO_PH(4);
     else GO_PH(8);
 #undef GO_PH
 #undef GO_P
@@ -486,7 +571,8 @@ int launch(const Shape& sh, bool vec, const void* x, const void* w, const float*
 #undef GO_V
 #undef GO_S
 #undef ARGS
-  return (int)blocks;
+#undef GO_K
+  return (int)used_blocks;
 }
 
 int check(const char* what, int64_t b, int64_t t, int64_t h, int64_t d, int x_dtype, int w_dtype, Shape* sh) {

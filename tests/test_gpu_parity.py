@@ -1114,7 +1114,12 @@ def test_swiglu_split_fwd_bwd(rows, h, dt):
                                               # heads of four or eight vectors (one vector per lane, partner by lane
                                               # permute): 1, 2 and 4 heads per lane group, several tiles
                                               (2, 9, 6, 32, BF16, F32), (1, 5, 3, 32, BF16, BF16), (2, 7, 8, 16, BF16, F32),
-                                              (3, 4, 5, 16, F32, F32), (2, 300, 8, 32, BF16, F32), (1, 130, 2, 8, F32, F32)])
+                                              (3, 4, 5, 16, F32, F32), (2, 300, 8, 32, BF16, F32), (1, 130, 2, 8, F32, F32),
+                                              # halves of 5, 6, 3, 7 and 12 vectors (head sizes 80, 96, 48, 112, 192; 24 in
+                                              # fp32): lane groups of exactly that width, idle lanes at the end of a wave,
+                                              # odd and even head counts, several tiles
+                                              (2, 37, 8, 40, BF16, F32), (1, 301, 3, 48, BF16, BF16), (2, 9, 4, 24, F16, F16),
+                                              (1, 50, 6, 56, BF16, F32), (2, 11, 2, 96, BF16, F32), (3, 21, 5, 12, F32, F32)])
 def test_qk_norm_rope_fwd_bwd(b, t, h, hd, dt, wdt):
     # shapes of reference tests/kernel_interp_check.py:82-89, then realistic head sizes
     g = gen(41)
