@@ -306,29 +306,38 @@ def kl_div_logits_topk(student: torch.Tensor, teacher: torch.Tensor, k: int,
                               index_dtype, bool(retain))
 
 
+def _distill_piece(rows_s: torch.Tensor, rows_t: torch.Tensor, w_t: torch.Tensor, teacher_head) -> torch.Tensor:
+    """Summed KL of one block of rows. The student logits of the block are a temporary of this
+    call, so the kernel may write their gradient over them (``reuse=True``)."""
+    with torch.no_grad():
+        teacher_logits = teacher_head(rows_t)
+    student_logits = rows_s @ w_t
+    return kl_div_logits(student_logits, teacher_logits.detach().to(student_logits.dtype), "sum", reuse=True)
+
+
 def kl_distill_loss(hs: torch.Tensor, ht: torch.Tensor, w: torch.Tensor, teacher_head,
                     chunk: int = 4096) -> torch.Tensor:
-    """Mean forward KL of ``softmax(teacher_head(ht)) || softmax(hs @ w.T)`` in row chunks.
+    """Mean forward KL of ``softmax(teacher_head(ht)) || softmax(hs @ w.T)`` over all rows, computed
+    ``chunk`` rows at a time (call surface and meaning of the reference's ``kernels/kl.py:209-233``).
 
-    Same structure as the reference's ``kl.py:209-233``: the teacher head runs under
-    ``no_grad``; one chunk of student logits exists at a time in the forward, and its gradient
-    is written over it (``reuse=True``, as in the reference).
+    The teacher head runs under ``no_grad``. Only one block of student logits exists at a time in
+    the forward; what each block leaves behind for the backward is its gradient buffer (the
+    logits' own storage), so with a student that needs gradients the blocks add up to N x V again,
+    as the reference's docstring says of its own.
     """
-    hs2 = hs.reshape(-1, hs.shape[-1])
-    ht2 = ht.reshape(-1, ht.shape[-1])
-    n = hs2.shape[0]
-    total = None
-    for lo in range(0, n, chunk):
-        hi = min(n, lo + chunk)
-        with torch.no_grad():
-            t_log = teacher_head(ht2[lo:hi]).detach()
-        s_log = hs2[lo:hi] @ w.t()
-        # the chunk's student logits are a temporary of this loop: the gradient may overwrite them
-        piece = kl_div_logits(s_log, t_log.to(s_log.dtype), "sum", reuse=True)
-        total = piece if total is None else total + piece
-    if total is None:
-        return hs2.new_zeros((), dtype=torch.float32)
-    return total / n
+    if chunk < 1:
+        raise ValueError(f"chunk must be positive, got {chunk}")
+    student_rows = hs.flatten(0, -2) if hs.dim() > 1 else hs.unsqueeze(0)
+    teacher_rows = ht.flatten(0, -2) if ht.dim() > 1 else ht.unsqueeze(0)
+    n = student_rows.size(0)
+    if teacher_rows.size(0) != n:
+        raise ValueError(f"student has {n} rows, teacher {teacher_rows.size(0)}")
+    if n == 0:
+        return student_rows.new_zeros((), dtype=torch.float32)
+    w_t = w.t()
+    pieces = [_distill_piece(s_blk, t_blk, w_t, teacher_head)
+              for s_blk, t_blk in zip(student_rows.split(chunk), teacher_rows.split(chunk))]
+    return torch.stack(pieces).sum() / n
 
 
 kl_div = kl_div_logits
