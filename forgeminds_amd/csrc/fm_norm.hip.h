@@ -353,7 +353,10 @@ __global__ __launch_bounds__(kBwdBlock) void norm_bwd_kernel(
 template <typename WT>
 __global__ __launch_bounds__(1024) void colsum_kernel(const float* __restrict__ partial,
                                                        WT* __restrict__ dw, int p, int d,
-                                                       int stride) {
+                                                       int stride, WT* __restrict__ dw_second) {
+  // a launch with two rows of workgroups sums two column sets at once: the second row takes the
+  // columns d .. 2d - 1 of every partial row into `dw_second` (LayerNorm: weight and bias gradient)
+  if (blockIdx.y == 1) { partial += d; dw = dw_second; }
   __shared__ float s[64][64 + 4];
   const int q = threadIdx.x & 15;
   const int g = threadIdx.x >> 4;
@@ -395,7 +398,8 @@ __global__ __launch_bounds__(1024) void colsum_kernel(const float* __restrict__ 
 template <typename WT>
 __global__ __launch_bounds__(1024) void colsum_scalar_kernel(const float* __restrict__ partial,
                                                               WT* __restrict__ dw, int p, int d,
-                                                              int stride) {
+                                                              int stride, WT* __restrict__ dw_second) {
+  if (blockIdx.y == 1) { partial += d; dw = dw_second; }
   __shared__ float s[16][64];
   const int lane = threadIdx.x & 63;
   const int g = threadIdx.x >> 6;
@@ -535,7 +539,8 @@ __global__ __launch_bounds__(256) void dw_generic(const T* __restrict__ x,
 template <typename WT>
 __global__ __launch_bounds__(1024) void colsum16_kernel(const float* __restrict__ partial,
                                                          WT* __restrict__ dw, int p, int d,
-                                                         int stride) {
+                                                         int stride, WT* __restrict__ dw_second) {
+  if (blockIdx.y == 1) { partial += d; dw = dw_second; }
   __shared__ float s[256][16 + 1];
   __shared__ float s2[16][16 + 1];
   const int q = threadIdx.x & 3;
@@ -1069,22 +1074,26 @@ int launch_bwd(const Plan& p, const void* x, const void* w, const float* mean, c
     }
   }
   if (partial != nullptr) {
-    const dim3 grid((unsigned)((d + 63) / 64));
+    // LayerNorm with both parameter gradients wanted: one launch, two rows of workgroups
+    const bool both = LN && dw != nullptr && db != nullptr;
     void* outs[2] = {dw, LN ? db : nullptr};
-    for (int which = 0; which < (LN ? 2 : 1); ++which) {
+    for (int which = 0; which < (LN && !both ? 2 : 1); ++which) {
       if (outs[which] == nullptr) continue;
       const float* src = partial + (int64_t)which * d;
+      WT* first = static_cast<WT*>(outs[which]);
+      WT* second = both ? static_cast<WT*>(db) : nullptr;
+      const unsigned gy = both ? 2u : 1u;
       // narrow weights: 16 columns a workgroup, so that a column sum of few columns still spreads
       // over the device (no difference from 8192 columns on)
       if (d % 4 == 0 && d <= 4096)
-        hipLaunchKernelGGL((colsum16_kernel<WT>), dim3((unsigned)((d + 15) / 16)), dim3(1024), 0, st, src,
-                           static_cast<WT*>(outs[which]), p.bwd_blocks, (int)d, pcols);
+        hipLaunchKernelGGL((colsum16_kernel<WT>), dim3((unsigned)((d + 15) / 16), gy), dim3(1024), 0, st, src,
+                           first, p.bwd_blocks, (int)d, pcols, second);
       else if (d % 4 == 0)
-        hipLaunchKernelGGL((colsum_kernel<WT>), grid, dim3(1024), 0, st, src, static_cast<WT*>(outs[which]),
-                           p.bwd_blocks, (int)d, pcols);
+        hipLaunchKernelGGL((colsum_kernel<WT>), dim3((unsigned)((d + 63) / 64), gy), dim3(1024), 0, st, src, first,
+                           p.bwd_blocks, (int)d, pcols, second);
       else
-        hipLaunchKernelGGL((colsum_scalar_kernel<WT>), grid, dim3(1024), 0, st, src,
-                           static_cast<WT*>(outs[which]), p.bwd_blocks, (int)d, pcols);
+        hipLaunchKernelGGL((colsum_scalar_kernel<WT>), dim3((unsigned)((d + 63) / 64), gy), dim3(1024), 0, st, src,
+                           first, p.bwd_blocks, (int)d, pcols, second);
     }
   }
   return FM_OK;

@@ -647,10 +647,10 @@ int fm_qk_norm_rope_bwd(const void* x, const void* w, const float* cosv, const f
   if (partial != nullptr) {                                                                            \
     if (d % 4 == 0)                                                                                    \
       hipLaunchKernelGGL((colsum_kernel<WT>), dim3((unsigned)((d + 63) / 64)), dim3(1024), 0, st,       \
-                         partial, static_cast<WT*>(dw), used, (int)d, (int)d);                         \
+                         partial, static_cast<WT*>(dw), used, (int)d, (int)d, static_cast<WT*>(nullptr));                         \
     else                                                                                               \
       hipLaunchKernelGGL((colsum_scalar_kernel<WT>), dim3((unsigned)((d + 63) / 64)), dim3(1024), 0, st, \
-                         partial, static_cast<WT*>(dw), used, (int)d, (int)d);                         \
+                         partial, static_cast<WT*>(dw), used, (int)d, (int)d, static_cast<WT*>(nullptr));                         \
   }
   if (x_dtype == FM_F32) { CALL(float, float); }
   else if (x_dtype == FM_BF16 && w_dtype == FM_BF16) { CALL(bf16_t, bf16_t); }
