@@ -501,7 +501,10 @@ int launch(const void* x, void* values, void* indices, int64_t n, int v, int k, 
   FM_LAUNCH((topk_lds_kernel<T, TH, UN, BIG_>), grid, dim3(TH), (size_t)(nvec + 8) * 2, st, xp, vp, \
                      i32, i64, v, k, vec_ok)
   const bool big = k > 256;               // twice the candidate slots (1024-thread forms only)
-  int variant = nvec <= 3072 ? 1 : (nvec <= 12288 ? 2 : 3);
+  // 512 threads up to 140 K bf16 columns: three such workgroups share a compute unit, and while one
+  // is in its selection phases two keep the loads going (top-64 of [4096,128256]: 163 against 166.5 us
+  // with 1024 threads, k = 256: 215 against 254; at 152 K columns only two fit and 1024 threads win)
+  int variant = nvec <= 3072 ? 1 : (nvec <= 17600 ? 2 : 3);
   {
     // The threshold search needs k <= 63 x (full waves of the row); more threads give more of
     // them while the row has a vector for each, and it pays while k stays within half of that
