@@ -333,7 +333,8 @@ def make_workload(name, torch, L, dev):
         w.check = check
         w.step = step
         w.dominant_launch = bwd
-        w.dominant = "norm_bwd_kernel<bf16,f32,512,2,LN> + 2 colsum_kernel"
+        w.floor = [lambda i: ((x, dl), (xn, y)), lambda i: ((xn, gy, gxn), (dx,))]
+        w.dominant = "norm_bwd_kernel<bf16,f32,512,2,LN> + colsum_kernel"
         w.dominant_bytes = n * d * 8
         w.bytes = n * d * 16
         w.desc = f"add-LayerNorm fwd+bwd x,delta bf16 [{n},{d}], w,b fp32, eps 1e-5, with residual grad"
@@ -609,6 +610,9 @@ def make_workload(name, torch, L, dev):
         w.step = step
         w.dominant_launch = bwd
         w.dominant = "swiglu_split_bwd_kernel<bf16>"
+        xa, xb = x.view(-1)[:rows * h], x.view(-1)[rows * h:]      # streams of the size of gate and up
+        da, db_ = dx.view(-1)[:rows * h], dx.view(-1)[rows * h:]
+        w.floor = [lambda i: ((xa, xb), (y,)), lambda i: ((xa, xb, dy), (da, db_))]
         w.dominant_bytes = rows * h * 2 * 5          # gate, up, dy in; dgate, dup out
         w.bytes = rows * h * 2 * 8                   # + gate, up in; y out
         w.desc = f"SwiGLU on a fused projection fwd+bwd, x bf16 [{rows},{2 * h}] -> y [{rows},{h}]"
@@ -654,6 +658,7 @@ def make_workload(name, torch, L, dev):
         w.check = check
         w.step = step
         w.dominant_launch = bwd
+        w.floor = [lambda i: ((x,), (out,)), lambda i: ((x, do), (dx,))]
         w.dominant = "qk_norm_rope_bwd_kernel<bf16,f32>"
         w.dominant_bytes = b * t * hh * d * 2 * 3
         w.bytes = b * t * hh * d * 2 * 5
@@ -817,6 +822,8 @@ def make_workload(name, torch, L, dev):
         w.check = check
         w.step = step
         w.dominant_launch = combine
+        xs_a, xs_b = xs[:n], xs[n:]
+        w.floor = [lambda i: ((x,), (xs_a, xs_b)), lambda i: ((xs_a, xs_b), (out,))]
         w.dominant = "combine_kernel<bf16>"
         w.dominant_bytes = n * d * 2 * (k + 1)
         w.bytes = 2 * n * d * 2 * (k + 1)

@@ -109,7 +109,7 @@ int launch_mix(int reads, int writes, const u32x4* a, const u32x4* b, const u32x
                        st, a, b, c, o1, o2, sink, tiles, store_kind);                           \
     return FM_OK;                                                                               \
   }
-  GO(1, 0) GO(2, 0) GO(1, 1) GO(2, 1) GO(3, 1) GO(1, 2) GO(2, 2)
+  GO(1, 0) GO(2, 0) GO(3, 0) GO(1, 1) GO(2, 1) GO(3, 1) GO(1, 2) GO(2, 2) GO(3, 2)
 #undef GO
   fm_host::set_error("fm_stream_probe_mix: no kernel for %d reads + %d writes", reads, writes);
   return FM_ERR_UNSUPPORTED;
