@@ -117,14 +117,37 @@ __device__ __forceinline__ void kl_merge(const KLState& k, float* smem, float* l
   *kl2 = A / Dt - *l2t + *l2s;
 }
 
-// One sweep over a row that writes (softmax(s) - softmax(t)) * mul from the row's base-2
-// log-sum-exps: the body of the backward, shared by the kernels that append it to a forward.
+// (softmax(s) - softmax(t)) * mul of one 16-byte vector of each, from the row's base-2 log-sum-exps.
+template <typename T, typename GT>
+__device__ __forceinline__ void kl_grad_vec(const u32x4& rs, const u32x4& rt, GT* dst, float c1, float l2s,
+                                            float l2t, float mul) {
+  constexpr int EPV = Elem<T>::kVec;
+  float zs[EPV], zt[EPV], o[EPV];
+  Elem<T>::unpack(rs, zs);
+  Elem<T>::unpack(rt, zt);
+#pragma unroll
+  for (int e = 0; e < EPV; ++e)
+    o[e] = (fast_exp2(zs[e] * c1 - l2s) - fast_exp2(zt[e] * c1 - l2t)) * mul;
+  if constexpr (sizeof(GT) == sizeof(T)) {
+    store16_stream(dst, Elem<GT>::pack(o));
+  } else {  // fp32 gradient next to 16-bit logits: two 16-byte stores
+    static_assert(sizeof(GT) == 4 && EPV == 8, "gradient is the logits' dtype or fp32");
+    float lo[4] = {o[0], o[1], o[2], o[3]}, hi[4] = {o[4], o[5], o[6], o[7]};
+    store16_stream(dst, Elem<float>::pack(lo));
+    store16_stream(dst + 4, Elem<float>::pack(hi));
+  }
+}
+
+// One sweep over a row (from vector c_begin on) that writes (softmax(s) - softmax(t)) * mul from the
+// row's base-2 log-sum-exps: the body of the backward, shared by the kernels that append it to a
+// forward.
 template <typename T, typename GT, int THREADS, int UNROLL>
 __device__ __forceinline__ void kl_grad_sweep(const T* sp_, const T* tp_, GT* gp, const RowSplit& sp,
-                                              int v, float c1, float l2s, float l2t, float mul) {
+                                              int v, float c1, float l2s, float l2t, float mul,
+                                              int c_begin = 0) {
   constexpr int EPV = Elem<T>::kVec;
   const int tid = threadIdx.x;
-  for (int c0 = 0; c0 < sp.nvec; c0 += THREADS * UNROLL) {
+  for (int c0 = c_begin; c0 < sp.nvec; c0 += THREADS * UNROLL) {
     u32x4 rs[UNROLL], rt[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
@@ -591,6 +614,109 @@ __global__ __launch_bounds__(THREADS) void kl_loss_grad_wide_kernel(const T* stu
     row_kl[row] = kl2 * kLn2;
   }
   kl_grad_sweep<T, GT, THREADS, UNROLL>(sp_, tp_, gp, sp, v, c1, l2s, l2t, mul);
+}
+
+// The same for rows that fit the CHIP: one 512-thread workgroup per compute unit has 256 registers a
+// thread and 128 KB of LDS to itself, which hold 24 + 8 vectors of each row per thread, 16384 vector
+// pairs (a 131072-column bf16 pair of rows, 512 KB) in all. The row is then read from memory once:
+// 6 bytes per logit pair cross the L2 boundary instead of the 10 of the two sweeps above (which run
+// at the bandwidth of that boundary). Vectors past the 16384th, if any, are streamed and re-read
+// as above. Every thread parks and fetches only its own LDS slots: no barrier between the passes.
+constexpr int kHeldThreads = 512;
+constexpr int kHeldRegs = 24;    // vector pairs a thread keeps in registers
+constexpr int kHeldLds = 8;      // and in LDS
+template <typename T, typename GT>
+__global__ __launch_bounds__(kHeldThreads) void kl_loss_grad_held_kernel(const T* student,
+                                                                          const T* __restrict__ teacher,
+                                                                          float* __restrict__ lse_s,
+                                                                          float* __restrict__ lse_t,
+                                                                          float* __restrict__ row_kl,
+                                                                          GT* dstudent, int v, float inv_temp,
+                                                                          float mul, bool vec_ok) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int THREADS = kHeldThreads, RI = kHeldRegs, LI = kHeldLds;
+  constexpr int NW = THREADS / 64;
+  extern __shared__ u32x4 parked[];          // [LI][2][THREADS]
+  __shared__ float smem[5 * NW];
+  const int64_t row = blockIdx.x;
+  const T* sp_ = student + row * (int64_t)v;
+  const T* tp_ = teacher + row * (int64_t)v;
+  GT* gp = dstudent + row * (int64_t)v;
+  const RowSplit sp = split_row<EPV>(row, v, vec_ok);
+  const int tid = threadIdx.x;
+  const int ne = edge_count(sp, v);
+  const float c1 = kLog2e * inv_temp;
+
+  // all of a thread's loads are issued before the first is used
+  u32x4 hs[RI], ht[RI];
+#pragma unroll
+  for (int i = 0; i < RI; ++i) {
+    const int c = clamp_col(i * THREADS + tid, sp.nvec);
+    hs[i] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
+    ht[i] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
+  }
+  KLState k{kNegBig, 0.f, kNegBig, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < LI; j += 2) {
+    u32x4 rs[2], rt[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = clamp_col((RI + j + u) * THREADS + tid, sp.nvec);
+      rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
+      rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
+    }
+    kl_update<T, 2>(k, rs, rt, (RI + j) * THREADS + tid, THREADS, sp.nvec, c1);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      parked[((j + u) * 2 + 0) * THREADS + tid] = rs[u];
+      parked[((j + u) * 2 + 1) * THREADS + tid] = rt[u];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < RI; i += 2) {
+    const u32x4 rs[2] = {hs[i], hs[i + 1]}, rt[2] = {ht[i], ht[i + 1]};
+    kl_update<T, 2>(k, rs, rt, i * THREADS + tid, THREADS, sp.nvec, c1);
+  }
+  constexpr int HELD = (RI + LI) * THREADS;
+  for (int c0 = HELD; c0 < sp.nvec; c0 += THREADS * 2) {
+    u32x4 rs[2], rt[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      rs[u] = load16(sp_ + sp.head + (int64_t)c * EPV);
+      rt[u] = load16(tp_ + sp.head + (int64_t)c * EPV);
+    }
+    kl_update<T, 2>(k, rs, rt, c0 + tid, THREADS, sp.nvec, c1);
+  }
+  for (int e = tid; e < ne; e += THREADS) {
+    const int col = edge_col(sp, e);
+    kl_update1(k, Elem<T>::load1(sp_ + col) * c1, Elem<T>::load1(tp_ + col) * c1);
+  }
+  float l2s, l2t, kl2;
+  kl_merge<NW>(k, smem, &l2s, &l2t, &kl2);
+  if (tid == 0) {
+    if (lse_s != nullptr) lse_s[row] = l2s * kLn2;
+    if (lse_t != nullptr) lse_t[row] = l2t * kLn2;
+    row_kl[row] = kl2 * kLn2;
+  }
+#pragma unroll
+  for (int i = 0; i < RI; ++i) {
+    const int c = i * THREADS + tid;
+    // (behind an empty asm, so that the compiler unpacks the vector again here instead of keeping
+    // the floats of the first pass alive for all 24 pairs)
+    touch(hs[i]);
+    touch(ht[i]);
+    if (c < sp.nvec) kl_grad_vec<T, GT>(hs[i], ht[i], gp + sp.head + (int64_t)c * EPV, c1, l2s, l2t, mul);
+  }
+#pragma unroll
+  for (int j = 0; j < LI; ++j) {
+    const int c = (RI + j) * THREADS + tid;
+    if (c < sp.nvec)
+      kl_grad_vec<T, GT>(parked[(j * 2 + 0) * THREADS + tid], parked[(j * 2 + 1) * THREADS + tid],
+                         gp + sp.head + (int64_t)c * EPV, c1, l2s, l2t, mul);
+  }
+  // what was not held, and the row's unaligned edges
+  kl_grad_sweep<T, GT, THREADS, 2>(sp_, tp_, gp, sp, v, c1, l2s, l2t, mul, HELD < sp.nvec ? HELD : sp.nvec);
 }
 
 // Narrow rows (at most 1024 classes: classifier distillation, not vocabularies): TPR lanes per
@@ -1068,10 +1194,28 @@ int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, floa
                         fm_host::aligned16(dstudent);
     const float mul_w = inv_temperature * scale;
     const dim3 wgrid((unsigned)n);
+    // Aligned rows of the right width: the form that keeps the row pair on the chip (a workgroup per
+    // compute unit with 128 KB of LDS, which the device has to grant once per kernel). It reads the
+    // row once where the two sweeps read it twice, but leaves a compute unit one workgroup of eight
+    // waves, and the 16-bit rows are bound by their four exponentials per logit pair as much as by
+    // bytes. Measured against the two sweeps (us, 2^28 bf16 or 2^27 fp32 logits per tensor):
+    //   bf16 columns  40000: 530 / 381   65536: 417 / 370   100000: 376 / 372   110000: 411 / 373
+    //                128256: 355 / 372  151936: 312 / 338   180000: 351 / 363   200000: 385 / 382
+    //                262144: 437 / 420
+    //   fp32 columns  20000: 375 / 336   30000: 331 / 358    40000: 311 / 368    65536: 342 / 379
+    //                128256: 322 / 409  262144: 386 / 440
+    const int64_t wvec = v / (dtype == FM_F32 ? 4 : 8);
+    const bool held = vec_ok && (dtype == FM_F32 ? wvec >= 7168 : (wvec >= 15360 && wvec <= 24576));
 #define WIDE(T, GT)                                                                                \
-  FM_LAUNCH((kl_loss_grad_wide_kernel<T, GT, 1024, 2>), wgrid, dim3(1024), 0, st,         \
-                     static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t,  \
-                     row_kl, static_cast<GT*>(dstudent), (int)v, inv_temperature, mul_w, vec_ok)
+  if (held && fm_host::allow_wide_lds<&kl_loss_grad_held_kernel<T, GT>>())                         \
+    FM_LAUNCH((kl_loss_grad_held_kernel<T, GT>), wgrid, dim3(kHeldThreads),                        \
+              (size_t)kHeldLds * 2 * kHeldThreads * 16, st, static_cast<const T*>(student),        \
+              static_cast<const T*>(teacher), lse_s, lse_t, row_kl, static_cast<GT*>(dstudent),    \
+              (int)v, inv_temperature, mul_w, vec_ok);                                             \
+  else                                                                                             \
+    FM_LAUNCH((kl_loss_grad_wide_kernel<T, GT, 1024, 2>), wgrid, dim3(1024), 0, st,                \
+              static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t,        \
+              row_kl, static_cast<GT*>(dstudent), (int)v, inv_temperature, mul_w, vec_ok)
     FM_KL_BY_DTYPES(dtype, grad_dtype, WIDE);
 #undef WIDE
     FM_CHECK_LAUNCH("fm_kl_loss_grad");

@@ -468,7 +468,11 @@ KL1_CASES = [(64, 32000, BF16, 2.0, BF16), (6, 5000, F32, 1.0, F32), (3, 1, F32,
              (37, 2048, BF16, 1.5, F32), (33, 96, F32, 1.0, F32), (19, 1024, F32, 2.0, F32),
              # rows past the register path: two sweeps in one launch
              (4, 70000, BF16, 2.0, BF16), (3, 40000, F32, 1.0, F32), (3, 128256, BF16, 2.0, F32),
-             (5, 65537, F16, 1.0, F16)]
+             (5, 65537, F16, 1.0, F16),
+             # rows that stay on the chip between the passes (registers + LDS of one workgroup per
+             # compute unit): aligned and odd widths, in place, and rows past what the chip holds
+             (3, 128256, BF16, 1.0, BF16), (2, 151937, F16, 2.0, F16), (2, 140000, F32, 1.0, F32),
+             (2, 196608, BF16, 1.0, BF16), (3, 28673, F32, 2.0, F32)]
 
 
 @pytest.mark.parametrize("n,v,dt,T,gdt", KL1_CASES)
