@@ -453,6 +453,137 @@ __global__ __launch_bounds__(THREADS) void ce_loss_grad_kernel(const T* logits,
   }
 }
 
+// The same for rows past eight vectors a thread that still fit the CHIP: a 1024-thread workgroup, one
+// per compute unit, keeps 16 vectors a thread in registers and 8 more in 128 KB of LDS (every thread
+// parks and fetches its own slots only: no barrier for them): 24576 vectors, 196608 bf16 columns, the
+// vocabularies of 100 K to 152 K entries among them. One read and one write of the row, where the two
+// sweeps of ce_loss_grad_wide_kernel read it twice.
+constexpr int kCeHeldThreads = 1024;
+constexpr int kCeHeldRegs = 16;
+constexpr int kCeHeldLds = 8;
+constexpr int kCeHeldMaxVec = kCeHeldThreads * (kCeHeldRegs + kCeHeldLds);
+template <typename T>
+__global__ __launch_bounds__(kCeHeldThreads) void ce_loss_grad_held_kernel(const T* logits,
+                                                                            const int64_t* __restrict__ labels,
+                                                                            const float* __restrict__ n_valid,
+                                                                            float* __restrict__ lse,
+                                                                            float* __restrict__ row_loss,
+                                                                            T* dlogits, int v,
+                                                                            int64_t ignore_index) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int THREADS = kCeHeldThreads, RI = kCeHeldRegs, LI = kCeHeldLds;
+  constexpr int NW = THREADS / 64;
+  extern __shared__ u32x4 parked[];          // [LI][THREADS]
+  __shared__ float smem[2 * NW];
+  const int64_t row = blockIdx.x;
+  const T* rp = logits + row * (int64_t)v;
+  T* gp = dlogits + row * (int64_t)v;
+  const RowSplit sp = split_row<EPV>(row, v, true);
+  const int tid = threadIdx.x;
+  const int ne = edge_count(sp, v);
+  const int64_t y64 = labels[row];
+
+  if (y64 == ignore_index) {  // ignored row: zeros, and the logits are never read
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    for (int c = tid; c < sp.nvec; c += THREADS) store16_stream(gp + sp.head + (int64_t)c * EPV, zero);
+    for (int e = tid; e < ne; e += THREADS) Elem<T>::store1(gp + edge_col(sp, e), 0.f);
+    if (tid == 0) {
+      row_loss[row] = 0.f;
+      if (lse != nullptr) lse[row] = 0.f;
+    }
+    return;
+  }
+  const int y = (y64 >= 0 && y64 < v) ? (int)y64 : -1;
+  float ylogit = 0.f;
+  if (tid == 0 && y >= 0) ylogit = Elem<T>::load1(rp + y);   // early: overlaps the row loads
+
+  // every load of the thread is issued before the first is used (clamped columns: no load sits
+  // behind a branch); the LDS share is parked as it arrives
+  u32x4 raw[RI];
+#pragma unroll
+  for (int i = 0; i < RI; ++i)
+    raw[i] = load16_stream(rp + sp.head + (int64_t)clamp_col(i * THREADS + tid, sp.nvec) * EPV);
+  {
+    u32x4 late[LI];
+#pragma unroll
+    for (int j = 0; j < LI; ++j)
+      late[j] = load16_stream(rp + sp.head + (int64_t)clamp_col((RI + j) * THREADS + tid, sp.nvec) * EPV);
+#pragma unroll
+    for (int j = 0; j < LI; ++j) parked[j * THREADS + tid] = late[j];
+  }
+  float edge = -INFINITY;
+  int edge_at = -1;
+  if (tid < ne) {
+    edge_at = edge_col(sp, tid);
+    edge = Elem<T>::load1(rp + edge_at) * kLog2e;
+  }
+  // maximum first, then the sum: the data sits on the chip, a second sweep costs no traffic.
+  // Each pass unpacks afresh (behind an empty asm): converted floats kept from pass to pass would
+  // take the registers the row itself needs.
+  float mz = fmaxf(edge, kNegBig);
+#pragma unroll
+  for (int i = 0; i < RI + LI; ++i) {
+    const int c = i * THREADS + tid;
+    if (c < sp.nvec) {
+      u32x4 r;
+      if (i < RI) { touch(raw[i < RI ? i : 0]); r = raw[i < RI ? i : 0]; }
+      else r = parked[(i - RI) * THREADS + tid];
+      float z[EPV];
+      Elem<T>::unpack(r, z);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) mz = fmaxf(mz, z[e] * kLog2e);
+    }
+  }
+  float ssum = edge_at >= 0 ? fast_exp2(edge - mz) : 0.f;
+#pragma unroll
+  for (int i = 0; i < RI + LI; ++i) {
+    const int c = i * THREADS + tid;
+    if (c < sp.nvec) {
+      u32x4 r;
+      if (i < RI) { touch(raw[i < RI ? i : 0]); r = raw[i < RI ? i : 0]; }
+      else r = parked[(i - RI) * THREADS + tid];
+      float z[EPV];
+      Elem<T>::unpack(r, z);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) ssum += fast_exp2(z[e] * kLog2e - mz);
+    }
+  }
+  const MaxSum tot = block_merge<NW>(MaxSum{mz, ssum}, smem);
+  const float l2 = tot.m + fast_log2(tot.s);
+  const float scale = 1.f / (n_valid != nullptr ? *n_valid : 1.f);
+  if (tid == 0) {
+    const float l = l2 * kLn2;
+    if (lse != nullptr) lse[row] = l;
+    row_loss[row] = y >= 0 ? l - ylogit : __builtin_nanf("");
+  }
+#pragma unroll
+  for (int i = 0; i < RI + LI; ++i) {
+    const int c = i * THREADS + tid;
+    if (c < sp.nvec) {
+      u32x4 r;
+      if (i < RI) { touch(raw[i < RI ? i : 0]); r = raw[i < RI ? i : 0]; }
+      else r = parked[(i - RI) * THREADS + tid];
+      float z[EPV], o[EPV];
+      Elem<T>::unpack(r, z);
+      const int col0 = sp.head + c * EPV;
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) o[e] = fast_exp2(z[e] * kLog2e - l2);
+      if (y >= col0 && y < col0 + EPV) {
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] -= (col0 + e == y) ? 1.f : 0.f;
+      }
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) o[e] *= scale;
+      store16_stream(gp + col0, Elem<T>::pack(o));
+    }
+  }
+  if (edge_at >= 0) {
+    float p = fast_exp2(edge - l2);
+    if (edge_at == y) p -= 1.f;
+    Elem<T>::store1(gp + edge_at, p * scale);
+  }
+}
+
 // x *= *factor in place, skipped altogether when the factor is exactly 1 (the usual upstream
 // gradient of a loss): the gradient written by ce_loss_grad_kernel then costs no second pass.
 template <typename T>
@@ -836,6 +967,32 @@ int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float
   }
   const bool one_pass = n > 0 && fm_host::aligned16(logits) && fm_host::aligned16(dlogits) &&
                         nvec <= 8 * 1024;
+  // wider, up to what a compute unit holds: the row stays on the chip (needs 128 KB of LDS granted)
+  if (!one_pass && n > 0 && fm_host::aligned16(logits) && fm_host::aligned16(dlogits) &&
+      nvec + 2 <= kCeHeldMaxVec) {
+    bool granted = false;
+#define GRANT(T) granted = fm_host::grant_dynamic_lds<&ce_loss_grad_held_kernel<T>>(kCeHeldLds * kCeHeldThreads * 16)
+    FM_CE_BY_DTYPE(dtype, GRANT);
+#undef GRANT
+    if (granted) {
+      const bool mean_ = reduction == FM_REDUCE_MEAN;
+      if (mean_) {
+        hipLaunchKernelGGL(ce_count_kernel, dim3(1), dim3(1024), 0, st, labels, n, ignore_index, n_valid);
+        FM_CHECK_LAUNCH("fm_ce_loss_grad(count)");
+      }
+#define HELD(T)                                                                                    \
+  FM_LAUNCH((ce_loss_grad_held_kernel<T>), dim3((unsigned)n), dim3(kCeHeldThreads),                \
+            (size_t)kCeHeldLds * kCeHeldThreads * 16, st, static_cast<const T*>(logits), labels,    \
+            mean_ ? n_valid : nullptr, lse, row_loss, static_cast<T*>(dlogits), (int)v, ignore_index)
+      FM_CE_BY_DTYPE(dtype, HELD);
+#undef HELD
+      FM_CHECK_LAUNCH("fm_ce_loss_grad");
+      hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, st, row_loss, labels, n, ignore_index,
+                         mean_ ? 1 : 0, loss, n_valid);
+      FM_CHECK_LAUNCH("fm_ce_loss_grad(finalize)");
+      return FM_OK;
+    }
+  }
   if (!one_pass) {
     // rows too wide for the register file (or unaligned buffers): two sweeps in one launch
     if (n > 0) {

@@ -9,6 +9,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/fm_hip.h"
 
 namespace fm {
@@ -321,6 +323,24 @@ void note_kernel(const void* host_function);
   } while (0)
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Dynamic LDS beyond 64 KB has to be allowed per kernel and device before the first such launch;
+// K is the kernel's address, `bytes` the most it will ever ask for. False when the device says no
+// (the caller then takes a form that needs less).
+template <auto K>
+bool grant_dynamic_lds(int bytes) {
+  static std::atomic<uint64_t> allowed{0};   // one bit per device
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+  if ((allowed.load(std::memory_order_acquire) >> dev) & 1u) return true;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(K), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          bytes) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  allowed.fetch_or(1ull << dev, std::memory_order_release);
+  return true;
+}
 
 #define FM_CHECK_ARG(cond, ...)                 \
   do {                                          \

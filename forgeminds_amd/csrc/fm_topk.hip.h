@@ -822,16 +822,6 @@ static_assert(sizeof(fm::TopkShared<1024, fm::kVecMaxLds, fm::kTopkBig>) + (size
               "prefixes of the widest row plus the selection state must fit one compute unit's LDS");
 template <auto K>
 bool allow_wide_lds() {
-  static std::atomic<uint64_t> allowed{0};   // one bit per device
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
-  if ((allowed.load(std::memory_order_acquire) >> dev) & 1u) return true;
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(K), hipFuncAttributeMaxDynamicSharedMemorySize,
-                          (kLdsWideMaxVec + 8) * 2) != hipSuccess) {
-    (void)hipGetLastError();   // not fatal: the caller has a form without the prefixes
-    return false;
-  }
-  allowed.fetch_or(1ull << dev, std::memory_order_release);
-  return true;
+  return grant_dynamic_lds<K>((kLdsWideMaxVec + 8) * 2);
 }
 }  // namespace fm_host

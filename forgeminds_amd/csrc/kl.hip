@@ -1207,7 +1207,7 @@ int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, floa
     const int64_t wvec = v / (dtype == FM_F32 ? 4 : 8);
     const bool held = vec_ok && (dtype == FM_F32 ? wvec >= 7168 : (wvec >= 15360 && wvec <= 24576));
 #define WIDE(T, GT)                                                                                \
-  if (held && fm_host::allow_wide_lds<&kl_loss_grad_held_kernel<T, GT>>())                         \
+  if (held && fm_host::grant_dynamic_lds<&kl_loss_grad_held_kernel<T, GT>>(kHeldLds * 2 * kHeldThreads * 16))                         \
     FM_LAUNCH((kl_loss_grad_held_kernel<T, GT>), wgrid, dim3(kHeldThreads),                        \
               (size_t)kHeldLds * 2 * kHeldThreads * 16, st, static_cast<const T*>(student),        \
               static_cast<const T*>(teacher), lse_s, lse_t, row_kl, static_cast<GT*>(dstudent),    \
