@@ -5,6 +5,8 @@
 // Rows of up to 128 KiB whose width is a whole number of 16-byte vectors stay in registers:
 // a row is owned by TPR threads (a lane group, a wave or the waves of one workgroup, several
 // rows per workgroup when they are narrow), read once, reduced (maximum, then sum) and written.
+// Aligned rows from 8192 vectors on stay on the chip instead (registers and LDS of one workgroup
+// per compute unit; what a row has beyond that is streamed and read again).
 // Other rows take one workgroup each: an online (max, sum-exp) pass, then a second pass over
 // the row (served by L2 for rows that fit) that writes exp2(z - m) / s.
 //
@@ -357,6 +359,264 @@ bool rows_plan(int64_t nvec, int* tpr, int* iters) {
 }
 
 // lanes per row and elements per lane of the scalar lane-group kernels (v <= 1024): about
+// Rows past the register kernels that still fit the CHIP, one workgroup per compute unit, the row
+// read once. Forward: 1024 threads keep 16 vectors each in registers and 8 more in 128 KB of LDS
+// (24576 vectors, 196608 bf16 columns); the three passes (maximum, sum, output) unpack the packed
+// vectors afresh. Backward (two rows, y and dy): 512 threads with twice the registers each, 24 + 8
+// vector pairs a thread (16384 pairs). Every thread parks and fetches its own LDS slots only, so
+// the passes need no barrier for them.
+constexpr int kHeldFwdThreads = 1024, kHeldFwdRegs = 16, kHeldFwdLds = 8;
+constexpr int kHeldFwdMaxVec = kHeldFwdThreads * (kHeldFwdRegs + kHeldFwdLds);
+constexpr int kHeldBwdThreads = 512, kHeldBwdRegs = 24, kHeldBwdLds = 8;
+constexpr int kHeldBwdMaxVec = kHeldBwdThreads * (kHeldBwdRegs + kHeldBwdLds);
+
+template <typename T>
+__global__ __launch_bounds__(kHeldFwdThreads) void softmax_held_kernel(const T* __restrict__ x,
+                                                                        T* __restrict__ y, int v) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int THREADS = kHeldFwdThreads, RI = kHeldFwdRegs, LI = kHeldFwdLds;
+  constexpr int NW = THREADS / 64;
+  extern __shared__ u32x4 parked[];          // [LI][THREADS]
+  __shared__ float smem[2 * NW];
+  const int64_t row = blockIdx.x;
+  const T* rp = x + row * (int64_t)v;
+  T* op = y + row * (int64_t)v;
+  const RowSplit sp = split_row<EPV>(row, v, true);
+  const int tid = threadIdx.x;
+  const int ne = edge_count(sp, v);
+  u32x4 raw[RI];
+#pragma unroll
+  for (int i = 0; i < RI; ++i)
+    raw[i] = load16_stream(rp + sp.head + (int64_t)clamp_col(i * THREADS + tid, sp.nvec) * EPV);
+  {
+    u32x4 late[LI];
+#pragma unroll
+    for (int j = 0; j < LI; ++j)
+      late[j] = load16_stream(rp + sp.head + (int64_t)clamp_col((RI + j) * THREADS + tid, sp.nvec) * EPV);
+#pragma unroll
+    for (int j = 0; j < LI; ++j) parked[j * THREADS + tid] = late[j];
+  }
+  float edge = -INFINITY;   // the unaligned ends of the row (at most EPV - 1 elements each): thread e keeps edge e
+  int edge_at = -1;
+  if (tid < ne) {
+    edge_at = edge_col(sp, tid);
+    edge = Elem<T>::load1(rp + edge_at) * kLog2e;
+  }
+  auto vec = [&](int i) -> u32x4 {
+    if (i < RI) { touch(raw[i < RI ? i : 0]); return raw[i < RI ? i : 0]; }
+    return parked[(i - RI) * THREADS + tid];
+  };
+  float mz = fmaxf(edge, kNegBig);
+#pragma unroll
+  for (int i = 0; i < RI + LI; ++i) {
+    if (i * THREADS + tid < sp.nvec) {
+      float z[EPV];
+      Elem<T>::unpack(vec(i), z);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) mz = fmaxf(mz, z[e] * kLog2e);
+    }
+  }
+  // a NaN anywhere must reach the whole row: fmaxf drops it, so it is carried in the sum
+  float ssum = edge_at >= 0 ? fast_exp2(edge - mz) : 0.f;
+#pragma unroll
+  for (int i = 0; i < RI + LI; ++i) {
+    if (i * THREADS + tid < sp.nvec) {
+      float z[EPV];
+      Elem<T>::unpack(vec(i), z);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) ssum += fast_exp2(z[e] * kLog2e - mz);
+    }
+  }
+  // vectors past what the chip holds: streamed with a running (maximum, sum), read again below
+  MaxSum st{mz, ssum};
+  for (int c0 = kHeldFwdMaxVec; c0 < sp.nvec; c0 += THREADS * 2) {
+    u32x4 more[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      more[u] = load16(rp + sp.head + (int64_t)clamp_col(c0 + u * THREADS + tid, sp.nvec) * EPV);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      touch(more[u]);
+      if (c0 + u * THREADS + tid < sp.nvec) {
+        float z[EPV];
+        Elem<T>::unpack(more[u], z);
+        float cm = st.m;
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) { z[e] *= kLog2e; cm = fmaxf(cm, z[e]); }
+        float acc = st.s * fast_exp2(st.m - cm);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) acc += fast_exp2(z[e] - cm);
+        st.m = cm;
+        st.s = acc;
+      }
+    }
+  }
+  const MaxSum tot = block_merge<NW>(st, smem);
+  // a row whose maximum is -inf has sum 0: 0 * inf = NaN, which is what torch returns
+  const float inv = 1.f / tot.s;
+#pragma unroll
+  for (int i = 0; i < RI + LI; ++i) {
+    const int c = i * THREADS + tid;
+    if (c < sp.nvec) {
+      float z[EPV], o[EPV];
+      Elem<T>::unpack(vec(i), z);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) o[e] = fast_exp2(z[e] * kLog2e - tot.m) * inv;
+      store16_stream(op + sp.head + (int64_t)c * EPV, Elem<T>::pack(o));
+    }
+  }
+  for (int c0 = kHeldFwdMaxVec; c0 < sp.nvec; c0 += THREADS * 2) {
+    u32x4 more[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      more[u] = load16_stream(rp + sp.head + (int64_t)clamp_col(c0 + u * THREADS + tid, sp.nvec) * EPV);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      touch(more[u]);
+      if (c < sp.nvec) {
+        float z[EPV], o[EPV];
+        Elem<T>::unpack(more[u], z);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] = fast_exp2(z[e] * kLog2e - tot.m) * inv;
+        store16_stream(op + sp.head + (int64_t)c * EPV, Elem<T>::pack(o));
+      }
+    }
+  }
+  if (edge_at >= 0) Elem<T>::store1(op + edge_at, fast_exp2(edge - tot.m) * inv);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kHeldBwdThreads) void softmax_bwd_held_kernel(const T* __restrict__ y,
+                                                                            const T* __restrict__ dy,
+                                                                            T* __restrict__ dx, int v) {
+  constexpr int EPV = Elem<T>::kVec;
+  constexpr int THREADS = kHeldBwdThreads, RI = kHeldBwdRegs, LI = kHeldBwdLds;
+  constexpr int NW = THREADS / 64;
+  extern __shared__ u32x4 parked[];          // [LI][2][THREADS]
+  __shared__ float smem[NW];
+  const int64_t row = blockIdx.x;
+  const T* yp = y + row * (int64_t)v;
+  const T* gp = dy + row * (int64_t)v;
+  T* op = dx + row * (int64_t)v;
+  const RowSplit sp = split_row<EPV>(row, v, true);
+  const int tid = threadIdx.x;
+  const int ne = edge_count(sp, v);
+  u32x4 ry[RI], rg[RI];
+#pragma unroll
+  for (int i = 0; i < RI; ++i) {
+    const int c = clamp_col(i * THREADS + tid, sp.nvec);
+    ry[i] = load16_stream(yp + sp.head + (int64_t)c * EPV);
+    rg[i] = load16_stream(gp + sp.head + (int64_t)c * EPV);
+  }
+#pragma unroll
+  for (int j = 0; j < LI; j += 2) {
+    u32x4 ly[2], lg[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = clamp_col((RI + j + u) * THREADS + tid, sp.nvec);
+      ly[u] = load16_stream(yp + sp.head + (int64_t)c * EPV);
+      lg[u] = load16_stream(gp + sp.head + (int64_t)c * EPV);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      parked[((j + u) * 2 + 0) * THREADS + tid] = ly[u];
+      parked[((j + u) * 2 + 1) * THREADS + tid] = lg[u];
+    }
+  }
+  float ey = 0.f, eg = 0.f;   // thread e keeps edge e of both rows
+  int edge_at = -1;
+  if (tid < ne) {
+    edge_at = edge_col(sp, tid);
+    ey = Elem<T>::load1(yp + edge_at);
+    eg = Elem<T>::load1(gp + edge_at);
+  }
+  float dot = ey * eg;
+#pragma unroll
+  for (int i = 0; i < RI + LI; ++i) {
+    if (i * THREADS + tid < sp.nvec) {
+      u32x4 a4, b4;
+      if (i < RI) {
+        touch(ry[i < RI ? i : 0]);
+        touch(rg[i < RI ? i : 0]);
+        a4 = ry[i < RI ? i : 0]; b4 = rg[i < RI ? i : 0];
+      } else {
+        a4 = parked[((i - RI) * 2 + 0) * THREADS + tid]; b4 = parked[((i - RI) * 2 + 1) * THREADS + tid];
+      }
+      float a[EPV], b[EPV];
+      Elem<T>::unpack(a4, a);
+      Elem<T>::unpack(b4, b);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) dot += a[e] * b[e];
+    }
+  }
+  // vector pairs past what the chip holds: streamed here, read again below
+  for (int c0 = kHeldBwdMaxVec; c0 < sp.nvec; c0 += THREADS * 2) {
+    u32x4 my[2], mg[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      my[u] = load16(yp + sp.head + (int64_t)c * EPV);
+      mg[u] = load16(gp + sp.head + (int64_t)c * EPV);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      touch(my[u]);
+      if (c0 + u * THREADS + tid < sp.nvec) {
+        float a[EPV], b[EPV];
+        Elem<T>::unpack(my[u], a);
+        Elem<T>::unpack(mg[u], b);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) dot += a[e] * b[e];
+      }
+    }
+  }
+  dot = row_reduce<THREADS, OpSum>(dot, smem, 0, tid);
+#pragma unroll
+  for (int i = 0; i < RI + LI; ++i) {
+    const int c = i * THREADS + tid;
+    if (c < sp.nvec) {
+      u32x4 a4, b4;
+      if (i < RI) {
+        touch(ry[i < RI ? i : 0]);
+        touch(rg[i < RI ? i : 0]);
+        a4 = ry[i < RI ? i : 0]; b4 = rg[i < RI ? i : 0];
+      } else {
+        a4 = parked[((i - RI) * 2 + 0) * THREADS + tid]; b4 = parked[((i - RI) * 2 + 1) * THREADS + tid];
+      }
+      float a[EPV], b[EPV], o[EPV];
+      Elem<T>::unpack(a4, a);
+      Elem<T>::unpack(b4, b);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) o[e] = (b[e] - dot) * a[e];
+      store16_stream(op + sp.head + (int64_t)c * EPV, Elem<T>::pack(o));
+    }
+  }
+  for (int c0 = kHeldBwdMaxVec; c0 < sp.nvec; c0 += THREADS * 2) {
+    u32x4 my[2], mg[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+      my[u] = load16_stream(yp + sp.head + (int64_t)c * EPV);
+      mg[u] = load16_stream(gp + sp.head + (int64_t)c * EPV);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      touch(my[u]);
+      if (c < sp.nvec) {
+        float a[EPV], b[EPV], o[EPV];
+        Elem<T>::unpack(my[u], a);
+        Elem<T>::unpack(mg[u], b);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] = (b[e] - dot) * a[e];
+        store16_stream(op + sp.head + (int64_t)c * EPV, Elem<T>::pack(o));
+      }
+    }
+  }
+  if (edge_at >= 0) Elem<T>::store1(op + edge_at, (eg - dot) * ey);
+}
+
 // four elements a lane for the narrowest rows, so that rows of a few elements do not idle
 // most of a 16-lane group
 void scalar_plan(int v, int* tpr, int* iters) {
@@ -400,6 +660,14 @@ void launch(const void* x, void* y, int64_t n, int v, bool vec_ok, hipStream_t s
     GOS(16, 4) GOS(16, 8) GOS(16, 16) GOS(64, 8) GOS(64, 16)
 #undef GOS
   }
+  // (from 8192 vectors on: below that the streaming form, several rows a compute unit, is as fast
+  // or faster -- bf16 [5120,50257] 218 against 229 us, [3840,65544] 218 against 211)
+  if (vec_ok && v / EPV <= 2 * kHeldFwdMaxVec && v / EPV >= 8192 &&
+      fm_host::grant_dynamic_lds<&softmax_held_kernel<T>>(kHeldFwdLds * kHeldFwdThreads * 16)) {
+    FM_LAUNCH((softmax_held_kernel<T>), dim3((unsigned)n), dim3(kHeldFwdThreads),
+              (size_t)kHeldFwdLds * kHeldFwdThreads * 16, st, xp, yp, v);
+    return;
+  }
   const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 4);
   const dim3 grid((unsigned)n);
 #define LAUNCH(TH, UN) \
@@ -441,6 +709,14 @@ void launch_bwd(const void* y, const void* dy, void* dx, int64_t n, int v, bool 
     GOS(1, 1) GOS(1, 2) GOS(1, 4) GOS(2, 4) GOS(4, 4) GOS(8, 4)
     GOS(16, 4) GOS(16, 8) GOS(16, 16) GOS(64, 8) GOS(64, 16)
 #undef GOS
+  }
+  // (16-bit rows only when they fill most of what the chip holds: bf16 [2560,100000] 373 us streamed
+  // against 386 held, [2048,128256] 388 against 352; fp32 [3328,40000] 376 against 274)
+  if (vec_ok && v / EPV <= 2 * kHeldBwdMaxVec && v / EPV >= 8192 &&
+      fm_host::grant_dynamic_lds<&softmax_bwd_held_kernel<T>>(kHeldBwdLds * 2 * kHeldBwdThreads * 16)) {
+    FM_LAUNCH((softmax_bwd_held_kernel<T>), dim3((unsigned)n), dim3(kHeldBwdThreads),
+              (size_t)kHeldBwdLds * 2 * kHeldBwdThreads * 16, st, yp, gp, op, v);
+    return;
   }
   const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 1024, 4);
   const dim3 grid((unsigned)n);

@@ -845,7 +845,11 @@ def test_topk_unaligned_rows():
                                      (1000, 64, F32), (77, 16, BF16), (3, 4, F32), (33, 512, BF16),
                                      (130, 8, F16), (9, 8192, BF16), (5, 32768, F16), (3, 65536, BF16),
                                      (257, 2048, F32), (4, 32000, BF16), (1000, 33, BF16), (77, 7, F32),
-                                     (300, 257, F16), (65, 1023, BF16), (40, 100, F32), (9, 513, F32)])
+                                     (300, 257, F16), (65, 1023, BF16), (40, 100, F32), (9, 513, F32),
+                                     # rows kept on the chip between the passes (registers + LDS): odd widths,
+                                     # the widest that fits and one past it
+                                     (3, 151937, F16), (2, 98000, F32), (2, 196592, BF16), (2, 196608, BF16),
+                                     (3, 65543, BF16)])
 def test_softmax(n, v, dt):
     x = torch.randn(n, v, generator=gen(21)).to(dt)
     y = _hip.softmax_fwd(x.to(DEV))
@@ -858,7 +862,11 @@ def test_softmax(n, v, dt):
                                      (2, 128256, BF16), (1000, 64, F32), (77, 16, BF16), (33, 512, BF16),
                                      (9, 8192, BF16), (5, 32768, F16), (3, 65536, BF16), (257, 2048, F32),
                                      (4, 32000, BF16), (1000, 33, BF16), (65, 1023, BF16), (9, 513, F32),
-                                     (3, 40000, F32), (6, 16384, F32)])
+                                     (3, 40000, F32), (6, 16384, F32),
+                                     # both rows kept on the chip: 16-bit rows near the 16384 vectors it holds,
+                                     # fp32 rows from 8192 vectors on, odd widths, one past the capacity
+                                     (3, 128257, F16), (2, 131056, BF16), (2, 131072, BF16), (3, 65530, F32),
+                                     (2, 120000, BF16)])
 def test_softmax_bwd(n, v, dt):
     g = gen(22)
     y = torch.softmax(2 * torch.randn(n, v, generator=g), -1).to(dt)
