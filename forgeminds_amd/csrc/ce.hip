@@ -457,7 +457,8 @@ __global__ __launch_bounds__(THREADS) void ce_loss_grad_kernel(const T* logits,
 // per compute unit, keeps 16 vectors a thread in registers and 8 more in 128 KB of LDS (every thread
 // parks and fetches its own slots only: no barrier for them): 24576 vectors, 196608 bf16 columns, the
 // vocabularies of 100 K to 152 K entries among them. One read and one write of the row, where the two
-// sweeps of ce_loss_grad_wide_kernel read it twice.
+// sweeps of ce_loss_grad_wide_kernel read it twice. What a row has beyond the 24576 vectors is streamed
+// and read again (taken up to twice that width).
 constexpr int kCeHeldThreads = 1024;
 constexpr int kCeHeldRegs = 16;
 constexpr int kCeHeldLds = 8;
@@ -548,7 +549,31 @@ __global__ __launch_bounds__(kCeHeldThreads) void ce_loss_grad_held_kernel(const
       for (int e = 0; e < EPV; ++e) ssum += fast_exp2(z[e] * kLog2e - mz);
     }
   }
-  const MaxSum tot = block_merge<NW>(MaxSum{mz, ssum}, smem);
+  // vectors past what the chip holds: streamed with a running (maximum, sum), read again below
+  MaxSum run{mz, ssum};
+  for (int c0 = kCeHeldMaxVec; c0 < sp.nvec; c0 += THREADS * 2) {
+    u32x4 more[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      more[u] = load16(rp + sp.head + (int64_t)clamp_col(c0 + u * THREADS + tid, sp.nvec) * EPV);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      touch(more[u]);
+      if (c0 + u * THREADS + tid < sp.nvec) {
+        float z[EPV];
+        Elem<T>::unpack(more[u], z);
+        float cm = run.m;
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) { z[e] *= kLog2e; cm = fmaxf(cm, z[e]); }
+        float acc = run.s * fast_exp2(run.m - cm);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) acc += fast_exp2(z[e] - cm);
+        run.m = cm;
+        run.s = acc;
+      }
+    }
+  }
+  const MaxSum tot = block_merge<NW>(run, smem);
   const float l2 = tot.m + fast_log2(tot.s);
   const float scale = 1.f / (n_valid != nullptr ? *n_valid : 1.f);
   if (tid == 0) {
@@ -575,6 +600,31 @@ __global__ __launch_bounds__(kCeHeldThreads) void ce_loss_grad_held_kernel(const
 #pragma unroll
       for (int e = 0; e < EPV; ++e) o[e] *= scale;
       store16_stream(gp + col0, Elem<T>::pack(o));
+    }
+  }
+  for (int c0 = kCeHeldMaxVec; c0 < sp.nvec; c0 += THREADS * 2) {
+    u32x4 more[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+      more[u] = load16_stream(rp + sp.head + (int64_t)clamp_col(c0 + u * THREADS + tid, sp.nvec) * EPV);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = c0 + u * THREADS + tid;
+      touch(more[u]);
+      if (c < sp.nvec) {
+        float z[EPV], o[EPV];
+        Elem<T>::unpack(more[u], z);
+        const int col0 = sp.head + c * EPV;
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] = fast_exp2(z[e] * kLog2e - l2);
+        if (y >= col0 && y < col0 + EPV) {
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) o[e] -= (col0 + e == y) ? 1.f : 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) o[e] *= scale;
+        store16_stream(gp + col0, Elem<T>::pack(o));
+      }
     }
   }
   if (edge_at >= 0) {
@@ -969,7 +1019,7 @@ int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float
                         nvec <= 8 * 1024;
   // wider, up to what a compute unit holds: the row stays on the chip (needs 128 KB of LDS granted)
   if (!one_pass && n > 0 && fm_host::aligned16(logits) && fm_host::aligned16(dlogits) &&
-      nvec + 2 <= kCeHeldMaxVec) {
+      nvec <= 2 * kCeHeldMaxVec) {
     bool granted = false;
 #define GRANT(T) granted = fm_host::grant_dynamic_lds<&ce_loss_grad_held_kernel<T>>(kCeHeldLds * kCeHeldThreads * 16)
     FM_CE_BY_DTYPE(dtype, GRANT);

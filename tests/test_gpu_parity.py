@@ -288,7 +288,8 @@ def test_ce_fwd_bwd(n, v, dt):
 CE1_CASES = CE_CASES + [(5, 140000, BF16), (3, 70000, F32), (4, 600, BF16), (3, 9000, F16),
                         # rows kept on the chip (registers + LDS of one workgroup per compute unit): aligned and
                         # odd widths, the widest that fits, and one past it (two sweeps)
-                        (6, 128256, BF16), (5, 151937, F16), (4, 98000, F32), (4, 196560, BF16), (3, 196608, BF16)]
+                        (6, 128256, BF16), (5, 151937, F16), (4, 98000, F32), (4, 196560, BF16), (3, 196608, BF16),
+                        (3, 262147, BF16), (2, 128256, F32), (2, 393300, F16)]
 
 
 @pytest.mark.parametrize("n,v,dt", CE1_CASES)
