@@ -96,7 +96,7 @@ def measured_traffic(kernel):
     return int(round((kib[0] * TRAFFIC_SCALE[0] + kib[1] * TRAFFIC_SCALE[1]) * 1024))
 
 
-WORKLOADS = ["ce", "ce_one_pass", "rmsnorm", "add_rmsnorm", "add_layernorm", "kl", "kl_one_launch", "kl_topk",
+WORKLOADS = ["ce", "ce_one_pass", "ce_one_pass_128k", "rmsnorm", "add_rmsnorm", "add_layernorm", "kl", "kl_one_launch", "kl_topk",
              "kl_topk_one_launch", "topk", "route", "route_256x8", "route_train", "moe_dispatch", "swiglu", "qk_norm_rope"]
 
 
@@ -341,10 +341,20 @@ def make_workload(name, torch, L, dev):
         w.rows = n
         return w
 
-    if name in ("ce", "ce_one_pass"):
-        n, v = 8192, 32000
+    if name in ("ce", "ce_one_pass", "ce_one_pass_128k"):
+        wide = name == "ce_one_pass_128k"    # the vocabulary of config 5: rows of 250 KB, kept on the chip
+        n, v = (4096, 128256) if wide else (8192, 32000)
         g.manual_seed(1002)
-        lg = rn(n, v, scale=2.0)
+        if wide:
+            if "kl_st" not in _SHARED:       # the student logits of the KL workloads serve
+                g.manual_seed(1005)
+                s_ = rn(n, v, scale=3.0)
+                _SHARED["kl_st"] = (s_, rn(n, v, scale=0.5, base=s_))
+            lg = _SHARED["kl_st"][0]
+            g.manual_seed(1002)
+        else:
+            lg = rn(n, v, scale=2.0)
+        loss_rows = 256 if wide else 2048
         y = torch.randint(0, v, (n,), generator=g)
         y[torch.rand(n, generator=g) < 0.05] = -100
         y = y.to(dev)
@@ -369,14 +379,15 @@ def make_workload(name, torch, L, dev):
             yc = y[:rows].cpu()
             _, og = O.cross_entropy(lg[:rows].cpu(), yc)        # mean over the sample's valid rows
             og = og.float() * (max(1, int((yc != -100).sum())) / max(1, n_valid))
-            ol, _ = O.cross_entropy(lg[:2048].cpu(), y[:2048].cpu())   # loss: first 2048 rows against their own row losses
-            got = rl[:2048].sum().item() / max(1, int((y[:2048] != -100).sum().item()))
+            ol, _ = O.cross_entropy(lg[:loss_rows].cpu(), y[:loss_rows].cpu())   # loss: the first rows against their own row losses
+            got = rl[:loss_rows].sum().item() / max(1, int((y[:loss_rows] != -100).sum().item()))
             return _close(dlg[:rows], og) and abs(got - ol.item()) <= 1e-4 * abs(ol.item())
 
         def cpu():
             from oracle import oracle as O
-            lc, yc = lg.cpu(), y.cpu()
-            return (lambda: O.cross_entropy(lc, yc)), 1.0, f"all {n} rows"
+            rows_ = 512 if wide else n
+            lc, yc = lg[:rows_].cpu(), y[:rows_].cpu()
+            return (lambda: O.cross_entropy(lc, yc)), n / rows_, (f"{rows_} rows x {n // rows_}" if wide else f"all {n} rows")
 
         def eager():
             from forgeminds_amd.kernels import _fallback as fb
@@ -387,7 +398,7 @@ def make_workload(name, torch, L, dev):
         # bytes the dataflow has to move: rows whose label is ignored are never read
         w.valid_rows = n_valid
 
-        if name == "ce_one_pass":
+        if name in ("ce_one_pass", "ce_one_pass_128k"):
             one = torch.ones((), device=dev)
 
             def both():
@@ -402,7 +413,7 @@ def make_workload(name, torch, L, dev):
 
             w.step = step
             w.dominant_launch = both
-            w.dominant = "ce_loss_grad_kernel<bf16,512,8>"
+            w.dominant = "ce_loss_grad_held_kernel<bf16>" if wide else "ce_loss_grad_kernel<bf16,512,8>"
             w.dominant_bytes = w.bytes = n * v * 4
             w.required_bytes = w.dominant_required_bytes = n_valid * v * 2 + n * v * 2
             w.desc = (f"fused CE loss + gradient in one pass, logits bf16 [{n},{v}], 5% ignore_index, mean; "
