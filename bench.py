@@ -528,14 +528,12 @@ def make_workload(name, torch, L, dev):
 
             w.step = step
             w.dominant_launch = both
-            w.dominant = "kl_loss_grad_wide_kernel<bf16,bf16,1024,2>"
+            w.dominant = "kl_loss_grad_held_kernel<bf16,bf16>"
             w.dominant_bytes = w.bytes = n * v * 6
             w.desc = (f"KL loss + gradient in one launch bf16 [{n},{v}], T=2, mean; algorithmic 6 B/logit pair "
-                      "(read s,t + write g). Each row is swept a second time right after the first, inside the "
-                      "launch: the L2-side counters show 10 B/pair (both sweeps fetched); that the second sweep is "
-                      "served by the memory-side cache is an inference from the clock, no counter of this profiler "
-                      "sits behind that cache")
-            w.l2_bytes = n * v * 10
+                      "(read s,t + write g). The pair of rows stays in the registers and LDS of one workgroup per "
+                      "compute unit between the two passes: it is read once, and the L2-side counters show the "
+                      "algorithmic bytes")
             w.rows = n
             w.floor = [lambda i: ((s, t), (gs,))]
             return w
@@ -559,8 +557,8 @@ def make_workload(name, torch, L, dev):
             w.dominant = "kl_fwd_topk_kernel<bf16,512,2>"
             w.dominant_bytes = w.bytes = n * v * 6
             w.desc = (f"KL loss + gradient + teacher top-64 in one launch bf16 [{n},{v}], T=2, mean; algorithmic "
-                      "6 B/logit pair; two sweeps per row inside the launch, 10 B/pair at the L2 boundary (see "
-                      "kl_one_launch)")
+                      "6 B/logit pair; two sweeps per row inside the launch: the L2-side counters show 10 B/pair "
+                      "(both sweeps fetched)")
             w.l2_bytes = n * v * 10
             w.rows = n
             return w
