@@ -199,9 +199,11 @@ int fm_ce_bwd(const void* logits, const int64_t* labels, const float* lse, const
  * Rows stay in registers between the log-sum-exp and the store, so the step moves 2 + 2
  * bytes per 16-bit logit instead of 2 + 2 + 2. dlogits may be the logits buffer itself
  * (the way the reference's KL writes its gradient into an owned student tensor,
- * kernels/kl.py:146-150, 157-160); lse may be NULL. Rows wider than 128 KiB (or unaligned
- * buffers) are swept twice inside the same launch (the second sweep follows the first at
- * once, when the memory-side cache is most likely to still hold the row). lse of ignored rows is written as 0 (those rows are not read). */
+ * kernels/kl.py:146-150, 157-160); lse may be NULL. Rows wider than 128 KiB stay on the chip
+ * all the same (registers and LDS of one workgroup per compute unit hold 384 KiB; what a row has
+ * beyond that, up to twice that width, is streamed and read again); wider rows still and unaligned
+ * buffers are swept twice inside the same launch (faster than two launches, not single-read).
+ * lse of ignored rows is written as 0 (those rows are not read). */
 int fm_ce_loss_grad(const void* logits, const int64_t* labels, float* lse, float* row_loss,
                     float* loss, float* n_valid, void* dlogits, int64_t n, int64_t v, int dtype,
                     int64_t ignore_index, int reduction, fm_stream_t stream);
@@ -228,8 +230,9 @@ int fm_kl_fwd(const void* student, const void* teacher, float* lse_s, float* lse
  * fm_kl_fwd's outputs plus dstudent = fm_kl_bwd's result for grad_out = 1 and
  * scale = 1/n (FM_REDUCE_MEAN) or 1 (FM_REDUCE_SUM). Rows of at most 64 KiB stay in
  * registers between the log-sum-exps and the store (4 + 2 bytes per pair of 16-bit logits
- * instead of 4 + 4 + 2); wider rows are swept twice inside the same launch (the second
- * sweep follows the first at once, when the memory-side cache is most likely to still hold the row). dstudent may be the student buffer itself when
+ * instead of 4 + 4 + 2); wider rows are swept twice inside the same launch, or, where that is
+ * measured faster (fp32 rows from 112 KiB on, 16-bit rows of 240-384 KiB), kept in the registers and
+ * LDS of one workgroup per compute unit and read once. dstudent may be the student buffer itself when
  * grad_dtype == dtype (kl.py:146-150, reuse=True); lse_s / lse_t may be NULL.
  * fm_scale_inplace applies an upstream gradient other than 1. */
 int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, float* lse_t,
