@@ -146,6 +146,54 @@ def test_sweep_topk_softmax():
         assert _within(sb, O.softmax_bwd(smc, gy), dt, ulps=2.0, cancel=cancel), ("softmax bwd", case)
 
 
+def test_sweep_rows_kept_on_the_chip():
+    """The one-pass losses and the softmax pair on rows of 7168 to 49152 vectors, the range in which a
+    workgroup keeps the row (or the pair of rows) in its registers and LDS between the passes: widths
+    around the points where the registers, the LDS share and the streamed remainder begin, a few
+    elements either side, so that rows start at every alignment."""
+    rng = random.Random(SEED + 5)
+    g = torch.Generator().manual_seed(rng.randint(0, 1 << 30))
+    for i in range(12):
+        dt = rng.choice([BF16, F16, F32])
+        epv = 4 if dt == F32 else 8
+        v = rng.choice([7168, 8192, 12288, 15360, 16384, 24576, 32768, 49152]) * epv
+        v += rng.choice([-17, -8, -1, 0, 1, 7, 9, 16, 33, rng.randint(-3000, 3000)])
+        n = rng.randint(1, 3)
+        T = rng.choice([1.0, 2.0])
+        case = (i, n, v, dt, T)
+        s = (3 * torch.randn(n, v, generator=g)).to(dt)
+        t = (s.float() + 0.5 * torch.randn(n, v, generator=g)).to(dt)
+        lab = torch.randint(0, v, (n,), generator=g)
+        if n > 1:
+            lab[n - 1] = -100
+        sd, td, labd = s.to(DEV), t.to(DEV), lab.to(DEV)
+        o64, _ = O.cross_entropy(s, lab, acc=torch.float64)
+        _, og = O.cross_entropy(s, lab)
+        nv = max(1, int((lab != -100).sum()))
+        loss, dl, _, _ = _hip.ce_loss_grad(sd, labd, -100, "mean")
+        assert abs(loss.item() - o64.item()) <= 1e-4 * abs(o64.item()) + 1e-6, ("ce one-pass loss", case)
+        assert _within(dl, og, dt, cancel=1.0 / nv), ("ce one-pass grad", case)
+        own = sd.clone()
+        _, dl2, _, _ = _hip.ce_loss_grad(own, labd, -100, "mean", True)
+        assert dl2.data_ptr() == own.data_ptr() and torch.equal(dl2, dl), ("ce one-pass in place", case)
+        orow, _ = O.kl_div(s, t, "none", T, acc=torch.float64)
+        _, ogk = O.kl_div(s, t, "mean", T)
+        lm = 1.0 + float(torch.logsumexp(s.double() / T, -1).abs().max())
+        _, g1, r1 = _hip.kl_loss_grad(sd, td, 1.0 / T, "mean", dt)
+        assert _within(g1, ogk, dt, cancel=2 * lm / (T * n)), ("kl one-launch grad", case)
+        assert torch.allclose(r1.cpu().double(), orow, rtol=3e-4, atol=3e-6), ("kl one-launch rows", case)
+        own = sd.clone()
+        _, g2, _ = _hip.kl_loss_grad(own, td, 1.0 / T, "mean", dt, True)
+        assert g2.data_ptr() == own.data_ptr() and torch.equal(g2, g1), ("kl one-launch in place", case)
+        sm = _hip.softmax_fwd(sd)
+        assert _within(sm, O.softmax(s), dt, ulps=2.0), ("softmax", case)
+        gy = torch.randn(n, v, generator=g).to(dt)
+        smc = sm.cpu()
+        sb = _hip.softmax_bwd(sm, gy.to(DEV))
+        cancel = float((gy.float().abs().max() + 1) * smc.float().max())
+        assert _within(sb, O.softmax_bwd(smc, gy), dt, ulps=2.0, cancel=cancel), ("softmax bwd", case)
+
+
 def test_sweep_router():
     for i, rng, g in _cases(4):
         e = rng.choice([2, 3, 4, 8, 16, 32, 64, 100, 128, 256, 512])
