@@ -15,16 +15,22 @@ using namespace fm;
 
 namespace {
 
-template <typename T, int THREADS, int UNROLL>
+// KEEP: the rows are read with ordinary (cached) loads instead of streaming ones. The forward of a
+// training step takes it for the LAST rows, as many as the memory-side cache holds: the backward,
+// which follows at once and walks the rows in the same order, then finds them there when it gets to
+// them (its own loads and stores stream past that cache). A load's kind cannot be chosen at run
+// time -- two loads of one address that differ only in their cache hint are merged into a plain
+// one -- so the two kinds are two instantiations, launched over two row ranges (`row0`).
+template <typename T, int THREADS, int UNROLL, bool KEEP>
 __global__ __launch_bounds__(THREADS) void ce_fwd_kernel(const T* __restrict__ logits,
                                                           const int64_t* __restrict__ labels,
                                                           float* __restrict__ lse,
                                                           float* __restrict__ row_loss, int v,
-                                                          int64_t ignore_index, bool vec_ok) {
+                                                          int64_t ignore_index, bool vec_ok, int64_t row0) {
   constexpr int EPV = Elem<T>::kVec;
   constexpr int NW = THREADS / 64;
   __shared__ float smem[2 * NW];
-  const int64_t row = blockIdx.x;
+  const int64_t row = row0 + blockIdx.x;
   const T* rp = logits + row * (int64_t)v;
   const RowSplit sp = split_row<EPV>(row, v, vec_ok);
   const int tid = threadIdx.x;
@@ -44,7 +50,7 @@ __global__ __launch_bounds__(THREADS) void ce_fwd_kernel(const T* __restrict__ l
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
-      raw[u] = load16_stream(rp + sp.head + (int64_t)c * EPV);
+      raw[u] = KEEP ? load16(rp + sp.head + (int64_t)c * EPV) : load16_stream(rp + sp.head + (int64_t)c * EPV);
     }
     // the maximum is taken on the raw logits and scaled once per batch, so each element costs
     // one max, one fma and one exp2
@@ -82,7 +88,7 @@ __global__ __launch_bounds__(THREADS) void ce_fwd_kernel(const T* __restrict__ l
   const MaxSum tot = block_merge<NW>(st, smem);
   if (tid == 0) {
     const float l = (tot.m + fast_log2(tot.s)) * kLn2;
-    lse[row] = l;
+    if (lse != nullptr) lse[row] = l;
     float loss = 0.f;
     if (y != ignore_index) loss = (y >= 0 && y < v) ? l - ylogit : __builtin_nanf("");
     row_loss[row] = loss;
@@ -881,16 +887,32 @@ bool launch_rows(const void* logits, const int64_t* labels, const float* n_valid
     else { CALL(f16_t); }                        \
   } while (0)
 
+// What the memory-side cache of the part holds (MI355X: 256 MiB): the forward that expects a backward
+// reads that much of its input, the last rows, with cached loads. [8192,32000] bf16 forward + backward:
+// 250.0 us with streaming loads throughout, 242.9 with the last 50 % of the rows (262 MB) cached,
+// 248.1 / 246.5 / 247.0 with the last 40 / 60 / 70 %, 244.8 with all of them, 245.6 with the FIRST
+// half, 252.9 with the backward walking the rows in reverse (the forward alone is 12 % slower on the
+// rows it reads with cached loads).
+constexpr int64_t kKeepBytes = 256ll << 20;
+
 template <typename T>
 int launch_fwd(const void* logits, const int64_t* labels, float* lse, float* row_loss, int64_t n,
-               int v, int64_t ignore_index, bool vec_ok, hipStream_t st) {
+               int v, int64_t ignore_index, bool vec_ok, bool backward_follows, hipStream_t st) {
   const T* lp = static_cast<const T*>(logits);
   // the forward alone keeps 256 threads up to 24 KiB rows (16 KiB rows: 50 against 65 us per 256 MiB)
   const fm_host::VocabShape sh = fm_host::vocab_shape(v, sizeof(T), 512, 4, 24 * 1024);
-  const dim3 grid((unsigned)n);
+  int64_t kept = backward_follows ? kKeepBytes / ((int64_t)v * (int64_t)sizeof(T)) : 0;
+  if (kept > n) kept = n;
+  const int64_t streamed = n - kept;
 #define LAUNCH(TH, UN)                                                                          \
-  FM_LAUNCH((ce_fwd_kernel<T, TH, UN>), grid, dim3(TH), 0, st, lp, labels, lse, row_loss, \
-                     v, ignore_index, vec_ok)
+  do {                                                                                          \
+    if (streamed > 0)                                                                           \
+      FM_LAUNCH((ce_fwd_kernel<T, TH, UN, false>), dim3((unsigned)streamed), dim3(TH), 0, st, lp, labels, lse, \
+                row_loss, v, ignore_index, vec_ok, (int64_t)0);                                 \
+    if (kept > 0)                                                                               \
+      FM_LAUNCH((ce_fwd_kernel<T, TH, UN, true>), dim3((unsigned)kept), dim3(TH), 0, st, lp, labels, lse, \
+                row_loss, v, ignore_index, vec_ok, streamed);                                   \
+  } while (0)
   FM_VOCAB_DISPATCH(sh, LAUNCH);
 #undef LAUNCH
   return FM_OK;
@@ -939,7 +961,7 @@ int fm_ce_fwd(const void* logits, const int64_t* labels, float* lse, float* row_
   FM_CHECK_ARG(reduction == FM_REDUCE_SUM || reduction == FM_REDUCE_MEAN,
                "fm_ce_fwd: reduction must be sum or mean (got %d)", reduction);
   FM_CHECK_ARG(loss && n_valid, "fm_ce_fwd: NULL scalar output");
-  FM_CHECK_ARG(n == 0 || (logits && labels && lse && row_loss), "fm_ce_fwd: NULL pointer");
+  FM_CHECK_ARG(n == 0 || (logits && labels && row_loss), "fm_ce_fwd: NULL pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
   bool narrow = false;
   if (n > 0) {
@@ -949,9 +971,10 @@ int fm_ce_fwd(const void* logits, const int64_t* labels, float* lse, float* row_
   }
   if (n > 0 && !narrow) {
     const bool vec_ok = fm_host::aligned16(logits);
-    if (dtype == FM_F32) launch_fwd<float>(logits, labels, lse, row_loss, n, (int)v, ignore_index, vec_ok, st);
-    else if (dtype == FM_BF16) launch_fwd<bf16_t>(logits, labels, lse, row_loss, n, (int)v, ignore_index, vec_ok, st);
-    else launch_fwd<f16_t>(logits, labels, lse, row_loss, n, (int)v, ignore_index, vec_ok, st);
+    const bool bwd = lse != nullptr;   // the saved log-sum-exps are what a backward needs: no lse, no backward
+    if (dtype == FM_F32) launch_fwd<float>(logits, labels, lse, row_loss, n, (int)v, ignore_index, vec_ok, bwd, st);
+    else if (dtype == FM_BF16) launch_fwd<bf16_t>(logits, labels, lse, row_loss, n, (int)v, ignore_index, vec_ok, bwd, st);
+    else launch_fwd<f16_t>(logits, labels, lse, row_loss, n, (int)v, ignore_index, vec_ok, bwd, st);
   }
   if (n > 0) FM_CHECK_LAUNCH("fm_ce_fwd");
   hipLaunchKernelGGL(ce_finalize_kernel, dim3(1), dim3(1024), 0, st, row_loss, labels, n,

@@ -311,12 +311,16 @@ def layernorm_bwd(x2, w, mean, rstd, dy2, gxn2=None, want_dw: bool = True, want_
 
 
 # ------------------------------------------------------------------ cross entropy
-def ce_fwd(logits2, labels, ignore_index: int, reduction: str):
-    """logits2 [n, v], labels [n] int64 -> (loss fp32 scalar, lse [n], n_valid fp32 scalar)."""
+def ce_fwd(logits2, labels, ignore_index: int, reduction: str, for_backward: bool = True):
+    """logits2 [n, v], labels [n] int64 -> (loss fp32 scalar, lse [n], n_valid fp32 scalar, row_loss).
+
+    ``for_backward=False`` (no gradient will be asked for) passes no ``lse`` buffer: the library then
+    streams the logits past the caches throughout instead of leaving their last 256 MB where a
+    backward would find them, and ``lse`` comes back as None."""
     _dense(logits2, labels)
     n, v = logits2.shape
     dev = logits2.device
-    lse = torch.empty(n, device=dev, dtype=torch.float32)
+    lse = torch.empty(n, device=dev, dtype=torch.float32) if for_backward else None
     row_loss = torch.empty(n, device=dev, dtype=torch.float32)
     scal = torch.empty(2, device=dev, dtype=torch.float32)
     with _guard(dev):

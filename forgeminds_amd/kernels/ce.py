@@ -32,7 +32,7 @@ class _CrossEntropyFn(torch.autograd.Function):
         ctx.mode = "none"
         ctx.args = (ignore_index, reduction)
         if not ctx.needs_input_grad[0]:
-            loss, _lse, _n_valid, _rows = _hip.ce_fwd(lg2, y, ignore_index, reduction)
+            loss, _lse, _n_valid, _rows = _hip.ce_fwd(lg2, y, ignore_index, reduction, for_backward=False)
             return loss.clone()     # `loss` is a view into a 2-element scratch tensor
         if logits.dtype == torch.float16:
             # (softmax - onehot) / n_valid stored in fp16 before the upstream gradient is applied

@@ -178,7 +178,10 @@ int fm_layernorm_bwd(const void* x, const void* w, const float* mean, const floa
  *          sum(row_loss) for FM_REDUCE_SUM (one chunk of loss.py:36-38)
  * logits: [n, v] of dtype; labels: [n] int64; lse, row_loss: [n] fp32 (lse is what the
  * backward re-uses instead of a stored softmax); loss, n_valid: fp32 scalars on device.
- * One read of logits. n == 0 yields loss 0 and n_valid 1. */
+ * One read of logits. n == 0 yields loss 0 and n_valid 1.
+ * lse may be NULL when no backward will follow (evaluation): the logits are then streamed past
+ * the caches throughout. With lse the last 256 MiB of them (what the part's memory-side cache
+ * holds) are read with cached loads, and fm_ce_bwd, called next, finds those rows there. */
 int fm_ce_fwd(const void* logits, const int64_t* labels, float* lse, float* row_loss,
               float* loss, float* n_valid, int64_t n, int64_t v, int dtype,
               int64_t ignore_index, int reduction, fm_stream_t stream);

@@ -285,6 +285,25 @@ def test_ce_fwd_bwd(n, v, dt):
     assert torch.allclose(lse.cpu().double(), lse_ref, rtol=1e-5, atol=1e-5)
 
 
+def test_ce_forward_with_and_without_a_backward_to_follow():
+    """With an lse buffer the forward reads the last rows (what the memory-side cache holds) with cached
+    loads for the backward to find, without one it streams every row: two kernels over two row ranges
+    or one, the same numbers either way, also where the split falls inside the tensor."""
+    g = gen(1019)
+    for n, v, dt in ((9000, 32000, BF16), (300, 1000, F32), (5, 70001, F16)):
+        lg = (2 * torch.randn(n, v, generator=g)).to(dt).to(DEV)
+        y = torch.randint(0, v, (n,), generator=g)
+        y[::7] = -100
+        y = y.to(DEV)
+        loss, lse, nv, rows = _hip.ce_fwd(lg, y, -100, "mean")
+        loss2, lse2, nv2, rows2 = _hip.ce_fwd(lg, y, -100, "mean", for_backward=False)
+        assert lse2 is None and torch.equal(rows, rows2) and loss.item() == loss2.item() and nv.item() == nv2.item()
+        ref = torch.nn.functional.cross_entropy(lg.float(), y, ignore_index=-100)
+        assert loss.item() == pytest.approx(ref.item(), rel=1e-4)
+        ok = y != -100
+        assert torch.allclose(lse[ok], torch.logsumexp(lg.float(), -1)[ok], rtol=1e-5, atol=1e-5)
+
+
 CE1_CASES = CE_CASES + [(5, 140000, BF16), (3, 70000, F32), (4, 600, BF16), (3, 9000, F16),
                         # rows kept on the chip (registers + LDS of one workgroup per compute unit): aligned and
                         # odd widths, the widest that fits, and one past it (two sweeps)
