@@ -154,6 +154,18 @@ __device__ __forceinline__ void store16_stream(T* p, const u32x4& v) {
   __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
 }
 
+// 16 bytes per lane from global memory straight into LDS, no register in between
+// (global_load_lds_dwordx4): lane i of the wave writes wave_base[i]. `wave_base` is the same for
+// every lane of the wave; `src` is the lane's own address. Non-temporal like load16_stream.
+// The data is in LDS once the wave's outstanding vector-memory count says so (wait_vmem_all).
+template <typename T>
+__device__ __forceinline__ void load16_stream_to_lds(const T* src, u32x4* wave_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                   (__attribute__((address_space(3))) void*)wave_base, 16, 0, /*nt*/ 2);
+}
+// every vector-memory operation of this wave issued so far has completed
+__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 // Unpack a vector that is used by several passes without letting the compiler keep the
 // converted floats of the first pass alive for the later ones (fp16 conversions are otherwise
 // hoisted, and eight vectors per lane then take 230 registers instead of 60). FRESH = false is
@@ -340,6 +352,23 @@ bool grant_dynamic_lds(int bytes) {
   }
   allowed.fetch_or(1ull << dev, std::memory_order_release);
   return true;
+}
+
+// Workgroups of kernel K (`threads` threads, `dynamic_lds` bytes) one compute unit holds at once,
+// asked of the runtime once per kernel: the grid of a persistent kernel is this many per compute
+// unit and no more (a workgroup beyond them would start when the others have done their whole share).
+template <auto K>
+int resident_per_cu(int threads, size_t dynamic_lds) {
+  static std::atomic<int> cached{0};
+  int o = cached.load(std::memory_order_relaxed);
+  if (o == 0) {
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&o, K, threads, dynamic_lds) != hipSuccess || o < 1) {
+      (void)hipGetLastError();
+      o = 1;
+    }
+    cached.store(o, std::memory_order_relaxed);
+  }
+  return o;
 }
 
 #define FM_CHECK_ARG(cond, ...)                 \

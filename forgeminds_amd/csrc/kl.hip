@@ -28,8 +28,8 @@ struct KLState {
 };
 
 // Folds UNROLL vectors of student / teacher logits (vector u is column c_first + u * stride,
-// live when that is below nvec) into the running state.
-template <typename T, int UNROLL>
+// live when that is below nvec, or always with ALL) into the running state.
+template <typename T, int UNROLL, bool ALL = false>
 __device__ __forceinline__ void kl_update(KLState& k, const u32x4 (&rs)[UNROLL],
                                           const u32x4 (&rt)[UNROLL], int c_first, int stride,
                                           int nvec, float c1) {
@@ -41,7 +41,7 @@ __device__ __forceinline__ void kl_update(KLState& k, const u32x4 (&rs)[UNROLL],
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
     const int c = c_first + u * stride;
-    if (c < nvec) {
+    if (ALL || c < nvec) {
       Elem<T>::unpack(rs[u], zs[u]);
       Elem<T>::unpack(rt[u], zt[u]);
 #pragma unroll
@@ -59,7 +59,7 @@ __device__ __forceinline__ void kl_update(KLState& k, const u32x4 (&rs)[UNROLL],
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
     const int c = c_first + u * stride;
-    if (c < nvec) {   // uniform per vector; keeps (-inf) - (-inf) out of the A term
+    if (ALL || c < nvec) {   // uniform per vector; keeps (-inf) - (-inf) out of the A term
 #pragma unroll
       for (int e = 0; e < EPV; ++e) {
         ds += fast_exp2(__builtin_fmaf(zs[u][e], c1, -cms));
@@ -617,106 +617,165 @@ __global__ __launch_bounds__(THREADS) void kl_loss_grad_wide_kernel(const T* stu
 }
 
 // The same for rows that fit the CHIP: one 512-thread workgroup per compute unit has 256 registers a
-// thread and 128 KB of LDS to itself, which hold 24 + 8 vectors of each row per thread, 16384 vector
-// pairs (a 131072-column bf16 pair of rows, 512 KB) in all. The row is then read from memory once:
+// thread and 144 KB of LDS to itself, which hold 22 + 9 vectors of each row per thread, 15872 vector
+// pairs (a 126976-column bf16 pair of rows, 496 KB) in all. The row is then read from memory once:
 // 6 bytes per logit pair cross the L2 boundary instead of the 10 of the two sweeps above (which run
-// at the bandwidth of that boundary). Vectors past the 16384th, if any, are streamed and re-read
-// as above. Every thread parks and fetches only its own LDS slots: no barrier between the passes.
+// at the bandwidth of that boundary). Vectors past those, if any, are streamed and re-read
+// as above. Every thread fetches only its own LDS slots: no barrier between the passes.
+//
+// The grid is persistent (a workgroup per compute unit walks rows blockIdx.x, + gridDim.x, ...), and
+// the one workgroup a compute unit holds would otherwise load, then compute, then store in turn,
+// so the NEXT row's loads are issued from inside the gradient pass: as soon as a held vector pair has
+// given its gradient, its registers (or its LDS slots, filled straight from memory without a register
+// in between) take the same columns of the next row, and the loads run under the
+// exponentials of the rest of the pass. (A spilled register in that pass undoes this: its reload is
+// a vector-memory operation too, and waiting for it means waiting for every load issued before it.)
 constexpr int kHeldThreads = 512;
-constexpr int kHeldRegs = 24;    // vector pairs a thread keeps in registers
-constexpr int kHeldLds = 8;      // and in LDS
+constexpr int kHeldRegs = 22;    // vector pairs a thread keeps in registers
+constexpr int kHeldLds = 9;      // and in LDS
+constexpr int kHeldLdsBytes = kHeldLds * 2 * kHeldThreads * 16;
 template <typename T, typename GT>
 __global__ __launch_bounds__(kHeldThreads) void kl_loss_grad_held_kernel(const T* student,
                                                                           const T* __restrict__ teacher,
                                                                           float* __restrict__ lse_s,
                                                                           float* __restrict__ lse_t,
                                                                           float* __restrict__ row_kl,
-                                                                          GT* dstudent, int v, float inv_temp,
-                                                                          float mul, bool vec_ok) {
+                                                                          GT* dstudent, int64_t n, int v,
+                                                                          float inv_temp, float mul,
+                                                                          bool vec_ok) {
   constexpr int EPV = Elem<T>::kVec;
   constexpr int THREADS = kHeldThreads, RI = kHeldRegs, LI = kHeldLds;
   constexpr int NW = THREADS / 64;
   extern __shared__ u32x4 parked[];          // [LI][2][THREADS]
-  __shared__ float smem[5 * NW];
-  const int64_t row = blockIdx.x;
-  const T* sp_ = student + row * (int64_t)v;
-  const T* tp_ = teacher + row * (int64_t)v;
-  GT* gp = dstudent + row * (int64_t)v;
-  const RowSplit sp = split_row<EPV>(row, v, vec_ok);
+  __shared__ float smem[2][5 * NW];          // by row parity: a wave may reach the next row's merge
+                                             // while another still reads this row's
   const int tid = threadIdx.x;
-  const int ne = edge_count(sp, v);
+  const int wave_first = __builtin_amdgcn_readfirstlane(tid & ~63);   // (a scalar, and known to be one)
+  const uint32_t lane_el = (uint32_t)tid * EPV;   // this thread's first element inside a slot
   const float c1 = kLog2e * inv_temp;
+  // slot i of a row: THREADS vectors from vector i * THREADS on, one per thread. The row's base is
+  // the same for the whole workgroup; a thread adds its own 32-bit offset.
+  auto slot = [&](auto* row_base, int i) { return row_base + (int64_t)i * (THREADS * EPV) + lane_el; };
+  auto park = [&](int j, int which) { return parked + (j * 2 + which) * THREADS; };
 
-  // all of a thread's loads are issued before the first is used
   u32x4 hs[RI], ht[RI];
+  int64_t row = blockIdx.x;
+  if (row >= n) return;
+  // A slot is held only when every thread has a column in it (`full` of them, the same for the
+  // whole workgroup); the ragged end of the row is streamed with the remainder.
+  auto full_slots = [](const RowSplit& sp) {
+    const int f = sp.nvec / THREADS;
+    return f < RI + LI ? f : RI + LI;
+  };
+  {
+    const RowSplit sp = split_row<EPV>(row, v, vec_ok);
+    const T* sb = student + row * (int64_t)v + sp.head;
+    const T* tb = teacher + row * (int64_t)v + sp.head;
+    const int full = full_slots(sp);
 #pragma unroll
-  for (int i = 0; i < RI; ++i) {
-    const int c = clamp_col(i * THREADS + tid, sp.nvec);
-    hs[i] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
-    ht[i] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
-  }
-  KLState k{kNegBig, 0.f, kNegBig, 0.f, 0.f};
-#pragma unroll
-  for (int j = 0; j < LI; j += 2) {
-    u32x4 rs[2], rt[2];
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int c = clamp_col((RI + j + u) * THREADS + tid, sp.nvec);
-      rs[u] = load16_stream(sp_ + sp.head + (int64_t)c * EPV);
-      rt[u] = load16_stream(tp_ + sp.head + (int64_t)c * EPV);
+    for (int i = 0; i < RI; ++i) {
+      if (i < full) {
+        hs[i] = load16_stream(slot(sb, i));
+        ht[i] = load16_stream(slot(tb, i));
+      }
     }
-    kl_update<T, 2>(k, rs, rt, (RI + j) * THREADS + tid, THREADS, sp.nvec, c1);
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      parked[((j + u) * 2 + 0) * THREADS + tid] = rs[u];
-      parked[((j + u) * 2 + 1) * THREADS + tid] = rt[u];
+    for (int j = 0; j < LI; ++j) {
+      if (RI + j < full) {
+        load16_stream_to_lds(slot(sb, RI + j), park(j, 0) + wave_first);
+        load16_stream_to_lds(slot(tb, RI + j), park(j, 1) + wave_first);
+      }
     }
   }
+  for (int flip = 0; row < n; row += gridDim.x, flip ^= 1) {
+    const T* sp_ = student + row * (int64_t)v;
+    const T* tp_ = teacher + row * (int64_t)v;
+    GT* gp = dstudent + row * (int64_t)v;
+    const RowSplit sp = split_row<EPV>(row, v, vec_ok);
+    const int ne = edge_count(sp, v);
+    const int full = full_slots(sp);
+
+    // (one vector pair at a time: two at a time need 16 more registers, and then one held pair
+    // is spilled)
+    KLState k{kNegBig, 0.f, kNegBig, 0.f, 0.f};
 #pragma unroll
-  for (int i = 0; i < RI; i += 2) {
-    const u32x4 rs[2] = {hs[i], hs[i + 1]}, rt[2] = {ht[i], ht[i + 1]};
-    kl_update<T, 2>(k, rs, rt, i * THREADS + tid, THREADS, sp.nvec, c1);
-  }
-  constexpr int HELD = (RI + LI) * THREADS;
-  for (int c0 = HELD; c0 < sp.nvec; c0 += THREADS * 2) {
-    u32x4 rs[2], rt[2];
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
-      rs[u] = load16(sp_ + sp.head + (int64_t)c * EPV);
-      rt[u] = load16(tp_ + sp.head + (int64_t)c * EPV);
+    for (int i = 0; i < RI; ++i) {
+      if (i < full) {
+        const u32x4 rs[1] = {hs[i]}, rt[1] = {ht[i]};
+        kl_update<T, 1, true>(k, rs, rt, 0, 0, 0, c1);
+      }
     }
-    kl_update<T, 2>(k, rs, rt, c0 + tid, THREADS, sp.nvec, c1);
-  }
-  for (int e = tid; e < ne; e += THREADS) {
-    const int col = edge_col(sp, e);
-    kl_update1(k, Elem<T>::load1(sp_ + col) * c1, Elem<T>::load1(tp_ + col) * c1);
-  }
-  float l2s, l2t, kl2;
-  kl_merge<NW>(k, smem, &l2s, &l2t, &kl2);
-  if (tid == 0) {
-    if (lse_s != nullptr) lse_s[row] = l2s * kLn2;
-    if (lse_t != nullptr) lse_t[row] = l2t * kLn2;
-    row_kl[row] = kl2 * kLn2;
-  }
+    wait_vmem_all();   // the LDS slots were filled by loads that name no register
 #pragma unroll
-  for (int i = 0; i < RI; ++i) {
-    const int c = i * THREADS + tid;
-    // (behind an empty asm, so that the compiler unpacks the vector again here instead of keeping
-    // the floats of the first pass alive for all 24 pairs)
-    touch(hs[i]);
-    touch(ht[i]);
-    if (c < sp.nvec) kl_grad_vec<T, GT>(hs[i], ht[i], gp + sp.head + (int64_t)c * EPV, c1, l2s, l2t, mul);
-  }
+    for (int j = 0; j < LI; ++j) {
+      if (RI + j < full) {
+        const u32x4 rs[1] = {park(j, 0)[tid]}, rt[1] = {park(j, 1)[tid]};
+        kl_update<T, 1, true>(k, rs, rt, 0, 0, 0, c1);
+      }
+    }
+    const int held = full * THREADS;
+    for (int c0 = held; c0 < sp.nvec; c0 += THREADS * 2) {
+      u32x4 rs[2], rt[2];
 #pragma unroll
-  for (int j = 0; j < LI; ++j) {
-    const int c = (RI + j) * THREADS + tid;
-    if (c < sp.nvec)
-      kl_grad_vec<T, GT>(parked[(j * 2 + 0) * THREADS + tid], parked[(j * 2 + 1) * THREADS + tid],
-                         gp + sp.head + (int64_t)c * EPV, c1, l2s, l2t, mul);
+      for (int u = 0; u < 2; ++u) {
+        const int c = clamp_col(c0 + u * THREADS + tid, sp.nvec);
+        rs[u] = load16(sp_ + sp.head + (int64_t)c * EPV);
+        rt[u] = load16(tp_ + sp.head + (int64_t)c * EPV);
+      }
+      kl_update<T, 2>(k, rs, rt, c0 + tid, THREADS, sp.nvec, c1);
+    }
+    for (int e = tid; e < ne; e += THREADS) {
+      const int col = edge_col(sp, e);
+      kl_update1(k, Elem<T>::load1(sp_ + col) * c1, Elem<T>::load1(tp_ + col) * c1);
+    }
+    float l2s, l2t, kl2;
+    kl_merge<NW>(k, smem[flip], &l2s, &l2t, &kl2);
+    if (tid == 0) {
+      if (lse_s != nullptr) lse_s[row] = l2s * kLn2;
+      if (lse_t != nullptr) lse_t[row] = l2t * kLn2;
+      row_kl[row] = kl2 * kLn2;
+    }
+
+    // the gradient of every held pair, and in its place the same columns of the next row
+    const int64_t next = row + gridDim.x;
+    const bool more = next < n;   // the same for the whole workgroup
+    const RowSplit nsp = split_row<EPV>(more ? next : row, v, vec_ok);
+    const int nfull = more ? full_slots(nsp) : 0;
+    const T* nsb = student + (more ? next : row) * (int64_t)v + nsp.head;
+    const T* ntb = teacher + (more ? next : row) * (int64_t)v + nsp.head;
+    GT* gb = gp + sp.head;
+#pragma unroll
+    for (int i = 0; i < RI; ++i) {
+      if (i < full) {
+        // (behind an empty asm, so that the compiler unpacks the vector again here instead of
+        // keeping the floats of the first pass alive for all the pairs)
+        touch(hs[i]);
+        touch(ht[i]);
+        kl_grad_vec<T, GT>(hs[i], ht[i], slot(gb, i), c1, l2s, l2t, mul);
+      }
+      if (i < nfull) {
+        hs[i] = load16_stream(slot(nsb, i));
+        ht[i] = load16_stream(slot(ntb, i));
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < LI; ++j) {
+      u32x4 rs, rt;
+      if (RI + j < full) {
+        rs = park(j, 0)[tid];
+        rt = park(j, 1)[tid];
+        touch(rs);   // in registers before the slots are given away
+        touch(rt);
+      }
+      if (RI + j < nfull) {
+        load16_stream_to_lds(slot(nsb, RI + j), park(j, 0) + wave_first);
+        load16_stream_to_lds(slot(ntb, RI + j), park(j, 1) + wave_first);
+      }
+      if (RI + j < full) kl_grad_vec<T, GT>(rs, rt, slot(gb, RI + j), c1, l2s, l2t, mul);
+    }
+    // what was not held, and the row's unaligned edges
+    kl_grad_sweep<T, GT, THREADS, 2>(sp_, tp_, gp, sp, v, c1, l2s, l2t, mul, held);
   }
-  // what was not held, and the row's unaligned edges
-  kl_grad_sweep<T, GT, THREADS, 2>(sp_, tp_, gp, sp, v, c1, l2s, l2t, mul, HELD < sp.nvec ? HELD : sp.nvec);
 }
 
 // Narrow rows (at most 1024 classes: classifier distillation, not vocabularies): TPR lanes per
@@ -1207,12 +1266,14 @@ int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, floa
     const int64_t wvec = v / (dtype == FM_F32 ? 4 : 8);
     const bool held = vec_ok && (dtype == FM_F32 ? wvec >= 7168 : (wvec >= 15360 && wvec <= 24576));
 #define WIDE(T, GT)                                                                                \
-  if (held && fm_host::grant_dynamic_lds<&kl_loss_grad_held_kernel<T, GT>>(kHeldLds * 2 * kHeldThreads * 16))                         \
-    FM_LAUNCH((kl_loss_grad_held_kernel<T, GT>), wgrid, dim3(kHeldThreads),                        \
-              (size_t)kHeldLds * 2 * kHeldThreads * 16, st, static_cast<const T*>(student),        \
+  if (held && fm_host::grant_dynamic_lds<&kl_loss_grad_held_kernel<T, GT>>(kHeldLdsBytes)) {        \
+    const int64_t fit = (int64_t)fm_host::num_cus() *                                              \
+        fm_host::resident_per_cu<&kl_loss_grad_held_kernel<T, GT>>(kHeldThreads, kHeldLdsBytes);   \
+    FM_LAUNCH((kl_loss_grad_held_kernel<T, GT>), dim3((unsigned)(n < fit ? n : fit)),              \
+              dim3(kHeldThreads), (size_t)kHeldLdsBytes, st, static_cast<const T*>(student),       \
               static_cast<const T*>(teacher), lse_s, lse_t, row_kl, static_cast<GT*>(dstudent),    \
-              (int)v, inv_temperature, mul_w, vec_ok);                                             \
-  else                                                                                             \
+              n, (int)v, inv_temperature, mul_w, vec_ok);                                          \
+  } else                                                                                           \
     FM_LAUNCH((kl_loss_grad_wide_kernel<T, GT, 1024, 2>), wgrid, dim3(1024), 0, st,                \
               static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t,        \
               row_kl, static_cast<GT*>(dstudent), (int)v, inv_temperature, mul_w, vec_ok)
