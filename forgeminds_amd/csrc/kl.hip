@@ -1239,8 +1239,23 @@ int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, floa
       return FM_OK;
     }
   }
-  const bool one_pass = n > 0 && fm_host::aligned16(student) && fm_host::aligned16(teacher) &&
-                        fm_host::aligned16(dstudent) && nvec <= kOnePassMaxVec;
+  // Aligned rows of more than 2048 vectors: the form that keeps the row pair on the chip (a workgroup
+  // per compute unit with 144 KB of LDS, which the device has to grant once per kernel), the next
+  // row's loads under this row's gradient. It reads the row once where the two sweeps of the wide
+  // form read it twice, and below 4096 vectors it beats the register form wherever that one's
+  // power-of-two vectors per thread leave lanes idle. Measured against what ran before (us, 2^28
+  // bf16 or 2^27 fp32 logits per tensor; r = the register form, w = the two sweeps):
+  //   bf16 columns  8192: 538 / 272 r   16384: 389 / 308 r   18432: 417 / 442 r   20480: 374 / 405 r
+  //                24576: 331 / 374 r   32000: 350 / 364 r   40000: 352 / 351 w   50304: 326 / 347 w
+  //                65536: 311 / 372 w  100000: 329 / 368 w  128256: 330 / 372 w  151936: 317 / 338 w
+  //               200000: 374 / 380 w  262144: 407 / 416 w
+  //   fp32 columns  8192: 316 / 263 r    9216: 319 / 364 r   12288: 284 / 343 r   16384: 304 / 333 r
+  //                20000: 297 / 336 w   40000: 302 / 368 w   65536: 302 / 379 w  128256: 336 / 409 w
+  //               262144: 393 / 440 w
+  const bool aligned = fm_host::aligned16(student) && fm_host::aligned16(teacher) &&
+                       fm_host::aligned16(dstudent);
+  const bool held = n > 0 && aligned && nvec > 2048 && nvec <= 32768;
+  const bool one_pass = n > 0 && aligned && nvec <= kOnePassMaxVec && !held;
   if (!one_pass) {
     if (n == 0) {
       return fm_kl_fwd(student, teacher, lse_s, lse_t, row_kl, loss, n, v, dtype, inv_temperature, reduction,
@@ -1253,18 +1268,6 @@ int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, floa
                         fm_host::aligned16(dstudent);
     const float mul_w = inv_temperature * scale;
     const dim3 wgrid((unsigned)n);
-    // Aligned rows of the right width: the form that keeps the row pair on the chip (a workgroup per
-    // compute unit with 128 KB of LDS, which the device has to grant once per kernel). It reads the
-    // row once where the two sweeps read it twice, but leaves a compute unit one workgroup of eight
-    // waves, and the 16-bit rows are bound by their four exponentials per logit pair as much as by
-    // bytes. Measured against the two sweeps (us, 2^28 bf16 or 2^27 fp32 logits per tensor):
-    //   bf16 columns  40000: 530 / 381   65536: 417 / 370   100000: 376 / 372   110000: 411 / 373
-    //                128256: 355 / 372  151936: 312 / 338   180000: 351 / 363   200000: 385 / 382
-    //                262144: 437 / 420
-    //   fp32 columns  20000: 375 / 336   30000: 331 / 358    40000: 311 / 368    65536: 342 / 379
-    //                128256: 322 / 409  262144: 386 / 440
-    const int64_t wvec = v / (dtype == FM_F32 ? 4 : 8);
-    const bool held = vec_ok && (dtype == FM_F32 ? wvec >= 7168 : (wvec >= 15360 && wvec <= 24576));
 #define WIDE(T, GT)                                                                                \
   if (held && fm_host::grant_dynamic_lds<&kl_loss_grad_held_kernel<T, GT>>(kHeldLdsBytes)) {        \
     const int64_t fit = (int64_t)fm_host::num_cus() *                                              \

@@ -346,6 +346,48 @@ def test_ce_loss_and_gradient_in_one_pass(n, v, dt, reduction):
     assert_close_lowp(dl, dl3.float().cpu(), dt, "vs two-pass", ulps=2.0, cancel=cancel)
 
 
+@pytest.mark.parametrize("n,v,dt", [(600, 66000, BF16), (300, 70001, F16), (530, 33032, F32)])
+def test_ce_one_pass_many_wide_rows_with_ignored_ones(n, v, dt):
+    """More rows than the chip has compute units, at widths kept on the chip (one workgroup per
+    compute unit at a time), with ignored rows first, last, 256 apart and two in a row. Checked
+    against the two-pass kernels (which the other tests pin to the oracle) and, on a sample of
+    rows, against the oracle itself."""
+    g = gen(1051)
+    lg = (2 * torch.randn(n, v, generator=g)).to(dt)
+    y = torch.randint(0, v, (n,), generator=g)
+    y[torch.rand(n, generator=g) < 0.15] = -100
+    y[3] = -100
+    y[5::256] = -100                # every row a compute unit would get in turn
+    y[7 + 256] = -100
+    y[9] = -100
+    y[9 + 256] = -100
+    y[n - 1] = -100                 # the last row of all
+    y[10] = v - 1                   # labels at both ends of the row
+    y[11] = 0
+    lgd, yd = lg.to(DEV), y.to(DEV)
+    keep = lgd.clone()
+    for reduction in ("mean", "sum"):
+        loss, dl, nv, rows = _hip.ce_loss_grad(lgd, yd, -100, reduction)
+        torch.cuda.synchronize()
+        assert torch.equal(lgd, keep)
+        n_valid = int((y != -100).sum())
+        assert nv.item() == n_valid
+        cancel = 1.0 / n_valid if reduction == "mean" else 1.0
+        loss3, lse, nv3, _ = _hip.ce_fwd(keep, yd, -100, reduction)
+        dl3 = _hip.ce_bwd(keep, yd, lse, nv3 if reduction == "mean" else None, None, -100)
+        assert loss3.item() == pytest.approx(loss.item(), rel=1e-6, abs=1e-7)
+        assert_close_lowp(dl, dl3.float().cpu(), dt, "vs two-pass", ulps=2.0, cancel=cancel)
+        ign = (y == -100)
+        assert not dl.cpu()[ign].any() and not rows.cpu()[ign].any()
+        sample = torch.tensor([0, 3, 5, 9, 10, 11, 255, 256, 257, 261, 263, 265, 299, n - 2, n - 1])
+        _, og = O.cross_entropy(lg[sample].float(), y[sample])
+        ov = max(1, int((y[sample] != -100).sum()))
+        want = og * ov * (1.0 / n_valid if reduction == "mean" else 1.0)
+        assert_close_lowp(dl[sample.to(DEV)], want.float(), dt, "sampled rows vs oracle", ulps=3.0, cancel=cancel)
+        loss2, dl2, _, _ = _hip.ce_loss_grad(lgd.clone(), yd, -100, reduction, inplace=True)
+        assert torch.equal(dl2, dl) and loss2.item() == loss.item()
+
+
 def test_ce_kl_vector_rows_agree_with_the_scalar_form():
     """Narrow rows of whole aligned vectors take 16-byte loads; the same rows one element per
     load (the form for other widths and alignments, reached here by buffers that start one element
@@ -495,7 +537,12 @@ KL1_CASES = [(64, 32000, BF16, 2.0, BF16), (6, 5000, F32, 1.0, F32), (3, 1, F32,
              # rows that stay on the chip between the passes (registers + LDS of one workgroup per
              # compute unit): aligned and odd widths, in place, and rows past what the chip holds
              (3, 128256, BF16, 1.0, BF16), (2, 151937, F16, 2.0, F16), (2, 140000, F32, 1.0, F32),
-             (2, 196608, BF16, 1.0, BF16), (3, 28673, F32, 2.0, F32)]
+             (2, 196608, BF16, 1.0, BF16), (3, 28673, F32, 2.0, F32),
+             # the same with more rows than the chip has compute units: a workgroup then walks two or
+             # three rows and loads the next one from inside this one's gradient pass (even and odd
+             # widths, rows of fewer slots than a thread holds, the last row of a workgroup)
+             (600, 20000, BF16, 2.0, BF16), (300, 17001, F16, 1.0, F32), (530, 9001, F32, 1.0, F32),
+             (257, 40008, BF16, 1.0, BF16), (520, 16392, BF16, 1.0, F32)]
 
 
 @pytest.mark.parametrize("n,v,dt,T,gdt", KL1_CASES)
