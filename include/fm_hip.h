@@ -231,11 +231,12 @@ int fm_kl_fwd(const void* student, const void* teacher, float* lse_s, float* lse
 /* KL AND its gradient from one read of both rows, the dataflow of the reference's kernel
  * (kl.py:73-135 writes dKL/dstudent in the forward, _KLDivFn.forward kl.py:154-176):
  * fm_kl_fwd's outputs plus dstudent = fm_kl_bwd's result for grad_out = 1 and
- * scale = 1/n (FM_REDUCE_MEAN) or 1 (FM_REDUCE_SUM). Rows of at most 64 KiB stay in
+ * scale = 1/n (FM_REDUCE_MEAN) or 1 (FM_REDUCE_SUM). Rows of at most 32 KiB stay in
  * registers between the log-sum-exps and the store (4 + 2 bytes per pair of 16-bit logits
- * instead of 4 + 4 + 2); wider rows are swept twice inside the same launch, or, where that is
- * measured faster (fp32 rows from 112 KiB on, 16-bit rows of 240-384 KiB), kept in the registers and
- * LDS of one workgroup per compute unit and read once. dstudent may be the student buffer itself when
+ * instead of 4 + 4 + 2); rows of up to 512 KiB are kept in the registers and LDS of one workgroup
+ * per compute unit (496 KiB of each row pair; the rest is read twice) while that workgroup already
+ * loads its next row; wider rows and unaligned buffers are swept twice inside the same launch.
+ * dstudent may be the student buffer itself when
  * grad_dtype == dtype (kl.py:146-150, reuse=True); lse_s / lse_t may be NULL.
  * fm_scale_inplace applies an upstream gradient other than 1. */
 int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, float* lse_t,
