@@ -541,8 +541,8 @@ KL1_CASES = [(64, 32000, BF16, 2.0, BF16), (6, 5000, F32, 1.0, F32), (3, 1, F32,
              # the same with more rows than the chip has compute units: a workgroup then walks two or
              # three rows and loads the next one from inside this one's gradient pass (even and odd
              # widths, rows of fewer slots than a thread holds, the last row of a workgroup)
-             (600, 20000, BF16, 2.0, BF16), (300, 17001, F16, 1.0, F32), (530, 9001, F32, 1.0, F32),
-             (257, 40008, BF16, 1.0, BF16), (520, 16392, BF16, 1.0, F32)]
+             (600, 20000, BF16, 2.0, BF16), (300, 17001, F16, 2.0, F32), (530, 9001, F32, 1.0, F32),
+             (257, 40008, BF16, 1.0, BF16), (520, 16392, BF16, 1.0, BF16)]
 
 
 @pytest.mark.parametrize("n,v,dt,T,gdt", KL1_CASES)
