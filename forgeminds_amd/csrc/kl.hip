@@ -633,9 +633,8 @@ __global__ __launch_bounds__(THREADS) void kl_loss_grad_wide_kernel(const T* stu
 constexpr int kHeldThreads = 512;
 constexpr int kHeldRegs = 22;    // vector pairs a thread keeps in registers
 constexpr int kHeldLds = 9;      // and in LDS
-constexpr int kHeldLdsBytes = kHeldLds * 2 * kHeldThreads * 16;
-template <typename T, typename GT>
-__global__ __launch_bounds__(kHeldThreads) void kl_loss_grad_held_kernel(const T* student,
+template <typename T, typename GT, int THREADS = kHeldThreads, int RI = kHeldRegs, int LI = kHeldLds>
+__global__ __launch_bounds__(THREADS) void kl_loss_grad_held_kernel(const T* student,
                                                                           const T* __restrict__ teacher,
                                                                           float* __restrict__ lse_s,
                                                                           float* __restrict__ lse_t,
@@ -644,7 +643,6 @@ __global__ __launch_bounds__(kHeldThreads) void kl_loss_grad_held_kernel(const T
                                                                           float inv_temp, float mul,
                                                                           bool vec_ok) {
   constexpr int EPV = Elem<T>::kVec;
-  constexpr int THREADS = kHeldThreads, RI = kHeldRegs, LI = kHeldLds;
   constexpr int NW = THREADS / 64;
   extern __shared__ u32x4 parked[];          // [LI][2][THREADS]
   __shared__ float smem[2][5 * NW];          // by row parity: a wave may reach the next row's merge
@@ -776,6 +774,45 @@ __global__ __launch_bounds__(kHeldThreads) void kl_loss_grad_held_kernel(const T
     // what was not held, and the row's unaligned edges
     kl_grad_sweep<T, GT, THREADS, 2>(sp_, tp_, gp, sp, v, c1, l2s, l2t, mul, held);
   }
+}
+
+// One launch shape of the kernel above; false when the device does not grant the LDS it needs.
+template <typename T, typename GT, int TH, int RI, int LI>
+bool launch_held_shape(const T* student, const T* teacher, float* lse_s, float* lse_t, float* row_kl,
+                       GT* dstudent, int64_t n, int v, float inv_temp, float mul, bool vec_ok,
+                       hipStream_t st) {
+  constexpr int lds = LI * 2 * TH * 16;
+  if (lds > 65536 && !fm_host::grant_dynamic_lds<&kl_loss_grad_held_kernel<T, GT, TH, RI, LI>>(lds)) return false;
+  const int64_t fit = (int64_t)fm_host::num_cus() *
+                      fm_host::resident_per_cu<&kl_loss_grad_held_kernel<T, GT, TH, RI, LI>>(TH, lds);
+  FM_LAUNCH((kl_loss_grad_held_kernel<T, GT, TH, RI, LI>), dim3((unsigned)(n < fit ? n : fit)), dim3(TH),
+            (size_t)lds, st, student, teacher, lse_s, lse_t, row_kl, dstudent, n, v, inv_temp, mul, vec_ok);
+  return true;
+}
+
+// The shape by row width. 16-bit rows are bound by arithmetic, and a compute unit that holds
+// SEVERAL workgroups, each on a row of its own, keeps its vector ALUs busy while one of them waits
+// for memory or at its barrier: three 256-thread workgroups (13 + 3 slots: at most 168 registers
+// and 24 KB of LDS each) up to 4096 vectors a row, two (22 + 9 slots) up to 7936, one 512-thread
+// workgroup beyond. us for bf16 rows, three / two / one workgroup a unit: [8192,20000] 204 / 226 /
+// 264, [16384,24576] 446 / 463 / 504, [16384,32000] 598 / 638 / 769, [8192,50304] 510 / 494 / 511,
+// [4096,65536] 344 / 325 / 325. fp32 rows are bound by bytes and run the same in every shape
+// ([8192,32000]: 588 / 576 / 568), so they take the one.
+template <typename T, typename GT>
+bool launch_held(const T* student, const T* teacher, float* lse_s, float* lse_t, float* row_kl,
+                 GT* dstudent, int64_t n, int v, int64_t nvec, float inv_temp, float mul, bool vec_ok,
+                 hipStream_t st) {
+  if constexpr (sizeof(T) == 2) {
+    if (nvec <= 4608)
+      return launch_held_shape<T, GT, 256, 13, 3>(student, teacher, lse_s, lse_t, row_kl, dstudent, n, v,
+                                                  inv_temp, mul, vec_ok, st);
+    if (nvec <= 8192 &&
+        launch_held_shape<T, GT, 256, 22, 9>(student, teacher, lse_s, lse_t, row_kl, dstudent, n, v, inv_temp,
+                                             mul, vec_ok, st))
+      return true;
+  }
+  return launch_held_shape<T, GT, kHeldThreads, kHeldRegs, kHeldLds>(student, teacher, lse_s, lse_t, row_kl,
+                                                                     dstudent, n, v, inv_temp, mul, vec_ok, st);
 }
 
 // Narrow rows (at most 1024 classes: classifier distillation, not vocabularies): TPR lanes per
@@ -1239,19 +1276,18 @@ int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, floa
       return FM_OK;
     }
   }
-  // Aligned rows of more than 2048 vectors: the form that keeps the row pair on the chip (a workgroup
-  // per compute unit with 144 KB of LDS, which the device has to grant once per kernel), the next
-  // row's loads under this row's gradient. It reads the row once where the two sweeps of the wide
-  // form read it twice, and below 4096 vectors it beats the register form wherever that one's
-  // power-of-two vectors per thread leave lanes idle. Measured against what ran before (us, 2^28
-  // bf16 or 2^27 fp32 logits per tensor; r = the register form, w = the two sweeps):
-  //   bf16 columns  8192: 538 / 272 r   16384: 389 / 308 r   18432: 417 / 442 r   20480: 374 / 405 r
-  //                24576: 331 / 374 r   32000: 350 / 364 r   40000: 352 / 351 w   50304: 326 / 347 w
-  //                65536: 311 / 372 w  100000: 329 / 368 w  128256: 330 / 372 w  151936: 317 / 338 w
-  //               200000: 374 / 380 w  262144: 407 / 416 w
-  //   fp32 columns  8192: 316 / 263 r    9216: 319 / 364 r   12288: 284 / 343 r   16384: 304 / 333 r
-  //                20000: 297 / 336 w   40000: 302 / 368 w   65536: 302 / 379 w  128256: 336 / 409 w
-  //               262144: 393 / 440 w
+  // Aligned rows of more than 2048 vectors: the form that keeps the row pair on the chip (registers
+  // and LDS of one to three workgroups per compute unit; more than 64 KB of LDS has to be granted
+  // by the device once per kernel), the next row's loads under this row's gradient. It reads the row
+  // once where the two sweeps of the wide form read it twice, and below 4096 vectors it beats the
+  // register form wherever that one's power-of-two vectors per thread leave lanes idle. Measured
+  // against what it replaced (us, 2^28 bf16 or 2^27 fp32 logits per tensor; r = the register form,
+  // w = the two sweeps):
+  //   bf16 columns 16384: 289 / 270 r (stays)   18432: 291 / 442 r   24576: 286 / 374 r
+  //                32000: 292 / 364 r   40000: 321 / 351 w   50304: 310 / 347 w   65536: 315 / 372 w
+  //                80000: 335 / 368 w  128256: 335 / 372 w  151936: 317 / 338 w  262144: 407 / 416 w
+  //   fp32 columns  8192: 318 / 261 r (stays)    9216: 320 / 364 r   16384: 292 / 333 r
+  //                32000: 294 / 358 w   65536: 306 / 379 w  128256: 336 / 409 w  262144: 393 / 440 w
   const bool aligned = fm_host::aligned16(student) && fm_host::aligned16(teacher) &&
                        fm_host::aligned16(dstudent);
   const bool held = n > 0 && aligned && nvec > 2048 && nvec <= 32768;
@@ -1269,14 +1305,9 @@ int fm_kl_loss_grad(const void* student, const void* teacher, float* lse_s, floa
     const float mul_w = inv_temperature * scale;
     const dim3 wgrid((unsigned)n);
 #define WIDE(T, GT)                                                                                \
-  if (held && fm_host::grant_dynamic_lds<&kl_loss_grad_held_kernel<T, GT>>(kHeldLdsBytes)) {        \
-    const int64_t fit = (int64_t)fm_host::num_cus() *                                              \
-        fm_host::resident_per_cu<&kl_loss_grad_held_kernel<T, GT>>(kHeldThreads, kHeldLdsBytes);   \
-    FM_LAUNCH((kl_loss_grad_held_kernel<T, GT>), dim3((unsigned)(n < fit ? n : fit)),              \
-              dim3(kHeldThreads), (size_t)kHeldLdsBytes, st, static_cast<const T*>(student),       \
-              static_cast<const T*>(teacher), lse_s, lse_t, row_kl, static_cast<GT*>(dstudent),    \
-              n, (int)v, inv_temperature, mul_w, vec_ok);                                          \
-  } else                                                                                           \
+  if (!(held && launch_held<T, GT>(static_cast<const T*>(student), static_cast<const T*>(teacher), \
+                                   lse_s, lse_t, row_kl, static_cast<GT*>(dstudent), n, (int)v,   \
+                                   nvec, inv_temperature, mul_w, vec_ok, st)))                     \
     FM_LAUNCH((kl_loss_grad_wide_kernel<T, GT, 1024, 2>), wgrid, dim3(1024), 0, st,                \
               static_cast<const T*>(student), static_cast<const T*>(teacher), lse_s, lse_t,        \
               row_kl, static_cast<GT*>(dstudent), (int)v, inv_temperature, mul_w, vec_ok)

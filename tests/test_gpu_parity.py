@@ -538,11 +538,13 @@ KL1_CASES = [(64, 32000, BF16, 2.0, BF16), (6, 5000, F32, 1.0, F32), (3, 1, F32,
              # compute unit): aligned and odd widths, in place, and rows past what the chip holds
              (3, 128256, BF16, 1.0, BF16), (2, 151937, F16, 2.0, F16), (2, 140000, F32, 1.0, F32),
              (2, 196608, BF16, 1.0, BF16), (3, 28673, F32, 2.0, F32),
-             # the same with more rows than the chip has compute units: a workgroup then walks two or
-             # three rows and loads the next one from inside this one's gradient pass (even and odd
-             # widths, rows of fewer slots than a thread holds, the last row of a workgroup)
+             # the same with more rows than the chip holds workgroups (one to three per compute unit
+             # by row width): a workgroup then walks two or three rows and loads the next one from
+             # inside this one's gradient pass (even and odd widths, rows of fewer slots than a thread
+             # holds, the last row of a workgroup)
              (600, 20000, BF16, 2.0, BF16), (300, 17001, F16, 2.0, F32), (530, 9001, F32, 1.0, F32),
-             (257, 40008, BF16, 1.0, BF16), (520, 16392, BF16, 1.0, BF16)]
+             (257, 40008, BF16, 1.0, BF16), (520, 16392, BF16, 1.0, BF16),
+             (1700, 16400, BF16, 2.0, BF16), (1100, 36880, BF16, 2.0, BF16), (300, 70000, BF16, 2.0, BF16)]
 
 
 @pytest.mark.parametrize("n,v,dt,T,gdt", KL1_CASES)
