@@ -534,18 +534,18 @@ def make_workload(name, torch, L, dev):
                                          st), "fm_kl_loss_grad")
 
             def step():
-                both()      # forward: loss, and the gradient from a second sweep of each row
+                both()      # forward: loss and gradient, the row pair read once
                 _check(L.fm_scale_inplace(gs.data_ptr(), one.data_ptr(), n * v, BF, st),
                        "fm_scale_inplace")   # backward: upstream gradient 1, nothing to move
 
             w.step = step
             w.dominant_launch = both
-            w.dominant = "kl_loss_grad_held_kernel<bf16,bf16>"
+            w.dominant = "kl_loss_grad_held_kernel<bf16,bf16,512,22,9>"
             w.dominant_bytes = w.bytes = n * v * 6
             w.desc = (f"KL loss + gradient in one launch bf16 [{n},{v}], T=2, mean; algorithmic 6 B/logit pair "
                       "(read s,t + write g). The pair of rows stays in the registers and LDS of one workgroup per "
-                      "compute unit between the two passes: it is read once, and the L2-side counters show the "
-                      "algorithmic bytes")
+                      "compute unit between the two passes (which loads its next row under this row's "
+                      "gradient): it is read once, and the L2-side counters show the algorithmic bytes")
             w.rows = n
             w.floor = [lambda i: ((s, t), (gs,))]
             return w
