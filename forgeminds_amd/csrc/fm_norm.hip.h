@@ -728,12 +728,21 @@ __global__ __launch_bounds__(kWideThreads) void norm_bwd_wide(
 // Rows just past the register path (up to ITERS vectors per thread of a 1024-thread workgroup,
 // ITERS * EPV <= 32: 32768 columns): the per-thread fp32 column sums of the weight gradient still
 // fit the registers, so one persistent kernel does the whole backward. A workgroup walks a
-// contiguous chunk of rows and holds the packed x and dy of a row in registers between the
+// contiguous chunk of rows and holds the packed x and dy of a row on the chip between the
 // reduction and the output sweep (2 reads + 1 write from HBM, as on the register path; re-reading
 // them through the caches instead was 1.5 times slower). The weight comes from cache each time,
-// not from registers or LDS. The widest forms spill a few registers and still beat two kernels
-// that read the row three times; only fp32 LayerNorm past six vectors per thread does not.
-template <typename T, typename WT, bool LN, int ITERS>
+// not from registers or LDS.
+//
+// Loads are unconditional, from clamped columns (a load behind a lane-dependent branch is waited
+// for at once). With PARK the dy vectors live in LDS instead of registers, filled straight from
+// memory (16 bytes a lane, no register in between): the forms with the most accumulators
+// (LayerNorm from four vectors a thread, fp32 rows) otherwise push registers out to scratch.
+// With PIPE the NEXT row is loaded from inside the output sweep (a vector that has given its
+// output hands its registers, or its LDS slot, to the same columns of the next row): the one
+// workgroup a compute unit holds otherwise loads, reduces and stores in turn. That pays for the
+// widest fp32 rows only; elsewhere the wait for the previous row's stores at the top of a row
+// (one counter for a wave's loads and stores) costs what the overlap gains.
+template <typename T, typename WT, bool LN, int ITERS, bool PARK = false, bool PIPE = false>
 __global__ __launch_bounds__(kWideThreads) void norm_bwd_wide_acc(
     const T* __restrict__ x, const WT* __restrict__ w, const float* __restrict__ mean,
     const float* __restrict__ rstd, const T* __restrict__ dy, const T* __restrict__ gxn,
@@ -742,7 +751,9 @@ __global__ __launch_bounds__(kWideThreads) void norm_bwd_wide_acc(
   constexpr int EPV = Elem<T>::kVec;
   constexpr int NB = LN ? ITERS : 1;
   __shared__ float smem[kWideThreads / 64];
+  extern __shared__ u32x4 parked[];   // PARK: [ITERS][threads], dy of the row (64 KB at four vectors)
   const int tid = threadIdx.x;
+  const int wave_first = __builtin_amdgcn_readfirstlane(tid & ~63);
   const int nvec = d / EPV;
   const float inv_d = 1.f / (float)d;
   float acc[ITERS][EPV], accb[NB][EPV];
@@ -758,28 +769,45 @@ __global__ __launch_bounds__(kWideThreads) void norm_bwd_wide_acc(
   }
   const int64_t r0 = (int64_t)blockIdx.x * rows_per_chunk;
   const int64_t r1 = (r0 + rows_per_chunk < n) ? r0 + rows_per_chunk : n;
+  // column of this thread in slot i, clamped into the row for the loads
+  int col[ITERS];
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int c = i * kWideThreads + tid;
+    col[i] = (c < nvec ? c : nvec - 1) * EPV;
+  }
+  u32x4 rx[ITERS], rg[PARK ? 1 : ITERS];
+  auto fetch = [&](int i, int64_t base) {
+    rx[i] = load16_stream(x + base + col[i]);
+    if constexpr (PARK) load16_stream_to_lds(dy + base + col[i], parked + i * kWideThreads + wave_first);
+    else rg[i] = load16_stream(dy + base + col[i]);
+  };
+  if (PIPE && r0 < r1) {
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) fetch(i, r0 * (int64_t)d);
+  }
   for (int64_t row = r0; row < r1; ++row) {
     const int64_t base = row * (int64_t)d;
+    if constexpr (!PIPE) {
+#pragma unroll
+      for (int i = 0; i < ITERS; ++i) fetch(i, base);
+    }
     const float r = rstd[row];
     float mu = 0.f;
     if constexpr (LN) mu = mean[row];
-    u32x4 rx[ITERS], rg[ITERS];
-#pragma unroll
-    for (int i = 0; i < ITERS; ++i) {
-      const int c = i * kWideThreads + tid;
-      if (c < nvec) {
-        rx[i] = load16_stream(x + base + (int64_t)c * EPV);
-        rg[i] = load16_stream(dy + base + (int64_t)c * EPV);
-      }
-    }
+    if constexpr (PARK) wait_vmem_all();   // the LDS slots were filled by loads that name no register
     float dot = 0.f, gsum = 0.f;
 #pragma unroll
     for (int i = 0; i < ITERS; ++i) {
       const int c = i * kWideThreads + tid;
+      touch(rx[i]);
+      u32x4 g;
+      if constexpr (PARK) g = parked[i * kWideThreads + tid];
+      else { touch(rg[i]); g = rg[i]; }
       if (c < nvec) {
         float xv[EPV], gv[EPV], wv[EPV];
         Elem<T>::unpack(rx[i], xv);
-        Elem<T>::unpack(rg[i], gv);
+        Elem<T>::unpack(g, gv);
         load_w<T, WT>(w, c * EPV, wv);
 #pragma unroll
         for (int e = 0; e < EPV; ++e) {
@@ -797,13 +825,25 @@ __global__ __launch_bounds__(kWideThreads) void norm_bwd_wide_acc(
     const float cmean = dot * inv_d;
     float gmean = 0.f;
     if constexpr (LN) gmean = row_reduce<kWideThreads, OpSum>(gsum, smem, 0, tid) * inv_d;
+    const bool more = row + 1 < r1;   // the same for the whole workgroup
 #pragma unroll
     for (int i = 0; i < ITERS; ++i) {
       const int c = i * kWideThreads + tid;
+      touch(rx[i]);
+      u32x4 g;
+      if constexpr (PARK) {
+        g = parked[i * kWideThreads + tid];
+        touch(g);   // in registers before the slot is given away
+      } else {
+        touch(rg[i]);
+        g = rg[i];
+      }
+      const u32x4 xr = rx[i];
+      if (PIPE && more) fetch(i, base + d);
       if (c < nvec) {
         float xv[EPV], gv[EPV], wv[EPV], o[EPV];
-        Elem<T>::unpack(rx[i], xv);
-        Elem<T>::unpack(rg[i], gv);
+        Elem<T>::unpack(xr, xv);
+        Elem<T>::unpack(g, gv);
         load_w<T, WT>(w, c * EPV, wv);
 #pragma unroll
         for (int e = 0; e < EPV; ++e) o[e] = ((gv[e] * wv[e] - gmean) - ((xv[e] - mu) * r) * cmean) * r;
@@ -1031,14 +1071,33 @@ int launch_bwd(const Plan& p, const void* x, const void* w, const float* mean, c
   if (p.bwd_wide && acc_fits) {
     // the column sums fit the registers: one persistent kernel, a chunk of rows per workgroup
     const dim3 grid((unsigned)p.bwd_blocks);
-#define GOA(IT_)                                                                                  \
-  FM_LAUNCH((norm_bwd_wide_acc<T, WT, LN, IT_>), grid, dim3(kWideThreads), 0, st, xp, wp, mean, rstd, dyp, \
-            gp, dxp, ddp, partial, n, (int)d, p.rows_per_chunk)
+    // dy in LDS (PARK) where it would otherwise push registers out to scratch, the next row loaded
+    // under the output sweep (PIPE) where that pays; measured per form (us, RMSNorm / LayerNorm,
+    // plain | PARK | PARK + PIPE): bf16 [7281,18432] 167 / 186 | 171 / 191 | 174 / 217;
+    // bf16 [4096,32768] 167 / 345 | 173 / 214 | 167 / 236; fp32 [3276,20480] 173 / 257 | 160 / 202 |
+    // 160 / 223; fp32 [2048,32768] 291 | 211 | 181.
     constexpr int kMaxIt = 32 / Elem<T>::kVec;
+#define GOA(IT_)                                                                                  \
+  do {                                                                                            \
+    constexpr bool park_ = LN ? (IT_ >= 4) : (sizeof(T) == 4);                                    \
+    constexpr bool pipe_ = sizeof(T) == 4 && IT_ == 8;                                            \
+    constexpr int lds_ = park_ ? IT_ * kWideThreads * 16 : 0;                                     \
+    if (lds_ == 0 || fm_host::grant_dynamic_lds<&norm_bwd_wide_acc<T, WT, LN, IT_, park_, pipe_>>(lds_)) \
+      FM_LAUNCH((norm_bwd_wide_acc<T, WT, LN, IT_, park_, pipe_>), grid, dim3(kWideThreads), (size_t)lds_, \
+                st, xp, wp, mean, rstd, dyp, gp, dxp, ddp, partial, n, (int)d, p.rows_per_chunk); \
+    else                                                                                          \
+      FM_LAUNCH((norm_bwd_wide_acc<T, WT, LN, IT_, false, false>), grid, dim3(kWideThreads), 0, st, xp, wp, \
+                mean, rstd, dyp, gp, dxp, ddp, partial, n, (int)d, p.rows_per_chunk);             \
+  } while (0)
     if (wide_iters <= 3 && kMaxIt >= 3) GOA(3);
     else if (wide_iters <= 4 || kMaxIt < 8) GOA(4);
-    else if (wide_iters <= 6) GOA((kMaxIt >= 6 ? 6 : 4));
-    else GOA((kMaxIt >= 8 ? 8 : 4));
+    else if (wide_iters <= 6) {
+      if constexpr (kMaxIt >= 6) GOA(6);
+      else GOA(4);
+    } else {
+      if constexpr (kMaxIt >= 8) GOA(8);
+      else GOA(4);
+    }
 #undef GOA
   } else if (p.bwd_wide) {
     FM_LAUNCH((norm_bwd_wide<T, WT, LN>), dim3((unsigned)n), dim3(kWideThreads), 0, st, xp, wp,
