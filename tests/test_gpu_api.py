@@ -596,6 +596,9 @@ def test_loss_selection_and_routing_launches_replay_in_a_graph():
     yn = torch.randint(0, 100, (700,), generator=g).to(DEV)
     s_, t_ = lg, (lg.float() + 0.5 * torch.randn(300, 4096, generator=g).to(DEV)).bfloat16()
     wide = (3 * torch.randn(8, 128256, generator=g)).bfloat16().to(DEV)
+    wide2 = (wide.float() + 0.5 * torch.randn(8, 128256, generator=g).to(DEV)).bfloat16()
+    mid = (3 * torch.randn(900, 20000, generator=g)).bfloat16().to(DEV)
+    mid2 = (mid.float() + 0.5 * torch.randn(900, 20000, generator=g).to(DEV)).bfloat16()
     short = torch.randn(500, 1000, generator=g).to(DEV)
     logits = torch.randn(2048, 64, generator=g).to(DEV)
     xs = torch.randn(2048, 512, generator=g).bfloat16().to(DEV)
@@ -634,6 +637,9 @@ def test_loss_selection_and_routing_launches_replay_in_a_graph():
         l3, d3, _, r3 = _hip.ce_loss_grad(aligned, ya, -100, "mean")
         k3, g3, rk3 = _hip.kl_loss_grad(aligned, aligned2, 1.0, "mean", torch.bfloat16)
         out += [l3, d3, r3, k3, g3, rk3]
+        # rows kept on the chip by workgroups that walk several rows (one and three per compute unit)
+        out += list(_hip.kl_loss_grad(wide, wide2, 0.5, "mean", torch.bfloat16))
+        out += list(_hip.kl_loss_grad(mid, mid2, 1.0, "sum", torch.bfloat16))
         out += [_hip.swiglu_split_fwd(xs), _hip.swiglu_split_bwd(xs, xs[:, :256].contiguous())]
         return out
 
