@@ -183,6 +183,11 @@ __device__ __forceinline__ void unpack_again(u32x4 raw, float (&f)[N]) {
 __device__ __forceinline__ void touch(u32x4& raw) {
   asm volatile("" : "+v"(raw.x), "+v"(raw.y), "+v"(raw.z), "+v"(raw.w));
 }
+// The same with the vector as ONE operand: its four registers stay a tuple. (With four operands
+// they become four values of their own, which the register allocator may keep apart; where it
+// does, the halves are copied out of the load's destination right behind the load, behind a wait
+// for it.) For kernels that keep many loaded vectors alive across several passes.
+__device__ __forceinline__ void touch_whole(u32x4& raw) { asm("" : "+v"(raw)); }
 
 // ---------------------------------------------------------------- wave reductions (DPP)
 __device__ __forceinline__ int lane_id() {
