@@ -384,51 +384,59 @@ __global__ __launch_bounds__(kHeldFwdThreads) void softmax_held_kernel(const T* 
   const RowSplit sp = split_row<EPV>(row, v, true);
   const int tid = threadIdx.x;
   const int ne = edge_count(sp, v);
-  u32x4 raw[RI];
-#pragma unroll
-  for (int i = 0; i < RI; ++i)
-    raw[i] = load16_stream(rp + sp.head + (int64_t)clamp_col(i * THREADS + tid, sp.nvec) * EPV);
-  {
-    u32x4 late[LI];
-#pragma unroll
-    for (int j = 0; j < LI; ++j)
-      late[j] = load16_stream(rp + sp.head + (int64_t)clamp_col((RI + j) * THREADS + tid, sp.nvec) * EPV);
-#pragma unroll
-    for (int j = 0; j < LI; ++j) parked[j * THREADS + tid] = late[j];
-  }
-  float edge = -INFINITY;   // the unaligned ends of the row (at most EPV - 1 elements each): thread e keeps edge e
+  // the unaligned ends of the row first (at most EPV - 1 elements each, thread e keeps edge e): a
+  // wait for them then waits for nothing that was issued behind them
+  float edge = -INFINITY;
   int edge_at = -1;
   if (tid < ne) {
     edge_at = edge_col(sp, tid);
     edge = Elem<T>::load1(rp + edge_at) * kLog2e;
   }
+  u32x4 raw[RI];
+#pragma unroll
+  for (int i = 0; i < RI; ++i)
+    raw[i] = load16_stream(rp + sp.head + (int64_t)clamp_col(i * THREADS + tid, sp.nvec) * EPV);
   auto vec = [&](int i) -> u32x4 {
     if (i < RI) { touch(raw[i < RI ? i : 0]); return raw[i < RI ? i : 0]; }
     return parked[(i - RI) * THREADS + tid];
   };
-  float mz = fmaxf(edge, kNegBig);
+  // Running (maximum, sum), one vector at a time in the order the loads were issued: the wait
+  // before vector i counts the loads issued after it, so the arithmetic on the first vectors runs
+  // while the later ones are still on their way. The LDS share is filled straight from memory, and
+  // requested only behind that (with a load into LDS outstanding the compiler waits for ALL
+  // vector-memory operations wherever it has to wait for one). A NaN anywhere must reach the whole
+  // row: fmaxf drops it, the sum carries it.
+  MaxSum st{fmaxf(edge, kNegBig), 0.f};
+  if (edge_at >= 0) st.s = fast_exp2(edge - st.m);
+  auto fold = [&](const u32x4& r) {
+    float z[EPV];
+    Elem<T>::unpack(r, z);
+    float cm = st.m;
 #pragma unroll
-  for (int i = 0; i < RI + LI; ++i) {
-    if (i * THREADS + tid < sp.nvec) {
-      float z[EPV];
-      Elem<T>::unpack(vec(i), z);
+    for (int e = 0; e < EPV; ++e) { z[e] *= kLog2e; cm = fmaxf(cm, z[e]); }
+    float acc = st.s * fast_exp2(st.m - cm);
 #pragma unroll
-      for (int e = 0; e < EPV; ++e) mz = fmaxf(mz, z[e] * kLog2e);
-    }
+    for (int e = 0; e < EPV; ++e) acc += fast_exp2(z[e] - cm);
+    st.m = cm;
+    st.s = acc;
+  };
+#pragma unroll
+  for (int i = 0; i < RI; ++i) {
+    if (i * THREADS + tid < sp.nvec) fold(raw[i]);
   }
-  // a NaN anywhere must reach the whole row: fmaxf drops it, so it is carried in the sum
-  float ssum = edge_at >= 0 ? fast_exp2(edge - mz) : 0.f;
+  {
+    const int wave_first = __builtin_amdgcn_readfirstlane(tid & ~63);
 #pragma unroll
-  for (int i = 0; i < RI + LI; ++i) {
-    if (i * THREADS + tid < sp.nvec) {
-      float z[EPV];
-      Elem<T>::unpack(vec(i), z);
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) ssum += fast_exp2(z[e] * kLog2e - mz);
-    }
+    for (int j = 0; j < LI; ++j)
+      load16_stream_to_lds(rp + sp.head + (int64_t)clamp_col((RI + j) * THREADS + tid, sp.nvec) * EPV,
+                           parked + j * THREADS + wave_first);
   }
-  // vectors past what the chip holds: streamed with a running (maximum, sum), read again below
-  MaxSum st{mz, ssum};
+  wait_vmem_all();   // those loads name no register the compiler could wait on
+#pragma unroll
+  for (int j = 0; j < LI; ++j) {
+    if ((RI + j) * THREADS + tid < sp.nvec) fold(parked[j * THREADS + tid]);
+  }
+  // vectors past what the chip holds: streamed into the same running pair, read again below
   for (int c0 = kHeldFwdMaxVec; c0 < sp.nvec; c0 += THREADS * 2) {
     u32x4 more[2];
 #pragma unroll
