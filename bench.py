@@ -17,7 +17,8 @@ descriptions, warm-cache, graph-replay, torch-eager and CPU columns to a file). 
   checked       one step's output compared with the CPU oracle on a bounded row sample before
                 anything is timed (per workload too);
   roofline      the dominant kernel of the headline workload against the 8 TB/s HBM peak, timed
-                with HIP events around that kernel's launches, on the bytes it has to move;
+                with HIP events around that kernel's launches (each behind the forward that precedes
+                it in every step, as in the timed region), on the bytes it has to move;
                 `traffic` = that kernel's HBM bytes from the committed profiler counter runs,
                 looked up by the name of the kernel that actually ran (null when unknown);
                 `configs` = one row per BASELINE configuration (cfg1 RMSNorm, cfg2 CE, cfg3 router,
@@ -54,49 +55,49 @@ METRIC = "HBM GB/s & % roofline: RMSNorm, CE/KL fwd+bwd; MoE top-k rows/s"
 # (profiles/all_workloads_hbm_traffic_pmc.txt). Each counter is scaled by what it reads for the
 # library's own 1 GiB copy (probe_copy_kernel, `bench.py --copy-probe 1024` under the same counters).
 # A kernel that is not in the table (a retune changed its template arguments) reports null.
-TRAFFIC_SCALE = (1048576.0 / 524299.6, 1048576.0 / 1049359.9)
+TRAFFIC_SCALE = (1048576.0 / 524299.6, 1048576.0 / 1049327.4)
 TRAFFIC_KIB = {
-    "ce_bwd_kernel<bf16_t, 1024, 4>": (244221.8, 512230.4),
-    "ce_fwd_kernel<bf16_t, 512, 4, false>": (125275.8, 250.2),
-    "ce_fwd_kernel<bf16_t, 512, 4, true>": (131370.4, 266.4),
-    "ce_loss_grad_held_kernel<bf16_t>": (487093.6, 1028556.2),
-    "ce_loss_grad_kernel<bf16_t, 512, 8>": (243962.6, 512522.0),
+    "ce_bwd_kernel<bf16_t, 1024, 4>": (244222.2, 512255.2),
+    "ce_fwd_kernel<bf16_t, 512, 4, false>": (125276.7, 250.2),
+    "ce_fwd_kernel<bf16_t, 512, 4, true>": (131370.3, 266.6),
+    "ce_loss_grad_held_kernel<bf16_t>": (487096.0, 1028488.8),
+    "ce_loss_grad_kernel<bf16_t, 512, 8>": (243962.6, 512532.8),
     "colsum16_kernel<bf16_t>": (4111.0, 8.0),
     "colsum16_kernel<float>": (1039.0, 4.0),
     "colsum_kernel<float>": (8208.0, 64.0),
     "combine_kernel<bf16_t, true>": (133143.1, 131072.0),
-    "kl_bwd_kernel<bf16_t, bf16_t, 1024, 8>": (1026898.1, 1026057.7),
-    "kl_fwd_kernel<bf16_t, 512, 4>": (1026888.6, 385.0),
-    "kl_fwd_topk_kernel<bf16_t, 512, 2, false>": (1054176.8, 2433.5),
-    "kl_fwd_topk_kernel<bf16_t, 512, 2, true>": (2057669.9, 1028505.8),
-    "kl_loss_grad_held_kernel<bf16_t, bf16_t, 512, 22, 9>": (1026391.4, 1026433.2),
-    "norm_bwd_kernel<bf16_t, bf16_t, 256, 2, false>": (65813.1, 69632.8),
-    "norm_bwd_kernel<bf16_t, float, 512, 2, false>": (393631.7, 270336.0),
-    "norm_bwd_kernel<bf16_t, float, 512, 2, true>": (393893.3, 278528.0),
+    "kl_bwd_kernel<bf16_t, bf16_t, 1024, 8>": (1026899.3, 1026058.2),
+    "kl_fwd_kernel<bf16_t, 512, 4>": (1026878.1, 384.9),
+    "kl_fwd_topk_kernel<bf16_t, 512, 2, false>": (1054172.7, 2433.4),
+    "kl_fwd_topk_kernel<bf16_t, 512, 2, true>": (2057462.7, 1028505.3),
+    "kl_loss_grad_held_kernel<bf16_t, bf16_t, 512, 22, 9>": (1026392.2, 1026433.1),
+    "norm_bwd_kernel<bf16_t, bf16_t, 256, 2, false>": (65814.0, 69632.9),
+    "norm_bwd_kernel<bf16_t, float, 512, 2, false>": (393631.7, 270336.1),
+    "norm_bwd_kernel<bf16_t, float, 512, 2, true>": (393893.2, 278528.0),
     "norm_bwd_kernel<bf16_t, float, 64, 2, false>": (16461.6, 17408.0),
-    "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, false, false>": (32820.5, 65845.8),
-    "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, true, false>": (65585.1, 131373.1),
-    "norm_fwd_kernel<bf16_t, float, 512, 2, true, false>": (262295.8, 524843.9),
-    "norm_fwd_kernel<bf16_t, float, 512, 2, true, true>": (262429.4, 525343.3),
-    "norm_fwd_kernel<bf16_t, float, 64, 2, false, false>": (8227.6, 16448.4),
-    "permute_kernel": (1584.9, 10728.8),
+    "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, false, false>": (32820.5, 65844.4),
+    "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, true, false>": (65585.1, 131370.3),
+    "norm_fwd_kernel<bf16_t, float, 512, 2, true, false>": (262295.8, 524843.4),
+    "norm_fwd_kernel<bf16_t, float, 512, 2, true, true>": (262429.3, 525339.7),
+    "norm_fwd_kernel<bf16_t, float, 64, 2, false, false>": (8227.6, 16448.1),
+    "permute_kernel": (1584.9, 10760.3),
     "probe_read_kernel": (524298.8, 0.0),
-    "rope_vec_kernel<bf16_t, float, 8, false, 2>": (105921.1, 213464.6),
-    "rope_vec_kernel<bf16_t, float, 8, true, 2>": (216510.7, 214215.3),
+    "rope_vec_kernel<bf16_t, float, 8, false, 2>": (105921.1, 213464.5),
+    "rope_vec_kernel<bf16_t, float, 8, true, 2>": (216510.7, 214215.7),
     "route_bwd_kernel<float, 8, true>": (2273.0, 4096.0),
-    "route_group_kernel<float, 32, true, 2>": (32845.1, 6179.5),
-    "route_group_kernel<float, 8, true, 0>": (2109.0, 328.5),
+    "route_group_kernel<float, 32, true, 2>": (32845.1, 6179.8),
+    "route_group_kernel<float, 8, true, 0>": (2109.0, 328.4),
     "route_scan_stats_kernel": (1893.5, 1026.0),
-    "scatter_kernel<bf16_t, true>": (66086.3, 262274.6),
+    "scatter_kernel<bf16_t, true>": (66086.2, 262267.7),
     "softmax_bwd_rows_kernel<bf16_t, 16, 1>": (2061.5, 2048.0),
-    "softmax_bwd_rows_kernel<bf16_t, 256, 2>": (65553.0, 65577.3),
-    "softmax_rows_kernel<bf16_t, 16, 1>": (1039.6, 2048.0),
-    "softmax_rows_kernel<bf16_t, 256, 2>": (32788.6, 65597.9),
-    "swiglu_bwd_kernel<bf16_t, true>": (264214.2, 352258.2),
+    "softmax_bwd_rows_kernel<bf16_t, 256, 2>": (65553.0, 65558.6),
+    "softmax_rows_kernel<bf16_t, 16, 1>": (1039.7, 2048.0),
+    "softmax_rows_kernel<bf16_t, 256, 2>": (32788.6, 65594.8),
+    "swiglu_bwd_kernel<bf16_t, true>": (264214.2, 352258.4),
     "swiglu_fwd_kernel<bf16_t, true>": (176147.3, 176128.0),
-    "swiglu_split_kernel<bf16_t, true, false>": (458770.1, 458752.0),
-    "swiglu_split_kernel<bf16_t, true, true>": (688148.4, 917504.8),
-    "topk_lds_kernel<bf16_t, 512, 4, 0>": (539853.1, 1024.0),
+    "swiglu_split_kernel<bf16_t, true, false>": (458770.2, 458752.1),
+    "swiglu_split_kernel<bf16_t, true, true>": (688148.4, 917505.6),
+    "topk_lds_kernel<bf16_t, 512, 4, 0>": (539853.6, 1024.0),
 }
 TRAFFIC_SOURCE = "profiles/all_workloads_hbm_traffic_pmc.txt"
 
@@ -238,7 +239,11 @@ def make_workload(name, torch, L, dev):
         w.check, w.cpu, w.eager = check, cpu, eager
         w.graph_steps = [(lambda i=i: (fwd(i), bwd(i))) for i in range(sets)]
         w.step, w.warm_step = step, warm_step
-        w.dominant_launch = lambda: bwd(state["i"])
+        def next_forward():       # the step's own order: the next buffer set, forward, then the backward timed
+            state["i"] = (state["i"] + 1) % sets
+            fwd(state["i"])
+
+        w.dominant_launch, w.dominant_before = (lambda: bwd(state["i"])), next_forward
         w.dominant = "norm_bwd_kernel<bf16,f32,64,2> + colsum_kernel"
         w.dominant_bytes = n * d * 6
         w.bytes = n * d * 10
@@ -299,7 +304,7 @@ def make_workload(name, torch, L, dev):
 
         w.check, w.cpu, w.eager = check, cpu, eager
         w.step = step
-        w.dominant_launch = bwd
+        w.dominant_launch, w.dominant_before = bwd, fwd
         w.dominant = "norm_bwd_kernel<bf16,f32,512,2> + colsum_kernel"
         w.dominant_bytes = n * d * 8
         w.bytes = n * d * 16
@@ -345,7 +350,7 @@ def make_workload(name, torch, L, dev):
 
         w.check = check
         w.step = step
-        w.dominant_launch = bwd
+        w.dominant_launch, w.dominant_before = bwd, fwd
         w.floor = [lambda i: ((x, dl), (xn, y)), lambda i: ((xn, gy, gxn), (dx,))]
         w.dominant = "norm_bwd_kernel<bf16,f32,512,2,LN> + colsum_kernel"
         w.dominant_bytes = n * d * 8
@@ -441,7 +446,7 @@ def make_workload(name, torch, L, dev):
             bwd()
 
         w.step = step
-        w.dominant_launch = bwd
+        w.dominant_launch, w.dominant_before = bwd, fwd
         w.dominant = "ce_bwd_kernel<bf16,1024,4>"
         w.dominant_bytes = n * v * 4
         w.bytes = n * v * 6
@@ -589,7 +594,7 @@ def make_workload(name, torch, L, dev):
             bwd()
 
         w.step = step
-        w.dominant_launch = bwd
+        w.dominant_launch, w.dominant_before = bwd, fwd
         w.dominant = "kl_bwd_kernel<bf16,bf16,1024,8>"
         w.dominant_bytes = n * v * 6
         w.bytes = n * v * 10
@@ -880,11 +885,15 @@ def time_steps(torch, fn, steps, warmup):
     return (time.perf_counter() - t0) * 1e3 / steps     # ms per step
 
 
-def time_kernel_events(torch, fn, steps):
+def time_kernel_events(torch, fn, steps, before=None):
     """Average duration of the launches `fn` enqueues, HIP events on the launch stream (the
-    benchmark's own stream is torch's current stream, so these events are recorded on it)."""
+    benchmark's own stream is torch's current stream, so these events are recorded on it).
+    `before` (untimed) is what precedes those launches in every step of the workload: a backward
+    is timed behind its forward, as it runs in the timed region and in a profile of this run."""
     pairs = []
     for _ in range(steps):
+        if before is not None:
+            before()
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record()
         fn()
@@ -966,7 +975,7 @@ def measure(torch, w, steps, warmup, L, cpu=True):
     # reference's kbench gate, forgemind/cli/kbench.py:197-213, 264-278); outside every timed region
     checked = bool(w.check()) if hasattr(w, "check") else None
     ms = time_steps(torch, w.step, steps, warmup)
-    avg, best, med = time_kernel_events(torch, w.dominant_launch, steps)
+    avg, best, med = time_kernel_events(torch, w.dominant_launch, steps, getattr(w, "dominant_before", None))
     kernel = L.fm_last_kernel().decode()
     out = {
         "desc": w.desc,
