@@ -257,6 +257,40 @@ def test_last_kernel_names_what_ran():
     assert _hip.last_kernel().startswith("topk_lds_kernel<bf16_t, ")
 
 
+def test_row_width_picks_the_form_that_was_measured_faster():
+    """The one-launch KL and the norm backward choose a kernel form by row width and dtype; the
+    names say which ran (what each choice rests on is written next to the dispatch in the source)."""
+    def kl_kernel(v, dt):
+        s = torch.randn(4, v, device=DEV).to(dt)
+        _hip.kl_loss_grad(s, s.flip(0).contiguous(), 1.0, "mean", dt)
+        return _hip.last_kernel()
+
+    bf, f32 = torch.bfloat16, torch.float32
+    assert kl_kernel(16384, bf).startswith("kl_loss_grad_kernel<bf16_t, bf16_t")          # registers
+    assert kl_kernel(20000, bf) == "kl_loss_grad_held_kernel<bf16_t, bf16_t, 256, 13, 3>"  # 3 workgroups a unit
+    assert kl_kernel(50304, bf) == "kl_loss_grad_held_kernel<bf16_t, bf16_t, 256, 22, 9>"  # 2
+    assert kl_kernel(128256, bf) == "kl_loss_grad_held_kernel<bf16_t, bf16_t, 512, 22, 9>"  # 1
+    assert kl_kernel(32000, f32) == "kl_loss_grad_held_kernel<float, float, 512, 22, 9>"
+    assert kl_kernel(300000, bf).startswith("kl_loss_grad_wide_kernel<bf16_t, bf16_t")    # two sweeps
+
+    def norm_kernel(d, dt, ln):
+        x = torch.randn(3, d, device=DEV).to(dt)
+        w = torch.ones(d, device=DEV, dtype=dt)
+        if ln:
+            _, _, mean, rstd = _hip.layernorm_fwd(x, w, w, 1e-5)
+            _hip.layernorm_bwd(x, w, mean, rstd, x)
+        else:
+            _, rstd = _hip.rmsnorm_fwd(x, w, 1e-6)
+            _hip.rmsnorm_bwd(x, w, rstd, x)
+        return _hip.last_kernel()
+
+    # <T, WT, LayerNorm, vectors a thread, dy in LDS, next row under the output sweep>
+    assert norm_kernel(32768, bf, False) == "norm_bwd_wide_acc<bf16_t, bf16_t, false, 4, false, false>"
+    assert norm_kernel(32768, bf, True) == "norm_bwd_wide_acc<bf16_t, bf16_t, true, 4, true, false>"
+    assert norm_kernel(20480, f32, False) == "norm_bwd_wide_acc<float, float, false, 6, true, false>"
+    assert norm_kernel(32768, f32, False) == "norm_bwd_wide_acc<float, float, false, 8, true, true>"
+
+
 def test_fp16_losses_apply_the_upstream_gradient_before_rounding():
     # a loss scaler multiplies the loss by 65536; (softmax - onehot) / 8192 rounded to fp16 FIRST
     # would lose most entries (p / 8192 < 6e-5 is subnormal or zero in fp16)
