@@ -15,7 +15,7 @@ using namespace fm;
 
 namespace {
 
-constexpr int kMaxK = 8;
+constexpr int kMaxK = 16;   // the kernels keep a token's slots in registers: built for 8 and for 16
 
 // dst[s, :] = scale * src[order[s] / k, :],  scale = w[order[s]] if w else 1
 // A destination row is owned by `g` threads (a power of two up to 256: as many as the row has
@@ -71,7 +71,7 @@ __global__ __launch_bounds__(256) void gather_kernel(const T* __restrict__ src,
 // above reads it k times). The copies alternate between plain and non-temporal stores: two
 // write streams of one kind share one path through the memory system and reach 5.5 TB/s in a
 // bare 1-read-2-writes sweep, one of each kind reaches 6.9 TB/s.
-template <typename T, bool VEC>
+template <typename T, bool VEC, int KMAX = 8>
 __global__ __launch_bounds__(256) void scatter_kernel(const T* __restrict__ src,
                                                        const int32_t* __restrict__ slot,
                                                        const float* __restrict__ w,
@@ -80,10 +80,10 @@ __global__ __launch_bounds__(256) void scatter_kernel(const T* __restrict__ src,
   const int rib = threadIdx.x / g, l = threadIdx.x % g;
   const int64_t t = (int64_t)blockIdx.x * (256 / g) + rib;
   if (t >= n) return;
-  int64_t to[kMaxK];
-  float sc[kMaxK];
+  int64_t to[KMAX];
+  float sc[KMAX];
 #pragma unroll
-  for (int j = 0; j < kMaxK; ++j) {
+  for (int j = 0; j < KMAX; ++j) {
     to[j] = j < k ? (int64_t)slot[t * k + j] * d : 0;
     sc[j] = j < k && w != nullptr ? w[t * k + j] : 1.f;
   }
@@ -98,7 +98,7 @@ __global__ __launch_bounds__(256) void scatter_kernel(const T* __restrict__ src,
         if (c < nvec) raw[u] = load16_stream(sp + c * EPV);
       }
 #pragma unroll
-      for (int j = 0; j < kMaxK; ++j) {
+      for (int j = 0; j < KMAX; ++j) {
         if (j < k) {
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
@@ -128,17 +128,17 @@ __global__ __launch_bounds__(256) void scatter_kernel(const T* __restrict__ src,
 }
 
 // out[t, :] = sum_j w[t*k+j] * ys[slot[t*k+j], :]   (w == NULL: unit weights)
-template <typename T, bool VEC>
+template <typename T, bool VEC, int KMAX = 8>
 __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ ys,
                                                        const float* __restrict__ w,
                                                        const int32_t* __restrict__ slot,
                                                        T* __restrict__ out, int d, int k) {
   constexpr int EPV = Elem<T>::kVec;
   const int64_t t = blockIdx.x;
-  int sl[kMaxK];
-  float wt[kMaxK];
+  int sl[KMAX];
+  float wt[KMAX];
 #pragma unroll
-  for (int j = 0; j < kMaxK; ++j) {
+  for (int j = 0; j < KMAX; ++j) {
     sl[j] = j < k ? slot[t * k + j] : 0;
     wt[j] = j < k ? (w != nullptr ? w[t * k + j] : 1.f) : 0.f;
   }
@@ -150,7 +150,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ ys,
 #pragma unroll
       for (int e = 0; e < EPV; ++e) acc[e] = 0.f;
 #pragma unroll
-      for (int j = 0; j < kMaxK; ++j) {
+      for (int j = 0; j < KMAX; ++j) {
         if (j < k) {
           float f[EPV];
           Elem<T>::unpack(load16_stream(ys + sl[j] * (int64_t)d + c * EPV), f);
@@ -170,7 +170,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const T* __restrict__ ys,
 }
 
 // Backward of the combine wrt the weights: dw[t*k+j] = <ys[slot[t*k+j], :], dout[t, :]>
-template <typename T, bool VEC>
+template <typename T, bool VEC, int KMAX = 8>
 __global__ __launch_bounds__(256) void combine_dw_kernel(const T* __restrict__ ys,
                                                           const T* __restrict__ dout,
                                                           const int32_t* __restrict__ slot,
@@ -178,10 +178,10 @@ __global__ __launch_bounds__(256) void combine_dw_kernel(const T* __restrict__ y
   constexpr int EPV = Elem<T>::kVec;
   __shared__ float smem[4];
   const int64_t t = blockIdx.x;
-  float dot[kMaxK];
-  int sl[kMaxK];
+  float dot[KMAX];
+  int sl[KMAX];
 #pragma unroll
-  for (int j = 0; j < kMaxK; ++j) { dot[j] = 0.f; sl[j] = j < k ? slot[t * k + j] : 0; }
+  for (int j = 0; j < KMAX; ++j) { dot[j] = 0.f; sl[j] = j < k ? slot[t * k + j] : 0; }
   const T* gp = dout + t * (int64_t)d;
   if constexpr (VEC) {
     const int nvec = d / EPV;
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(256) void combine_dw_kernel(const T* __restrict__ y
       float g[EPV];
       Elem<T>::unpack(load16(gp + c * EPV), g);
 #pragma unroll
-      for (int j = 0; j < kMaxK; ++j) {
+      for (int j = 0; j < KMAX; ++j) {
         if (j < k) {
           float f[EPV];
           Elem<T>::unpack(load16_stream(ys + sl[j] * (int64_t)d + c * EPV), f);
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(256) void combine_dw_kernel(const T* __restrict__ y
     }
   }
 #pragma unroll
-  for (int j = 0; j < kMaxK; ++j) {
+  for (int j = 0; j < KMAX; ++j) {
     if (j < k) {   // k is uniform, so every thread reaches the barriers inside row_reduce
       const float tot = row_reduce<256, OpSum>(dot[j], smem, 0, threadIdx.x);
       if (threadIdx.x == 0) dw[t * k + j] = tot;
@@ -282,11 +282,17 @@ int fm_moe_scatter(const void* x, const int32_t* slot, const float* scale, void*
     int g = 8;                                                                                   \
     while (g < 256 && g < units) g *= 2;                                                         \
     const dim3 grid((unsigned)((n + 256 / g - 1) / (256 / g)));                                  \
-    if (vec)                                                                                     \
+    if (vec && k <= 8)                                                                           \
       FM_LAUNCH((scatter_kernel<T, true>), grid, dim3(256), 0, st, static_cast<const T*>(x),     \
                 slot, scale, static_cast<T*>(xs), n, (int)d, k, g);                              \
-    else                                                                                         \
+    else if (vec)                                                                                \
+      FM_LAUNCH((scatter_kernel<T, true, 16>), grid, dim3(256), 0, st, static_cast<const T*>(x), \
+                slot, scale, static_cast<T*>(xs), n, (int)d, k, g);                              \
+    else if (k <= 8)                                                                             \
       FM_LAUNCH((scatter_kernel<T, false>), grid, dim3(256), 0, st, static_cast<const T*>(x),    \
+                slot, scale, static_cast<T*>(xs), n, (int)d, k, g);                              \
+    else                                                                                         \
+      FM_LAUNCH((scatter_kernel<T, false, 16>), grid, dim3(256), 0, st, static_cast<const T*>(x), \
                 slot, scale, static_cast<T*>(xs), n, (int)d, k, g);                              \
   }
   FM_BY_DTYPE(dtype, CALL);
@@ -303,15 +309,20 @@ int fm_moe_combine(const void* ys, const float* weights, const int32_t* slot, vo
   FM_CHECK_ARG(ys && slot && out, "fm_moe_combine: NULL pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)n);
+#define GO(T, VEC_, KMAX_)                                                                         \
+  FM_LAUNCH((combine_kernel<T, VEC_, KMAX_>), grid, dim3(256), 0, st, static_cast<const T*>(ys),   \
+            weights, slot, static_cast<T*>(out), (int)d, k)
 #define CALL(T)                                                                                    \
-  if (vec_ok<T>(d, ys, out))                                                                       \
-    FM_LAUNCH((combine_kernel<T, true>), grid, dim3(256), 0, st, static_cast<const T*>(ys), \
-                       weights, slot, static_cast<T*>(out), (int)d, k);                            \
-  else                                                                                             \
-    FM_LAUNCH((combine_kernel<T, false>), grid, dim3(256), 0, st, static_cast<const T*>(ys), \
-                       weights, slot, static_cast<T*>(out), (int)d, k)
+  if (vec_ok<T>(d, ys, out)) {                                                                     \
+    if (k <= 8) GO(T, true, 8);                                                                       \
+    else GO(T, true, 16);                                                                             \
+  } else {                                                                                         \
+    if (k <= 8) GO(T, false, 8);                                                                      \
+    else GO(T, false, 16);                                                                            \
+  }
   FM_BY_DTYPE(dtype, CALL);
 #undef CALL
+#undef GO
   FM_CHECK_LAUNCH("fm_moe_combine");
   return FM_OK;
 }
@@ -324,15 +335,20 @@ int fm_moe_combine_dw(const void* ys, const void* dout, const int32_t* slot, flo
   FM_CHECK_ARG(ys && dout && slot && dweights, "fm_moe_combine_dw: NULL pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)n);
+#define GO(T, VEC_, KMAX_)                                                                       \
+  FM_LAUNCH((combine_dw_kernel<T, VEC_, KMAX_>), grid, dim3(256), 0, st, static_cast<const T*>(ys), \
+            static_cast<const T*>(dout), slot, dweights, (int)d, k)
 #define CALL(T)                                                                                  \
-  if (vec_ok<T>(d, ys, dout))                                                                    \
-    FM_LAUNCH((combine_dw_kernel<T, true>), grid, dim3(256), 0, st,                     \
-                       static_cast<const T*>(ys), static_cast<const T*>(dout), slot, dweights, (int)d, k); \
-  else                                                                                           \
-    FM_LAUNCH((combine_dw_kernel<T, false>), grid, dim3(256), 0, st,                    \
-                       static_cast<const T*>(ys), static_cast<const T*>(dout), slot, dweights, (int)d, k)
+  if (vec_ok<T>(d, ys, dout)) {                                                                  \
+    if (k <= 8) GO(T, true, 8);                                                                     \
+    else GO(T, true, 16);                                                                           \
+  } else {                                                                                       \
+    if (k <= 8) GO(T, false, 8);                                                                    \
+    else GO(T, false, 16);                                                                          \
+  }
   FM_BY_DTYPE(dtype, CALL);
 #undef CALL
+#undef GO
   FM_CHECK_LAUNCH("fm_moe_combine_dw");
   return FM_OK;
 }

@@ -31,7 +31,7 @@ using namespace fm;
 namespace {
 
 constexpr int kMaxE = 512;
-constexpr int kMaxK = 8;
+constexpr int kMaxK = 16;             // picks a row; the forms tuned for few picks are built for 8
 constexpr int kMaxTiles = 1024;
 
 constexpr int kGroupThreads = 256;    // 4 waves per tile
@@ -140,13 +140,14 @@ __device__ __forceinline__ float group_max_f(float v) {
 // across the lanes in place of k rounds. The probability of a pick is read back from its key
 // (they are the same bits above the sign), so all forms give identical results (a NaN row's
 // weights are NaN either way, with whatever payload).
-template <typename T, int L, bool VEC, int SEL>
+template <typename T, int L, bool VEC, int SEL, int KMAX = 8>
 __global__ __launch_bounds__(kGroupThreads) void route_group_kernel(const T* __restrict__ logits,
                                                                      int32_t* __restrict__ idx,
                                                                      float* __restrict__ weights,
                                                                      int32_t* __restrict__ hist,
                                                                      float* __restrict__ fstat, int64_t n,
                                                                      int e, int k, int tile_rows) {
+  static_assert(KMAX <= L && (KMAX == 8 || SEL == kSelSorted), "pick j is kept by lane j of the group; more than 8 picks come from the sorted heads");
   constexpr int NW = kGroupThreads / 64;
   constexpr int GPW = 64 / L;           // rows per wave and pass
   __shared__ int lh[L * kGE];
@@ -316,7 +317,7 @@ __global__ __launch_bounds__(kGroupThreads) void route_group_kernel(const T* __r
         my_p[r] = pv;
         my_i[r] = 0xFFFF - (int)((uint32_t)c[r] & 0xFFFFu);
 #pragma unroll
-        for (int j = 0; j < kMaxK; ++j) {
+        for (int j = 0; j < KMAX; ++j) {
           if (j < k) wsum[r] += __shfl(pv, gbase + j, 64);   // in pick order, as the other forms add them
         }
       }
@@ -356,7 +357,7 @@ __global__ __launch_bounds__(kGroupThreads) void route_group_kernel(const T* __r
       }
       const int gbase = lane & ~(L - 1);
 #pragma unroll
-      for (int j = 0; j < kMaxK; ++j) {
+      for (int j = 0; j < KMAX; ++j) {
         if (j < k) {
           uint32_t gk[R];
 #pragma unroll
@@ -400,7 +401,7 @@ __global__ __launch_bounds__(kGroupThreads) void route_group_kernel(const T* __r
       }
     } else {
 #pragma unroll
-    for (int j = 0; j < kMaxK; ++j) {
+    for (int j = 0; j < KMAX; ++j) {
       if (j < k) {
         uint32_t bk[R], gk[R];
         int bq[R], gi[R];
@@ -552,7 +553,8 @@ __global__ __launch_bounds__(kGroupThreads) void route_bwd_kernel(const T* __res
   float s_loc = 0.f, d_loc = 0.f;
 #pragma unroll
   for (int j = 0; j < kMaxK; ++j) {
-    if (j < k && live) {
+    if (j >= k) break;
+    if (live) {
       const int ij = idx[row * (int64_t)k + j];
       const float gj = gw != nullptr ? gw[row * (int64_t)k + j] : 0.f;
 #pragma unroll
@@ -986,7 +988,23 @@ int launch_route(const void* logits, int32_t* idx, float* weights, int32_t* hist
   //   512 experts (32768 rows): scan 25 / 29 / 38 / 56, sorted heads 30 / 32 / 35 / 43, candidates 42-44
   // Up to 64 experts the scan and the sorted heads tie at four picks.
   const int sel = k >= (e > 64 ? 4 : 5) ? kSelSorted : kSelScan;
-  if (e <= 64) GOG(8);
+  if (k > 8) {
+    // more picks than the forms above are built for: sorted heads, 16 lanes a row at the least
+    // (lane j of a group keeps pick j)
+#define GOK(L_)                                                                                       \
+  do {                                                                                                \
+    if (vec)                                                                                          \
+      FM_LAUNCH((route_group_kernel<T, L_, true, kSelSorted, 16>), grid, dim3(kGroupThreads), 0, st, lp, idx, \
+                weights, hist, fstat, n, e, k, tl.tile_rows);                                         \
+    else                                                                                              \
+      FM_LAUNCH((route_group_kernel<T, L_, false, kSelSorted, 16>), grid, dim3(kGroupThreads), 0, st, lp, idx, \
+                weights, hist, fstat, n, e, k, tl.tile_rows);                                         \
+  } while (0)
+    if (e <= 128) GOK(16);
+    else if (e <= 256) GOK(32);
+    else GOK(64);
+#undef GOK
+  } else if (e <= 64) GOG(8);
   else if (e <= 128) GOG(16);
   else if (e <= 256) {
     if (k >= 5 && vec) GOS(32, true, kSelCands);

@@ -71,7 +71,7 @@ def moe_gather(x: torch.Tensor, order: torch.Tensor, k: int,
     """
     if x.dim() != 2 or order.dim() != 1 or order.numel() != x.shape[0] * k:
         raise ValueError(f"moe_gather: x {tuple(x.shape)}, order {tuple(order.shape)}, k={k} disagree")
-    if k > 8 or x.numel() == 0 or order.device != x.device:
+    if k > 16 or x.numel() == 0 or order.device != x.device:
         _note("moe_gather shape")
         return x[(order // k).long()]
     if tracing() or not fast_ok(x):      # a traced graph gets the tensor expression
@@ -96,7 +96,7 @@ def moe_combine(ys: torch.Tensor, weights: torch.Tensor, slot: torch.Tensor,
         picked = ys[slot.long()].view(n, k, ys.shape[1]).float()
         return (picked * weights.float().unsqueeze(-1)).sum(dim=1).to(ys.dtype)
 
-    if k > 8 or ys.numel() == 0 or slot.device != ys.device or weights.device != ys.device:
+    if k > 16 or ys.numel() == 0 or slot.device != ys.device or weights.device != ys.device:
         _note("moe_combine shape")
         return torch_path()
     if tracing() or not fast_ok(ys, weights):

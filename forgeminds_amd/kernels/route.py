@@ -19,7 +19,7 @@ from . import _hip
 from ._common import _note, fast_ok, tracing
 
 MAX_EXPERTS = 512
-MAX_TOP_K = 8
+MAX_TOP_K = 16
 
 
 class Routing(NamedTuple):

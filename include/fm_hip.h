@@ -309,7 +309,7 @@ int fm_softmax_bwd(const void* y, const void* dy, void* dx, int64_t n, int64_t v
  * losses of moe.py:92-95 and the sums behind them, without another pass over the logits:
  *   stats[j] = sum_rows probs[:, j] (j < e),  stats[e] = sum_rows logsumexp(logits)^2,
  *   stats[e+1] = aux = E * sum_j counts[j] / (n k) * stats[j] / n,  stats[e+2] = z = stats[e] / n,
- * summed in a fixed order. 1 <= k <= 8, k <= e <= 512, n*k < 2^31.
+ * summed in a fixed order. 1 <= k <= 16, k <= e <= 512, n*k < 2^31.
  * Probabilities below the smallest normal fp32 (a logit more than 87 below the row maximum) come
  * out as zero and tie by expert index; a row holding a NaN or +inf, or only -inf, has NaN
  * probabilities throughout, selects experts 0..k-1 and gets NaN weights. */
@@ -333,7 +333,8 @@ int fm_route_bwd(const void* logits, const int32_t* idx, const float* gweights, 
  * Replaces `xs = x[order // k]` (forgemind/moe.py:234-235): xs[s, :] = scale * x[order[s] / k, :]
  * with scale = scale_flat[order[s]] when scale_flat (fp32 [n*k], indexed by flat assignment)
  * is given, 1 otherwise. x: [n, d]; xs: [n*k, d]; order: [n*k] int32 from fm_route.
- * With a scale it is also the backward of fm_moe_combine wrt ys (x = dout, scale = weights). */
+ * With a scale it is also the backward of fm_moe_combine wrt ys (x = dout, scale = weights).
+ * 1 <= k <= 16 for all four token moves (fm_route's range). */
 int fm_moe_gather(const void* x, const int32_t* order, const float* scale_flat, void* xs, int64_t n,
                   int64_t d, int k, int dtype, fm_stream_t stream);
 

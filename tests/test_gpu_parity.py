@@ -987,7 +987,10 @@ ROUTE_CASES = [(16384, 64, 2), (1000, 8, 2), (513, 128, 4), (100, 300, 8), (1, 6
                # many tiles x many experts: the histograms are scanned by a kernel of their own
                (40000, 64, 2), (9000, 256, 8), (5000, 500, 3), (300000, 8, 1),
                # expert counts around the lane-group sizes, not multiples of eight
-               (700, 65, 2), (700, 129, 3), (700, 257, 8), (900, 60, 4), (64, 7, 7)]
+               (700, 65, 2), (700, 129, 3), (700, 257, 8), (900, 60, 4), (64, 7, 7),
+               # nine to sixteen picks (sorted heads, at least sixteen lanes a row)
+               (4000, 512, 10), (700, 128, 16), (300, 16, 16), (900, 24, 12), (2000, 384, 12),
+               (513, 200, 9), (70000, 64, 10)]
 
 
 @pytest.mark.parametrize("n,e,k", ROUTE_CASES)
@@ -1018,7 +1021,8 @@ def test_route_is_bit_exact(n, e, k):
 
 
 ROUTE_BWD_CASES = [(16384, 64, 2, F32), (1000, 8, 2, F32), (513, 128, 4, BF16), (100, 300, 8, F32), (1, 64, 2, F32),
-                   (257, 512, 8, F16), (4099, 60, 6, F32), (3, 2, 2, F32), (700, 65, 2, BF16), (900, 256, 8, F32)]
+                   (257, 512, 8, F16), (4099, 60, 6, F32), (3, 2, 2, F32), (700, 65, 2, BF16), (900, 256, 8, F32),
+                   (600, 512, 10, F32), (300, 40, 16, BF16), (900, 160, 12, F32)]
 
 
 @pytest.mark.parametrize("n,e,k,dt", ROUTE_BWD_CASES)
@@ -1128,7 +1132,8 @@ def test_route_statistics_from_one_or_two_kernels():
 
 # ------------------------------------------------------------------ gather / combine around the permutation
 @pytest.mark.parametrize("n,e,k,d,dt", [(1000, 8, 2, 1024, BF16), (257, 16, 4, 100, F32), (64, 4, 1, 7, F16),
-                                         (2048, 64, 2, 4096, BF16), (33, 8, 8, 256, F32)])
+                                         (2048, 64, 2, 4096, BF16), (33, 8, 8, 256, F32),
+                                         (500, 64, 10, 1024, BF16), (129, 16, 16, 100, F32), (77, 32, 12, 7, F16)])
 def test_moe_gather_and_combine(n, e, k, d, dt):
     g = gen(1007)
     lg = router_inputs(n, e, 77)
