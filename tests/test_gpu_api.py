@@ -698,10 +698,12 @@ def test_loss_selection_and_routing_launches_replay_in_a_graph():
             assert torch.equal(a, b)
 
 
-def test_moe_layer_matches_the_reference_expression():
-    """MoE.forward of forgemind/moe.py:227-251 written with aten ops vs the fused pipeline."""
+@pytest.mark.parametrize("e,k", [(8, 2), (32, 10)])
+def test_moe_layer_matches_the_reference_expression(e, k):
+    """MoE.forward of forgemind/moe.py:227-251 written with aten ops vs the fused pipeline (also
+    with more than eight experts a token: no step of the layer leaves the library)."""
     g = torch.Generator().manual_seed(7)
-    n, d, e, k, h = 300, 64, 8, 2, 128
+    n, d, h = 300, 64, 128
     layer = fm.moe.MoE(d, h, e, k).to(DEV)
     x = torch.randn(n, d, generator=g).to(DEV).requires_grad_(True)
     kernels.reset_stats()
