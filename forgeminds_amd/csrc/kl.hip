@@ -792,9 +792,10 @@ bool launch_held_shape(const T* student, const T* teacher, float* lse_s, float* 
 
 // The shape by row width. 16-bit rows are bound by arithmetic, and a compute unit that holds
 // SEVERAL workgroups, each on a row of its own, keeps its vector ALUs busy while one of them waits
-// for memory or at its barrier: three 256-thread workgroups (13 + 3 slots: at most 168 registers
-// and 24 KB of LDS each) up to 4096 vectors a row, two (22 + 9 slots) up to 7936, one 512-thread
-// workgroup beyond. us for bf16 rows, three / two / one workgroup a unit: [8192,20000] 204 / 226 /
+// for memory or at its barrier: three 256-thread workgroups (13 + 3 slots, which hold 4096 vectors:
+// at most 168 registers and 24 KB of LDS each) for rows of up to 4608 vectors, two (22 + 9 slots,
+// 7936 vectors) up to 8192, one 512-thread workgroup beyond; what a row has past the slots is
+// streamed. us for bf16 rows, three / two / one workgroup a unit: [8192,20000] 204 / 226 /
 // 264, [16384,24576] 446 / 463 / 504, [16384,32000] 598 / 638 / 769, [8192,50304] 510 / 494 / 511,
 // [4096,65536] 344 / 325 / 325. fp32 rows are bound by bytes and run the same in every shape
 // ([8192,32000]: 588 / 576 / 568), so they take the one.
