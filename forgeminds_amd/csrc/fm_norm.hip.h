@@ -156,7 +156,13 @@ __global__ __launch_bounds__(BlockOf<TPR>::value) void norm_fwd_kernel(
 // ---------------------------------------------------------------- backward (vector path)
 // grid-persistent; `partial` is [gridDim.x, d] fp32 (LN: [gridDim.x, 2 d], weight then bias
 // columns), or NULL when the parameter gradients are not wanted.
-template <typename T, typename WT, int TPR, int ITERS, bool LN>
+// XCACHED: x is read with cached loads instead of streaming ones. x is the one operand a forward
+// (or a recompute of it) may have written just before, with cached stores, and a cached load finds
+// it in the L2 / the memory-side cache where a streaming load does not: add-RMSNorm pair at
+// [16384,8192] bf16 334 -> 325 us, [8192,1024] 21.1 -> 20.0; on an x that is NOT there it costs 1 %
+// (183 -> 185 us). Only for an x that fits that cache: on a larger one the loads of its first
+// rows push out the last rows before they are read ([32768,8192]: pair 696 -> 768 us).
+template <typename T, typename WT, int TPR, int ITERS, bool LN, bool XCACHED = false>
 __global__ __launch_bounds__(kBwdBlock) void norm_bwd_kernel(
     const T* __restrict__ x, const WT* __restrict__ w, const float* __restrict__ mean,
     const float* __restrict__ rstd, const T* __restrict__ dy, const T* __restrict__ gxn,
@@ -248,7 +254,8 @@ __global__ __launch_bounds__(kBwdBlock) void norm_bwd_kernel(
     for (int i = 0; i < ITERS; ++i) {
       const int c = i * TPR + t;
       if (valid && c < nvec) {
-        rx[i] = load16_stream(x + base + (int64_t)c * EPV);
+        if constexpr (XCACHED) rx[i] = load16(x + base + (int64_t)c * EPV);
+        else rx[i] = load16_stream(x + base + (int64_t)c * EPV);
         rg[i] = load16_stream(dy + base + (int64_t)c * EPV);
         if constexpr (EARLY_RES) {
           if (gxn != nullptr) rr[i] = load16_stream(gxn + base + (int64_t)c * EPV);
@@ -1118,11 +1125,18 @@ int launch_bwd(const Plan& p, const void* x, const void* w, const float* mean, c
     }
   } else {
     bool done = false;
+    // an x that fits the 256 MiB memory-side cache is read with cached loads (see the kernel)
+    const bool x_cached = n * d * (int64_t)sizeof(T) <= (256ll << 20);
 #define X(TPR_, IT_)                                                                           \
   if (!done && p.tpr == TPR_ && p.iters == IT_) {                                              \
-    FM_LAUNCH((norm_bwd_kernel<T, WT, TPR_, IT_, LN>), dim3((unsigned)p.bwd_blocks),  \
-                       dim3(kBwdBlock), 0, st, xp, wp, mean, rstd, dyp, gp, dxp, ddp,          \
-                       partial, n, (int)d, p.bwd_tiles);                                       \
+    if (x_cached)                                                                              \
+      FM_LAUNCH((norm_bwd_kernel<T, WT, TPR_, IT_, LN, true>), dim3((unsigned)p.bwd_blocks),   \
+                dim3(kBwdBlock), 0, st, xp, wp, mean, rstd, dyp, gp, dxp, ddp, partial, n, (int)d, \
+                p.bwd_tiles);                                                                  \
+    else                                                                                       \
+      FM_LAUNCH((norm_bwd_kernel<T, WT, TPR_, IT_, LN, false>), dim3((unsigned)p.bwd_blocks),  \
+                dim3(kBwdBlock), 0, st, xp, wp, mean, rstd, dyp, gp, dxp, ddp, partial, n, (int)d, \
+                p.bwd_tiles);                                                                  \
     done = true;                                                                               \
   }
     FM_FOR_EACH_SHAPE(X)
