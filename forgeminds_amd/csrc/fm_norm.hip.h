@@ -45,7 +45,10 @@ __device__ __forceinline__ void load_w(const WT* w, int col, float (&o)[Elem<T>:
 // Persistent over row tiles: the grid holds a few workgroups per compute unit, each keeps its
 // columns of w (and the bias) in registers and walks tiles blockIdx.x, blockIdx.x + gridDim.x, ...
 // so the parameters are fetched once per workgroup instead of once per row.
-template <typename T, typename WT, int TPR, int ITERS, bool ADD, bool LN>
+// XKEEP: x is read with cached loads so that it stays in the memory-side cache for the backward
+// (or a recompute's backward) that reads it again; the launcher sets it for a plain norm whose x
+// fits that cache. Not for the fused add: its backward reads xn, and x kept there only evicts it.
+template <typename T, typename WT, int TPR, int ITERS, bool ADD, bool LN, bool XKEEP = false>
 __global__ __launch_bounds__(BlockOf<TPR>::value) void norm_fwd_kernel(
     const T* __restrict__ x, const T* __restrict__ delta, const WT* __restrict__ w,
     const WT* __restrict__ bias, T* __restrict__ xn, T* __restrict__ y, float* __restrict__ mean,
@@ -95,7 +98,9 @@ __global__ __launch_bounds__(BlockOf<TPR>::value) void norm_fwd_kernel(
     for (int i = 0; i < ITERS; ++i) {
       const int c = i * TPR + t;
       if (valid && c < nvec) {
-        u32x4 rx = load16_stream(x + base + (int64_t)c * EPV);
+        u32x4 rx;
+        if constexpr (XKEEP) rx = load16(x + base + (int64_t)c * EPV);
+        else rx = load16_stream(x + base + (int64_t)c * EPV);
         Elem<T>::unpack(rx, v[i]);
         if constexpr (ADD) {
           float dv[EPV];
@@ -1039,20 +1044,25 @@ int launch_fwd(const Plan& p, const void* x, const void* delta, const void* w, c
                        wp, bp, xnp, yp, mean, rstd, d, eps);
     return FM_OK;
   }
+  // measured on fwd + bwd pairs of a plain RMSNorm (us, streamed | kept): 128 MiB 119.6 | 116.6,
+  // 256 MiB 229.8 | 219.7; the fused add at [16384,8192] bf16 loses 60 us when x is kept
+  const bool keep = !ADD && n * d * (int64_t)sizeof(T) <= (256ll << 20);
 #define X(TPR_, IT_)                                                                            \
   if (p.tpr == TPR_ && p.iters == IT_) {                                                        \
-    static int occupancy = 0; /* workgroups of this kernel one compute unit holds */            \
-    if (occupancy == 0) {                                                                       \
-      int o = 0;                                                                                \
-      if (hipOccupancyMaxActiveBlocksPerMultiprocessor(                                         \
-              &o, norm_fwd_kernel<T, WT, TPR_, IT_, ADD, LN>, BlockOf<TPR_>::value, 0) != hipSuccess || \
-          o < 1)                                                                                \
-        o = 2048 / BlockOf<TPR_>::value;                                                        \
-      occupancy = o;                                                                            \
+    constexpr int block_ = BlockOf<TPR_>::value;                                                \
+    if (keep) {                                                                                 \
+      constexpr auto kern_ = norm_fwd_kernel<T, WT, TPR_, IT_, ADD, LN, !ADD>;                  \
+      const int occ_ = fm_host::resident_per_cu<kern_>(block_, 0);                              \
+      FM_LAUNCH((norm_fwd_kernel<T, WT, TPR_, IT_, ADD, LN, !ADD>),                             \
+                dim3((unsigned)fwd_grid(p, occ_)), dim3(block_), 0, st, xp, dp, wp, bp, xnp, yp, \
+                mean, rstd, n, (int)d, eps, p.tiles);                                           \
+    } else {                                                                                    \
+      constexpr auto kern_ = norm_fwd_kernel<T, WT, TPR_, IT_, ADD, LN, false>;                 \
+      const int occ_ = fm_host::resident_per_cu<kern_>(block_, 0);                              \
+      FM_LAUNCH((norm_fwd_kernel<T, WT, TPR_, IT_, ADD, LN, false>),                            \
+                dim3((unsigned)fwd_grid(p, occ_)), dim3(block_), 0, st, xp, dp, wp, bp, xnp, yp, \
+                mean, rstd, n, (int)d, eps, p.tiles);                                           \
     }                                                                                           \
-    FM_LAUNCH((norm_fwd_kernel<T, WT, TPR_, IT_, ADD, LN>),                            \
-                       dim3((unsigned)fwd_grid(p, occupancy)), dim3(BlockOf<TPR_>::value), 0, st, \
-                       xp, dp, wp, bp, xnp, yp, mean, rstd, n, (int)d, eps, p.tiles);           \
     return FM_OK;                                                                               \
   }
   FM_FOR_EACH_SHAPE(X)
