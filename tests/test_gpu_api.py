@@ -252,7 +252,10 @@ def test_last_kernel_names_what_ran():
     x = torch.randn(64, 1024, device=DEV).bfloat16()
     w = torch.ones(1024, device=DEV)
     _hip.rmsnorm_fwd(x, w, 1e-6)
-    assert _hip.last_kernel() == "norm_fwd_kernel<bf16_t, float, 64, 2, false, false>"
+    # a plain norm's forward keeps x cached for its backward, the fused add streams it
+    assert _hip.last_kernel() == "norm_fwd_kernel<bf16_t, float, 64, 2, false, false, true>"
+    _hip.add_rmsnorm_fwd(x, x, w, 1e-6)
+    assert _hip.last_kernel() == "norm_fwd_kernel<bf16_t, float, 64, 2, true, false, false>"
     _hip.topk(torch.randn(8, 128256, device=DEV).bfloat16(), 64, torch.int32)
     assert _hip.last_kernel().startswith("topk_lds_kernel<bf16_t, ")
 
