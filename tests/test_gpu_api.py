@@ -294,6 +294,28 @@ def test_row_width_picks_the_form_that_was_measured_faster():
     assert norm_kernel(32768, f32, False) == "norm_bwd_wide_acc<float, float, false, 8, true, true>"
 
 
+def test_norm_reads_x_cached_only_when_it_fits_the_memory_side_cache():
+    """Forward and backward of a plain norm read x with cached loads up to 256 MiB of x and with
+    streaming loads beyond; both forms give the same numbers (the load kind is the only difference)."""
+    w = torch.ones(2048, device=DEV)
+    names, outs = [], []
+    for n in (65536, 65544):             # 256 MiB of bf16 x exactly, and eight rows more
+        x = torch.randn(n, 2048, device=DEV).bfloat16()
+        y, rstd = _hip.rmsnorm_fwd(x, w, 1e-6)
+        names.append(_hip.last_kernel())
+        dx, dw = _hip.rmsnorm_bwd(x, w, rstd, y)[:2]
+        torch.cuda.synchronize()
+        outs.append((x, y, rstd, dx, dw))
+    assert names[0].startswith("norm_fwd_kernel<bf16_t, float, ") and names[0].endswith(", false, false, true>")
+    assert names[1].startswith("norm_fwd_kernel<bf16_t, float, ") and names[1].endswith(", false, false, false>")
+    # the larger call on the first call's rows: bit-identical y and dx for those rows
+    x0, y0, r0, dx0, _ = outs[0]
+    xb = torch.cat([x0, outs[1][0][-8:]])
+    yb, rb = _hip.rmsnorm_fwd(xb, w, 1e-6)
+    dxb = _hip.rmsnorm_bwd(xb, w, rb, yb)[0]
+    assert torch.equal(yb[:65536], y0) and torch.equal(rb[:65536], r0) and torch.equal(dxb[:65536], dx0)
+
+
 def test_fp16_losses_apply_the_upstream_gradient_before_rounding():
     # a loss scaler multiplies the loss by 65536; (softmax - onehot) / 8192 rounded to fp16 FIRST
     # would lose most entries (p / 8192 < 6e-5 is subnormal or zero in fp16)
