@@ -87,7 +87,19 @@ __global__ __launch_bounds__(BlockOf<TPR>::value) void norm_fwd_kernel(
     }
   }
 
-  for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+  int64_t first = blockIdx.x;
+  {
+    // One tile per workgroup (small inputs): the tiles are dealt so that a row is handled here by
+    // the same eighth of the device (workgroup index mod 8, one L2 each) that reads it in the
+    // backward, whose tiles are G of these and go round the same way. What this launch leaves in
+    // that L2 -- x read with cached loads, or the xn it wrote -- is what the backward reads first.
+    constexpr int G = kBwdBlock / BLOCK;
+    if (G >= 1 && gridDim.x == tiles && tiles % (8 * G) == 0) {
+      const int64_t j = blockIdx.x >> 3;
+      first = ((j / G) * 8 + (blockIdx.x & 7)) * G + (j % G);
+    }
+  }
+  for (int64_t tile = first; tile < tiles; tile += gridDim.x) {
     const int64_t row = tile * RPB + rib;
     const bool valid = row < n;
     const int64_t base = row * (int64_t)d;
