@@ -55,49 +55,49 @@ METRIC = "HBM GB/s & % roofline: RMSNorm, CE/KL fwd+bwd; MoE top-k rows/s"
 # (profiles/all_workloads_hbm_traffic_pmc.txt). Each counter is scaled by what it reads for the
 # library's own 1 GiB copy (probe_copy_kernel, `bench.py --copy-probe 1024` under the same counters).
 # A kernel that is not in the table (a retune changed its template arguments) reports null.
-TRAFFIC_SCALE = (1048576.0 / 524299.6, 1048576.0 / 1049341.9)
+TRAFFIC_SCALE = (1048576.0 / 524299.5, 1048576.0 / 1049433.3)
 TRAFFIC_KIB = {
-    "ce_bwd_kernel<bf16_t, 1024, 4>": (244222.0, 512262.9),
-    "ce_fwd_kernel<bf16_t, 512, 4, false>": (125275.3, 250.1),
-    "ce_fwd_kernel<bf16_t, 512, 4, true>": (131370.3, 266.6),
-    "ce_loss_grad_held_kernel<bf16_t>": (487092.2, 1028436.1),
-    "ce_loss_grad_kernel<bf16_t, 512, 8>": (243962.6, 512523.1),
+    "ce_bwd_kernel<bf16_t, 1024, 4>": (244221.5, 512256.4),
+    "ce_fwd_kernel<bf16_t, 512, 4, false>": (125276.5, 250.2),
+    "ce_fwd_kernel<bf16_t, 512, 4, true>": (131369.4, 266.4),
+    "ce_loss_grad_held_kernel<bf16_t>": (487092.0, 1028560.3),
+    "ce_loss_grad_kernel<bf16_t, 512, 8>": (243962.6, 512526.3),
     "colsum16_kernel<bf16_t>": (4111.0, 8.0),
     "colsum16_kernel<float>": (1039.0, 4.0),
-    "colsum_kernel<float>": (8206.5, 64.0),
+    "colsum_kernel<float>": (8208.0, 64.0),
     "combine_kernel<bf16_t, true, 8>": (133142.6, 131072.0),
-    "kl_bwd_kernel<bf16_t, bf16_t, 1024, 8>": (1026898.1, 1026058.4),
-    "kl_fwd_kernel<bf16_t, 512, 4>": (1026892.5, 385.0),
-    "kl_fwd_topk_kernel<bf16_t, 512, 2, false>": (1054175.7, 2433.4),
-    "kl_fwd_topk_kernel<bf16_t, 512, 2, true>": (2057558.5, 1028505.5),
-    "kl_loss_grad_held_kernel<bf16_t, bf16_t, 512, 22, 9>": (1026392.3, 1026433.1),
-    "norm_bwd_kernel<bf16_t, bf16_t, 256, 2, false, true>": (65814.9, 69632.1),
+    "kl_bwd_kernel<bf16_t, bf16_t, 1024, 8>": (1026898.0, 1026058.2),
+    "kl_fwd_kernel<bf16_t, 512, 4>": (1026880.6, 385.0),
+    "kl_fwd_topk_kernel<bf16_t, 512, 2, false>": (1054177.5, 2433.6),
+    "kl_fwd_topk_kernel<bf16_t, 512, 2, true>": (2057727.9, 1028505.4),
+    "kl_loss_grad_held_kernel<bf16_t, bf16_t, 512, 22, 9>": (1026391.4, 1026433.1),
+    "norm_bwd_kernel<bf16_t, bf16_t, 256, 2, false, true>": (65831.7, 69632.3),
     "norm_bwd_kernel<bf16_t, float, 512, 2, false, true>": (393631.7, 270336.0),
     "norm_bwd_kernel<bf16_t, float, 512, 2, true, true>": (393894.8, 278528.0),
-    "norm_bwd_kernel<bf16_t, float, 64, 2, false, true>": (16461.6, 17408.3),
-    "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, false, false, true>": (32820.5, 65843.8),
-    "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, true, false, false>": (65592.1, 131370.3),
-    "norm_fwd_kernel<bf16_t, float, 512, 2, true, false, false>": (262295.8, 524844.1),
-    "norm_fwd_kernel<bf16_t, float, 512, 2, true, true, false>": (262429.3, 525342.9),
-    "norm_fwd_kernel<bf16_t, float, 64, 2, false, false, true>": (8223.1, 16457.5),
-    "permute_kernel": (1585.1, 10678.9),
+    "norm_bwd_kernel<bf16_t, float, 64, 2, false, true>": (16461.6, 17409.4),
+    "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, false, false, true>": (32821.0, 65842.9),
+    "norm_fwd_kernel<bf16_t, bf16_t, 256, 2, true, false, false>": (65592.6, 131367.7),
+    "norm_fwd_kernel<bf16_t, float, 512, 2, true, false, false>": (262296.8, 524857.6),
+    "norm_fwd_kernel<bf16_t, float, 512, 2, true, true, false>": (262429.8, 525351.4),
+    "norm_fwd_kernel<bf16_t, float, 64, 2, false, false, true>": (8227.1, 16427.0),
+    "permute_kernel": (1585.1, 10651.3),
     "probe_read_kernel": (524298.8, 0.0),
-    "rope_vec_kernel<bf16_t, float, 8, false, 2>": (105921.1, 213465.1),
-    "rope_vec_kernel<bf16_t, float, 8, true, 2>": (216510.7, 214220.4),
+    "rope_vec_kernel<bf16_t, float, 8, false, 2>": (105921.2, 213461.3),
+    "rope_vec_kernel<bf16_t, float, 8, true, 2>": (216510.7, 214218.1),
     "route_bwd_kernel<float, 8, true>": (2221.5, 4096.0),
-    "route_group_kernel<float, 32, true, 2, 8>": (32845.1, 6179.0),
-    "route_group_kernel<float, 8, true, 0, 8>": (2106.0, 328.6),
+    "route_group_kernel<float, 32, true, 2, 8>": (32845.1, 6179.1),
+    "route_group_kernel<float, 8, true, 0, 8>": (2106.0, 328.5),
     "route_scan_stats_kernel": (1893.5, 1026.0),
-    "scatter_kernel<bf16_t, true, 8>": (66084.2, 262269.7),
+    "scatter_kernel<bf16_t, true, 8>": (66084.3, 262270.8),
     "softmax_bwd_rows_kernel<bf16_t, 16, 1>": (2061.5, 2048.0),
-    "softmax_bwd_rows_kernel<bf16_t, 256, 2>": (65553.0, 65576.2),
+    "softmax_bwd_rows_kernel<bf16_t, 256, 2>": (65553.0, 65550.5),
     "softmax_rows_kernel<bf16_t, 16, 1>": (1039.6, 2048.0),
-    "softmax_rows_kernel<bf16_t, 256, 2>": (32788.6, 65596.7),
-    "swiglu_bwd_kernel<bf16_t, true>": (264214.2, 352257.8),
+    "softmax_rows_kernel<bf16_t, 256, 2>": (32788.6, 65609.7),
+    "swiglu_bwd_kernel<bf16_t, true>": (264214.2, 352258.0),
     "swiglu_fwd_kernel<bf16_t, true>": (176147.3, 176128.0),
     "swiglu_split_kernel<bf16_t, true, false>": (458770.2, 458752.1),
-    "swiglu_split_kernel<bf16_t, true, true>": (688148.5, 917505.7),
-    "topk_lds_kernel<bf16_t, 512, 4, 0>": (539854.7, 1024.0),
+    "swiglu_split_kernel<bf16_t, true, true>": (688148.5, 917505.8),
+    "topk_lds_kernel<bf16_t, 512, 4, 0>": (539853.8, 1024.0),
 }
 TRAFFIC_SOURCE = "profiles/all_workloads_hbm_traffic_pmc.txt"
 
