@@ -73,6 +73,10 @@ NORM_CASES = [
     # sums in registers; more rows than workgroups, uneven chunks
     (700, 18432, BF16, F32, 1e-6), (513, 28672, F32, F32, 1e-6), (257, 32768, F16, F16, 1e-5),
     (300, 16392, BF16, BF16, 1e-6),
+    # one tile per workgroup and a tile count the forward can deal by L2 (a multiple of eight
+    # backward tiles): workgroups of 256, 512 and 1024 threads, one to many rounds
+    (96, 4096, BF16, F32, 1e-6), (16, 16384, BF16, BF16, 1e-6), (48, 8192, F32, F32, 1e-6),
+    (2048, 256, BF16, F32, 1e-6), (4096, 512, F16, F16, 1e-5),
 ]
 
 
@@ -129,7 +133,10 @@ def test_rmsnorm_unaligned_views_take_the_any_width_path():
 ADD_CASES = [(256, 8192, BF16, F32, 1e-5), (9, 24, F32, F32, 1e-6), (10, 33, BF16, BF16, 1e-6),
              (6, 8, F32, F32, 1e-6), (5, 7, F32, F32, 1e-6), (40, 4096, F16, F16, 1e-5),
              (12, 2048, BF16, F32, 1e-5), (7, 40960, BF16, F32, 1e-5), (5, 20480, F32, F32, 1e-6),
-             (260, 24576, F16, F16, 1e-5)]
+             (260, 24576, F16, F16, 1e-5),
+             # tile counts the forward deals by L2
+             (96, 4096, BF16, F32, 1e-5), (16, 16384, BF16, BF16, 1e-5), (4096, 512, F16, F16, 1e-5),
+             (48, 8192, F32, F32, 1e-6)]
 
 
 @pytest.mark.parametrize("n,d,dt,wdt,eps", ADD_CASES)
@@ -166,6 +173,8 @@ LN_CASES = [
     (5, 40960, BF16, F32, 1e-5, True), (3, 65536, F16, F16, 1e-5, False), (6, 20480, F32, F32, 1e-5, True),
     (270, 32768, BF16, BF16, 1e-5, True), (700, 18432, BF16, F32, 1e-5, True), (300, 24576, F32, F32, 1e-5, True),
     (260, 32768, F32, F32, 1e-5, True),
+    # tile counts the forward deals by L2
+    (96, 4096, BF16, F32, 1e-5, True), (48, 8192, F32, F32, 1e-5, True), (2048, 256, BF16, F32, 1e-5, False),
 ]
 
 
@@ -205,7 +214,7 @@ def test_layernorm_fwd_bwd(n, d, dt, wdt, eps, bias):
 
 @pytest.mark.parametrize("n,d,dt,wdt", [(128, 8192, BF16, F32), (9, 24, F32, F32), (10, 33, BF16, BF16),
                                         (40, 4096, F16, F16), (12, 2048, BF16, F32), (6, 40960, BF16, F32),
-                                        (4, 24576, F32, F32)])
+                                        (4, 24576, F32, F32), (96, 4096, BF16, F32), (1024, 1024, BF16, BF16)])
 def test_add_layernorm_fwd_bwd(n, d, dt, wdt):
     g = gen(1034)
     x = torch.randn(n, d, generator=g).to(dt)
